@@ -1,0 +1,142 @@
+"""The cache on the device: keys and values per run-order entry, per-slot state.
+
+Entries of the run order with the same needs (kv heads, head size, window, dtype)
+form a group; each group has storage, a page pool and block tables of its own:
+``K, V: [entry in group, page, kv head, position in page, head_dim]``. A page is
+``page_size`` positions of one sequence for every entry of the group. Beside it
+each entry may own a state area of fixed size per slot, ``[slot, elements]``,
+zeroed when the slot is handed out; the attention of this architecture asks for
+none (the reference has no such state either: J/inference/state/State.java:28-65).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from .pages import CacheFull, PagePool, SlotTable
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """What one run-order entry stores per position."""
+    n_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """What one run-order entry stores per sequence, whatever its length."""
+    elements: int
+    dtype: torch.dtype = torch.float32
+
+
+class CacheGroup:
+    def __init__(self, need, entries, n_pages, page_size, dtype, device):
+        self.need = need
+        self.entries = list(entries)
+        self.pool = PagePool(n_pages)
+        self.page_size = page_size
+        shape = (len(self.entries), n_pages, need.n_kv_heads, page_size, need.head_dim)
+        self.k = torch.zeros(shape, dtype=dtype, device=device)
+        self.v = torch.zeros(shape, dtype=dtype, device=device)
+
+
+class Cache:
+    """``kv_needs[e]`` / ``state_needs[e]`` give run-order entry e's needs (None: nothing).
+
+    ``max_tokens``: positions that all live sequences may hold together, each
+    sequence's count rounded up to whole pages. ``max_context``: longest sequence.
+    """
+
+    def __init__(self, kv_needs, state_needs, max_tokens, max_context, n_slots, dtype, device, page_size=64):
+        if max_tokens < 1 or max_context < 1 or n_slots < 1:
+            raise ValueError("cache sizes must be positive")
+        self.page_size = page_size
+        self.max_context = max_context
+        self.max_pages_per_seq = -(-max_context // page_size)
+        self.dtype = dtype
+        self.device = device
+        n_pages = -(-max_tokens // page_size) + 1           # + the sink page
+        self.groups = []
+        self.group_of = {}                                   # entry -> (group index, index inside the group)
+        by_need = {}
+        for e, need in enumerate(kv_needs):
+            if need is not None:
+                by_need.setdefault(need, []).append(e)
+        for need, entries in by_need.items():
+            g = CacheGroup(need, entries, n_pages, page_size, dtype, device)
+            for i, e in enumerate(entries):
+                self.group_of[e] = (len(self.groups), i)
+            self.groups.append(g)
+        self.slots = SlotTable(n_slots, len(self.groups))
+        self.state = {}
+        for e, need in enumerate(state_needs):
+            if need is not None and need.elements > 0:
+                self.state[e] = torch.zeros((n_slots, need.elements), dtype=need.dtype, device=device)
+
+    # ---- slots
+    def take_slot(self):
+        s = self.slots.take()
+        for t in self.state.values():
+            t[s].zero_()
+        return s
+
+    def give_back_slot(self, s):
+        self.slots.check(s)
+        for g, group in enumerate(self.groups):
+            group.pool.give_back(self.slots.pages[s][g])
+            self.slots.pages[s][g] = []
+        self.slots.give_back(s)
+
+    def length(self, s):
+        self.slots.check(s)
+        return self.slots.length[s]
+
+    def reserve(self, wanted):
+        """Make room for ``{slot: n new tokens}`` in every group, or change nothing."""
+        plan = []
+        for s, n in wanted.items():
+            self.slots.check(s)
+            new_len = self.slots.length[s] + n
+            if new_len > self.max_context:
+                raise CacheFull(f"slot {s}: {new_len} tokens exceed the longest sequence of {self.max_context}")
+            need_pages = -(-new_len // self.page_size)
+            for g in range(len(self.groups)):
+                plan.append((s, g, need_pages - len(self.slots.pages[s][g])))
+        for g, group in enumerate(self.groups):
+            total = sum(extra for _, gg, extra in plan if gg == g and extra > 0)
+            if total > group.pool.n_free:
+                raise CacheFull(f"{total} more pages wanted, {group.pool.n_free} free: the cache holds "
+                                f"{(group.pool.n_pages - 1) * self.page_size} tokens")
+        for s, g, extra in plan:
+            if extra > 0:
+                self.slots.pages[s][g].extend(self.groups[g].pool.take(extra))
+
+    def advance(self, s, n):
+        self.slots.length[s] += n
+
+    # ---- what the kernels read
+    def layer_kv(self, entry):
+        """(K, V) of one entry: [page, kv head, position in page, head_dim]."""
+        g, i = self.group_of[entry]
+        return self.groups[g].k[i], self.groups[g].v[i]
+
+    def group_index(self, entry):
+        return self.group_of[entry][0]
+
+    def block_rows(self, group, slots, width):
+        """Rows of page numbers for ``slots``, padded with the sink page."""
+        rows = []
+        for s in slots:
+            p = self.slots.pages[s][group]
+            rows.append(p + [0] * (width - len(p)))
+        return rows
+
+    def slot_state(self, entry):
+        return self.state.get(entry)
+
+    def tokens_free(self):
+        return min((g.pool.n_free for g in self.groups), default=0) * self.page_size

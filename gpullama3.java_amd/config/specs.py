@@ -1,0 +1,103 @@
+"""Descriptions of model parts as plain data.
+
+A model is described without any tensor: a list of block descriptions (each
+naming its norm, mixer and feed-forward with every size and constant), the order
+in which the blocks run, and the names under which each part's tensors are
+stored. The parts of ``parts/`` are built from these and from nothing else, so
+no part knows which architecture it serves.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional
+
+
+@dataclass(frozen=True)
+class Llama3RopeScaling:
+    """Frequency scaling of long wavelengths (the reference fixes the four numbers in
+    code, J/model/loader/ModelLoader.java:235-239; here they come from config.json)."""
+    factor: float
+    low_freq_factor: float
+    high_freq_factor: float
+    original_max_position: int
+
+
+@dataclass(frozen=True)
+class RotarySpec:
+    """Rotary position encoding of queries and keys."""
+    kind: str = "rotary"
+    head_dim: int = 0
+    theta: float = 10000.0
+    scaling: Optional[Llama3RopeScaling] = None
+    pairing: str = "half"        # "half": (j, j + hs/2); "adjacent": (2j, 2j+1)
+    max_positions: int = 0
+
+
+@dataclass(frozen=True)
+class NormSpec:
+    kind: str = "rmsnorm"
+    dim: int = 0
+    eps: float = 1e-5
+    names: dict = field(default_factory=dict)     # local tensor name -> stored name
+
+
+@dataclass(frozen=True)
+class AttentionSpec:
+    """Causal grouped-query attention over a cache of keys and values."""
+    kind: str = "attention"
+    hidden: int = 0
+    n_heads: int = 0
+    n_kv_heads: int = 0
+    head_dim: int = 0
+    position: Optional[RotarySpec] = None
+    window: Optional[int] = None      # None: every earlier key; n: the last n keys
+    scale: Optional[float] = None     # None: 1/sqrt(head_dim)
+    names: dict = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class GatedFeedForwardSpec:
+    """down(act(gate(x)) * up(x))."""
+    kind: str = "gated"
+    hidden: int = 0
+    intermediate: int = 0
+    activation: str = "silu"
+    names: dict = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class BlockSpec:
+    """One layer: how norm, mixer and feed-forward are arranged is ``kind``."""
+    kind: str = "prenorm"             # x += mixer(norm(x)); x += ffn(norm(x))
+    mixer_norm: object = None
+    mixer: object = None
+    ffn_norm: object = None
+    ffn: object = None
+
+
+@dataclass(frozen=True)
+class Run:
+    """One entry of the run order.
+
+    ``layer`` indexes ``ModelSpec.layers``. A layer may be named by several
+    entries; each entry then has storage of its own in the cache, unless
+    ``reads`` names an earlier entry of the run order, whose keys and values this
+    entry reads instead of making its own.
+    """
+    layer: int
+    reads: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    architecture: str
+    vocab_size: int
+    hidden: int
+    layers: tuple
+    run_order: tuple
+    final_norm: object
+    max_positions: int
+    tie_embeddings: bool
+    embedding_name: str
+    head_name: Optional[str]          # None when tied
+    stop_ids: tuple = ()

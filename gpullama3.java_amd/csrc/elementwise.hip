@@ -1,0 +1,146 @@
+// Embedding gather, RMSNorm and rotary encoding fused with the cache write.
+// Statistics and rotation are computed in 32-bit whatever the storage type.
+#include "common.h"
+
+// ----------------------------------------------------------------- embedding
+// out[t, :] = table[ids[t], :] as float (J/inference/InferenceCore.java:69).
+template <typename TW>
+__global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out, int d) {
+  const long t = blockIdx.x;
+  const TW* row = table + (long)ids[t] * d;
+  float* o = out + t * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = to_f32<TW>(row[i]);
+}
+
+extern "C" int gl3_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens, int d,
+                         hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(table && ids && out && n_tokens > 0 && d > 0, "gl3_embed: bad arguments (T=%d d=%d)", n_tokens, d);
+  dim3 grid(n_tokens), block(256);
+  if (table_dtype == GL3_F32) embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, ids, out, d);
+  else if (table_dtype == GL3_BF16) embed_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)table, ids, out, d);
+  else GL3_REQUIRE(false, "gl3_embed: unknown dtype %d", table_dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- rmsnorm
+// out[r, i] = w[i] * (ss * x[row(r), i]),  ss = 1/sqrt(mean(x^2) + eps)
+// (J/inference/InferenceCore.java:47-56). One block per row; `rows` (may be
+// null) picks the rows of x that are normalised, so that the final norm runs on
+// the wanted positions only. The order of the sum depends on d alone.
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows, const TW* __restrict__ w,
+                               TO* __restrict__ out, int d, float eps) {
+  __shared__ float scratch[16];
+  const long r = blockIdx.x;
+  const long src = rows ? rows[r] : r;
+  const float* xr = x + src * d;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float v = xr[i];
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  ss = ss / (float)d;
+  ss = ss + eps;
+  ss = 1.0f / sqrtf(ss);
+  TO* o = out + r * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_f32<TO>(to_f32<TW>(w[i]) * (ss * xr[i]));
+}
+
+extern "C" int gl3_rmsnorm(const float* x, const int* rows, const void* w, int w_dtype, void* out, int out_dtype,
+                           int n_rows, int d, float eps, hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  GL3_REQUIRE(x && w && out && n_rows > 0 && d > 0, "gl3_rmsnorm: bad arguments (rows=%d d=%d)", n_rows, d);
+  dim3 grid(n_rows), block(256);
+#define GO(TW, TO) rmsnorm_kernel<TW, TO><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, d, eps)
+  if (w_dtype == GL3_F32 && out_dtype == GL3_F32) GO(float, float);
+  else if (w_dtype == GL3_F32 && out_dtype == GL3_BF16) GO(float, bf16_t);
+  else if (w_dtype == GL3_BF16 && out_dtype == GL3_F32) GO(bf16_t, float);
+  else if (w_dtype == GL3_BF16 && out_dtype == GL3_BF16) GO(bf16_t, bf16_t);
+  else GL3_REQUIRE(false, "gl3_rmsnorm: unknown dtypes %d %d", w_dtype, out_dtype);
+#undef GO
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- rotary + cache write
+// qkv[t] holds [n_heads q heads | n_kv k heads | n_kv v heads], each of head_dim.
+// Queries are rotated in place; keys are rotated and written to the paged key
+// cache, values are copied to the value cache (rotation before the write, so
+// cached keys are already rotated: J/inference/InferenceCore.java:83-101).
+// Pair j of a head is (2j, 2j+1) for adjacent pairing, (j, j + rot/2) for
+// half pairing; the angle's cos and sin come from a table [position, rot/2]
+// built on the host (J/inference/operation/RoPE.java:29-31). Elements beyond
+// `rot_dim` pass through. A null table means no rotation at all.
+// The cache of one layer is [page][kv head][slot in page][head_dim]; the page of
+// position p of sequence s is block_table[s * table_stride + p / page_size].
+template <typename T>
+__global__ void rope_cache_kernel(T* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                                  const int* __restrict__ block_table, int table_stride, const float* __restrict__ cos_tab,
+                                  const float* __restrict__ sin_tab, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                  int n_heads, int n_kv, int head_dim, int rot_dim, int adjacent, int page_size,
+                                  int write_kv) {
+  const int t = blockIdx.x;
+  const int head = blockIdx.y;  // [0,H): q, [H,H+K): k, [H+K,H+2K): v
+  const int pos = positions[t];
+  const long row = (long)t * (n_heads + 2 * n_kv) * head_dim;
+  T* src = qkv + row + (long)head * head_dim;
+  const int half = rot_dim / 2;
+  T* dst = src;
+  if (head >= n_heads) {
+    if (!write_kv) return;
+    const int c = (head - n_heads) % n_kv;
+    const int page = block_table[(long)seq_of_token[t] * table_stride + pos / page_size];
+    T* base = (head < n_heads + n_kv) ? k_cache : v_cache;
+    dst = base + (((long)page * n_kv + c) * page_size + pos % page_size) * head_dim;
+  }
+  const bool rotate = cos_tab != nullptr && head < n_heads + n_kv;
+  if (!rotate) {
+    if (dst != src)
+      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
+    return;
+  }
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    const int i0 = adjacent ? 2 * j : j;
+    const int i1 = adjacent ? 2 * j + 1 : j + half;
+    const float c = cos_tab[(long)pos * half + j], s = sin_tab[(long)pos * half + j];
+    const float v0 = to_f32<T>(src[i0]), v1 = to_f32<T>(src[i1]);
+    dst[i0] = from_f32<T>(v0 * c - v1 * s);
+    dst[i1] = from_f32<T>(v0 * s + v1 * c);
+  }
+  if (dst != src)
+    for (int i = rot_dim + threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
+}
+
+extern "C" int gl3_rope_cache_write(void* qkv, int dtype, const int* positions, const int* seq_of_token,
+                                    const int* block_table, int table_stride, const float* cos_tab,
+                                    const float* sin_tab, void* k_cache, void* v_cache, int n_tokens, int n_heads,
+                                    int n_kv, int head_dim, int rot_dim, int adjacent, int page_size, int write_kv,
+                                    hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  GL3_REQUIRE(qkv && positions && n_tokens > 0 && n_heads > 0 && n_kv > 0 && head_dim > 0,
+              "gl3_rope_cache_write: bad arguments");
+  GL3_REQUIRE(rot_dim >= 0 && rot_dim <= head_dim && rot_dim % 2 == 0, "gl3_rope_cache_write: rot_dim %d of head_dim %d",
+              rot_dim, head_dim);
+  GL3_REQUIRE((cos_tab == nullptr) == (sin_tab == nullptr), "gl3_rope_cache_write: one table without the other");
+  if (write_kv)
+    GL3_REQUIRE(k_cache && v_cache && block_table && seq_of_token && page_size > 0 && table_stride > 0,
+                "gl3_rope_cache_write: cache arguments missing");
+  const int heads = write_kv ? n_heads + 2 * n_kv : n_heads;
+  GL3_REQUIRE(heads <= 65535, "gl3_rope_cache_write: %d heads exceed the grid", heads);
+  dim3 grid(n_tokens, heads), block(64);
+  if (dtype == GL3_F32)
+    rope_cache_kernel<float><<<grid, block, 0, stream>>>((float*)qkv, positions, seq_of_token, block_table, table_stride,
+                                                         cos_tab, sin_tab, (float*)k_cache, (float*)v_cache, n_heads, n_kv,
+                                                         head_dim, rot_dim, adjacent, page_size, write_kv);
+  else if (dtype == GL3_BF16)
+    rope_cache_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)qkv, positions, seq_of_token, block_table,
+                                                          table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
+                                                          (bf16_t*)v_cache, n_heads, n_kv, head_dim, rot_dim, adjacent,
+                                                          page_size, write_kv);
+  else GL3_REQUIRE(false, "gl3_rope_cache_write: unknown dtype %d", dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,130 @@
+// C[M,N] = A[M,K] . W[N,K]^T for any sizes and any mix of float / bfloat16
+// operands, with 32-bit multiply-adds only (no matrix-core, no reduced-precision
+// mode): the true 32-bit path of the model and the fallback for shapes that the
+// matrix-core kernels refuse. W is row-major [out, in] as the reference's matmul
+// reads it (J/core/model/tensor/FloatTensor.java:98-100).
+//
+// Every output element is the sum over k = 0..K-1 in ascending order, one
+// multiply-add per k, whatever M is and wherever the row sits in its tile: a
+// token's result does not depend on how many tokens share the step.
+//
+// Epilogues: store (as float or bfloat16), add into a float matrix in place (the
+// residual stream; the reference fuses the same, TransformerComputeKernelsLayered
+// .java:766-784), and gated: W holds [gate rows | up rows] and the kernel writes
+// silu(gate) * up (J/inference/InferenceCore.java:158-166).
+#include "common.h"
+
+#define GT 64   // tile edge
+#define GK 16   // k step
+
+enum { EPI_STORE = 0, EPI_ADD = 1, EPI_GATED = 2 };
+
+template <typename TA, typename TW, typename TC, int EPI>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
+                                                            TC* __restrict__ C, int M, int N, int K, long lda,
+                                                            long ldw, long ldc, long up_offset) {
+  // N is the number of output columns; for EPI_GATED the up rows of W start at
+  // row `up_offset`.
+  __shared__ float As[GK][GT + 1];
+  __shared__ float Ws[GK][GT + 1];
+  __shared__ float Us[EPI == EPI_GATED ? GK : 1][GT + 1];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;  // 16 x 16 threads, 4 x 4 outputs each
+  const long m0 = (long)blockIdx.y * GT, n0 = (long)blockIdx.x * GT;
+  float acc[4][4] = {};
+  float accu[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += GK) {
+    // 64 x 16 elements per operand, 4 per thread; consecutive threads read along k
+    for (int e = tid; e < GT * GK; e += 256) {
+      const int r = e / GK, kk = e % GK;
+      const int k = k0 + kk;
+      float a = 0.f, w = 0.f, u = 0.f;
+      if (k < K) {
+        if (m0 + r < M) a = to_f32<TA>(A[(m0 + r) * lda + k]);
+        if (n0 + r < N) {
+          w = to_f32<TW>(W[(n0 + r) * ldw + k]);
+          if (EPI == EPI_GATED) u = to_f32<TW>(W[(up_offset + n0 + r) * ldw + k]);
+        }
+      }
+      As[kk][r] = a;
+      Ws[kk][r] = w;
+      if (EPI == EPI_GATED) Us[kk][r] = u;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GK; ++kk) {
+      float a[4], w[4], u[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx * 4 + j];
+      if (EPI == EPI_GATED) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) u[j] = Us[kk][tx * 4 + j];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+          if (EPI == EPI_GATED) accu[i][j] = fmaf(a[i], u[j], accu[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const long m = m0 + ty * 4 + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const long n = n0 + tx * 4 + j;
+      if (n >= N) continue;
+      float v = acc[i][j];
+      if (EPI == EPI_GATED) {
+        v = v / (1.0f + expf(-v));
+        v = v * accu[i][j];
+      }
+      TC* c = C + m * ldc + n;
+      if (EPI == EPI_ADD) *c = from_f32<TC>(to_f32<TC>(*c) + v);
+      else *c = from_f32<TC>(v);
+    }
+  }
+}
+
+template <typename TA, typename TW, typename TC>
+static int launch_generic(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
+                          int epi, hipStream_t stream) {
+  dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT), block(256);
+  GL3_REQUIRE(grid.y <= 65535, "gl3_gemm_generic: M=%d is too large for one launch", M);
+  const TA* a = (const TA*)A;
+  const TW* w = (const TW*)W;
+  TC* c = (TC*)C;
+  if (epi == EPI_STORE) gemm_generic_kernel<TA, TW, TC, EPI_STORE><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0);
+  else if (epi == EPI_ADD) gemm_generic_kernel<TA, TW, TC, EPI_ADD><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0);
+  else gemm_generic_kernel<TA, TW, TC, EPI_GATED><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, N);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// N counts output columns: for the gated epilogue W has 2N rows (gate, then up).
+extern "C" int gl3_gemm_generic(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M,
+                                int N, int K, long lda, long ldw, long ldc, int epilogue, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_generic: bad arguments (M=%d N=%d K=%d)", M, N, K);
+  GL3_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gl3_gemm_generic: leading dimensions %ld %ld %ld too small", lda, ldw, ldc);
+  GL3_REQUIRE(epilogue >= 0 && epilogue <= 2, "gl3_gemm_generic: unknown epilogue %d", epilogue);
+  GL3_REQUIRE(epilogue != EPI_ADD || c_dtype == GL3_F32, "gl3_gemm_generic: the add epilogue needs a float output");
+  const int key = a_dtype * 4 + w_dtype * 2 + c_dtype;
+  switch (key) {
+    case 0: return launch_generic<float, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
+    case 2: return launch_generic<float, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
+    case 4: return launch_generic<bf16_t, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
+    case 5: return launch_generic<bf16_t, float, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
+    case 6: return launch_generic<bf16_t, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
+    case 7: return launch_generic<bf16_t, bf16_t, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
+    default:
+      GL3_REQUIRE(false, "gl3_gemm_generic: unsupported dtypes A=%d W=%d C=%d", a_dtype, w_dtype, c_dtype);
+  }
+  return 0;
+}

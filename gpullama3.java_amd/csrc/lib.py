@@ -1,0 +1,213 @@
+"""ctypes bindings of the HIP library, with the host-side checks every launch needs.
+
+Each wrapper checks, before anything reaches the GPU, that its tensors live on the
+device, are contiguous where the kernel assumes it, have the dtypes and shapes the
+kernel's indexing assumes, and that index tensors are int32. There is no CPU
+fallback: without a GPU, or without the library, the call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_uint32, c_void_p
+
+import torch
+
+from . import build as _build
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+EPI_STORE, EPI_ADD, EPI_GATED = 0, 1, 2
+
+_lib = None
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def library():
+    """The loaded library; built first if no build matches the sources."""
+    global _lib
+    if _lib is None:
+        path = _build.library_path() or _build.build()
+        lib = ctypes.CDLL(path)
+        lib.gl3_last_error.restype = ctypes.c_char_p
+        _declare(lib)
+        _lib = lib
+    return _lib
+
+
+def library_file():
+    library()
+    return _build.library_path()
+
+
+def _declare(lib):
+    P, I, L, F = c_void_p, c_int, c_long, c_float
+    sigs = {
+        "gl3_abi_version": [],
+        "gl3_fill_u32": [P, c_uint32, L, P],
+        "gl3_embed": [P, I, P, P, I, I, P],
+        "gl3_rmsnorm": [P, P, P, I, P, I, I, I, F, P],
+        "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
+        "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P],
+        "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
+        "gl3_sample": [P, L, P, P, P, P, P, I, I, P],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name, None)
+        if fn is None:
+            continue
+        fn.argtypes = args
+        fn.restype = c_int
+    lib._optional = set()
+
+
+def has(name):
+    return hasattr(library(), name)
+
+
+def _check(rc, name):
+    if rc != 0:
+        raise KernelError(f"{name}: {library().gl3_last_error().decode()}")
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(t, name, dtype=None, contiguous=True):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name} must be a tensor on the GPU (the kernels have no CPU path)")
+    if dtype is not None and t.dtype not in (dtype if isinstance(dtype, tuple) else (dtype,)):
+        raise KernelError(f"{name} has dtype {t.dtype}, expected {dtype}")
+    if contiguous and not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    return t
+
+
+def _code(t, name):
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise KernelError(f"{name} has dtype {t.dtype}; the kernels take float32 and bfloat16") from None
+
+
+def _ptr(t):
+    return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
+
+
+# ------------------------------------------------------------------ ops
+def fill_u32(t, value):
+    _dev(t, "tensor")
+    if t.element_size() * t.numel() % 4:
+        raise KernelError("fill_u32 needs a multiple of 4 bytes")
+    _check(library().gl3_fill_u32(_ptr(t), value, t.element_size() * t.numel() // 4, _stream()), "fill_u32")
+
+
+def embed(table, ids, out):
+    """out[t] = table[ids[t]] as float32. The caller has checked ids < rows."""
+    _dev(table, "table"); _dev(ids, "ids", torch.int32); _dev(out, "out", torch.float32)
+    T, d = out.shape
+    if table.dim() != 2 or table.shape[1] != d or ids.numel() != T:
+        raise KernelError(f"embed: table {tuple(table.shape)}, ids {tuple(ids.shape)}, out {tuple(out.shape)}")
+    _check(library().gl3_embed(_ptr(table), _code(table, "table"), _ptr(ids), _ptr(out), T, d, _stream()), "embed")
+
+
+def rmsnorm(x, weight, out, eps, rows=None):
+    """out[r] = weight * x[rows[r]] / rms (rows None: every row in order)."""
+    _dev(x, "x", torch.float32); _dev(weight, "weight"); _dev(out, "out")
+    d = x.shape[-1]
+    n = out.shape[0]
+    if x.dim() != 2 or out.dim() != 2 or out.shape[1] != d or weight.shape != (d,):
+        raise KernelError(f"rmsnorm: x {tuple(x.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+    if rows is not None:
+        _dev(rows, "rows", torch.int32)
+        if rows.numel() != n:
+            raise KernelError(f"rmsnorm: {rows.numel()} rows for {n} outputs")
+    elif x.shape[0] != n:
+        raise KernelError(f"rmsnorm: {x.shape[0]} inputs for {n} outputs")
+    _check(library().gl3_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _code(weight, "weight"), _ptr(out),
+                                 _code(out, "out"), n, d, float(eps), _stream()), "rmsnorm")
+
+
+def rope_cache_write(qkv, positions, seq_of_token, block_table, cos, sin, k_cache, v_cache, n_heads, n_kv,
+                     head_dim, rot_dim, adjacent, page_size, write_kv=True):
+    """Rotate q (in place) and k, and write k and v into one layer's paged cache.
+
+    qkv [T, (H+2K)*hs] (or [T, H*hs] when ``write_kv`` is false); caches
+    [pages, K, page_size, hs]; block_table [B, width] int32.
+    """
+    _dev(qkv, "qkv"); _dev(positions, "positions", torch.int32)
+    T = qkv.shape[0]
+    width = (n_heads + (2 * n_kv if write_kv else 0)) * head_dim
+    if qkv.dim() != 2 or qkv.shape[1] != width or positions.numel() != T:
+        raise KernelError(f"rope_cache_write: qkv {tuple(qkv.shape)} for {n_heads}+2*{n_kv} heads of {head_dim}")
+    if cos is not None:
+        _dev(cos, "cos", torch.float32); _dev(sin, "sin", torch.float32)
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != rot_dim // 2:
+            raise KernelError(f"rope_cache_write: table {tuple(cos.shape)} for rot_dim {rot_dim}")
+    stride = 0
+    if write_kv:
+        _dev(seq_of_token, "seq_of_token", torch.int32); _dev(block_table, "block_table", torch.int32)
+        _dev(k_cache, "k_cache", qkv.dtype); _dev(v_cache, "v_cache", qkv.dtype)
+        if seq_of_token.numel() != T or block_table.dim() != 2:
+            raise KernelError("rope_cache_write: seq_of_token / block_table shapes")
+        if k_cache.shape != v_cache.shape or k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim):
+            raise KernelError(f"rope_cache_write: cache {tuple(k_cache.shape)} for kv {n_kv} page {page_size} hs {head_dim}")
+        stride = block_table.shape[1]
+    _check(library().gl3_rope_cache_write(
+        _ptr(qkv), _code(qkv, "qkv"), _ptr(positions), _ptr(seq_of_token), _ptr(block_table), stride,
+        _ptr(cos), _ptr(sin), _ptr(k_cache), _ptr(v_cache), T, n_heads, n_kv, head_dim, rot_dim, int(adjacent),
+        page_size, int(write_kv), _stream()), "rope_cache_write")
+
+
+def gemm_generic(a, w, out, epilogue=EPI_STORE):
+    """out = a @ w.T with float multiply-adds; see gemm_generic.hip for the epilogues.
+    ``a`` and ``out`` may be row-strided views (last dimension contiguous)."""
+    _dev(a, "a", contiguous=False); _dev(w, "w"); _dev(out, "out", contiguous=False)
+    if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
+    M, K = a.shape
+    N = out.shape[1]
+    rows = 2 * N if epilogue == EPI_GATED else N
+    if w.shape != (rows, K) or out.shape[0] != M:
+        raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
+    _check(library().gl3_gemm_generic(_ptr(a), _code(a, "a"), _ptr(w), _code(w, "w"), _ptr(out), _code(out, "out"),
+                                      M, N, K, a.stride(0), w.stride(0), out.stride(0), epilogue, _stream()),
+           "gemm_generic")
+
+
+def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,
+                      page_size, window, scale):
+    """q: a [T, >= H*hs] view whose first H*hs columns of each row are the queries."""
+    _dev(q, "q", contiguous=False); _dev(out, "out", contiguous=False)
+    _dev(k_cache, "k_cache", q.dtype); _dev(v_cache, "v_cache", q.dtype)
+    _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
+    _dev(block_table, "block_table", torch.int32)
+    T = q.shape[0]
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < n_heads * head_dim or out.dtype != q.dtype:
+        raise KernelError(f"attention: q {tuple(q.shape)} for {n_heads} heads of {head_dim}")
+    if out.shape != (T, n_heads * head_dim) or out.stride(1) != 1:
+        raise KernelError(f"attention: out {tuple(out.shape)}")
+    if k_cache.shape != v_cache.shape or k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim):
+        raise KernelError(f"attention: cache {tuple(k_cache.shape)} for kv {n_kv} page {page_size} hs {head_dim}")
+    if positions.numel() != T or seq_of_token.numel() != T or block_table.dim() != 2:
+        raise KernelError("attention: positions / seq_of_token / block_table shapes")
+    _check(library().gl3_attention_generic(
+        _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _code(q, "q"), _ptr(positions), _ptr(seq_of_token),
+        _ptr(block_table), block_table.shape[1], _ptr(out), out.stride(0), T, n_heads, n_kv, head_dim, page_size,
+        int(window or 0), float(scale), _stream()), "attention_generic")
+
+
+def sample(logits, work, temperature, top_p, uniform, out):
+    _dev(logits, "logits", torch.float32, contiguous=False); _dev(work, "work", torch.float32)
+    for t, n in ((temperature, "temperature"), (top_p, "top_p"), (uniform, "uniform")):
+        _dev(t, n, torch.float32)
+    _dev(out, "out", torch.int32)
+    R, V = logits.shape
+    if logits.stride(1) != 1 or work.numel() < R * V or min(temperature.numel(), top_p.numel(), uniform.numel(),
+                                                              out.numel()) < R:
+        raise KernelError("sample: argument sizes")
+    _check(library().gl3_sample(_ptr(logits), logits.stride(0), _ptr(work), _ptr(temperature), _ptr(top_p),
+                                _ptr(uniform), _ptr(out), R, V, _stream()), "sample")

@@ -1,0 +1,62 @@
+"""What a step looks like to the parts: the packed tokens of a batch and where each
+belongs.
+
+All index arrays are int32 on the device: ``token_ids[T]``, ``positions[T]`` (a
+token's place in its own sequence), ``seq_of_token[T]`` (which row of the batch),
+``cu_seqlens[B+1]``, ``kv_before[B]`` (tokens a sequence held before this step),
+and one block table ``[B, width]`` per cache group. Host copies of the lengths are
+kept for launch decisions.
+"""
+from __future__ import annotations
+
+import torch
+
+
+class Workspace:
+    """Named scratch buffers that keep their address from step to step."""
+
+    def __init__(self, device):
+        self.device = device
+        self._flat = {}
+        self.frozen = False
+
+    def get(self, name, shape, dtype):
+        n = 1
+        for s in shape:
+            n *= s
+        key = (name, dtype)
+        flat = self._flat.get(key)
+        if flat is None or flat.numel() < n:
+            if self.frozen:
+                raise RuntimeError(f"workspace buffer {name!r} would grow while its address is fixed")
+            flat = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._flat[key] = flat
+        return flat[:n].view(shape)
+
+
+class StepContext:
+    def __init__(self, engine, n_tokens, n_seqs, q_lens, kv_before_host, slots, decode, max_q_len, max_kv_len):
+        self.engine = engine
+        self.cache = engine.cache
+        self.dtype = engine.dtype
+        self.device = engine.device
+        self.n_tokens, self.n_seqs = n_tokens, n_seqs
+        self.q_lens, self.kv_before_host, self.slots = q_lens, kv_before_host, slots
+        self.decode = decode
+        self.max_q_len, self.max_kv_len = max_q_len, max_kv_len
+        self.token_ids = self.positions = self.seq_of_token = self.cu_seqlens = self.kv_before = None
+        self.slot_ids = None
+        self._tables = []
+
+    def block_table(self, group):
+        return self._tables[group]
+
+    def buffer(self, name, shape, dtype):
+        return self.engine.workspace.get(name, shape, dtype)
+
+    def logits_buffer(self, n_rows, vocab):
+        return torch.empty((n_rows, vocab), dtype=torch.float32, device=self.device)
+
+    def slot_state(self, entry):
+        """``[n_slots, elements]`` state of one run-order entry; index with ``slot_ids``."""
+        return self.cache.slot_state(entry)

@@ -1,0 +1,157 @@
+"""The generation loop above the step function.
+
+The reference's loop serves one sequence: it feeds the prompt one token per
+forward pass, then samples, reports and checks stop tokens until the position
+bound (J/inference/InferenceEngine.java:83-131, GPU twin :278-366). Here requests
+are served in batches that start together: the prompts of a batch go through one
+step, then every live sequence gets one token per step; a sequence that ends
+leaves the batch and gives its slot back at once; when a batch has ended the next
+requests form the next one. Once a batch has started no request joins it.
+
+The loop only decides; the model is behind ``backend``:
+``take_slot()``, ``give_back_slot(slot)``, ``step(entries) -> logits handle`` (last
+row of each entry), ``sample(logits, temperatures, top_ps, uniforms) -> ids``,
+``max_context``, ``page_size``, ``tokens_capacity()``, ``n_slots``.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, Optional, Sequence
+
+from ..sampling import SamplingParams, uniform
+
+
+@dataclass
+class Request:
+    prompt: Sequence[int]
+    max_new_tokens: int
+    sampling: SamplingParams = SamplingParams()
+    stop_ids: frozenset = frozenset()
+
+
+@dataclass
+class Generated:
+    tokens: list = field(default_factory=list)      # generated ids only, a stop token included
+    finish_reason: Optional[str] = None             # "stop" | "length"
+
+
+@dataclass
+class RunMetrics:
+    """Prompt and generated tokens with their times, kept apart; the reference reports
+    one figure over both (J/auxiliary/LastRunMetrics.java:27-31)."""
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    prefill_seconds: float = 0.0
+    decode_seconds: float = 0.0
+    decode_steps: int = 0
+
+    @property
+    def total_tokens_per_second(self):
+        t = self.prefill_seconds + self.decode_seconds
+        return (self.prompt_tokens + self.generated_tokens) / t if t > 0 else 0.0
+
+
+def _rounded(n, page):
+    return -(-n // page) * page
+
+
+def plan_batch(requests, first, max_batch, capacity, page_size, max_context):
+    """How many requests from ``first`` on form the next batch: as many as there are
+    slots, and as their longest possible lengths fit into the cache together."""
+    held, n = 0, 0
+    for r in requests[first:first + max_batch]:
+        longest = min(len(r.prompt) + max(r.max_new_tokens - 1, 0), max_context)
+        need = _rounded(max(longest, 1), page_size)
+        if held + need > capacity:
+            break
+        held += need
+        n += 1
+    if n == 0:
+        r = requests[first]
+        raise ValueError(f"request {first} may hold {len(r.prompt)} + {r.max_new_tokens} tokens; "
+                         f"the cache holds {capacity}")
+    return n
+
+
+def generate(backend, requests, on_token: Optional[Callable[[int, int], None]] = None, max_batch=None,
+             metrics: Optional[RunMetrics] = None):
+    """Serve ``requests`` and return a ``Generated`` per request, in request order."""
+    for i, r in enumerate(requests):
+        if len(r.prompt) == 0:
+            raise ValueError(f"request {i} has an empty prompt")
+        if len(r.prompt) > backend.max_context:
+            raise ValueError(f"request {i}: a prompt of {len(r.prompt)} tokens exceeds the context of "
+                             f"{backend.max_context}")
+    results = [Generated() for _ in requests]
+    metrics = metrics if metrics is not None else RunMetrics()
+    max_batch = min(max_batch or backend.n_slots, backend.n_slots)
+    first = 0
+    while first < len(requests):
+        n = plan_batch(requests, first, max_batch, backend.tokens_capacity(), backend.page_size,
+                       backend.max_context)
+        _run_batch(backend, requests, results, range(first, first + n), on_token, metrics)
+        first += n
+    return results
+
+
+def _run_batch(backend, requests, results, ids, on_token, metrics):
+    live = []                     # (request index, slot), in request order
+    try:
+        for i in ids:
+            if requests[i].max_new_tokens <= 0:
+                results[i].finish_reason = "length"
+                continue
+            live.append((i, backend.take_slot()))
+        if not live:
+            return
+        held = {i: len(requests[i].prompt) for i, _ in live}
+        t0 = time.perf_counter()
+        logits = backend.step([(slot, list(requests[i].prompt)) for i, slot in live])
+        step_no = 0
+        prefill = True
+        while live:
+            rows = [i for i, _ in live]
+            ids_out = backend.sample(
+                logits,
+                [requests[i].sampling.temperature for i in rows],
+                [requests[i].sampling.top_p for i in rows],
+                [uniform(requests[i].sampling.seed, i, len(results[i].tokens)) for i in rows])
+            dt = time.perf_counter() - t0
+            if prefill:
+                metrics.prefill_seconds += dt
+                metrics.prompt_tokens += sum(len(requests[i].prompt) for i in rows)
+                prefill = False
+            else:
+                metrics.decode_seconds += dt
+                metrics.decode_steps += 1
+            t0 = time.perf_counter()
+            nxt = []
+            for (i, slot), tok in zip(live, ids_out):
+                r, out = requests[i], results[i]
+                out.tokens.append(int(tok))
+                metrics.generated_tokens += 1
+                if on_token is not None:
+                    on_token(i, int(tok))
+                if int(tok) in r.stop_ids:
+                    out.finish_reason = "stop"       # the stop token is part of the result
+                elif len(out.tokens) >= r.max_new_tokens or held[i] >= backend.max_context:
+                    out.finish_reason = "length"     # no room to feed this token back
+                if out.finish_reason is not None:
+                    backend.give_back_slot(slot)
+                else:
+                    nxt.append((i, slot))
+            live = nxt
+            if not live:
+                break
+            logits = backend.step([(slot, [results[i].tokens[-1]]) for i, slot in live])
+            for i, _ in live:
+                held[i] += 1
+            step_no += 1
+    except BaseException:
+        for _, slot in live:
+            try:
+                backend.give_back_slot(slot)
+            except Exception:
+                pass
+        raise

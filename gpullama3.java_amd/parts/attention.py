@@ -1,0 +1,76 @@
+"""Causal grouped-query attention over the paged cache.
+
+Order as the reference's layer (J/inference/InferenceCore.java:78-151): q, k, v
+projections (one product over the three matrices stacked by rows), rotation of q
+and k, cache write at the token's position, attention over positions lo..p of the
+token's own sequence, output projection added into the residual stream.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..cache import KVNeed
+from ..csrc import lib as K
+from ..weights.loader import TensorSpec
+from . import ops
+from .base import build_part, register_part
+
+
+class GQAAttention:
+    def __init__(self, spec, dtype, device):
+        self.spec, self.dtype = spec, dtype
+        self.d, self.H, self.Kh, self.hs = spec.hidden, spec.n_heads, spec.n_kv_heads, spec.head_dim
+        if self.H % self.Kh:
+            raise ValueError(f"{self.H} heads are not a multiple of {self.Kh} kv heads")
+        self.window = spec.window
+        self.scale = spec.scale if spec.scale is not None else 1.0 / math.sqrt(self.hs)
+        self.position = build_part("position", spec.position, device=device) if spec.position is not None else None
+        self.names = spec.names
+        self.w_qkv = self.w_q = self.w_o = None
+
+    def tensors(self):
+        n, d, hs = self.names, self.d, self.hs
+        return {n["q"]: TensorSpec((self.H * hs, d)), n["k"]: TensorSpec((self.Kh * hs, d)),
+                n["v"]: TensorSpec((self.Kh * hs, d)), n["o"]: TensorSpec((d, self.H * hs))}
+
+    def load(self, weights):
+        n = self.names
+        parts = [weights[n["q"]], weights[n["k"]], weights[n["v"]]]
+        dt = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
+        self.w_qkv = torch.cat([p.to(dt) for p in parts], dim=0).contiguous()
+        qn, kn = self.H * self.hs, self.Kh * self.hs
+        # the stored names stay addressable as views of the stacked matrix
+        weights[n["q"]], weights[n["k"]], weights[n["v"]] = (
+            self.w_qkv[:qn], self.w_qkv[qn:qn + kn], self.w_qkv[qn + kn:])
+        self.w_q = self.w_qkv[:qn]
+        self.w_o = weights[n["o"]]
+
+    def kv_need(self):
+        return KVNeed(self.Kh, self.hs, self.window)
+
+    def state_need(self):
+        return None
+
+    def forward(self, ctx, h, x, run):
+        T, H, Kh, hs = h.shape[0], self.H, self.Kh, self.hs
+        k_cache, v_cache = ctx.cache.layer_kv(run.kv_entry)
+        table = ctx.block_table(ctx.cache.group_index(run.kv_entry))
+        pos = self.position
+        if run.writes_kv:
+            qkv = ctx.buffer("qkv", (T, (H + 2 * Kh) * hs), self.dtype)
+            ops.linear(h, self.w_qkv, qkv)
+        else:
+            qkv = ctx.buffer("qkv", (T, H * hs), self.dtype)
+            ops.linear(h, self.w_q, qkv)
+        K.rope_cache_write(qkv, ctx.positions, ctx.seq_of_token, table,
+                           pos.cos if pos else None, pos.sin if pos else None, k_cache, v_cache,
+                           H, Kh, hs, pos.rot_dim if pos else 0, pos.adjacent if pos else False,
+                           ctx.cache.page_size, write_kv=run.writes_kv)
+        att = ctx.buffer("attn_out", (T, H * hs), self.dtype)
+        ops.attention(ctx, qkv, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale)
+        ops.linear(att, self.w_o, x, ops.EPI_ADD)
+
+
+register_part("mixer", "attention", GQAAttention)

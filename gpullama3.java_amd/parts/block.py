@@ -1,0 +1,29 @@
+"""A layer: the arrangement of norm, mixer and feed-forward.
+
+``prenorm`` is the reference's: the normalised copy feeds the mixer, the residual
+stream keeps the sum (J/inference/InferenceCore.java:74, :151, :154, :172).
+"""
+from __future__ import annotations
+
+from .base import build_part, register_part
+
+
+class PreNormBlock:
+    def __init__(self, spec, dtype, device):
+        self.mixer_norm = build_part("norm", spec.mixer_norm, dtype=dtype)
+        self.mixer = build_part("mixer", spec.mixer, dtype=dtype, device=device)
+        self.ffn_norm = build_part("norm", spec.ffn_norm, dtype=dtype) if spec.ffn is not None else None
+        self.ffn = build_part("ffn", spec.ffn, dtype=dtype, device=device) if spec.ffn is not None else None
+
+    def parts(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+
+    def forward(self, ctx, x, run):
+        h = self.mixer_norm(ctx, x)
+        self.mixer.forward(ctx, h, x, run)
+        if self.ffn is not None:
+            h = self.ffn_norm(ctx, x)
+            self.ffn.forward(ctx, h, x)
+
+
+register_part("block", "prenorm", PreNormBlock)

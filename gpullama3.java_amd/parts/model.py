@@ -1,0 +1,89 @@
+"""The decoder: embedding, blocks in their run order, final norm, head.
+
+Built from a ``ModelSpec`` alone. The run order is data: an entry names a layer
+(possibly one already named) and, optionally, an earlier entry whose keys and
+values it reads instead of making its own.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..csrc import lib as K
+from ..weights.loader import TensorSpec
+from . import ops
+from .base import RunInfo, build_part
+
+
+def expected_tensors(spec, dtype=torch.float32, device="cpu"):
+    """Stored name -> TensorSpec of every tensor the model needs (no memory is used)."""
+    out = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden))}
+    if spec.head_name is not None:
+        out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden))
+    out.update(_norm_tensors(spec.final_norm))
+    for b in spec.layers:
+        block = build_part("block", b, dtype=dtype, device=device)
+        for p in block.parts():
+            out.update(p.tensors())
+    return out
+
+
+def _norm_tensors(spec):
+    return build_part("norm", spec, dtype=torch.float32).tensors()
+
+
+class DecoderModel:
+    def __init__(self, spec, dtype, device):
+        self.spec, self.dtype, self.device = spec, dtype, device
+        self.blocks = [build_part("block", b, dtype=dtype, device=device) for b in spec.layers]
+        self.final_norm = build_part("norm", spec.final_norm, dtype=dtype)
+        self.runs = []
+        for e, r in enumerate(spec.run_order):
+            if not 0 <= r.layer < len(self.blocks):
+                raise ValueError(f"run order entry {e} names layer {r.layer} of {len(self.blocks)}")
+            if r.reads is not None and not (0 <= r.reads < e and spec.run_order[r.reads].reads is None):
+                raise ValueError(f"run order entry {e} reads entry {r.reads}, which is not an earlier entry "
+                                 "with keys and values of its own")
+            self.runs.append(RunInfo(entry=e, kv_entry=e if r.reads is None else r.reads,
+                                     writes_kv=r.reads is None))
+        self.embedding = self.head = None
+        self.weights = {}
+
+    def expected(self):
+        out = {self.spec.embedding_name: TensorSpec((self.spec.vocab_size, self.spec.hidden))}
+        if self.spec.head_name is not None:
+            out[self.spec.head_name] = TensorSpec((self.spec.vocab_size, self.spec.hidden))
+        out.update(self.final_norm.tensors())
+        for b in self.blocks:
+            for p in b.parts():
+                out.update(p.tensors())
+        return out
+
+    def load(self, weights):
+        self.weights = weights
+        self.embedding = weights[self.spec.embedding_name]
+        self.head = self.embedding if self.spec.head_name is None else weights[self.spec.head_name]
+        self.final_norm.load(weights)
+        for b in self.blocks:
+            for p in b.parts():
+                p.load(weights)
+
+    def cache_needs(self):
+        kv, state = [], []
+        for run, r in zip(self.runs, self.spec.run_order):
+            mixer = self.blocks[r.layer].mixer
+            kv.append(mixer.kv_need() if run.writes_kv else None)
+            state.append(mixer.state_need())
+        return kv, state
+
+    def forward(self, ctx, want_rows):
+        """Logits ``[len(want_rows), vocab]`` float32 at the wanted packed rows."""
+        x = ctx.buffer("residual", (ctx.n_tokens, self.spec.hidden), torch.float32)
+        K.embed(self.embedding, ctx.token_ids, x)
+        for run, r in zip(self.runs, self.spec.run_order):
+            self.blocks[r.layer].forward(ctx, x, run)
+        n = want_rows.numel()
+        logits = ctx.logits_buffer(n, self.spec.vocab_size)
+        if n:
+            h = self.final_norm(ctx, x, rows=want_rows, name="final_normed")
+            ops.linear(h, self.head, logits)
+        return logits
