@@ -1,0 +1,125 @@
+"""The cache's bookkeeping: no slot or page lost, held twice or freed twice (no GPU)."""
+import random
+
+import pytest
+import torch
+
+from gpullama3_java_amd.cache import Cache, CacheFull, KVNeed, PagePool, SlotTable, StateNeed
+
+
+def test_page_pool():
+    pool = PagePool(5)
+    a = pool.take(3)
+    assert 0 not in a and len(set(a)) == 3 and pool.n_free == 1
+    with pytest.raises(CacheFull):
+        pool.take(2)
+    assert pool.n_free == 1                                   # a refused request takes nothing
+    pool.give_back(a[:2])
+    with pytest.raises(RuntimeError):
+        pool.give_back(a[:1])                                 # freed twice
+    with pytest.raises(RuntimeError):
+        pool.give_back([0])                                   # the sink page is never held
+    assert pool.n_free == 3
+
+
+def test_slot_table():
+    st = SlotTable(3, 1)
+    s = [st.take() for _ in range(3)]
+    assert sorted(s) == [0, 1, 2]
+    with pytest.raises(CacheFull):
+        st.take()
+    st.give_back(s[1])
+    with pytest.raises(RuntimeError):
+        st.give_back(s[1])
+    assert st.take() == s[1]                                  # given back, used again
+
+
+def make(max_tokens=640, max_context=256, n_slots=4, needs=None, state=None):
+    needs = needs or [KVNeed(2, 16), KVNeed(2, 16), KVNeed(1, 32, window=8)]
+    state = state or [None, StateNeed(6), None]
+    return Cache(needs, state, max_tokens, max_context, n_slots, torch.float32, "cpu", page_size=64)
+
+
+def test_groups_have_storage_of_their_own():
+    c = make()
+    assert len(c.groups) == 2
+    assert c.groups[0].k.shape == (2, 11, 2, 64, 16) and c.groups[1].k.shape == (1, 11, 1, 64, 32)
+    assert c.group_of == {0: (0, 0), 1: (0, 1), 2: (1, 0)}
+    k, v = c.layer_kv(1)
+    assert k.shape == (11, 2, 64, 16) and k.data_ptr() == c.groups[0].k[1].data_ptr()
+    assert c.slot_state(1).shape == (4, 6) and c.slot_state(0) is None
+
+
+def test_reserve_is_all_or_nothing():
+    c = make()
+    a, b = c.take_slot(), c.take_slot()
+    c.reserve({a: 100, b: 10})
+    c.advance(a, 100); c.advance(b, 10)
+    third = c.take_slot()
+    c.reserve({third: 200}); c.advance(third, 200)             # 4 of the 10 pages
+    assert len(c.slots.pages[a][0]) == 2 and len(c.slots.pages[a][1]) == 2 and len(c.slots.pages[b][0]) == 1
+    free = [g.pool.n_free for g in c.groups]
+    with pytest.raises(CacheFull, match="longest"):
+        c.reserve({a: 1, b: 300})                             # b would pass max_context
+    with pytest.raises(CacheFull, match="pages"):
+        c.reserve({a: 156, b: 246})                           # 2 + 3 more pages, 3 are free
+    assert [g.pool.n_free for g in c.groups] == free and c.length(a) == 100
+    c.reserve({a: 28})                                        # fits the pages already held
+    assert [g.pool.n_free for g in c.groups] == free
+    with pytest.raises(RuntimeError):
+        c.reserve({3: 1})                                     # a slot nobody holds
+
+
+def test_state_is_zeroed_when_a_slot_is_handed_out():
+    c = make()
+    s = c.take_slot()
+    c.slot_state(1)[s] = 5.0
+    c.give_back_slot(s)
+    s2 = c.take_slot()
+    assert s2 == s and torch.all(c.slot_state(1)[s2] == 0)
+
+
+def test_random_traffic_keeps_the_books():
+    rng = random.Random(0)
+    c = make(max_tokens=64 * 12, max_context=300, n_slots=5)
+    total_pages = [g.pool.n_pages - 1 for g in c.groups]
+    live = {}
+    for _ in range(2000):
+        op = rng.random()
+        if op < 0.3 and len(live) < 5:
+            live[c.take_slot()] = 0
+        elif op < 0.8 and live:
+            s = rng.choice(list(live))
+            n = rng.randint(1, 90)
+            try:
+                c.reserve({s: n})
+                c.advance(s, n)
+                live[s] += n
+            except CacheFull:
+                pass
+        elif live:
+            s = rng.choice(list(live))
+            c.give_back_slot(s)
+            del live[s]
+            with pytest.raises(RuntimeError):
+                c.give_back_slot(s)
+        # the books: every page is free or held by exactly one live slot; lengths fit their pages
+        for g, group in enumerate(c.groups):
+            held = [p for s in live for p in c.slots.pages[s][g]]
+            assert len(held) == len(set(held)) and 0 not in held
+            assert len(held) + group.pool.n_free == total_pages[g]
+            assert set(held) == group.pool._held
+        for s, n in live.items():
+            assert c.length(s) == n and all(len(c.slots.pages[s][g]) == -(-n // 64) for g in range(2))
+        assert set(live) == c.slots.live and len(live) + len(c.slots._free) == 5
+    for s in list(live):
+        c.give_back_slot(s)
+    assert all(g.pool.n_free == t for g, t in zip(c.groups, total_pages))
+
+
+def test_block_rows_pad_with_the_sink():
+    c = make()
+    a = c.take_slot()
+    c.reserve({a: 70})
+    rows = c.block_rows(0, [a], 4)
+    assert rows[0][:2] == c.slots.pages[a][0] and rows[0][2:] == [0, 0]

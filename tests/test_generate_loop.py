@@ -1,0 +1,174 @@
+"""The generation loop's decisions, with a backend that needs no GPU."""
+import numpy as np
+import pytest
+
+import plain_llama as P
+from gpullama3_java_amd.cache import Cache, CacheFull, KVNeed
+from gpullama3_java_amd.engine.generate import Request, RunMetrics, generate, plan_batch
+from gpullama3_java_amd.sampling import SamplingParams, sample_host, uniform
+
+V = 50
+
+
+class FakeBackend:
+    """Logits are a fixed function of a sequence's tokens, so every request has one
+    right answer whatever it is batched with. The real cache does the bookkeeping."""
+
+    def __init__(self, max_tokens=1024, max_context=64, n_slots=4):
+        import torch
+        self.cache = Cache([KVNeed(1, 2)], [None], max_tokens, max_context, n_slots, torch.float32, "cpu", 16)
+        self.max_context, self.n_slots, self.page_size = max_context, n_slots, 16
+        self.seqs = {}
+        self.steps = []          # per step: list of (slot, n tokens)
+        self.taken = []
+
+    def tokens_capacity(self):
+        return self.cache.tokens_free()
+
+    def take_slot(self):
+        s = self.cache.take_slot()
+        assert s not in self.seqs
+        self.seqs[s] = []
+        self.taken.append(s)
+        return s
+
+    def give_back_slot(self, s):
+        self.cache.give_back_slot(s)
+        del self.seqs[s]
+
+    @staticmethod
+    def logits_of(seq):
+        rng = np.random.default_rng([len(seq), sum(seq) % 9973, seq[-1]])
+        return rng.standard_normal(V).astype(np.float32) * 3
+
+    def step(self, entries):
+        self.cache.reserve({s: len(t) for s, t in entries})
+        rows = []
+        for s, toks in entries:
+            self.cache.advance(s, len(toks))
+            self.seqs[s].extend(toks)
+            rows.append(self.logits_of(self.seqs[s]))
+        self.steps.append([(s, len(t)) for s, t in entries])
+        return np.stack(rows)
+
+    def sample(self, logits, temperatures, top_ps, uniforms):
+        return [sample_host(l, t, p, u) for l, t, p, u in zip(logits, temperatures, top_ps, uniforms)]
+
+
+def alone(prompt, n, sampling=SamplingParams(), stops=(), index=0, max_context=64):
+    seq, out = list(prompt), []
+    while len(out) < n:
+        tok = P.sample(FakeBackend.logits_of(seq), sampling.temperature, sampling.top_p,
+                       uniform(sampling.seed, index, len(out)))
+        out.append(tok)
+        if tok in stops or len(seq) >= max_context:
+            break
+        seq.append(tok)
+    return out
+
+
+def prompts(lens, seed=0):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, V, n).tolist() for n in lens]
+
+
+def test_unequal_prompts_in_one_step_then_one_token_each():
+    be = FakeBackend()
+    ps = prompts([5, 11, 3])
+    res = generate(be, [Request(p, 6) for p in ps])
+    assert [r.tokens for r in res] == [alone(p, 6) for p in ps]
+    assert all(r.finish_reason == "length" for r in res)
+    assert sorted(n for _, n in be.steps[0]) == [3, 5, 11]                 # whole prompts, one step
+    assert all(n == 1 for st in be.steps[1:] for _, n in st) and len(be.steps) == 6
+    assert not be.seqs and be.cache.slots.live == set()                    # every slot came back
+
+
+def test_stop_token_ends_only_its_own_sequence_and_is_kept():
+    be = FakeBackend()
+    ps = prompts([4, 9, 6], seed=1)
+    free_run = [alone(p, 12) for p in ps]
+    stop = free_run[1][3]                                # request 1 meets it at its 4th token (or earlier)
+    res = generate(be, [Request(p, 12, stop_ids=frozenset([stop])) for p in ps])
+    for r, p in zip(res, ps):
+        want = alone(p, 12, stops=(stop,))
+        assert r.tokens == want
+        assert r.finish_reason == ("stop" if want[-1] == stop else "length")
+    assert res[1].tokens[-1] == stop and len(res[1].tokens) <= 4
+    # a stop token inside a prompt stops nothing
+    res2 = generate(FakeBackend(), [Request([stop, stop] + ps[0], 3)])
+    assert len(res2[0].tokens) >= 1 and res2[0].tokens == alone([stop, stop] + ps[0], 3)
+
+
+def test_finished_sequences_leave_the_batch_at_once():
+    be = FakeBackend()
+    ps = prompts([4, 4, 4], seed=2)
+    res = generate(be, [Request(ps[0], 2), Request(ps[1], 7), Request(ps[2], 4)])
+    assert [len(r.tokens) for r in res] == [2, 7, 4]
+    assert [len(st) for st in be.steps] == [3, 3, 2, 2, 1, 1, 1]
+
+
+def test_batches_follow_one_another_and_slots_are_used_again():
+    be = FakeBackend(n_slots=2)
+    ps = prompts([3, 8, 5, 2, 7], seed=3)
+    res = generate(be, [Request(p, 4) for p in ps])
+    assert [r.tokens for r in res] == [alone(p, 4, index=i) for i, p in enumerate(ps)]   # request order kept
+    assert len(be.taken) == 5 and set(be.taken) == {0, 1}                  # five requests over two slots
+    assert [len(st) for st in be.steps if st[0][1] > 1 or len(st) > 0][0] == 2
+    firsts = [st for st in be.steps if any(n > 1 for _, n in st)]
+    assert [len(st) for st in firsts] == [2, 2, 1]                         # nobody joins a running batch
+
+
+def test_batch_is_cut_by_the_cache_size():
+    reqs = [Request([1] * 20, 13), Request([1] * 20, 13), Request([1] * 5, 4)]
+    assert plan_batch(reqs, 0, 8, capacity=64, page_size=16, max_context=64) == 2     # 32 + 32 tokens
+    assert plan_batch(reqs, 0, 1, capacity=640, page_size=16, max_context=64) == 1
+    assert plan_batch(reqs, 2, 8, capacity=16, page_size=16, max_context=64) == 1
+    with pytest.raises(ValueError, match="cache holds"):
+        plan_batch(reqs, 0, 8, capacity=16, page_size=16, max_context=64)
+    be = FakeBackend(max_tokens=64, n_slots=4)
+    res = generate(be, reqs)
+    assert [len(r.tokens) for r in res] == [13, 13, 4]
+
+
+def test_context_bound_and_bad_prompts():
+    be = FakeBackend(max_context=16)
+    p = prompts([14], seed=4)[0]
+    res = generate(be, [Request(p, 10)])
+    # 14 held; tokens 1 and 2 are fed back (15, 16 held); the third is sampled but cannot be fed
+    assert len(res[0].tokens) == 3 and res[0].finish_reason == "length"
+    assert res[0].tokens == alone(p, 10, max_context=16)[:3]
+    full = prompts([16], seed=5)[0]
+    assert len(generate(FakeBackend(max_context=16), [Request(full, 5)])[0].tokens) == 1
+    with pytest.raises(ValueError, match="exceeds the context"):
+        generate(be, [Request([1] * 17, 1)])
+    with pytest.raises(ValueError, match="empty"):
+        generate(be, [Request([], 1)])
+    assert generate(be, [Request(p, 0)])[0].tokens == []
+    assert be.cache.slots.live == set()
+
+
+def test_sampled_tokens_do_not_depend_on_batch_mates():
+    sp = SamplingParams(0.8, 0.95, seed=7)
+    ps = prompts([6, 3, 9], seed=6)
+    together = generate(FakeBackend(), [Request(p, 8, sp) for p in ps])
+    for i, p in enumerate(ps):
+        assert together[i].tokens == alone(p, 8, sp, index=i)
+    other = generate(FakeBackend(), [Request(p, 8, SamplingParams(0.8, 0.95, seed=8)) for p in ps])
+    assert [r.tokens for r in other] != [r.tokens for r in together]
+
+
+def test_callback_and_metrics():
+    seen = []
+    m = RunMetrics()
+    ps = prompts([4, 6], seed=8)
+    res = generate(FakeBackend(), [Request(p, 3) for p in ps], on_token=lambda i, t: seen.append((i, t)), metrics=m)
+    assert [t for i, t in seen if i == 0] == res[0].tokens and [t for i, t in seen if i == 1] == res[1].tokens
+    assert m.prompt_tokens == 10 and m.generated_tokens == 6 and m.decode_steps == 2
+
+
+def test_a_failing_step_gives_the_slots_back():
+    be = FakeBackend(max_tokens=32, n_slots=4)
+    be.tokens_capacity = lambda: 10**6          # let the plan through so that the step itself fails
+    with pytest.raises(CacheFull):
+        generate(be, [Request([1] * 30, 2), Request([1] * 30, 2)])
+    assert be.cache.slots.live == set() and be.cache.groups[0].pool.n_free == 2
