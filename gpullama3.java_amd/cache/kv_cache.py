@@ -139,4 +139,7 @@ class Cache:
         return self.state.get(entry)
 
     def tokens_free(self):
-        return min((g.pool.n_free for g in self.groups), default=0) * self.page_size
+        """Positions that can still be handed out (no per-position storage: no bound but the slots)."""
+        if not self.groups:
+            return self.slots.n_slots * self.max_context
+        return min(g.pool.n_free for g in self.groups) * self.page_size

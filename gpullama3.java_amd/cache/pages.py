@@ -55,6 +55,10 @@ class SlotTable:
         self.length = [0] * n_slots
         self.pages = [[[] for _ in range(n_groups)] for _ in range(n_slots)]
 
+    @property
+    def n_free(self):
+        return len(self._free)
+
     def take(self):
         if not self._free:
             raise CacheFull(f"all {self.n_slots} slots are held")

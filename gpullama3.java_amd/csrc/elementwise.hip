@@ -81,11 +81,11 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const int* __restrict__ p
                                   const int* __restrict__ block_table, int table_stride, const float* __restrict__ cos_tab,
                                   const float* __restrict__ sin_tab, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   int n_heads, int n_kv, int head_dim, int rot_dim, int adjacent, int page_size,
-                                  int write_kv) {
+                                  int write_kv, long row_stride) {
   const int t = blockIdx.x;
   const int head = blockIdx.y;  // [0,H): q, [H,H+K): k, [H+K,H+2K): v
   const int pos = positions[t];
-  const long row = (long)t * (n_heads + 2 * n_kv) * head_dim;
+  const long row = (long)t * row_stride;
   T* src = qkv + row + (long)head * head_dim;
   const int half = rot_dim / 2;
   T* dst = src;
@@ -128,18 +128,19 @@ extern "C" int gl3_rope_cache_write(void* qkv, int dtype, const int* positions, 
   if (write_kv)
     GL3_REQUIRE(k_cache && v_cache && block_table && seq_of_token && page_size > 0 && table_stride > 0,
                 "gl3_rope_cache_write: cache arguments missing");
-  const int heads = write_kv ? n_heads + 2 * n_kv : n_heads;
+  const int heads = write_kv ? n_heads + 2 * n_kv : n_heads;   // without the write a row holds queries only
+  const long row_stride = (long)heads * head_dim;
   GL3_REQUIRE(heads <= 65535, "gl3_rope_cache_write: %d heads exceed the grid", heads);
   dim3 grid(n_tokens, heads), block(64);
   if (dtype == GL3_F32)
     rope_cache_kernel<float><<<grid, block, 0, stream>>>((float*)qkv, positions, seq_of_token, block_table, table_stride,
                                                          cos_tab, sin_tab, (float*)k_cache, (float*)v_cache, n_heads, n_kv,
-                                                         head_dim, rot_dim, adjacent, page_size, write_kv);
+                                                         head_dim, rot_dim, adjacent, page_size, write_kv, row_stride);
   else if (dtype == GL3_BF16)
     rope_cache_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)qkv, positions, seq_of_token, block_table,
                                                           table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
                                                           (bf16_t*)v_cache, n_heads, n_kv, head_dim, rot_dim, adjacent,
-                                                          page_size, write_kv);
+                                                          page_size, write_kv, row_stride);
   else GL3_REQUIRE(false, "gl3_rope_cache_write: unknown dtype %d", dtype);
   GL3_LAUNCH_CHECK();
   return 0;

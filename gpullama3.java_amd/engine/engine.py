@@ -106,6 +106,9 @@ class Engine:
     def page_size(self):
         return self.cache.page_size
 
+    def slots_free(self):
+        return self.cache.slots.n_free
+
     def tokens_capacity(self):
         return self.cache.tokens_free()
 

@@ -11,7 +11,7 @@ requests form the next one. Once a batch has started no request joins it.
 The loop only decides; the model is behind ``backend``:
 ``take_slot()``, ``give_back_slot(slot)``, ``step(entries) -> logits handle`` (last
 row of each entry), ``sample(logits, temperatures, top_ps, uniforms) -> ids``,
-``max_context``, ``page_size``, ``tokens_capacity()``, ``n_slots``.
+``max_context``, ``page_size``, ``tokens_capacity()``, ``slots_free()``.
 """
 from __future__ import annotations
 
@@ -19,6 +19,7 @@ import time
 from dataclasses import dataclass, field
 from typing import Callable, Optional, Sequence
 
+from ..cache.pages import CacheFull
 from ..sampling import SamplingParams, uniform
 
 
@@ -85,11 +86,13 @@ def generate(backend, requests, on_token: Optional[Callable[[int, int], None]] =
                              f"{backend.max_context}")
     results = [Generated() for _ in requests]
     metrics = metrics if metrics is not None else RunMetrics()
-    max_batch = min(max_batch or backend.n_slots, backend.n_slots)
     first = 0
     while first < len(requests):
-        n = plan_batch(requests, first, max_batch, backend.tokens_capacity(), backend.page_size,
-                       backend.max_context)
+        slots = backend.slots_free()
+        if slots < 1:
+            raise CacheFull("no slot is free for the next batch")
+        n = plan_batch(requests, first, min(max_batch or slots, slots), backend.tokens_capacity(),
+                       backend.page_size, backend.max_context)
         _run_batch(backend, requests, results, range(first, first + n), on_token, metrics)
         first += n
     return results

@@ -25,6 +25,9 @@ class FakeBackend:
     def tokens_capacity(self):
         return self.cache.tokens_free()
 
+    def slots_free(self):
+        return self.cache.slots.n_free
+
     def take_slot(self):
         s = self.cache.take_slot()
         assert s not in self.seqs

@@ -1,0 +1,193 @@
+"""The engine against the plain implementation under every way of cutting the work."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_helpers import CONFIGS, DTYPES, close, first_bad_row, model, plain_logits, rand_tokens
+
+pytestmark = pytest.mark.gpu
+
+CASES = [(n, d) for n in ("A", "B", "C") for d in DTYPES]
+
+
+def engine(name, dtype, **kw):
+    from gpullama3_java_amd.engine import Engine
+    folder, _, _ = model(name)
+    kw.setdefault("max_tokens", 2048)
+    return Engine.from_folder(folder, dtype=dtype, **kw)
+
+
+def lengths(name):
+    return {"A": [5, 11, 64, 100], "B": [3, 17, 40, 129, 200], "C": [1, 63, 65, 300]}[name]
+
+
+@pytest.mark.parametrize("name, dtype", CASES)
+def test_each_request_alone_and_whole(name, dtype):
+    eng = engine(name, dtype)
+    for i, n in enumerate(lengths(name)):
+        toks = rand_tokens(name, i, n)
+        s = eng.take_slot()
+        got = eng.step([(s, toks)], want="all").cpu().numpy()
+        eng.give_back_slot(s)
+        close(got, plain_logits(name, toks), dtype, f"{name} {dtype} whole n={n}")
+
+
+@pytest.mark.parametrize("name, dtype", CASES)
+def test_last_32_tokens_one_by_one(name, dtype):
+    eng = engine(name, dtype)
+    for i, n in enumerate(lengths(name)):
+        if n <= 33:
+            continue
+        toks = rand_tokens(name, 10 + i, n)
+        ref = plain_logits(name, toks)
+        s = eng.take_slot()
+        rows = [eng.step([(s, toks[:n - 32])], want="all").cpu().numpy()]
+        rows += [eng.step([(s, [t])], want="all").cpu().numpy() for t in toks[n - 32:]]
+        eng.give_back_slot(s)
+        got = np.concatenate(rows)
+        bad = first_bad_row(got, ref, dtype)
+        assert bad is None, f"{name} {dtype} n={n}: first wrong row {bad} (prompt ends at {n - 32})"
+        close(got, ref, dtype)
+
+
+@pytest.mark.parametrize("name, dtype", CASES)
+def test_unequal_batches_one_after_another_reuse_slots(name, dtype):
+    """Batches start together with unequal prompts, decode one token each, shorter
+    requests end earlier; three batches run over three slots and a cache that holds
+    one batch only, so slots and pages are used again with old data in them."""
+    cfgd = CONFIGS[name]
+    limit = cfgd["max_position_embeddings"]
+    eng = engine(name, dtype, n_slots=3, max_tokens=3 * 64 * (-(-min(limit, 200) // 64)))
+    rng = np.random.default_rng(5)
+    for batch in range(3):
+        prompt_lens = [int(x) for x in rng.integers(1, min(limit, 200) - 40, size=3)]
+        new = [int(x) for x in rng.integers(1, 30, size=3)]
+        seqs = [rand_tokens(name, 100 * batch + j, p + n) for j, (p, n) in enumerate(zip(prompt_lens, new))]
+        slots = [eng.take_slot() for _ in seqs]
+        got = [[] for _ in seqs]
+        out = eng.step([(s, q[:p]) for s, q, p in zip(slots, seqs, prompt_lens)], want="all").cpu().numpy()
+        o = 0
+        for j, p in enumerate(prompt_lens):
+            got[j].append(out[o:o + p]); o += p
+        live = list(range(3))
+        k = 0
+        while live:
+            live = [j for j in live if k < new[j]]
+            for j in range(3):                       # a request that has ended gives its slot back at once
+                if j not in live and slots[j] is not None and k >= new[j]:
+                    eng.give_back_slot(slots[j]); slots[j] = None
+            if not live:
+                break
+            out = eng.step([(slots[j], [seqs[j][prompt_lens[j] + k]]) for j in live]).cpu().numpy()
+            for r, j in enumerate(live):
+                got[j].append(out[r:r + 1])
+            k += 1
+        for j, q in enumerate(seqs):
+            g_ = np.concatenate(got[j])
+            ref = plain_logits(name, q)
+            bad = first_bad_row(g_, ref, dtype)
+            assert bad is None, (f"{name} {dtype} batch {batch} request {j}: first wrong row {bad} "
+                                 f"(prompt {prompt_lens[j]}, total {len(q)})")
+    assert eng.cache.slots.live == set()
+
+
+@pytest.mark.parametrize("name, dtype", [("B", "float32"), ("B", "bfloat16"), ("C", "float32"), ("C", "bfloat16")])
+def test_long_decoding(name, dtype):
+    n = {"B": 250, "C": 400}[name]
+    toks = rand_tokens(name, 77, n)
+    ref = plain_logits(name, toks)
+    eng = engine(name, dtype)
+    s = eng.take_slot()
+    rows = [eng.step([(s, toks[:3])], want="all").cpu().numpy()]
+    rows += [eng.step([(s, [t])]).cpu().numpy() for t in toks[3:]]
+    got = np.concatenate(rows)
+    bad = first_bad_row(got, ref, dtype)
+    assert bad is None, f"first wrong row {bad}"
+
+
+@pytest.mark.parametrize("name, dtype", CASES)
+def test_first_tokens_of_a_sequence(name, dtype):
+    eng = engine(name, dtype)
+    toks = rand_tokens(name, 5, 6)
+    ref = plain_logits(name, toks)
+    s = eng.take_slot()                                          # from the very first token, one by one
+    got = np.concatenate([eng.step([(s, [t])]).cpu().numpy() for t in toks])
+    eng.give_back_slot(s)
+    close(got, ref, dtype, "one by one from position 0")
+    for n in (1, 2, 3):                                          # prompts of 1, 2, 3 tokens in one batch
+        pass
+    slots = [eng.take_slot() for _ in range(3)]
+    out = eng.step([(slots[i], toks[:i + 1]) for i in range(3)], want="all").cpu().numpy()
+    close(out, np.concatenate([ref[:1], ref[:2], ref[:3]]), dtype, "prompts of 1, 2, 3")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_batch_mates_order_and_slot_change_nothing(dtype):
+    name = "B"
+    a, b, c = rand_tokens(name, 1, 50), rand_tokens(name, 2, 7), rand_tokens(name, 3, 120)
+    eng = engine(name, dtype, n_slots=8)
+    s = eng.take_slot()
+    alone = eng.step([(s, a)], want="all").cpu().numpy()
+    eng.give_back_slot(s)
+    for _ in range(3):
+        eng.take_slot()                                           # other slots, other pages
+    sb, sa, sc = eng.take_slot(), eng.take_slot(), eng.take_slot()
+    out = eng.step([(sc, c), (sa, a), (sb, b)], want="all").cpu().numpy()
+    mixed = out[120:170]
+    if dtype == "float32":
+        np.testing.assert_array_equal(mixed, alone)               # same kernels, same order of sums
+    else:
+        close(mixed, alone, dtype)
+    close(mixed, plain_logits(name, a), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_wanted_places_and_errors(dtype):
+    from gpullama3_java_amd.engine import CacheFull
+    name = "A"
+    eng = engine(name, dtype, max_tokens=128, n_slots=2)
+    a, b = rand_tokens(name, 1, 20), rand_tokens(name, 2, 9)
+    sa, sb = eng.take_slot(), eng.take_slot()
+    out = eng.step([(sa, a), (sb, b)], want=[[0, 19, 7], []]).cpu().numpy()
+    ref = plain_logits(name, a)
+    close(out, ref[[0, 19, 7]], dtype)
+    assert eng.step([(sb, [1])], want="none").shape == (0, 256)
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.step([(sa, [256])])
+    with pytest.raises(ValueError, match="twice"):
+        eng.step([(sa, [1]), (sa, [2])])
+    with pytest.raises(CacheFull):
+        eng.step([(sa, [1] * 60)])                                 # 20 + 60 needs a second page; b holds it
+    assert eng.cache.length(sa) == 20                              # a refused step changed nothing
+    more = eng.step([(sa, [5])]).cpu().numpy()
+    close(more, plain_logits(name, a + [5])[-1:], dtype)
+    with pytest.raises(CacheFull, match="longest"):
+        eng.step([(sb, [1] * 200)])
+
+
+def test_float32_and_bfloat16_pick_the_same_greedy_tokens():
+    for name in ("A", "B"):
+        prompts = [rand_tokens(name, 1, 5), rand_tokens(name, 2, 11)]
+        out = {}
+        for dtype in DTYPES:
+            out[dtype] = [r.tokens for r in engine(name, dtype).generate(prompts, max_new_tokens=8)]
+        # where they differ, the two logits must be a near tie in the plain implementation
+        for p, x, y in zip(prompts, out["float32"], out["bfloat16"]):
+            seq = list(p)
+            for tx, ty in zip(x, y):
+                if tx != ty:
+                    l = plain_logits(name, seq)[-1]
+                    assert abs(l[tx] - l[ty]) < 2e-2 * np.abs(l).max()
+                    break
+                seq.append(tx)
+
+
+def test_no_gpu_library_no_engine(monkeypatch):
+    """Without the device library the engine must fail, not fall back."""
+    from gpullama3_java_amd.csrc import lib
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib._build, "library_path", lambda: None)
+    monkeypatch.setattr(lib._build, "build", lambda: (_ for _ in ()).throw(RuntimeError("hipcc not found")))
+    with pytest.raises(RuntimeError, match="hipcc"):
+        lib.rmsnorm(torch.zeros(1, 8, device="cuda"), torch.zeros(8, device="cuda"),
+                    torch.zeros(1, 8, device="cuda"), 1e-5)

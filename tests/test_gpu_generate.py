@@ -1,0 +1,116 @@
+"""Greedy generation through the entry point and the command line, against the plain
+implementation; sampled generation against the replayed logits."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import plain_llama as P
+from gpu_helpers import DTYPES, model, plain_logits, rand_tokens
+from gpullama3_java_amd.sampling import uniform
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_greedy(name, prompt, n, tie=0.0):
+    seq, out = list(prompt), []
+    for _ in range(n):
+        out.append(int(np.argmax(plain_logits(name, seq)[-1])))
+        seq.append(out[-1])
+    return out
+
+
+def agrees_with_plain(name, prompt, got, dtype):
+    """Token by token: the plain argmax, or a logit within rounding of it (then follow the engine)."""
+    seq = list(prompt)
+    for t in got:
+        l = plain_logits(name, seq)[-1]
+        best = int(np.argmax(l))
+        margin = {"float32": 1e-5, "bfloat16": 2e-2}[dtype] * np.abs(l).max()
+        assert t == best or l[best] - l[t] <= margin, (seq, t, best, l[best] - l[t])
+        seq.append(t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_entry_point_greedy(name, dtype):
+    import gpullama3_java_amd as g
+    folder, cfgd, _ = model(name)
+    eng = g.load_model(folder, context_length=-1, dtype=dtype)
+    sampler = g.select_sampler(cfgd["vocab_size"], 0.0, 0.95, seed=1)
+    prompt = rand_tokens(name, 3, 11)
+    seen = []
+    out = eng.generate_tokens(prompt, stop_tokens=set(), max_tokens=11 + 8 - 1, sampler=sampler,
+                              on_token_generated=seen.append)
+    assert len(out) == 8 and seen == out                  # max_tokens bounds the position, as in the reference
+    agrees_with_plain(name, prompt, out, dtype)
+    if dtype == "float32":
+        assert out == plain_greedy(name, prompt, 8)
+    # a stop token ends the sequence and is kept
+    out2 = eng.generate_tokens(prompt, stop_tokens={out[2]}, max_tokens=-1, sampler=sampler)
+    assert out2 == out[:out.index(out[2]) + 1]
+    assert eng.cache.slots.live == set()
+    assert eng.metrics.prompt_tokens == 11 and eng.metrics.generated_tokens == len(out2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_batched_generation_equals_each_alone(dtype):
+    from gpullama3_java_amd.engine import Engine
+    name = "B"
+    folder, _, _ = model(name)
+    eng = Engine.from_folder(folder, dtype=dtype, max_tokens=1024, n_slots=2)     # 5 requests over 2 slots
+    prompts = [rand_tokens(name, 20 + i, n) for i, n in enumerate((3, 17, 40, 9, 64))]
+    res = eng.generate(prompts, max_new_tokens=12)
+    for p, r in zip(prompts, res):
+        assert len(r.tokens) == 12 and r.finish_reason == "length"
+        agrees_with_plain(name, p, r.tokens, dtype)
+    alone = [eng.generate([p], max_new_tokens=12)[0].tokens for p in prompts]
+    if dtype == "float32":
+        assert alone == [r.tokens for r in res]
+    stop = res[1].tokens[4]
+    res2 = eng.generate(prompts, max_new_tokens=12, stop_ids=[stop])
+    for r, r0 in zip(res2, res):
+        cut = r0.tokens.index(stop) + 1 if stop in r0.tokens else 12
+        assert r.tokens == r0.tokens[:cut] and r.finish_reason == ("stop" if stop in r0.tokens else "length")
+
+
+def test_sampled_generation_follows_the_logits():
+    """With temperature and top-p every drawn token is what the plain rule draws from the
+    plain logits of the sequence so far, with the draw's own uniform number."""
+    from gpullama3_java_amd.engine import Engine
+    name = "B"
+    folder, _, _ = model(name)
+    eng = Engine.from_folder(folder, dtype="float32", max_tokens=1024)
+    prompts = [rand_tokens(name, 30 + i, n) for i, n in enumerate((3, 17, 40))]
+    res = eng.generate(prompts, max_new_tokens=12, temperature=0.8, top_p=0.95, seed=9)
+    for i, (p, r) in enumerate(zip(prompts, res)):
+        seq = list(p)
+        for k, t in enumerate(r.tokens):
+            u = uniform(9, i, k)
+            l = plain_logits(name, seq)[-1]
+            want = P.sample(l, 0.8, 0.95, u)
+            if t != want:                                   # allowed only at an edge of the running sum
+                assert any(P.sample(l, 0.8, 0.95, min(max(u + d, 0), 0.9999999)) == t for d in (-2e-5, 2e-5)), (i, k)
+            seq.append(t)
+    again = eng.generate(prompts[::-1], max_new_tokens=12, temperature=0.8, top_p=0.95, seed=9)
+    assert [r.tokens for r in again] != [r.tokens for r in res[::-1]]      # the request index is part of the draw
+    same = eng.generate(prompts, max_new_tokens=12, temperature=0.8, top_p=0.95, seed=9)
+    assert [r.tokens for r in same] == [r.tokens for r in res]
+
+
+def test_command_line(tmp_path):
+    folder, cfgd, _ = model("A")
+    prompt = rand_tokens("A", 4, 6)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "llama-hip"), "--model", folder, "--prompt-ids",
+           ",".join(map(str, prompt)), "--temperature=0", "-n", "13", "--stream", "false", "--dtype", "float32"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert [int(t) for t in r.stdout.split()] == plain_greedy("A", prompt, 8)
+    assert "achieved tok/s" in r.stderr and "Tokens: 14" in r.stderr
+    bad = subprocess.run(cmd[:4] + ["--top-p", "1.5", "--prompt-ids", "1"], capture_output=True, text=True, timeout=300)
+    assert bad.returncode != 0 and "--top-p must be within [0, 1]" in bad.stderr
+    noprompt = subprocess.run(cmd[:4] + ["--prompt", "hello"], capture_output=True, text=True, timeout=300)
+    assert noprompt.returncode != 0 and "tokenizer.json" in noprompt.stderr

@@ -1,0 +1,322 @@
+"""Each kernel alone against its plain reference, at sizes the engine's tests do not use."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from gpullama3_java_amd.sampling import sample_host
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TD = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def K():
+    from gpullama3_java_amd.csrc import lib
+    return lib
+
+
+def dev(a, dtype=torch.float32):
+    return torch.as_tensor(np.ascontiguousarray(a)).to(DEV).to(dtype)
+
+
+def rounded(a, dtype):
+    """The values the kernel really sees after storage in ``dtype``."""
+    return torch.as_tensor(np.asarray(a, np.float32)).to(TD[dtype]).float().numpy()
+
+
+def tol(dtype, k=1):
+    return {"float32": 2e-5, "bfloat16": 1e-2}[dtype]
+
+
+# ------------------------------------------------------------------ embedding, norm
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed(dtype):
+    rng = np.random.default_rng(0)
+    table = rounded(rng.standard_normal((1000, 70)), dtype)
+    ids = rng.integers(0, 1000, 37)
+    out = torch.empty(37, 70, device=DEV)
+    K().embed(dev(table, TD[dtype]), dev(ids, torch.int32), out)
+    np.testing.assert_array_equal(out.cpu().numpy(), table[ids])
+
+
+@pytest.mark.parametrize("d", [70, 2048, 5000])
+@pytest.mark.parametrize("wdtype, odtype", [("float32", "float32"), ("bfloat16", "bfloat16"), ("float32", "bfloat16")])
+def test_rmsnorm(d, wdtype, odtype):
+    rng = np.random.default_rng(d)
+    x = (rng.standard_normal((9, d)) * 3).astype(np.float32)
+    w = rounded(1 + 0.2 * rng.standard_normal(d), wdtype)
+    out = torch.empty(9, d, device=DEV, dtype=TD[odtype])
+    K().rmsnorm(dev(x), dev(w, TD[wdtype]), out, 1e-6)
+    ref = P.rmsnorm(x, w, 1e-6)
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref, rtol=1e-5 if odtype == "float32" else 5e-3, atol=1e-6)
+    rows = np.array([7, 0, 7, 3])
+    out2 = torch.empty(4, d, device=DEV, dtype=TD[odtype])
+    K().rmsnorm(dev(x), dev(w, TD[wdtype]), out2, 1e-6, dev(rows, torch.int32))
+    assert torch.equal(out2, out[torch.as_tensor(rows).to(DEV)])
+    zero = torch.empty(1, d, device=DEV)
+    K().rmsnorm(torch.zeros(1, d, device=DEV), dev(w), zero, 1e-5)
+    assert torch.all(zero == 0)
+
+
+# ------------------------------------------------------------------ generic product
+@pytest.mark.parametrize("M, N, Kd", [(1, 130, 70), (37, 257, 129), (200, 64, 64), (3, 1000, 112)])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gemm_generic_epilogues(M, N, Kd, dtype):
+    rng = np.random.default_rng(M * N)
+    a = rounded(rng.standard_normal((M, Kd)), dtype)
+    w = rounded(rng.standard_normal((2 * N, Kd)) / math.sqrt(Kd), dtype)
+    A, W = dev(a, TD[dtype]), dev(w, TD[dtype])
+    lib = K()
+    out = torch.empty(M, N, device=DEV, dtype=TD[dtype])
+    lib.gemm_generic(A, W[:N], out, lib.EPI_STORE)
+    ref = P.linear(a, w[:N])
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref, atol=tol(dtype) * np.abs(ref).max())
+    logits = torch.empty(M, N, device=DEV)                         # float output from bfloat16 operands
+    lib.gemm_generic(A, W[:N], logits, lib.EPI_STORE)
+    np.testing.assert_allclose(logits.cpu().numpy(), ref, atol=2e-5 * np.abs(ref).max())
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    x = dev(res)
+    lib.gemm_generic(A, W[:N], x, lib.EPI_ADD)
+    np.testing.assert_allclose(x.cpu().numpy(), res + ref, atol=2e-5 * np.abs(ref).max())
+    gated = torch.empty(M, N, device=DEV, dtype=TD[dtype])
+    lib.gemm_generic(A, W, gated, lib.EPI_GATED)
+    refg = P.silu(P.linear(a, w[:N])) * P.linear(a, w[N:])
+    np.testing.assert_allclose(gated.float().cpu().numpy(), refg, atol=tol(dtype) * max(np.abs(refg).max(), 1e-3))
+
+
+def test_gemm_generic_rows_do_not_depend_on_their_company():
+    rng = np.random.default_rng(3)
+    a, w = dev(rng.standard_normal((130, 96))), dev(rng.standard_normal((77, 96)))
+    lib = K()
+    full = torch.empty(130, 77, device=DEV)
+    lib.gemm_generic(a, w, full)
+    one = torch.empty(1, 77, device=DEV)
+    for r in (0, 63, 64, 129):
+        lib.gemm_generic(a[r:r + 1], w, one)
+        assert torch.equal(one[0], full[r])
+
+
+def test_gemm_generic_mixed_storage_and_strides():
+    rng = np.random.default_rng(4)
+    a = rounded(rng.standard_normal((5, 40)), "bfloat16")
+    w = rng.standard_normal((9, 40)).astype(np.float32)               # a matrix stored in 32-bit stays so
+    lib = K()
+    out = torch.empty(5, 9, device=DEV, dtype=torch.bfloat16)
+    lib.gemm_generic(dev(a, torch.bfloat16), dev(w), out)
+    np.testing.assert_allclose(out.float().cpu().numpy(), P.linear(a, w), atol=0.05)
+    wide = torch.zeros(5, 30, device=DEV)                              # output is a view with a row stride
+    lib.gemm_generic(dev(a), dev(w), wide[:, 3:12])
+    np.testing.assert_allclose(wide[:, 3:12].cpu().numpy(), P.linear(a, w), atol=1e-4)
+    assert torch.all(wide[:, :3] == 0) and torch.all(wide[:, 12:] == 0)
+    with pytest.raises(lib.KernelError):
+        lib.gemm_generic(dev(a), dev(w[:, :39]), wide[:, 3:12])
+
+
+# ------------------------------------------------------------------ paged cache helpers
+def paged(seqs_k, seqs_v, n_kv, hs, page, dtype, rng, n_pages=None):
+    """Scatter per-sequence ``[len, n_kv, hs]`` keys and values into shuffled pages."""
+    need = [-(-len(k) // page) for k in seqs_k]
+    n_pages = n_pages or sum(need) + 3
+    ids = rng.permutation(np.arange(1, n_pages))[:sum(need)].tolist()
+    kc = torch.full((n_pages, n_kv, page, hs), 777.0, dtype=TD[dtype])        # garbage where nothing was written
+    vc = torch.full((n_pages, n_kv, page, hs), -777.0, dtype=TD[dtype])
+    width = max(need)
+    table = np.zeros((len(seqs_k), width), np.int32)
+    for s, (k, v) in enumerate(zip(seqs_k, seqs_v)):
+        for p in range(need[s]):
+            pid = ids.pop()
+            table[s, p] = pid
+            chunk = slice(p * page, min(len(k), (p + 1) * page))
+            n = chunk.stop - chunk.start
+            kc[pid, :, :n] = torch.as_tensor(k[chunk]).to(TD[dtype]).transpose(0, 1)
+            vc[pid, :, :n] = torch.as_tensor(v[chunk]).to(TD[dtype]).transpose(0, 1)
+    return kc.to(DEV), vc.to(DEV), torch.as_tensor(table).to(DEV)
+
+
+# ------------------------------------------------------------------ rotary + cache write
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("pairing", ["adjacent", "half"])
+@pytest.mark.parametrize("H, Kh, hs", [(6, 2, 16), (5, 5, 48), (8, 1, 128)])
+def test_rope_cache_write(dtype, pairing, H, Kh, hs):
+    rng = np.random.default_rng(hs + H)
+    page = 64
+    lens_before, new = [70, 0, 129], [3, 40, 1]
+    T = sum(new)
+    qkv = rounded(rng.standard_normal((T, (H + 2 * Kh) * hs)), dtype)
+    positions = np.concatenate([np.arange(b, b + n) for b, n in zip(lens_before, new)])
+    seq_of = np.concatenate([[i] * n for i, n in enumerate(new)])
+    total = [b + n for b, n in zip(lens_before, new)]
+    zk = [np.zeros((t, Kh, hs), np.float32) for t in total]
+    kc, vc, table = paged(zk, zk, Kh, hs, page, dtype, rng)
+    before_k = kc.clone()
+    cos, sin = P.rope_table(256, hs, 50000.0, dict(factor=4.0, low_freq_factor=1.0, high_freq_factor=2.0,
+                                                   original_max_position_embeddings=64))
+    buf = dev(qkv, TD[dtype])
+    K().rope_cache_write(buf, dev(positions, torch.int32), dev(seq_of, torch.int32), table, dev(cos), dev(sin),
+                         kc, vc, H, Kh, hs, hs, pairing == "adjacent", page)
+    q = qkv[:, :H * hs].reshape(T, H, hs)
+    k = qkv[:, H * hs:(H + Kh) * hs].reshape(T, Kh, hs)
+    v = qkv[:, (H + Kh) * hs:].reshape(T, Kh, hs)
+    qr = P.rope_rotate(q, positions, cos, sin, pairing)
+    kr = P.rope_rotate(k, positions, cos, sin, pairing)
+    out = buf.float().cpu().numpy()
+    t = tol(dtype)
+    np.testing.assert_allclose(out[:, :H * hs].reshape(T, H, hs), qr, atol=t * 4)
+    np.testing.assert_array_equal(out[:, H * hs:], qkv[:, H * hs:])           # k and v in the buffer are left alone
+    kcpu, vcpu, tab = kc.float().cpu().numpy(), vc.float().cpu().numpy(), table.cpu().numpy()
+    touched = np.zeros(kc.shape[0], bool)
+    for i in range(T):
+        pid = tab[seq_of[i], positions[i] // page]
+        touched[pid] = True
+        np.testing.assert_allclose(kcpu[pid, :, positions[i] % page], kr[i], atol=t * 4)
+        np.testing.assert_array_equal(vcpu[pid, :, positions[i] % page], v[i])  # values are copied, never rotated
+    # nothing else in the cache moved
+    mask = torch.ones_like(kc, dtype=torch.bool)
+    for i in range(T):
+        mask[tab[seq_of[i], positions[i] // page], :, positions[i] % page] = False
+    assert torch.equal(kc[mask], before_k[mask])
+
+
+def test_rope_position_zero_and_no_table():
+    rng = np.random.default_rng(1)
+    qkv = rng.standard_normal((2, 4 * 16)).astype(np.float32)
+    cos, sin = P.rope_table(8, 16, 10000.0)
+    kc = torch.zeros(3, 1, 64, 16, device=DEV); vc = torch.zeros_like(kc)
+    table = dev(np.array([[1], [2]]), torch.int32)
+    for cs in ((dev(cos), dev(sin)), (None, None)):
+        buf = dev(qkv)
+        K().rope_cache_write(buf, dev([0, 0], torch.int32), dev([0, 1], torch.int32), table, cs[0], cs[1], kc, vc,
+                             2, 1, 16, 16 if cs[0] is not None else 0, True, 64)
+        np.testing.assert_array_equal(buf.cpu().numpy(), qkv)
+        np.testing.assert_array_equal(kc[1, 0, 0].cpu().numpy(), qkv[0, 32:48])
+
+
+# ------------------------------------------------------------------ attention
+def attention_case(rng, H, Kh, hs, lens_before, new, dtype, scale_hot=None):
+    seqs_k, seqs_v, qs = [], [], []
+    for b, n in zip(lens_before, new):
+        seqs_k.append(rounded(rng.standard_normal((b + n, Kh, hs)), dtype))
+        seqs_v.append(rounded(rng.standard_normal((b + n, Kh, hs)), dtype))
+        qs.append(rounded(rng.standard_normal((b + n, H, hs)), dtype))
+    return seqs_k, seqs_v, qs
+
+
+def run_attention(fn, seqs_k, seqs_v, qs, lens_before, new, H, Kh, hs, dtype, rng, window=None, page=64):
+    kc, vc, table = paged(seqs_k, seqs_v, Kh, hs, page, dtype, rng)
+    positions = np.concatenate([np.arange(b, b + n) for b, n in zip(lens_before, new)])
+    seq_of = np.concatenate([[i] * n for i, n in enumerate(new)])
+    q = np.concatenate([qq[b:b + n] for qq, b, n in zip(qs, lens_before, new)]).reshape(len(positions), H * hs)
+    wide = torch.zeros(len(positions), H * hs + 2 * Kh * hs, device=DEV, dtype=TD[dtype])   # q sits in a wider row
+    wide[:, :H * hs] = dev(q, TD[dtype])
+    out = torch.empty(len(positions), H * hs, device=DEV, dtype=TD[dtype])
+    fn(wide, kc, vc, dev(positions, torch.int32), dev(seq_of, torch.int32), table, out, H, Kh, hs, page, window,
+       1.0 / math.sqrt(hs))
+    ref = np.concatenate([P.attention(qq, k, v, window=window)[b:b + n]
+                          for qq, k, v, b, n in zip(qs, seqs_k, seqs_v, lens_before, new)])
+    return out.float().cpu().numpy().reshape(-1, H, hs), ref
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H, Kh, hs", [(6, 2, 16), (5, 5, 48), (8, 1, 128), (2, 1, 256), (4, 2, 80)])
+def test_attention_generic(dtype, H, Kh, hs):
+    rng = np.random.default_rng(H * hs)
+    lens_before, new = [0, 70, 130, 5], [33, 1, 2, 1]          # a prompt, decodes at page edges, a short one
+    sk, sv, qs = attention_case(rng, H, Kh, hs, lens_before, new, dtype)
+    got, ref = run_attention(K().attention_generic, sk, sv, qs, lens_before, new, H, Kh, hs, dtype, rng)
+    np.testing.assert_allclose(got, ref, atol=tol(dtype) * np.abs(ref).max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_generic_far_key_and_window_edge(dtype):
+    """One far key among hundreds carries the whole weight; with a window the key just
+    inside it counts and the key just outside does not."""
+    rng = np.random.default_rng(9)
+    H, Kh, hs, n = 4, 2, 32, 700
+    k = rng.standard_normal((n, Kh, hs)).astype(np.float32) * 0.1
+    v = rng.standard_normal((n, Kh, hs)).astype(np.float32)
+    q = rng.standard_normal((n, H, hs)).astype(np.float32) * 0.1
+    far = 13
+    k[far, 1] = 0; k[far, 1, 5] = 30.0                                      # stands out for kv head 1 only
+    q[n - 1, 2] = 0; q[n - 1, 2, 5] = 30.0                                  # head 2 -> kv head 1
+    q[n - 1, 0] = 0; q[n - 1, 0, 5] = 30.0                                  # head 0 -> kv head 0: no hot key there
+    k, v, q = (rounded(a, dtype) for a in (k, v, q))
+    got, ref = run_attention(K().attention_generic, [k], [v], [q], [n - 1], [1], H, Kh, hs, dtype, rng)
+    np.testing.assert_allclose(got, ref, atol=tol(dtype) * np.abs(ref).max())
+    np.testing.assert_allclose(got[0, 2], v[far, 1], atol=tol(dtype) * 4)   # the far value, nothing else
+    assert np.abs(got[0, 0] - v[far, 0]).max() > 0.3
+    # window: the query at n-1 sees keys n-w .. n-1
+    w = 100
+    for hot, inside in ((n - w, True), (n - w - 1, False)):
+        k2 = k.copy(); k2[far, 1] = 0.0; k2[hot, 1] = 0; k2[hot, 1, 5] = 30.0
+        k2 = rounded(k2, dtype)
+        got, ref = run_attention(K().attention_generic, [k2], [v], [q], [n - 1], [1], H, Kh, hs, dtype, rng, window=w)
+        np.testing.assert_allclose(got, ref, atol=tol(dtype) * np.abs(ref).max())
+        assert (np.abs(got[0, 2] - v[hot, 1]).max() < tol(dtype) * 4) == inside
+
+
+def test_attention_generic_is_the_same_for_every_cut():
+    rng = np.random.default_rng(11)
+    H, Kh, hs, n = 4, 2, 48, 150
+    sk, sv, qs = attention_case(rng, H, Kh, hs, [0], [n], "float32")
+    whole, _ = run_attention(K().attention_generic, sk, sv, qs, [0], [n], H, Kh, hs, "float32", rng)
+    for p in (0, 63, 64, 149):
+        one, _ = run_attention(K().attention_generic, sk, sv, qs, [p], [1], H, Kh, hs, "float32", rng)
+        np.testing.assert_array_equal(one[0], whole[p])
+
+
+# ------------------------------------------------------------------ sampling
+def check_draw(logits, temperature, top_p, u, tok):
+    """The drawn token is the twin's, or u sits within rounding of the edge between them."""
+    want = sample_host(logits, temperature, top_p, u)
+    if tok == want:
+        return
+    for du in (-1e-6, 1e-6):
+        if sample_host(logits, temperature, top_p, min(max(u + du, 0.0), 0.99999994)) == tok:
+            return
+    for dp in (-1e-6, 1e-6):
+        if 0 < top_p < 1 and sample_host(logits, temperature, top_p + dp, u) == tok:
+            return
+    raise AssertionError(f"T={temperature} p={top_p} u={u}: kernel {tok}, twin {want}")
+
+
+@pytest.mark.parametrize("V", [2, 50, 1000, 5000, 128256])
+def test_sample_kernel(V):
+    rng = np.random.default_rng(V)
+    R = 24
+    logits = (rng.standard_normal((R, V)) * rng.uniform(0.3, 4, (R, 1))).astype(np.float32)
+    logits[3, : min(V, 7)] = logits[3].max() + 1.0                        # ties at the top
+    temps = np.array([0, 0, 0.8, 1.0, 1.0, 0.3, 2.0, 1.0] * 3, np.float32)
+    tops = np.array([0.95, 1.0, 0.95, 1.0, 0.0, 0.5, 0.9, 1e-6] * 3, np.float32)
+    us = rng.random(R).astype(np.float32)
+    us[4] = 0.0; us[6] = np.float32(0.99999994)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    K().sample(dev(logits), torch.empty(R * V, device=DEV), dev(temps), dev(tops), dev(us), out)
+    for r, tok in enumerate(out.tolist()):
+        assert 0 <= tok < V
+        check_draw(logits[r], float(temps[r]), float(tops[r]), float(us[r]), tok)
+    assert out[3].item() == 0 if temps[3] == 0 else True
+
+
+def test_sample_kernel_frequencies_and_rules():
+    rng = np.random.default_rng(5)
+    V, R = 12, 4000
+    row = rng.standard_normal(V).astype(np.float32) * 1.5
+    logits = np.tile(row, (R, 1))
+    us = rng.random(R).astype(np.float32)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    lib = K()
+    work = torch.empty(R * V, device=DEV)
+    lib.sample(dev(logits), work, dev(np.full(R, 1.0)), dev(np.full(R, 1.0)), dev(us), out)
+    p = P.probabilities(row, 1.0)
+    counts = np.bincount(out.cpu().numpy(), minlength=V)
+    assert np.sum((counts - R * p) ** 2 / (R * p)) < 40                 # 11 degrees of freedom
+    lib.sample(dev(logits), work, dev(np.full(R, 1.0)), dev(np.full(R, 0.6)), dev(us), out)
+    kept, _ = P.top_p_set(p, 0.6)
+    assert set(out.cpu().numpy().tolist()) == set(kept)                 # the smallest prefix, all of it, only it
+    lib.sample(dev(logits), work, dev(np.zeros(R)), dev(np.full(R, 0.6)), dev(us), out)
+    assert torch.all(out == int(np.argmax(row)))
+    lib.sample(dev(logits), work, dev(np.full(R, 1e-3)), dev(np.full(R, 1.0)), dev(us), out)
+    assert torch.all(out == int(np.argmax(row)))                        # T -> 0+ is greedy

@@ -1,0 +1,317 @@
+"""Each part alone, the run order as data, and a toy mixer with state of its own that is
+registered, built and stepped without a change to the framework's files."""
+import json
+import math
+import os
+from dataclasses import dataclass, field
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import save_file
+
+import plain_llama as P
+from gpu_helpers import close, model, rand_tokens
+from tiny import TINY_A
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TD = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+class Harness:
+    """What a part needs of an engine: a cache, a workspace, dtype and device."""
+
+    def __init__(self, kv_needs, state_needs, dtype, max_tokens=1024, n_slots=4):
+        from gpullama3_java_amd.cache import Cache
+        from gpullama3_java_amd.engine.context import Workspace
+        self.dtype, self.device = TD[dtype], torch.device(DEV)
+        self.cache = Cache(kv_needs, state_needs, max_tokens, 512, n_slots, self.dtype, self.device)
+        self.workspace = Workspace(self.device)
+
+    def context(self, entries):
+        """entries: [(slot, n new tokens)] -> a step context (no token ids: parts do not need them)."""
+        from gpullama3_java_amd.engine.context import StepContext
+        slots = [s for s, _ in entries]
+        q_lens = [n for _, n in entries]
+        before = [self.cache.length(s) for s in slots]
+        self.cache.reserve(dict(entries))
+        ctx = StepContext(self, sum(q_lens), len(entries), q_lens, before, slots, all(n == 1 for n in q_lens),
+                          max(q_lens), max(b + n for b, n in zip(before, q_lens)))
+        i32 = lambda a: torch.as_tensor(np.asarray(a, np.int32)).to(DEV)
+        ctx.positions = i32(np.concatenate([np.arange(b, b + n) for b, n in zip(before, q_lens)]))
+        ctx.seq_of_token = i32(np.concatenate([[i] * n for i, n in enumerate(q_lens)]))
+        ctx.cu_seqlens = i32(np.concatenate([[0], np.cumsum(q_lens)]))
+        ctx.kv_before, ctx.slot_ids = i32(before), i32(slots)
+        width = max(1, -(-ctx.max_kv_len // self.cache.page_size))
+        ctx._tables = [i32(self.cache.block_rows(g, slots, width)) for g in range(len(self.cache.groups))]
+        for s, n in entries:
+            self.cache.advance(s, n)
+        return ctx
+
+
+def stored(a, dtype):
+    return torch.as_tensor(np.asarray(a, np.float32)).to(TD[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_norm_part(dtype):
+    from gpullama3_java_amd.config import NormSpec
+    from gpullama3_java_amd.parts import build_part
+    rng = np.random.default_rng(0)
+    part = build_part("norm", NormSpec(dim=100, eps=1e-3, names={"weight": "w"}), dtype=TD[dtype])
+    assert {k: v.shape for k, v in part.tensors().items()} == {"w": (100,)}
+    w = stored(1 + 0.3 * rng.standard_normal(100), dtype)
+    part.load({"w": w.to(DEV)})
+    x = rng.standard_normal((7, 100)).astype(np.float32) * 0.01        # small: eps matters
+    out = part(Harness([], [], dtype).context([]) if False else _ctx_only(dtype), torch.as_tensor(x).to(DEV))
+    ref = P.rmsnorm(x, w.float().numpy(), 1e-3)
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref, atol=(1e-6 if dtype == "float32" else 5e-3) * np.abs(ref).max())
+
+
+def _ctx_only(dtype):
+    from gpullama3_java_amd.cache import KVNeed
+    h = Harness([KVNeed(1, 16)], [None], dtype)
+    return h.context([(h.cache.take_slot(), 7)])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H, Kh, hs, d, pairing, window", [(6, 2, 16, 40, "adjacent", None), (3, 1, 48, 72, "half", None),
+                                                           (4, 4, 32, 64, "half", 20)])
+def test_attention_part_whole_and_in_pieces(dtype, H, Kh, hs, d, pairing, window):
+    from gpullama3_java_amd.config import AttentionSpec, RotarySpec
+    from gpullama3_java_amd.parts import RunInfo, build_part
+    rng = np.random.default_rng(H * d)
+    names = {k: k for k in "qkvo"}
+    spec = AttentionSpec(hidden=d, n_heads=H, n_kv_heads=Kh, head_dim=hs, window=window, names=names,
+                         position=RotarySpec(head_dim=hs, theta=1000.0, pairing=pairing, max_positions=512))
+    part = build_part("mixer", spec, dtype=TD[dtype], device=torch.device(DEV))
+    assert {k: tuple(v.shape) for k, v in part.tensors().items()} == {
+        "q": (H * hs, d), "k": (Kh * hs, d), "v": (Kh * hs, d), "o": (d, H * hs)}
+    W = {n: stored(rng.standard_normal(s.shape) * 0.3, dtype) for n, s in part.tensors().items()}
+    part.load({n: t.to(DEV) for n, t in W.items()})
+    Wn = {n: t.float().numpy() for n, t in W.items()}
+    n_tok = [70, 9]
+    hs_in = [stored(rng.standard_normal((n, d)), dtype) for n in n_tok]
+    cos, sin = P.rope_table(512, hs, 1000.0)
+
+    def plain(h):
+        h = h.float().numpy()
+        T = len(h)
+        pos = np.arange(T)
+        q = P.rope_rotate(P.linear(h, Wn["q"]).reshape(T, H, hs), pos, cos, sin, pairing)
+        k = P.rope_rotate(P.linear(h, Wn["k"]).reshape(T, Kh, hs), pos, cos, sin, pairing)
+        v = P.linear(h, Wn["v"]).reshape(T, Kh, hs)
+        return P.linear(P.attention(q, k, v, window=window).reshape(T, H * hs), Wn["o"])
+
+    refs = [plain(h) for h in hs_in]
+    harness = Harness([part.kv_need()], [part.state_need()], dtype)
+    assert part.kv_need().window == window and part.state_need() is None
+    run = RunInfo(entry=0, kv_entry=0, writes_kv=True)
+    slots = [harness.cache.take_slot() for _ in n_tok]
+    # both sequences whole in one step; the output is added into x
+    x = torch.ones(sum(n_tok), d, device=DEV)
+    part.forward(harness.context(list(zip(slots, n_tok))), torch.cat(hs_in).to(DEV), x, run)
+    ref = np.concatenate(refs)
+    t = (2e-5 if dtype == "float32" else 2e-2) * np.abs(ref).max()
+    np.testing.assert_allclose(x.cpu().numpy() - 1, ref, atol=t)
+    # again in pieces: 60 + 1 + ... for the first, the second one token at a time
+    for s in slots:
+        harness.cache.give_back_slot(s)
+    s0 = harness.cache.take_slot()
+    outs = []
+    for lo, hi in [(0, 60)] + [(i, i + 1) for i in range(60, 70)]:
+        x = torch.zeros(hi - lo, d, device=DEV)
+        part.forward(harness.context([(s0, hi - lo)]), hs_in[0][lo:hi].to(DEV), x, run)
+        outs.append(x.cpu().numpy())
+    np.testing.assert_allclose(np.concatenate(outs), refs[0], atol=t)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_feed_forward_part(dtype):
+    from gpullama3_java_amd.config import GatedFeedForwardSpec
+    from gpullama3_java_amd.parts import build_part
+    rng = np.random.default_rng(2)
+    d, F = 72, 200
+    part = build_part("ffn", GatedFeedForwardSpec(hidden=d, intermediate=F, names={"gate": "g", "up": "u", "down": "dn"}),
+                      dtype=TD[dtype], device=torch.device(DEV))
+    assert {k: tuple(v.shape) for k, v in part.tensors().items()} == {"g": (F, d), "u": (F, d), "dn": (d, F)}
+    W = {n: stored(rng.standard_normal(s.shape) * 0.2, dtype) for n, s in part.tensors().items()}
+    weights = {n: t.to(DEV) for n, t in W.items()}
+    part.load(weights)
+    assert torch.equal(weights["u"].cpu(), W["u"])                       # stacked, still addressable by name
+    h = stored(rng.standard_normal((11, d)), dtype)
+    x = torch.full((11, d), 2.0, device=DEV)
+    part.forward(_ctx_only(dtype), h.to(DEV), x)
+    ref = P.feed_forward(h.float().numpy(), *(W[n].float().numpy() for n in ("g", "u", "dn")))
+    np.testing.assert_allclose(x.cpu().numpy() - 2, ref, atol=(2e-5 if dtype == "float32" else 2e-2) * np.abs(ref).max())
+    with pytest.raises(ValueError, match="gelu"):
+        build_part("ffn", GatedFeedForwardSpec(hidden=d, intermediate=F, activation="gelu"), dtype=TD[dtype], device=DEV)
+
+
+def test_unknown_part_kind_lists_the_known():
+    from gpullama3_java_amd.parts import build_part
+
+    @dataclass
+    class Odd:
+        kind: str = "odd"
+    with pytest.raises(KeyError, match="rmsnorm"):
+        build_part("norm", Odd(), dtype=torch.float32)
+
+
+# ------------------------------------------------------------------ the run order is data
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_run_order_names_a_layer_twice_and_reads_another_entry_s_cache(dtype):
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.config import Run
+    from gpullama3_java_amd.engine import Engine
+    from gpullama3_java_amd.weights import load_weights
+    from gpullama3_java_amd.parts import DecoderModel
+    folder, cfgd, W = model("A")
+    order = [(0, None), (1, None), (1, None), (0, 1)]          # layer 1 twice; the last run reads entry 1's keys
+
+    class Reordered(g.LlamaConfiguration):
+        def model_spec(self):
+            from dataclasses import replace
+            return replace(super().model_spec(), run_order=tuple(Run(layer=l, reads=r) for l, r in order))
+
+    cfg = Reordered(**g.config_from_dict(cfgd).__dict__)
+    probe = DecoderModel(cfg.model_spec(), TD[dtype], "cpu")
+    eng = Engine(cfg, load_weights(folder, probe.expected(), TD[dtype], torch.device(DEV)), dtype=dtype, max_tokens=512)
+    assert len(eng.cache.groups[0].entries) == 3                # three entries store keys, the fourth reads
+    toks = rand_tokens("A", 3, 50)
+    ref = P.forward(cfgd, W, toks, schedule=order)
+    s = eng.take_slot()
+    got = np.concatenate([eng.step([(s, toks[:30])], want="all").cpu().numpy()]
+                         + [eng.step([(s, [t])]).cpu().numpy() for t in toks[30:]])
+    close(got, ref, dtype, "reordered run")
+    assert np.abs(ref - P.forward(cfgd, W, toks)).max() > 1e-3   # the order matters
+
+    with pytest.raises(ValueError, match="reads entry"):
+        class Bad(g.LlamaConfiguration):
+            def model_spec(self):
+                from dataclasses import replace
+                return replace(super().model_spec(), run_order=(Run(0), Run(1, reads=1)))
+        DecoderModel(Bad(**cfg.__dict__).model_spec(), torch.float32, "cpu")
+
+
+# ------------------------------------------------------------------ a toy mixer with state of its own
+@dataclass(frozen=True)
+class DecaySpec:
+    """y_t = s_t . W with s_t = decay * s_{t-1} + h_t: a running sum per sequence, kept per slot."""
+    kind: str = "toy_decay"
+    hidden: int = 0
+    decay: float = 0.5
+    names: dict = field(default_factory=dict)
+
+
+class DecayMixer:
+    def __init__(self, spec, dtype, device):
+        self.spec, self.dtype = spec, dtype
+        self.w = None
+
+    def tensors(self):
+        from gpullama3_java_amd.weights import TensorSpec
+        return {self.spec.names["w"]: TensorSpec((self.spec.hidden, self.spec.hidden))}
+
+    def load(self, weights):
+        self.w = weights[self.spec.names["w"]]
+
+    def kv_need(self):
+        return None                                         # nothing per position
+
+    def state_need(self):
+        from gpullama3_java_amd.cache import StateNeed
+        return StateNeed(self.spec.hidden, torch.float32)
+
+    def forward(self, ctx, h, x, run):
+        state = ctx.slot_state(run.entry)                   # [n_slots, hidden], zero for a fresh slot
+        o = 0
+        for slot, n in zip(ctx.slots, ctx.q_lens):
+            s = state[slot].clone()
+            for i in range(n):                              # a chunk advances the state token by token
+                s = self.spec.decay * s + h[o + i].float()
+                x[o + i] += (s.to(self.dtype).float() @ self.w.float().t())
+            state[slot] = s
+            o += n
+
+
+def toy_plain(cfg, W, toks):
+    x = W["emb"][toks].astype(np.float32)
+    for l in range(cfg["n_layers"]):
+        h = P.rmsnorm(x, W[f"l{l}.norm"], cfg["eps"])
+        s = np.zeros(cfg["hidden"], np.float32)
+        out = np.zeros_like(x)
+        for t in range(len(toks)):
+            s = np.float32(cfg["decay"]) * s + h[t]
+            out[t] = s @ W[f"l{l}.w"].T
+        x = x + out
+    return P.rmsnorm(x, W["final"], cfg["eps"]) @ W["emb"].T
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.config import BlockSpec, ModelSpec, NormSpec, Run
+    from gpullama3_java_amd.engine import Engine
+    from gpullama3_java_amd.parts import register_part
+
+    register_part("mixer", "toy_decay", DecayMixer)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        hidden: int
+        n_layers: int
+        vocab: int
+        decay: float
+        eps: float
+        max_position_embeddings: int = 512
+        stop_ids: tuple = ()
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(d["hidden"], d["n_layers"], d["vocab"], d["decay"], d["eps"])
+
+        def with_context_length(self, n):
+            return self
+
+        def model_spec(self):
+            layers = tuple(BlockSpec(kind="prenorm",
+                                     mixer_norm=NormSpec(dim=self.hidden, eps=self.eps, names={"weight": f"l{i}.norm"}),
+                                     mixer=DecaySpec(hidden=self.hidden, decay=self.decay, names={"w": f"l{i}.w"}),
+                                     ffn_norm=None, ffn=None) for i in range(self.n_layers))
+            return ModelSpec(architecture="ToyForCausalLM", vocab_size=self.vocab, hidden=self.hidden, layers=layers,
+                             run_order=tuple(Run(i) for i in range(self.n_layers)),
+                             final_norm=NormSpec(dim=self.hidden, eps=self.eps, names={"weight": "final"}),
+                             max_positions=512, tie_embeddings=True, embedding_name="emb", head_name=None)
+
+    g.register_architecture("ToyForCausalLM", ToyConfig)
+    cfg = {"architectures": ["ToyForCausalLM"], "hidden": 24, "n_layers": 2, "vocab": 40, "decay": 0.7, "eps": 1e-5}
+    rng = np.random.default_rng(0)
+    W = {"emb": rng.standard_normal((40, 24)).astype(np.float32), "final": np.ones(24, np.float32)}
+    for l in range(2):
+        W[f"l{l}.norm"] = (1 + 0.1 * rng.standard_normal(24)).astype(np.float32)
+        W[f"l{l}.w"] = (rng.standard_normal((24, 24)) * 0.2).astype(np.float32)
+    folder = str(tmp_path / "toy")
+    os.makedirs(folder)
+    json.dump(cfg, open(os.path.join(folder, "config.json"), "w"))
+    save_file({k: torch.as_tensor(v) for k, v in W.items()}, os.path.join(folder, "model.safetensors"))
+
+    eng = Engine.from_folder(folder, dtype="float32", max_tokens=256, n_slots=2)
+    assert not eng.cache.groups and sorted(eng.cache.state) == [0, 1]        # state, no keys and values
+    a, b = rng.integers(0, 40, 30).tolist(), rng.integers(0, 40, 12).tolist()
+    sa, sb = eng.take_slot(), eng.take_slot()
+    out = eng.step([(sa, a[:20]), (sb, b[:5])], want="all").cpu().numpy()
+    got_a, got_b = [out[:20]], [out[20:]]
+    for i in range(7):                                                        # both go on one token at a time
+        o = eng.step([(sa, [a[20 + i]]), (sb, [b[5 + i]])]).cpu().numpy()
+        got_a.append(o[:1]); got_b.append(o[1:])
+    eng.give_back_slot(sb)                                                    # b ends earlier
+    got_a.append(eng.step([(sa, a[27:])], want="all").cpu().numpy())
+    np.testing.assert_allclose(np.concatenate(got_a), toy_plain(cfg, W, a), atol=2e-4)
+    np.testing.assert_allclose(np.concatenate(got_b), toy_plain(cfg, W, b), atol=2e-4)
+    eng.give_back_slot(sa)
+    s = eng.take_slot()                                                       # a used slot starts from zero state
+    again = eng.step([(s, b)], want="all").cpu().numpy()
+    np.testing.assert_allclose(again, toy_plain(cfg, W, b), atol=2e-4)
+    res = eng.generate([a[:4], b[:6]], max_new_tokens=5)                      # and the generation loop runs it
+    assert [len(r.tokens) for r in res] == [5, 5]
