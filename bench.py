@@ -1,0 +1,178 @@
+"""Decode and prefill throughput of the Llama-3.2-1B shape with random weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+
+A step is one decode step of the generation loop: the engine's step for B sequences (one
+token each, from the cache left by 512-token prompts) and the greedy pick of the next
+token on the device. ``value`` is decoded tokens a second at the default batch of 8.
+The same line carries the prefill of one 2,048-token prompt, the decode step's share of
+the memory roofline, and decode at batch 1 and 64. Peaks are the published ones of the
+MI355X: 8 TB/s HBM3E, 2.5 PFLOP/s dense bf16 matrix throughput.
+"""
+import argparse
+import json
+import os
+import shutil
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_GBS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+
+# BASELINE.json configs[2]: the Llama-3.2-1B shape
+SHAPE = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 2048, "intermediate_size": 8192,
+    "num_hidden_layers": 16, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
+    "vocab_size": 128256, "max_position_embeddings": 4096, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "tie_word_embeddings": True, "hidden_act": "silu",
+}
+CONTEXT = 4096
+PROMPT = 512
+PREFILL = 2048
+
+
+def weight_bytes(c, esize):
+    per_layer = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
+        + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size \
+        + 2 * c.hidden_size
+    return esize * (c.num_hidden_layers * per_layer + c.vocab_size * c.hidden_size + c.hidden_size)
+
+
+def decode_bytes(c, esize, kv_lens):
+    """Every weight once (the head too; of the embedding only the rows used) and the cache
+    of the live requests."""
+    cache = sum(kv_lens) * 2 * c.num_hidden_layers * c.num_key_value_heads * c.head_dim * esize
+    return weight_bytes(c, esize) + len(kv_lens) * c.hidden_size * esize + cache
+
+
+def prefill_flops(c, T, rows=1):
+    linear = 2 * T * c.num_hidden_layers * (
+        c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim
+        + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size)
+    attention = c.num_hidden_layers * 4 * c.num_attention_heads * c.head_dim * T * (T + 1) // 2
+    return linear + attention + 2 * rows * c.hidden_size * c.vocab_size
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
+                    help="fewer layers than the shape has (reported as such); never smaller layers")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma-separated")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
+        return 2
+
+    import numpy as np
+    import torch
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.engine import Engine
+
+    cfg = g.config_from_dict({**SHAPE, "num_hidden_layers": args.layers})
+    esize = 2 if args.dtype == "bfloat16" else 4
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    K, W = args.steps, args.warmup
+    points = [int(b) for b in args.points.split(",") if b]
+    biggest = max([args.batch] + points)
+    per_seq = -(-(PROMPT + K + W + 1) // 64) * 64
+    tmp = tempfile.mkdtemp(prefix="gl3-bench-")
+    try:
+        t0 = time.time()
+        g.write_random_model(tmp, cfg, args.seed)
+        print(f"[bench] random {args.layers}-layer model written in {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
+        eng = Engine.from_folder(tmp, dtype=args.dtype, max_context=CONTEXT,
+                                 max_tokens=max(biggest * per_seq, PREFILL + 64), n_slots=biggest)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    rng = np.random.default_rng(args.seed)
+    V = cfg.vocab_size
+
+    def sync():
+        torch.cuda.synchronize()
+
+    # ---- prefill: one prompt of 2,048 tokens, logits at its last token
+    def prefill_once():
+        s = eng.take_slot()
+        toks = rng.integers(0, V, PREFILL).tolist()
+        sync(); t = time.perf_counter()
+        eng.step([(s, toks)])
+        sync(); dt = time.perf_counter() - t
+        eng.give_back_slot(s)
+        return dt
+    prefill_once()
+    prefill_s = min(prefill_once() for _ in range(3))
+    print(f"[bench] prefill {PREFILL} tokens: {prefill_s * 1e3:.2f} ms", file=sys.stderr, flush=True)
+
+    # ---- decode at batch B after 512-token prompts
+    def decode(B):
+        slots = [eng.take_slot() for _ in range(B)]
+        for lo in range(0, B, 8):                              # prompts in groups of 8 to bound the step's memory
+            eng.step([(s, rng.integers(0, V, PROMPT).tolist()) for s in slots[lo:lo + 8]], want="none")
+        temps, tops, us = [0.0] * B, [1.0] * B, [0.0] * B
+        toks = rng.integers(0, V, B).tolist()
+
+        def one(toks):
+            logits = eng.step([(s, [t]) for s, t in zip(slots, toks)])
+            return eng.sample(logits, temps, tops, us)
+        for _ in range(W):
+            toks = one(toks)
+        kv = [eng.cache.length(s) for s in slots]
+        sync(); t = time.perf_counter()
+        for _ in range(K):
+            toks = one(toks)
+        sync(); dt = time.perf_counter() - t
+        for s in slots:
+            eng.give_back_slot(s)
+        mean_kv = [n + (K + 1) / 2 for n in kv]               # the cache read grows by one token a step
+        return dt, decode_bytes(cfg, esize, mean_kv)
+
+    results = {}
+    for B in [args.batch] + [b for b in points if b != args.batch]:
+        dt, nbytes = decode(B)
+        results[B] = (dt, nbytes)
+        print(f"[bench] decode B={B}: {dt / K * 1e3:.3f} ms/step, {B * K / dt:.0f} tok/s, "
+              f"{nbytes / (dt / K) / 1e9:.0f} GB/s", file=sys.stderr, flush=True)
+
+    dt, nbytes = results[args.batch]
+    ms = dt / K * 1e3
+    achieved = nbytes / (dt / K) / 1e9
+    flops = prefill_flops(cfg, PREFILL)
+    line = {
+        "metric": "decode tok/s at batch 8 (Llama-3.2-1B shape, 512-token prompts)" if args.batch == 8
+        else f"decode tok/s at batch {args.batch} (Llama-3.2-1B shape, 512-token prompts)",
+        "value": round(args.batch * K / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic: random N(0,0.02) weights, uniform random token ids",
+        "config": {
+            "model": "Llama-3.2-1B shape", "layers": args.layers, "layers_of_shape": SHAPE["num_hidden_layers"],
+            "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
+            "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+            "vocab_size": cfg.vocab_size, "tied_head": cfg.tie_word_embeddings, "rope_theta": cfg.rope_theta,
+            "rope_scaling_factor": cfg.rope_scaling.factor, "rms_norm_eps": cfg.rms_norm_eps,
+            "global_batch": args.batch, "context_length": CONTEXT, "prompt_len": PROMPT,
+            "prefill_len": PREFILL, "parallelism": "single GPU", "sampling": "greedy on device",
+        },
+        "prefill": {"value": round(PREFILL / prefill_s, 1), "tokens": PREFILL, "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(flops / prefill_s / (PEAK_TFLOPS[short] * 1e12), 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBS, 4)},
+        "points": {f"decode_b{B}": round(B * K / results[B][0], 1) for B in results if B != args.batch},
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

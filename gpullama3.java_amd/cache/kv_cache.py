@@ -2,7 +2,8 @@
 
 Entries of the run order with the same needs (kv heads, head size, window, dtype)
 form a group; each group has storage, a page pool and block tables of its own:
-``K, V: [entry in group, page, kv head, position in page, head_dim]``. A page is
+``K: [entry in group, page, kv head, position in page, head_dim]``, ``V`` the same with its
+last two axes exchanged. A page is
 ``page_size`` positions of one sequence for every entry of the group. Beside it
 each entry may own a state area of fixed size per slot, ``[slot, elements]``,
 zeroed when the slot is handed out; the attention of this architecture asks for
@@ -39,9 +40,11 @@ class CacheGroup:
         self.entries = list(entries)
         self.pool = PagePool(n_pages)
         self.page_size = page_size
-        shape = (len(self.entries), n_pages, need.n_kv_heads, page_size, need.head_dim)
-        self.k = torch.zeros(shape, dtype=dtype, device=device)
-        self.v = torch.zeros(shape, dtype=dtype, device=device)
+        n = len(self.entries)
+        self.k = torch.zeros((n, n_pages, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
+        # values lie transposed inside a page (positions contiguous): the order in which the
+        # attention kernels' second product reads them
+        self.v = torch.zeros((n, n_pages, need.n_kv_heads, need.head_dim, page_size), dtype=dtype, device=device)
 
 
 class Cache:
@@ -120,7 +123,7 @@ class Cache:
 
     # ---- what the kernels read
     def layer_kv(self, entry):
-        """(K, V) of one entry: [page, kv head, position in page, head_dim]."""
+        """(K, V) of one entry: K [page, kv head, position in page, head_dim], V [page, kv head, head_dim, position]."""
         g, i = self.group_of[entry]
         return self.groups[g].k[i], self.groups[g].v[i]
 

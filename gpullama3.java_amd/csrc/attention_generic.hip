@@ -54,12 +54,13 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     for (int r = 0; r < ATT_MAX_HS / 64; ++r) acc[r] *= alpha;
     for (int j = 0; j < n_valid; ++j) {
       const int kj = base + j;
-      const T* vp = v_cache + (((long)bt[kj / page_size] * n_kv + c) * page_size + kj % page_size) * head_dim;
+      // values lie transposed in a page: [head_dim][position in page]
+      const T* vp = v_cache + ((long)bt[kj / page_size] * n_kv + c) * page_size * head_dim + kj % page_size;
       const float w = ps[j];
 #pragma unroll
       for (int r = 0; r < ATT_MAX_HS / 64; ++r) {
         const int i = lane + 64 * r;
-        if (i < head_dim) acc[r] = fmaf(w, to_f32<T>(vp[i]), acc[r]);
+        if (i < head_dim) acc[r] = fmaf(w, to_f32<T>(vp[(long)i * page_size]), acc[r]);
       }
     }
     m = m_new;

@@ -74,8 +74,10 @@ extern "C" int gl3_rmsnorm(const float* x, const int* rows, const void* w, int w
 // half pairing; the angle's cos and sin come from a table [position, rot/2]
 // built on the host (J/inference/operation/RoPE.java:29-31). Elements beyond
 // `rot_dim` pass through. A null table means no rotation at all.
-// The cache of one layer is [page][kv head][slot in page][head_dim]; the page of
-// position p of sequence s is block_table[s * table_stride + p / page_size].
+// One layer's key cache is [page][kv head][position in page][head_dim]; its value cache
+// is [page][kv head][head_dim][position in page]: values lie transposed, positions
+// contiguous, which is the operand order the attention kernels' matrix-core products
+// read. The page of position p of sequence s is block_table[s * table_stride + p / page_size].
 template <typename T>
 __global__ void rope_cache_kernel(T* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                                   const int* __restrict__ block_table, int table_stride, const float* __restrict__ cos_tab,
@@ -93,8 +95,12 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const int* __restrict__ p
     if (!write_kv) return;
     const int c = (head - n_heads) % n_kv;
     const int page = block_table[(long)seq_of_token[t] * table_stride + pos / page_size];
-    T* base = (head < n_heads + n_kv) ? k_cache : v_cache;
-    dst = base + (((long)page * n_kv + c) * page_size + pos % page_size) * head_dim;
+    if (head >= n_heads + n_kv) {   // a value head: transposed, no rotation
+      T* vt = v_cache + ((long)page * n_kv + c) * page_size * head_dim + pos % page_size;
+      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) vt[(long)i * page_size] = src[i];
+      return;
+    }
+    dst = k_cache + (((long)page * n_kv + c) * page_size + pos % page_size) * head_dim;
   }
   const bool rotate = cos_tab != nullptr && head < n_heads + n_kv;
   if (!rotate) {

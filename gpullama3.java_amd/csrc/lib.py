@@ -53,6 +53,9 @@ def _declare(lib):
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P],
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P],
+        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P],
+        "gl3_attention_decode_supports": [I, I],
+        "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name, None)
@@ -95,6 +98,14 @@ def _code(t, name):
 
 def _ptr(t):
     return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
+
+
+def _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, who):
+    """Keys [pages, kv heads, page, head_dim]; values transposed [pages, kv heads, head_dim, page]."""
+    if (k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim)
+            or tuple(v_cache.shape) != (k_cache.shape[0], n_kv, head_dim, page_size)):
+        raise KernelError(f"{who}: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for kv {n_kv} "
+                          f"page {page_size} hs {head_dim}")
 
 
 # ------------------------------------------------------------------ ops
@@ -153,8 +164,7 @@ def rope_cache_write(qkv, positions, seq_of_token, block_table, cos, sin, k_cach
         _dev(k_cache, "k_cache", qkv.dtype); _dev(v_cache, "v_cache", qkv.dtype)
         if seq_of_token.numel() != T or block_table.dim() != 2:
             raise KernelError("rope_cache_write: seq_of_token / block_table shapes")
-        if k_cache.shape != v_cache.shape or k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim):
-            raise KernelError(f"rope_cache_write: cache {tuple(k_cache.shape)} for kv {n_kv} page {page_size} hs {head_dim}")
+        _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "rope_cache_write")
         stride = block_table.shape[1]
     _check(library().gl3_rope_cache_write(
         _ptr(qkv), _code(qkv, "qkv"), _ptr(positions), _ptr(seq_of_token), _ptr(block_table), stride,
@@ -190,8 +200,7 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
         raise KernelError(f"attention: q {tuple(q.shape)} for {n_heads} heads of {head_dim}")
     if out.shape != (T, n_heads * head_dim) or out.stride(1) != 1:
         raise KernelError(f"attention: out {tuple(out.shape)}")
-    if k_cache.shape != v_cache.shape or k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim):
-        raise KernelError(f"attention: cache {tuple(k_cache.shape)} for kv {n_kv} page {page_size} hs {head_dim}")
+    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention")
     if positions.numel() != T or seq_of_token.numel() != T or block_table.dim() != 2:
         raise KernelError("attention: positions / seq_of_token / block_table shapes")
     _check(library().gl3_attention_generic(
@@ -211,3 +220,67 @@ def sample(logits, work, temperature, top_p, uniform, out):
         raise KernelError("sample: argument sizes")
     _check(library().gl3_sample(_ptr(logits), logits.stride(0), _ptr(work), _ptr(temperature), _ptr(top_p),
                                 _ptr(uniform), _ptr(out), R, V, _stream()), "sample")
+
+
+# ------------------------------------------------------------------ bfloat16 product for few rows
+def gemm_skinny_fits(a, w, out, epilogue):
+    M, K = a.shape
+    return (M <= 64 and K % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and (out.dtype == torch.float32 or (out.dtype == torch.bfloat16 and epilogue != EPI_ADD)))
+
+
+def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0):
+    """out (=, +=, gated) a @ w.T on the matrix cores for at most 64 rows of ``a``."""
+    _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
+    if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
+    M, K = a.shape
+    N = out.shape[1]
+    rows = 2 * N if epilogue == EPI_GATED else N
+    if w.shape != (rows, K) or out.shape[0] != M:
+        raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
+    _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
+                                     out.stride(0), epilogue, waves, _stream()), "gemm_skinny")
+
+
+# ------------------------------------------------------------------ bfloat16 attention of a decode step
+def attention_decode_fits(head_dim, n_heads, n_kv, page_size):
+    return bool(library().gl3_attention_decode_supports(head_dim, page_size)) and n_heads % n_kv == 0
+
+
+def decode_splits(n_tokens, n_heads, n_kv, kv_len):
+    """Blocks that share a sequence's keys: enough blocks for the chip, a wave keeps at least one
+    chunk of 32 keys."""
+    blocks = n_tokens * n_kv * -(-(n_heads // n_kv) // 16)
+    most = max(1, kv_len // 128)
+    return int(max(1, min(most, -(-768 // blocks), 64)))
+
+
+def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,
+                     page_size, window, scale, n_splits, part_o=None, part_ml=None):
+    """One token per sequence. ``part_o`` [T, H, splits, hs] and ``part_ml`` [T, H, splits, 2] float32
+    are needed when ``n_splits`` > 1 (contiguous, adjacent is not required)."""
+    _dev(q, "q", torch.bfloat16, contiguous=False); _dev(out, "out", torch.bfloat16, contiguous=False)
+    _dev(k_cache, "k_cache", torch.bfloat16); _dev(v_cache, "v_cache", torch.bfloat16)
+    _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
+    _dev(block_table, "block_table", torch.int32)
+    T = q.shape[0]
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < n_heads * head_dim:
+        raise KernelError(f"attention: q {tuple(q.shape)} for {n_heads} heads of {head_dim}")
+    if out.shape != (T, n_heads * head_dim) or out.stride(1) != 1:
+        raise KernelError(f"attention: out {tuple(out.shape)}")
+    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention")
+    if positions.numel() != T or seq_of_token.numel() != T or block_table.dim() != 2:
+        raise KernelError("attention: positions / seq_of_token / block_table shapes")
+    floats = 0
+    if n_splits > 1:
+        _dev(part_o, "part_o", torch.float32); _dev(part_ml, "part_ml", torch.float32)
+        if part_o.numel() < T * n_heads * n_splits * head_dim or part_ml.numel() < T * n_heads * n_splits * 2:
+            raise KernelError("attention: the workspace of the splits is too small")
+        floats = T * n_heads * n_splits * (head_dim + 2)
+    _check(library().gl3_attention_decode(
+        _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
+        block_table.shape[1], _ptr(part_o), _ptr(part_ml), floats, _ptr(out), out.stride(0), T, n_heads, n_kv,
+        head_dim, page_size, int(window or 0), float(scale), n_splits, _stream()), "attention_decode")

@@ -19,6 +19,7 @@ class Workspace:
         self.device = device
         self._flat = {}
         self.frozen = False
+        self.generation = 0        # counts reallocations: captured graphs hold the old addresses
 
     def get(self, name, shape, dtype):
         n = 1
@@ -29,6 +30,8 @@ class Workspace:
         if flat is None or flat.numel() < n:
             if self.frozen:
                 raise RuntimeError(f"workspace buffer {name!r} would grow while its address is fixed")
+            if flat is not None:
+                self.generation += 1
             flat = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._flat[key] = flat
         return flat[:n].view(shape)
@@ -44,6 +47,7 @@ class StepContext:
         self.q_lens, self.kv_before_host, self.slots = q_lens, kv_before_host, slots
         self.decode = decode
         self.max_q_len, self.max_kv_len = max_q_len, max_kv_len
+        self.kv_len_hint = max_kv_len      # what launch shapes are sized for; a replayed graph keeps its own
         self.token_ids = self.positions = self.seq_of_token = self.cu_seqlens = self.kv_before = None
         self.slot_ids = None
         self._tables = []

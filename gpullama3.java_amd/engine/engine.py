@@ -40,11 +40,17 @@ def _require_gpu(device):
     return torch.device(device)
 
 
+class _DecodeGraph:
+    """A captured decode step for one batch bucket: its fixed input buffer and its logits."""
+    graph = logits = host = dev = blank = None
+    width = off_before = off_slots = off_tables = 0
+
+
 class Engine:
     """``config``: a registered architecture's configuration; ``weights``: stored name -> device tensor."""
 
     def __init__(self, config, weights, dtype="bfloat16", device="cuda:0", max_tokens=None, max_context=None,
-                 n_slots=None, page_size=64):
+                 n_slots=None, page_size=64, use_graphs=True):
         self.device = _require_gpu(device)
         self.dtype = _dtype(dtype)
         limit = config.max_position_embeddings
@@ -64,6 +70,14 @@ class Engine:
         self.workspace = Workspace(self.device)
         self.sampler = DeviceSampler(self.device)
         self.metrics = RunMetrics()
+        # Decode steps are replayed from captured graphs when every part's work is made of kernel
+        # launches on the current stream alone and no part keeps per-slot state (a padded entry
+        # of a bucketed batch must not touch a real slot).
+        parts = [p for b in self.model.blocks for p in b.parts()]
+        self.use_graphs = bool(use_graphs and not self.cache.state
+                               and all(getattr(p, "graph_safe", False) for p in parts))
+        self._graphs = {}
+        self._graphs_generation = 0
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -131,6 +145,7 @@ class Engine:
         V = self.spec.vocab_size
         token_ids, positions, seq_of, cu, kv_before, want_rows = [], [], [], [0], [], []
         q_lens = []
+        last_only = True
         for b, (slot, toks) in enumerate(entries):
             toks = [int(t) for t in toks]
             if not toks:
@@ -150,6 +165,7 @@ class Engine:
                 idx = [int(i) for i in want[b]]
                 if any(not 0 <= i < n for i in idx):
                     raise ValueError(f"entry {b}: a wanted place is outside its {n} tokens")
+            last_only = last_only and idx == [n - 1]
             want_rows.extend(cu[-1] + i for i in idx)
             token_ids.extend(toks)
             positions.extend(range(start, start + n))
@@ -160,32 +176,125 @@ class Engine:
         self.cache.reserve({s: n for s, n in zip(slots, q_lens)})      # raises CacheFull, nothing changed
         T = cu[-1]
         max_kv = max(k + n for k, n in zip(kv_before, q_lens))
-        ctx = StepContext(self, T, B, q_lens, kv_before, slots, decode=all(n == 1 for n in q_lens),
-                          max_q_len=max(q_lens), max_kv_len=max_kv)
+        decode = all(n == 1 for n in q_lens)
+        with torch.cuda.device(self.device):
+            if self.use_graphs and decode and last_only:
+                logits = self._step_graph(B, token_ids, positions, slots, max_kv)
+            else:
+                logits = self._step_eager(B, T, token_ids, positions, seq_of, cu, kv_before, slots, want_rows,
+                                          q_lens, decode, max_kv)
+        for s, n in zip(slots, q_lens):
+            self.cache.advance(s, n)
+        return logits
+
+    def _step_eager(self, B, T, token_ids, positions, seq_of, cu, kv_before, slots, want_rows, q_lens, decode, max_kv):
+        ctx = StepContext(self, T, B, q_lens, kv_before, slots, decode=decode, max_q_len=max(q_lens),
+                          max_kv_len=max_kv)
         width = max(1, -(-max_kv // self.cache.page_size))
         tables = [self.cache.block_rows(g, slots, width) for g in range(len(self.cache.groups))]
         flat = token_ids + positions + seq_of + cu + kv_before + slots + want_rows
         for t in tables:
             for row in t:
                 flat.extend(row)
-        with torch.cuda.device(self.device):
-            dev = torch.tensor(flat, dtype=torch.int32).to(self.device)
-            o = 0
+        dev = torch.tensor(flat, dtype=torch.int32).to(self.device)
+        o = 0
 
-            def cut(n):
-                nonlocal o
-                t = dev[o:o + n]
-                o += n
-                return t
+        def cut(n):
+            nonlocal o
+            t = dev[o:o + n]
+            o += n
+            return t
 
-            ctx.token_ids, ctx.positions, ctx.seq_of_token = cut(T), cut(T), cut(T)
-            ctx.cu_seqlens, ctx.kv_before, ctx.slot_ids = cut(B + 1), cut(B), cut(B)
-            rows = cut(len(want_rows))
-            ctx._tables = [cut(B * width).view(B, width) for _ in tables]
-            logits = self.model.forward(ctx, rows)
-        for s, n in zip(slots, q_lens):
-            self.cache.advance(s, n)
-        return logits
+        ctx.token_ids, ctx.positions, ctx.seq_of_token = cut(T), cut(T), cut(T)
+        ctx.cu_seqlens, ctx.kv_before, ctx.slot_ids = cut(B + 1), cut(B), cut(B)
+        rows = cut(len(want_rows))
+        ctx._tables = [cut(B * width).view(B, width) for _ in tables]
+        return self.model.forward(ctx, rows)
+
+    # ------------------------------------------------------------------ decode steps from captured graphs
+    def _step_graph(self, B, token_ids, positions, slots, max_kv):
+        """One token for each of B sequences: the step's index arrays go into a fixed buffer and
+        the captured launches are replayed. The batch is padded to a bucket; a padded entry is a
+        one-token sequence whose block table names the sink page only, so it reads and writes
+        nothing that a real sequence owns, and its logits are not returned."""
+        if self._graphs_generation != self.workspace.generation:
+            self._graphs.clear()                 # a scratch buffer moved: the captured addresses are stale
+            self._graphs_generation = self.workspace.generation
+        B_pad = B if B <= 8 else -(-B // 8) * 8
+        kv_bucket = 256
+        while kv_bucket < max_kv:
+            kv_bucket *= 2
+        key = (B_pad, kv_bucket)
+        dg = self._graphs.get(key)
+        if dg is None:
+            dg = self._capture(B_pad, kv_bucket)
+            if self._graphs_generation != self.workspace.generation:    # the warm-up grew a buffer
+                self._graphs.clear()
+                self._graphs_generation = self.workspace.generation
+                dg = self._capture(B_pad, kv_bucket)
+            self._graphs[key] = dg
+        h = dg.host
+        W = dg.width
+        h[:] = dg.blank
+        h[0:B] = torch.tensor(token_ids, dtype=torch.int32)
+        h[B_pad:B_pad + B] = torch.tensor(positions, dtype=torch.int32)
+        h[dg.off_before:dg.off_before + B] = h[B_pad:B_pad + B]
+        h[dg.off_slots:dg.off_slots + B] = torch.tensor(slots, dtype=torch.int32)
+        for g in range(len(self.cache.groups)):
+            rows = torch.tensor(self.cache.block_rows(g, slots, W), dtype=torch.int32)
+            o = dg.off_tables + g * B_pad * W
+            h[o:o + B * W] = rows.view(-1)
+        dg.dev.copy_(h, non_blocking=True)
+        dg.graph.replay()
+        return dg.logits[:B]
+
+    def _capture(self, B_pad, kv_bucket):
+        W = self.cache.max_pages_per_seq
+        G = len(self.cache.groups)
+        dg = _DecodeGraph()
+        dg.width = W
+        # layout: tokens | positions | seq_of_token | cu_seqlens | kv_before | slots | rows | tables
+        dg.off_before = 3 * B_pad + B_pad + 1
+        dg.off_slots = dg.off_before + B_pad
+        off_rows = dg.off_slots + B_pad
+        dg.off_tables = off_rows + B_pad
+        n = dg.off_tables + G * B_pad * W
+        blank = torch.zeros(n, dtype=torch.int32)
+        ar = torch.arange(B_pad + 1, dtype=torch.int32)
+        blank[2 * B_pad:3 * B_pad] = ar[:B_pad]                   # seq_of_token
+        blank[3 * B_pad:3 * B_pad + B_pad + 1] = ar                # cu_seqlens
+        blank[off_rows:off_rows + B_pad] = ar[:B_pad]             # wanted rows: every entry's only token
+        dg.blank = blank
+        dg.host = torch.zeros(n, dtype=torch.int32).pin_memory()
+        dg.host[:] = blank
+        dg.dev = torch.zeros(n, dtype=torch.int32, device=self.device)
+        dg.dev.copy_(dg.host)
+        ctx = StepContext(self, B_pad, B_pad, [1] * B_pad, [0] * B_pad, [0] * B_pad, decode=True, max_q_len=1,
+                          max_kv_len=kv_bucket)
+        ctx.kv_len_hint = kv_bucket
+        d = dg.dev
+        ctx.token_ids, ctx.positions, ctx.seq_of_token = d[0:B_pad], d[B_pad:2 * B_pad], d[2 * B_pad:3 * B_pad]
+        ctx.cu_seqlens = d[3 * B_pad:4 * B_pad + 1]
+        ctx.kv_before = d[dg.off_before:dg.off_before + B_pad]
+        ctx.slot_ids = d[dg.off_slots:dg.off_slots + B_pad]
+        rows = d[off_rows:off_rows + B_pad]
+        ctx._tables = [d[dg.off_tables + g * B_pad * W:dg.off_tables + (g + 1) * B_pad * W].view(B_pad, W)
+                       for g in range(G)]
+        # once outside a capture: scratch buffers get their sizes, the library is loaded
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.model.forward(ctx, rows)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.workspace.frozen = True
+        try:
+            dg.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(dg.graph):
+                dg.logits = self.model.forward(ctx, rows)
+        finally:
+            self.workspace.frozen = False
+        return dg
 
     # ------------------------------------------------------------------ generation
     def sample(self, logits, temperatures, top_ps, uniforms):

@@ -19,6 +19,8 @@ from .base import build_part, register_part
 
 
 class GQAAttention:
+    graph_safe = True      # kernel launches on the current stream only, sizes fixed by (T, B)
+
     def __init__(self, spec, dtype, device):
         self.spec, self.dtype = spec, dtype
         self.d, self.H, self.Kh, self.hs = spec.hidden, spec.n_heads, spec.n_kv_heads, spec.head_dim

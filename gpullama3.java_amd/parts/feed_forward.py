@@ -11,6 +11,8 @@ from .base import register_part
 
 
 class GatedFeedForward:
+    graph_safe = True      # kernel launches on the current stream only, sizes fixed by (T, B)
+
     def __init__(self, spec, dtype, device):
         if spec.activation != "silu":
             raise ValueError(f"activation {spec.activation!r} is not built (silu)")

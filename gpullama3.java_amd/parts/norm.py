@@ -9,6 +9,8 @@ from .base import register_part
 
 
 class RMSNorm:
+    graph_safe = True      # kernel launches on the current stream only, sizes fixed by (T, B)
+
     def __init__(self, spec, dtype):
         self.dim, self.eps, self.dtype = spec.dim, spec.eps, dtype
         self.name = spec.names["weight"]

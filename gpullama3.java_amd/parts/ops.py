@@ -28,11 +28,18 @@ def linear(a, w, out, epilogue=EPI_STORE):
 
 
 def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale):
-    page = k_cache.shape[2]
+    page = k_cache.shape[2]          # keys are [page, kv head, position in page, head_dim]
     if q.dtype == torch.bfloat16:
         if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
                 and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):
-            return K.attention_decode(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale)
+            T = q.shape[0]
+            splits = K.decode_splits(T, n_heads, n_kv, ctx.kv_len_hint)
+            part_o = part_ml = None
+            if splits > 1:
+                part_o = ctx.buffer("attn_part_o", (T, n_heads, splits, head_dim), torch.float32)
+                part_ml = ctx.buffer("attn_part_ml", (T, n_heads, splits, 2), torch.float32)
+            return K.attention_decode(q, k_cache, v_cache, ctx.positions, ctx.seq_of_token, block_table, out, n_heads,
+                                      n_kv, head_dim, page, window, scale, splits, part_o, part_ml)
         if (not ctx.decode and "attn_prefill" not in disabled and K.has("gl3_attention_prefill")
                 and K.attention_prefill_fits(head_dim, n_heads, n_kv, page)):
             return K.attention_prefill(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale)

@@ -46,7 +46,7 @@ def test_groups_have_storage_of_their_own():
     assert c.groups[0].k.shape == (2, 11, 2, 64, 16) and c.groups[1].k.shape == (1, 11, 1, 64, 32)
     assert c.group_of == {0: (0, 0), 1: (0, 1), 2: (1, 0)}
     k, v = c.layer_kv(1)
-    assert k.shape == (11, 2, 64, 16) and k.data_ptr() == c.groups[0].k[1].data_ptr()
+    assert k.shape == (11, 2, 64, 16) and v.shape == (11, 2, 16, 64) and k.data_ptr() == c.groups[0].k[1].data_ptr()
     assert c.slot_state(1).shape == (4, 6) and c.slot_state(0) is None
 
 

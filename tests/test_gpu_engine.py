@@ -191,3 +191,35 @@ def test_no_gpu_library_no_engine(monkeypatch):
     with pytest.raises(RuntimeError, match="hipcc"):
         lib.rmsnorm(torch.zeros(1, 8, device="cuda"), torch.zeros(8, device="cuda"),
                     torch.zeros(1, 8, device="cuda"), 1e-5)
+
+
+@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+def test_replayed_graphs_equal_plain_launches(name, dtype):
+    """Decode steps replayed from captured graphs, with the batch padded to its bucket and other
+    work of the same engine between the replays, give what the same kernels give when launched
+    one by one."""
+    eager = engine(name, dtype, use_graphs=False, n_slots=16)
+    graph = engine(name, dtype, use_graphs=True, n_slots=16)
+    assert graph.use_graphs and not eager.use_graphs
+    B = 11                                                         # padded to a bucket of 16
+    seqs = [rand_tokens(name, 60 + i, 8 + 5 * i + 12) for i in range(B)]
+    outs = []
+    for eng in (eager, graph):
+        slots = [eng.take_slot() for _ in range(B)]
+        rows = [[] for _ in range(B)]
+        eng.step([(s, q[:8 + 5 * i]) for i, (s, q) in enumerate(zip(slots, seqs))], want="none")
+        for k in range(12):
+            o = eng.step([(s, [q[8 + 5 * i + k]]) for i, (s, q) in enumerate(zip(slots, seqs))]).cpu().numpy()
+            for i in range(B):
+                rows[i].append(o[i])
+            if k % 4 == 1:                                         # eager work between replays: a prompt elsewhere
+                extra = eng.take_slot()
+                eng.step([(extra, rand_tokens(name, k, 30))])
+                eng.give_back_slot(extra)
+        outs.append(rows)
+    assert len(graph._graphs) >= 1
+    for i in range(B):
+        got = np.stack(outs[1][i])
+        np.testing.assert_array_equal(got, np.stack(outs[0][i]))
+        n0 = 8 + 5 * i
+        close(got, plain_logits(name, seqs[i])[n0:n0 + 12], dtype, f"request {i}")

@@ -122,7 +122,7 @@ def paged(seqs_k, seqs_v, n_kv, hs, page, dtype, rng, n_pages=None):
     n_pages = n_pages or sum(need) + 3
     ids = rng.permutation(np.arange(1, n_pages))[:sum(need)].tolist()
     kc = torch.full((n_pages, n_kv, page, hs), 777.0, dtype=TD[dtype])        # garbage where nothing was written
-    vc = torch.full((n_pages, n_kv, page, hs), -777.0, dtype=TD[dtype])
+    vc = torch.full((n_pages, n_kv, hs, page), -777.0, dtype=TD[dtype])       # values lie transposed in a page
     width = max(need)
     table = np.zeros((len(seqs_k), width), np.int32)
     for s, (k, v) in enumerate(zip(seqs_k, seqs_v)):
@@ -132,7 +132,7 @@ def paged(seqs_k, seqs_v, n_kv, hs, page, dtype, rng, n_pages=None):
             chunk = slice(p * page, min(len(k), (p + 1) * page))
             n = chunk.stop - chunk.start
             kc[pid, :, :n] = torch.as_tensor(k[chunk]).to(TD[dtype]).transpose(0, 1)
-            vc[pid, :, :n] = torch.as_tensor(v[chunk]).to(TD[dtype]).transpose(0, 1)
+            vc[pid, :, :, :n] = torch.as_tensor(v[chunk]).to(TD[dtype]).permute(1, 2, 0)
     return kc.to(DEV), vc.to(DEV), torch.as_tensor(table).to(DEV)
 
 
@@ -172,7 +172,7 @@ def test_rope_cache_write(dtype, pairing, H, Kh, hs):
         pid = tab[seq_of[i], positions[i] // page]
         touched[pid] = True
         np.testing.assert_allclose(kcpu[pid, :, positions[i] % page], kr[i], atol=t * 4)
-        np.testing.assert_array_equal(vcpu[pid, :, positions[i] % page], v[i])  # values are copied, never rotated
+        np.testing.assert_array_equal(vcpu[pid, :, :, positions[i] % page], v[i])  # values are copied, never rotated
     # nothing else in the cache moved
     mask = torch.ones_like(kc, dtype=torch.bool)
     for i in range(T):
@@ -184,7 +184,7 @@ def test_rope_position_zero_and_no_table():
     rng = np.random.default_rng(1)
     qkv = rng.standard_normal((2, 4 * 16)).astype(np.float32)
     cos, sin = P.rope_table(8, 16, 10000.0)
-    kc = torch.zeros(3, 1, 64, 16, device=DEV); vc = torch.zeros_like(kc)
+    kc = torch.zeros(3, 1, 64, 16, device=DEV); vc = torch.zeros(3, 1, 16, 64, device=DEV)
     table = dev(np.array([[1], [2]]), torch.int32)
     for cs in ((dev(cos), dev(sin)), (None, None)):
         buf = dev(qkv)
@@ -320,3 +320,93 @@ def test_sample_kernel_frequencies_and_rules():
     assert torch.all(out == int(np.argmax(row)))
     lib.sample(dev(logits), work, dev(np.full(R, 1e-3)), dev(np.full(R, 1.0)), dev(us), out)
     assert torch.all(out == int(np.argmax(row)))                        # T -> 0+ is greedy
+
+
+# ------------------------------------------------------------------ bfloat16 product for few rows (matrix cores)
+@pytest.mark.parametrize("M", [1, 8, 17, 64])
+@pytest.mark.parametrize("N, Kd", [(2048, 2048), (130, 64), (48, 40), (3000, 512), (256, 8192)])
+def test_gemm_skinny(M, N, Kd):
+    rng = np.random.default_rng(M + N)
+    a = rounded(rng.standard_normal((M, Kd)), "bfloat16")
+    w = rounded(rng.standard_normal((2 * N, Kd)) / math.sqrt(Kd), "bfloat16")
+    A, W = dev(a, torch.bfloat16), dev(w, torch.bfloat16)
+    lib = K()
+    ref = P.linear(a, w[:N])
+    scale = np.abs(ref).max()
+    for waves in (0, 4, 8, 16):
+        out = torch.zeros(M, N, device=DEV)
+        lib.gemm_skinny(A, W[:N], out, lib.EPI_STORE, waves=waves)
+        np.testing.assert_allclose(out.cpu().numpy(), ref, atol=2e-5 * scale * math.sqrt(Kd / 64), err_msg=f"waves {waves}")
+        again = torch.zeros(M, N, device=DEV)
+        lib.gemm_skinny(A, W[:N], again, lib.EPI_STORE, waves=waves)       # one order of summation: same bits
+        assert torch.equal(out, again)
+    ob = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+    lib.gemm_skinny(A, W[:N], ob)
+    np.testing.assert_allclose(ob.float().cpu().numpy(), ref, atol=1e-2 * scale)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    x = dev(res)
+    lib.gemm_skinny(A, W[:N], x, lib.EPI_ADD)
+    np.testing.assert_allclose(x.cpu().numpy(), res + ref, atol=2e-5 * scale * math.sqrt(Kd / 64) + 1e-6)
+    refg = P.silu(P.linear(a, w[:N])) * P.linear(a, w[N:])
+    for waves in (0, 8):
+        g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+        lib.gemm_skinny(A, W, g_, lib.EPI_GATED, waves=waves)
+        np.testing.assert_allclose(g_.float().cpu().numpy(), refg, atol=1e-2 * max(np.abs(refg).max(), 1e-3))
+
+
+def test_gemm_skinny_refuses_what_it_cannot_do():
+    lib = K()
+    a = torch.zeros(65, 64, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(32, 64, device=DEV, dtype=torch.bfloat16)
+    assert not lib.gemm_skinny_fits(a, w, torch.zeros(65, 32, device=DEV), lib.EPI_STORE)
+    with pytest.raises(lib.KernelError, match="1..64"):
+        lib.gemm_skinny(a, w, torch.zeros(65, 32, device=DEV))
+    a2 = torch.zeros(4, 36, device=DEV, dtype=torch.bfloat16)
+    assert not lib.gemm_skinny_fits(a2, w[:, :36], torch.zeros(4, 32, device=DEV), lib.EPI_STORE)   # K % 8
+
+
+# ------------------------------------------------------------------ bfloat16 attention of a decode step
+def decode_fn(splits):
+    lib = K()
+
+    def fn(q, kc, vc, positions, seq_of, table, out, H, Kh, hs, page, window, scale):
+        T = q.shape[0]
+        po = torch.empty(T, H, splits, hs, device=DEV) if splits > 1 else None
+        pm = torch.empty(T, H, splits, 2, device=DEV) if splits > 1 else None
+        lib.attention_decode(q, kc, vc, positions, seq_of, table, out, H, Kh, hs, page, window, scale, splits, po, pm)
+    return fn
+
+
+@pytest.mark.parametrize("splits", [1, 3, 8])
+@pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 32), (5, 5, 96), (8, 1, 128), (40, 2, 64)])
+def test_attention_decode(H, Kh, hs, splits):
+    rng = np.random.default_rng(H * hs + splits)
+    lens_before, new = [0, 31, 32, 63, 64, 200, 511, 700], [1] * 8
+    sk, sv, qs = attention_case(rng, H, Kh, hs, lens_before, new, "bfloat16")
+    got, ref = run_attention(decode_fn(splits), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng)
+    np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+
+
+@pytest.mark.parametrize("splits", [1, 4])
+def test_attention_decode_far_key_and_window_edge(splits):
+    rng = np.random.default_rng(19)
+    H, Kh, hs, n = 4, 2, 64, 700
+    k = rng.standard_normal((n, Kh, hs)).astype(np.float32) * 0.1
+    v = rng.standard_normal((n, Kh, hs)).astype(np.float32)
+    q = rng.standard_normal((n, H, hs)).astype(np.float32) * 0.1
+    far = 13
+    k[far, 1] = 0; k[far, 1, 5] = 30.0
+    q[n - 1, 2] = 0; q[n - 1, 2, 5] = 30.0
+    q[n - 1, 0] = 0; q[n - 1, 0, 5] = 30.0
+    k, v, q = (rounded(a, "bfloat16") for a in (k, v, q))
+    got, ref = run_attention(decode_fn(splits), [k], [v], [q], [n - 1], [1], H, Kh, hs, "bfloat16", rng)
+    np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+    np.testing.assert_allclose(got[0, 2], v[far, 1], atol=4e-2)
+    assert np.abs(got[0, 0] - v[far, 0]).max() > 0.3
+    w = 100
+    for hot, inside in ((n - w, True), (n - w - 1, False)):
+        k2 = k.copy(); k2[far, 1] = 0.0; k2[hot, 1] = 0; k2[hot, 1, 5] = 30.0
+        k2 = rounded(k2, "bfloat16")
+        got, ref = run_attention(decode_fn(splits), [k2], [v], [q], [n - 1], [1], H, Kh, hs, "bfloat16", rng, window=w)
+        np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+        assert (np.abs(got[0, 2] - v[hot, 1]).max() < 4e-2) == inside
