@@ -54,7 +54,10 @@ def _declare(lib):
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P],
         "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P],
+        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, P],
         "gl3_attention_decode_supports": [I, I],
+        "gl3_attention_prefill_supports": [I, I],
+        "gl3_attention_prefill": [P, L, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, P],
         "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P],
     }
     for name, args in sigs.items():
@@ -284,3 +287,54 @@ def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, 
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
         block_table.shape[1], _ptr(part_o), _ptr(part_ml), floats, _ptr(out), out.stride(0), T, n_heads, n_kv,
         head_dim, page_size, int(window or 0), float(scale), n_splits, _stream()), "attention_decode")
+
+
+# ------------------------------------------------------------------ bfloat16 product for many rows
+def gemm_mfma_fits(a, w, out, epilogue):
+    M, K = a.shape
+    return (K % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and (out.dtype == torch.float32 or (out.dtype == torch.bfloat16 and epilogue != EPI_ADD)))
+
+
+def gemm_mfma(a, w, out, epilogue=EPI_STORE):
+    """out (=, +=, gated) a @ w.T on the matrix cores, tiled for many rows of ``a``."""
+    _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
+    if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
+    M, K = a.shape
+    N = out.shape[1]
+    rows = 2 * N if epilogue == EPI_GATED else N
+    if w.shape != (rows, K) or out.shape[0] != M:
+        raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
+    _check(library().gl3_gemm_mfma(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
+                                   out.stride(0), epilogue, _stream()), "gemm_mfma")
+
+
+# ------------------------------------------------------------------ bfloat16 attention of a prefill step
+def attention_prefill_fits(head_dim, n_heads, n_kv, page_size):
+    return bool(library().gl3_attention_prefill_supports(head_dim, page_size)) and n_heads % n_kv == 0
+
+
+def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, out, max_q_len, n_heads, n_kv,
+                      head_dim, page_size, window, scale):
+    """Any number of tokens per sequence; ``cu_seqlens`` [B+1] and ``kv_before`` [B] say which tokens
+    of the packed ``q`` belong to which sequence and where they sit in it."""
+    _dev(q, "q", torch.bfloat16, contiguous=False); _dev(out, "out", torch.bfloat16, contiguous=False)
+    _dev(k_cache, "k_cache", torch.bfloat16); _dev(v_cache, "v_cache", torch.bfloat16)
+    _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(kv_before, "kv_before", torch.int32)
+    _dev(block_table, "block_table", torch.int32)
+    T = q.shape[0]
+    B = kv_before.numel()
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < n_heads * head_dim:
+        raise KernelError(f"attention: q {tuple(q.shape)} for {n_heads} heads of {head_dim}")
+    if out.shape != (T, n_heads * head_dim) or out.stride(1) != 1:
+        raise KernelError(f"attention: out {tuple(out.shape)}")
+    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention")
+    if cu_seqlens.numel() != B + 1 or block_table.dim() != 2 or block_table.shape[0] < B or max_q_len < 1:
+        raise KernelError("attention: cu_seqlens / kv_before / block_table shapes")
+    _check(library().gl3_attention_prefill(
+        _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(cu_seqlens), _ptr(kv_before), _ptr(block_table),
+        block_table.shape[1], _ptr(out), out.stride(0), B, int(max_q_len), n_heads, n_kv, head_dim, page_size,
+        int(window or 0), float(scale), _stream()), "attention_prefill")

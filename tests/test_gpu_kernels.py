@@ -410,3 +410,75 @@ def test_attention_decode_far_key_and_window_edge(splits):
         got, ref = run_attention(decode_fn(splits), [k2], [v], [q], [n - 1], [1], H, Kh, hs, "bfloat16", rng, window=w)
         np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
         assert (np.abs(got[0, 2] - v[hot, 1]).max() < 4e-2) == inside
+
+
+# ------------------------------------------------------------------ bfloat16 product for many rows (matrix cores)
+@pytest.mark.parametrize("M, N, Kd", [(65, 130, 64), (128, 128, 64), (200, 257, 136), (300, 64, 2048), (1000, 1000, 112)])
+def test_gemm_mfma(M, N, Kd):
+    rng = np.random.default_rng(M + N + Kd)
+    a = rounded(rng.standard_normal((M, Kd)), "bfloat16")
+    w = rounded(rng.standard_normal((2 * N, Kd)) / math.sqrt(Kd), "bfloat16")
+    A, W = dev(a, torch.bfloat16), dev(w, torch.bfloat16)
+    lib = K()
+    ref = P.linear(a, w[:N])
+    scale = np.abs(ref).max()
+    out = torch.zeros(M, N, device=DEV)
+    lib.gemm_mfma(A, W[:N], out)
+    np.testing.assert_allclose(out.cpu().numpy(), ref, atol=2e-5 * scale * math.sqrt(Kd / 64))
+    ob = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+    lib.gemm_mfma(A, W[:N], ob)
+    np.testing.assert_allclose(ob.float().cpu().numpy(), ref, atol=1e-2 * scale)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    x = dev(res)
+    lib.gemm_mfma(A, W[:N], x, lib.EPI_ADD)
+    np.testing.assert_allclose(x.cpu().numpy(), res + ref, atol=2e-5 * scale * math.sqrt(Kd / 64) + 1e-6)
+    refg = P.silu(P.linear(a, w[:N])) * P.linear(a, w[N:])
+    g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+    lib.gemm_mfma(A, W, g_, lib.EPI_GATED)
+    np.testing.assert_allclose(g_.float().cpu().numpy(), refg, atol=1e-2 * max(np.abs(refg).max(), 1e-3))
+    wide = torch.zeros(M, N + 24, device=DEV, dtype=torch.bfloat16)      # a view with a row stride as output
+    lib.gemm_mfma(A, W[:N], wide[:, 8:8 + N])
+    assert torch.equal(wide[:, 8:8 + N], ob) and torch.all(wide[:, :8] == 0) and torch.all(wide[:, 8 + N:] == 0)
+
+
+# ------------------------------------------------------------------ bfloat16 attention of a prefill step
+def prefill_fn(lens_before, new):
+    lib = K()
+
+    def fn(q, kc, vc, positions, seq_of, table, out, H, Kh, hs, page, window, scale):
+        cu = dev(np.concatenate([[0], np.cumsum(new)]), torch.int32)
+        lib.attention_prefill(q, kc, vc, cu, dev(lens_before, torch.int32), table, out, max(new), H, Kh, hs, page,
+                              window, scale)
+    return fn
+
+
+@pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 32), (5, 5, 96), (8, 1, 128), (12, 2, 64)])
+def test_attention_prefill(H, Kh, hs):
+    rng = np.random.default_rng(H * hs)
+    lens_before, new = [0, 70, 0, 130, 5], [33, 1, 200, 17, 64]      # prompts, chunks after a prefix, one token
+    sk, sv, qs = attention_case(rng, H, Kh, hs, lens_before, new, "bfloat16")
+    got, ref = run_attention(prefill_fn(lens_before, new), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng)
+    np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+
+
+def test_attention_prefill_far_key_and_window_edge():
+    rng = np.random.default_rng(29)
+    H, Kh, hs, n = 4, 2, 64, 700
+    k = rng.standard_normal((n, Kh, hs)).astype(np.float32) * 0.1
+    v = rng.standard_normal((n, Kh, hs)).astype(np.float32)
+    q = rng.standard_normal((n, H, hs)).astype(np.float32) * 0.1
+    far = 13
+    k[far, 1] = 0; k[far, 1, 5] = 30.0
+    q[n - 1, 2] = 0; q[n - 1, 2, 5] = 30.0
+    k, v, q = (rounded(a, "bfloat16") for a in (k, v, q))
+    for before, new in ((0, n), (500, 200)):                       # the whole prompt; a chunk after a prefix
+        got, ref = run_attention(prefill_fn([before], [new]), [k], [v], [q], [before], [new], H, Kh, hs, "bfloat16", rng)
+        np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+        np.testing.assert_allclose(got[-1, 2], v[far, 1], atol=4e-2)
+    w = 100
+    for hot, inside in ((n - w, True), (n - w - 1, False)):
+        k2 = k.copy(); k2[far, 1] = 0.0; k2[hot, 1] = 0; k2[hot, 1, 5] = 30.0
+        k2 = rounded(k2, "bfloat16")
+        got, ref = run_attention(prefill_fn([0], [n]), [k2], [v], [q], [0], [n], H, Kh, hs, "bfloat16", rng, window=w)
+        np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+        assert (np.abs(got[-1, 2] - v[hot, 1]).max() < 4e-2) == inside
