@@ -120,18 +120,25 @@ def main():
         slots = [eng.take_slot() for _ in range(B)]
         for lo in range(0, B, 8):                              # prompts in groups of 8 to bound the step's memory
             eng.step([(s, rng.integers(0, V, PROMPT).tolist()) for s in slots[lo:lo + 8]], want="none")
-        temps, tops, us = [0.0] * B, [1.0] * B, [0.0] * B
+        temps, tops = [0.0] * B, [1.0] * B
         toks = rng.integers(0, V, B).tolist()
+        run = eng.decode_run_length
 
-        def one(toks):
-            logits = eng.step([(s, [t]) for s, t in zip(slots, toks)])
-            return eng.sample(logits, temps, tops, us)
-        for _ in range(W):
-            toks = one(toks)
+        def steps(toks, n):
+            """n decode steps: runs of steps on the device, the tokens fed back there, as the
+            generation loop does it."""
+            while n > 0:
+                m = min(run, n)
+                if m > 1:
+                    toks = eng.decode_run(list(zip(slots, toks)), m, temps, tops, [[0.0] * B] * m)[-1]
+                else:
+                    toks = eng.sample(eng.step([(s, [t]) for s, t in zip(slots, toks)]), temps, tops, [0.0] * B)
+                n -= m
+            return toks
+        toks = steps(toks, W)
         kv = [eng.cache.length(s) for s in slots]
         sync(); t = time.perf_counter()
-        for _ in range(K):
-            toks = one(toks)
+        toks = steps(toks, K)
         sync(); dt = time.perf_counter() - t
         for s in slots:
             eng.give_back_slot(s)

@@ -6,13 +6,17 @@
 // lo..p, softmax, weighted sum of the values; query head h reads kv head h / (H/K).
 //
 // A block works on (token, kv head, group of up to 16 query heads, split of the key
-// range); its four waves take chunks of 32 keys in turn. Per chunk, transposed:
+// range); its NW waves take chunks of 32 keys in turn, and a wave asks for the keys and
+// values of CB chunks at once before it works on the first: the work per chunk is short
+// next to a trip to memory, so the trips must overlap. Per chunk, transposed:
 //   S^T[key, head]  = K[key, :] . Q[head, :]^T      two 16x16 tiles, k = head_dim
 //   O^T[dim, head] += V^T[dim, key] . P^T[key, head]  head_dim/16 tiles, k = 32 keys
 // so a lane's 16 bytes of a key row, and of a row of the transposed value page, are the
 // operands as the instruction wants them, and the probabilities leave the first
-// product in the register order the second one takes (the 32 keys of a chunk are
-// consumed in the order 4q..4q+3, 16+4q..16+4q+3 by both operands). Softmax keeps a
+// product in the register order the second one takes: row i of the first score tile is
+// key 8*(i/4) + i%4 of the chunk and row i of the second is the key 4 further, so that
+// quarter q of the lanes ends up with keys 8q..8q+7, which is one 16-byte load from a
+// row of the transposed value page. Softmax keeps a
 // running maximum and sum per head in 32-bit. The waves' partial results are merged
 // in shared memory; with more than one split each block writes (max, sum, O) to a
 // workspace and a second kernel merges the splits in split order.
@@ -22,34 +26,36 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-template <int HS>
-__global__ __launch_bounds__(256) void attention_decode_kernel(
+template <int HS, int NW, int CB>
+__global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out,
     long out_stride, int n_heads, int n_kv, int page_size, int window, float scale, int n_splits) {
   constexpr int KK = HS / 32;   // k-steps of the first product
   constexpr int DT = HS / 16;   // row tiles of the second product
-  __shared__ float sm_m[4][16], sm_l[4][16];
-  __shared__ f32x4 sm_o[4][DT][64];
+  __shared__ float sm_m[NW][16], sm_l[NW][16];
+  __shared__ f32x4 sm_o[NW][DT][64];
   const int g = n_heads / n_kv;
   const int groups = (g + 15) / 16;
   const int t = blockIdx.x / (n_kv * groups);
   const int c = (blockIdx.x / groups) % n_kv;
   const int hg = blockIdx.x % groups;
   const int split = blockIdx.y;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // the wave's number as a scalar: what depends on it alone (chunk, page) then lives in scalar
+  // registers and its table look-ups are scalar loads, not a trip to memory per lane
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int j = lane & 15, qd = lane >> 4;
   const int heads_here = min(16, g - hg * 16);
   const int h0 = c * g + hg * 16;
 
-  const int kv_len = positions[t] + 1;
+  const int kv_len = __builtin_amdgcn_readfirstlane(positions[t]) + 1;
   const int lo = (window > 0 && kv_len > window) ? kv_len - window : 0;
   const int chunk_lo = lo / 32, chunk_hi = (kv_len + 31) / 32;
   const int per_split = (chunk_hi - chunk_lo + n_splits - 1) / n_splits;
   const int c_begin = chunk_lo + split * per_split;
   const int c_end = min(chunk_hi, c_begin + per_split);
-  const int* bt = block_table + (long)seq_of_token[t] * table_stride;
+  const int* bt = block_table + (long)__builtin_amdgcn_readfirstlane(seq_of_token[t]) * table_stride;
 
   // Q^T operand: lane (head j, quarter qd) holds Q[h0 + j][kk*32 + 8*qd .. +7]
   bf16x8 qt[KK];
@@ -63,61 +69,75 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int ck = c_begin + wave; ck < c_end; ck += 4) {
-    const int key0 = ck * 32;
-    const long page = bt[key0 / page_size];
-    const int po = key0 % page_size;
-    const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
-    const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + po;
-    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+  for (int ck0 = c_begin + wave; ck0 < c_end; ck0 += NW * CB) {
+    // operands of CB chunks, all asked for before any is used
+    bf16x8 ka[CB][KK], kb2[CB][KK], vt[CB][DT];
+    const int krow = 8 * (j >> 2) + (j & 3);   // which key of the chunk is row j of the first score tile
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      const bf16x8 ka = *(const bf16x8*)(kb + (long)j * HS + kk * 32 + 8 * qd);
-      const bf16x8 kb2 = *(const bf16x8*)(kb + (long)(16 + j) * HS + kk * 32 + 8 * qd);
-      sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qt[kk], sa, 0, 0, 0);
-      sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb2, qt[kk], sb, 0, 0, 0);
+    for (int b = 0; b < CB; ++b) {
+      const int ck = ck0 + b * NW;
+      if (ck < c_end) {
+        const int key0 = ck * 32;
+        const long page = __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
+        const int po = key0 % page_size;
+        const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
+        const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + po;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          ka[b][kk] = *(const bf16x8*)(kb + (long)krow * HS + kk * 32 + 8 * qd);
+          kb2[b][kk] = *(const bf16x8*)(kb + (long)(krow + 4) * HS + kk * 32 + 8 * qd);
+        }
+        // values: lane (dim j of the tile, quarter qd) takes keys 8qd..8qd+7 of the chunk
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vt[b][dt] = *(const bf16x8*)(vb + (long)(dt * 16 + j) * page_size + 8 * qd);
+      }
     }
-    // values: lane (dim i = j, quarter qd) takes keys 4qd..4qd+3 and 16+4qd..16+4qd+3 of the chunk
-    bf16x8 vt[DT];
+    __builtin_amdgcn_sched_barrier(0);   // every load above is issued before the first is waited for
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const bf16_t* vr = vb + (long)(dt * 16 + j) * page_size + 4 * qd;
-      const bf16x4 v0 = *(const bf16x4*)vr, v1 = *(const bf16x4*)(vr + 16);
-      vt[dt] = bf16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-    }
-    // lane (head j, quarter qd) holds scores of keys key0 + 4qd + v (sa) and key0 + 16 + 4qd + v (sb)
-    float s[8];
-    float mx = -INFINITY;
+    for (int b = 0; b < CB; ++b) {
+      const int ck = ck0 + b * NW;
+      if (ck >= c_end) break;
+      const int key0 = ck * 32;
+      f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int ka_i = key0 + 4 * qd + v, kb_i = ka_i + 16;
-      s[v] = (ka_i >= lo && ka_i < kv_len) ? sa[v] * scale : -INFINITY;
-      s[4 + v] = (kb_i >= lo && kb_i < kv_len) ? sb[v] * scale : -INFINITY;
-      mx = fmaxf(mx, fmaxf(s[v], s[4 + v]));
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = __expf(m_run - m_use);   // m_run = -inf gives 0
-    float ps = 0.f;
-    bf16x8 pb;
+      for (int kk = 0; kk < KK; ++kk) {
+        sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[b][kk], qt[kk], sa, 0, 0, 0);
+        sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb2[b][kk], qt[kk], sb, 0, 0, 0);
+      }
+      // lane (head j, quarter qd) holds scores of keys key0 + 8qd + v (sa) and key0 + 8qd + 4 + v (sb)
+      float s[8];
+      float mx = -INFINITY;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float p = __expf(s[e] - m_use);
-      ps += p;
-      pb[e] = static_cast<bf16_t>(p);
-    }
-    l_run = l_run * alpha + ps;
-    m_run = m_new;
+      for (int v = 0; v < 4; ++v) {
+        const int ka_i = key0 + 8 * qd + v, kb_i = ka_i + 4;
+        s[v] = (ka_i >= lo && ka_i < kv_len) ? sa[v] * scale : -INFINITY;
+        s[4 + v] = (kb_i >= lo && kb_i < kv_len) ? sb[v] * scale : -INFINITY;
+        mx = fmaxf(mx, fmaxf(s[v], s[4 + v]));
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __expf(m_run - m_use);   // m_run = -inf gives 0
+      float ps = 0.f;
+      bf16x8 pb;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      o[dt] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt], pb, o[dt], 0, 0, 0);
+      for (int e = 0; e < 8; ++e) {
+        const float p = __expf(s[e] - m_use);
+        ps += p;
+        pb[e] = static_cast<bf16_t>(p);
+      }
+      l_run = l_run * alpha + ps;
+      m_run = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        o[dt] *= alpha;
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[b][dt], pb, o[dt], 0, 0, 0);
+      }
     }
   }
 
-  // merge the four waves
+  // merge the waves, in wave order
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
   if (qd == 0) { sm_m[wave][j] = m_run; sm_l[wave][j] = l_run; }
@@ -126,18 +146,18 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   __syncthreads();
   float M = sm_m[0][j];
 #pragma unroll
-  for (int w = 1; w < 4; ++w) M = fmaxf(M, sm_m[w][j]);
-  float f[4], L = 0.f;
+  for (int w = 1; w < NW; ++w) M = fmaxf(M, sm_m[w][j]);
+  float f[NW], L = 0.f;
 #pragma unroll
-  for (int w = 0; w < 4; ++w) {
+  for (int w = 0; w < NW; ++w) {
     f[w] = sm_m[w][j] == -INFINITY ? 0.f : __expf(sm_m[w][j] - M);
     L += f[w] * sm_l[w][j];
   }
   const int h = h0 + j;
-  for (int dt = wave; dt < DT; dt += 4) {
+  for (int dt = wave; dt < DT; dt += NW) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < 4; ++w) acc += sm_o[w][dt][lane] * f[w];
+    for (int w = 0; w < NW; ++w) acc += sm_o[w][dt][lane] * f[w];
     if (j >= heads_here) continue;
     const int dim = dt * 16 + 4 * qd;   // lane holds O^T[dim .. dim+3][head j]
     if (n_splits == 1) {
@@ -204,9 +224,10 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
   const int groups = (n_heads / n_kv + 15) / 16;
   const long blocks = (long)n_tokens * n_kv * groups;
   GL3_REQUIRE(blocks < (1L << 31), "gl3_attention_decode: too many blocks");
-  dim3 grid((unsigned)blocks, n_splits), block(256);
+  dim3 grid((unsigned)blocks, n_splits);
+  // 8 waves where their partial results fit the block's shared memory, else 4
 #define GO(HS)                                                                                                        \
-  attention_decode_kernel<HS><<<grid, block, 0, stream>>>(                                                            \
+  attention_decode_kernel<HS, (HS <= 64 ? 8 : 4), (HS <= 64 ? 4 : 2)><<<grid, dim3(HS <= 64 ? 512 : 256), 0, stream>>>(  \
       (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token, block_table, \
       table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, n_splits)
   switch (head_dim) {

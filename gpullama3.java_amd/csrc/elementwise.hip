@@ -4,21 +4,35 @@
 
 // ----------------------------------------------------------------- embedding
 // out[t, :] = table[ids[t], :] as float (J/inference/InferenceCore.java:69).
+// ssq (may be null; then n_tokens <= 64): ssq[t] = sum of squares of row t, for a norm that is
+// folded into the product that follows.
 template <typename TW>
-__global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out, int d) {
+__global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out, int d,
+                             float* __restrict__ ssq) {
+  __shared__ float scratch[16];
   const long t = blockIdx.x;
   const TW* row = table + (long)ids[t] * d;
   float* o = out + t * d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = to_f32<TW>(row[i]);
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const float v = to_f32<TW>(row[i]);
+    o[i] = v;
+    ss += v * v;
+  }
+  if (ssq) {
+    ss = block_sum(ss, scratch);
+    if (threadIdx.x == 0) ssq[t] = ss;
+  }
 }
 
 extern "C" int gl3_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens, int d,
-                         hipStream_t stream) {
+                         float* ssq, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(table && ids && out && n_tokens > 0 && d > 0, "gl3_embed: bad arguments (T=%d d=%d)", n_tokens, d);
+  GL3_REQUIRE(!ssq || n_tokens <= 64, "gl3_embed: sums of squares are kept for at most 64 rows");
   dim3 grid(n_tokens), block(256);
-  if (table_dtype == GL3_F32) embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, ids, out, d);
-  else if (table_dtype == GL3_BF16) embed_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)table, ids, out, d);
+  if (table_dtype == GL3_F32) embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, ids, out, d, ssq);
+  else if (table_dtype == GL3_BF16) embed_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)table, ids, out, d, ssq);
   else GL3_REQUIRE(false, "gl3_embed: unknown dtype %d", table_dtype);
   GL3_LAUNCH_CHECK();
   return 0;
@@ -148,6 +162,36 @@ extern "C" int gl3_rope_cache_write(void* qkv, int dtype, const int* positions, 
                                                           (bf16_t*)v_cache, n_heads, n_kv, head_dim, rot_dim, adjacent,
                                                           page_size, write_kv, row_stride);
   else GL3_REQUIRE(false, "gl3_rope_cache_write: unknown dtype %d", dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- between the steps of a run
+// After a decode step whose tokens were sampled on the device: the sampled tokens become the next
+// step's input, each sequence moves on by one position, the tokens are kept in a history row, and
+// the step counter goes up. One block; n <= 1024.
+__global__ void decode_advance_kernel(int* __restrict__ token_ids, int* __restrict__ positions,
+                                      int* __restrict__ kv_before, const int* __restrict__ sampled,
+                                      int* __restrict__ history, int history_stride, int* __restrict__ step, int n) {
+  const int i = threadIdx.x;
+  const int s = step[0];
+  __syncthreads();
+  if (i < n) {
+    const int t = sampled[i];
+    token_ids[i] = t;
+    history[(long)s * history_stride + i] = t;
+    positions[i] += 1;
+    kv_before[i] += 1;
+  }
+  if (i == 0) step[0] = s + 1;
+}
+
+extern "C" int gl3_decode_advance(int* token_ids, int* positions, int* kv_before, const int* sampled, int* history,
+                                  int history_stride, int* step, int n, hipStream_t stream) {
+  GL3_REQUIRE(token_ids && positions && kv_before && sampled && history && step, "gl3_decode_advance: null argument");
+  GL3_REQUIRE(n > 0 && n <= 1024 && history_stride >= n, "gl3_decode_advance: n=%d stride=%d", n, history_stride);
+  decode_advance_kernel<<<dim3(1), dim3(1024), 0, stream>>>(token_ids, positions, kv_before, sampled, history,
+                                                            history_stride, step, n);
   GL3_LAUNCH_CHECK();
   return 0;
 }

@@ -11,64 +11,144 @@
 // chip a block that waits for another block's stores has to push them through the
 // per-XCD second-level caches, which costs more than the product itself.
 //
-// Epilogues as in gemm_generic.hip: store, add into a float matrix, gated
-// (silu(gate) * up with the up rows `N` rows below the gate rows).
+// A decode step is a chain of small kernels, each of which costs a few microseconds
+// before it does any work, so what would be kernels of their own is folded into the
+// products' ends:
+//  * XNORM: A is the float residual stream and the product is that of its RMSNorm
+//    (J/inference/InferenceCore.java:47-56): a lane multiplies x by the norm's weight as
+//    it loads it, and the row's 1/rms, which is a factor of the whole row, is applied to
+//    the sums at the end. The sum of squares of a row arrives as partial sums (one per
+//    16 columns of the row, written by the kernel that produced the row), added up here
+//    in a fixed order.
+//  * SSQ: the add epilogue also writes those partial sums of squares of the rows it
+//    completes, for the norm that follows.
+//  * SK_QKV: the rows of W are [q heads | k heads | v heads]; the end rotates q and k by
+//    the token's position and writes q to its buffer, k and v into the paged cache
+//    (J/inference/InferenceCore.java:83-101). For half-split pairing a strip is made of 8
+//    rows and the 8 rows half a head further, so both elements of a pair are in one tile.
+// Other epilogues as in gemm_generic.hip: store, add into a float matrix, gated.
+//
+// Two kernels share the strip's end. The streaming one reloads its share of A for every
+// strip and takes any K. The resident one is for K up to 32*NW*KS: a wave keeps the A
+// operands of its own k-steps in registers (with the norm's weight already applied) and
+// the block walks over several strips with them, asking for the next strip's rows of W
+// before it finishes the current strip; then the first-level cache carries W and nothing
+// else, which is what limits the streaming kernel when the same A is read for every strip.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-enum { SK_STORE = 0, SK_ADD = 1, SK_GATED = 2 };
+enum { SK_STORE = 0, SK_ADD = 1, SK_GATED = 2, SK_QKV = 3 };
 
-#define SK_UNROLL 8
+struct SkNorm {
+  const float* weight;    // [K] norm weight, float
+  const float* ssq;       // [n_partials][64] partial sums of squares of the rows of A
+  int n_partials;
+  float eps;
+  const int* rows;        // may be null: row m of the product reads row rows[m] of A
+};
 
-template <int MT, int NW, int EPI, typename TC>
-__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
-                                                              TC* __restrict__ C, int M, int N, int K, long lda,
-                                                              long ldw, long ldc) {
+struct SkRope {
+  const int* positions;
+  const int* seq_of_token;
+  const int* block_table;
+  int table_stride;
+  const float* cos_tab;   // null: no rotation
+  const float* sin_tab;
+  bf16_t* k_cache;
+  bf16_t* v_cache;
+  int n_heads, n_kv, head_dim, adjacent, page_size;
+};
+
+// Which row of W is row r of a strip's tile, and for SK_QKV which head the strip belongs to.
+template <int EPI>
+__device__ __forceinline__ int sk_strip_row(int strip, int r, int N, const SkRope& rp, int& hd, int& sub, bool& rotated) {
+  int wr = min(strip * 16 + r, N - 1);
+  hd = 0; sub = 0; rotated = false;
+  if (EPI == SK_QKV) {
+    const int per_head = rp.head_dim / 16;
+    hd = strip / per_head;
+    sub = strip % per_head;
+    rotated = rp.cos_tab != nullptr && hd < rp.n_heads + rp.n_kv;
+    if (rotated && !rp.adjacent)
+      wr = hd * rp.head_dim + 8 * sub + (r < 8 ? r : rp.head_dim / 2 + r - 8);
+  }
+  return wr;
+}
+
+template <bool XNORM>
+__device__ __forceinline__ const void* sk_x_row(const void* Av, long lda, int m, const SkNorm& nrm) {
+  if (XNORM) {
+    if (nrm.rows) m = nrm.rows[m];
+    return (const float*)Av + (long)m * lda;
+  }
+  return (const bf16_t*)Av + (long)m * lda;
+}
+
+// A operands of one k-step for MT token tiles: elements k .. k+7 of each tile's row.
+template <int MT, bool XNORM>
+__device__ __forceinline__ void sk_load_x(bf16x8 (&xf)[MT], const void* const (&xrow)[MT], int k, bool ok,
+                                          const SkNorm& nrm) {
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  if (XNORM) {
+    const float* gp = (const float*)nrm.weight + k;
+    const f32x4 g0 = ok ? *(const f32x4*)gp : zero4;
+    const f32x4 g1 = ok ? *(const f32x4*)(gp + 4) : zero4;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const float* xp = (const float*)xrow[mt] + k;
+      const f32x4 x0 = ok ? *(const f32x4*)xp : zero4;
+      const f32x4 x1 = ok ? *(const f32x4*)(xp + 4) : zero4;
+      bf16x8 h;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        h[e] = static_cast<bf16_t>(g0[e] * x0[e]);
+        h[4 + e] = static_cast<bf16_t>(g1[e] * x1[e]);
+      }
+      xf[mt] = h;
+    }
+  } else {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xf[mt] = ok ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
+  }
+}
+
+// Partial sums of squares of the rows: wave w adds the partials w, w+NW, ... of row `lane`.
+template <int NW>
+__device__ __forceinline__ void sk_ssq_partials(float (*sm_ssq)[64], int M, const SkNorm& nrm) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float sp = 0.f;
+  if (lane < M) {
+    const int row = nrm.rows ? nrm.rows[lane] : lane;   // the partial sums are stored by row of A
+    for (int p0 = wave; p0 < nrm.n_partials; p0 += NW * 16) {
+      float v[16];   // sixteen loads in flight, then added in order
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int p = p0 + NW * i;
+        v[i] = p < nrm.n_partials ? nrm.ssq[(long)p * 64 + row] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sp += v[i];
+    }
+  }
+  sm_ssq[wave][lane] = sp;
+}
+
+// The end of a strip: the waves' partial tiles are summed in wave order by the wave that owns
+// the tile, then the epilogue runs. `sub`, `hd`, `rotated` describe the strip for SK_QKV.
+template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ>
+__device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 1) * MT][64], float (*sm_ssq)[64],
+                                          const f32x4 (&acc)[(EPI == SK_GATED) ? 2 : 1][MT], int strip, int hd, int sub,
+                                          bool rotated, TC* __restrict__ C, int M, int N, int K, long ldc,
+                                          const SkNorm& nrm, float* __restrict__ ssq_out, const SkRope& rp) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
-  __shared__ f32x4 red[NW][NG * MT][64];
-  const int strip = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
   const int n0 = strip * 16;
-  const int wr = min(n0 + r, N - 1);
-  const bf16_t* wrow = W + (long)wr * ldw + q * 8;
-  const bf16_t* urow = wrow + (long)N * ldw;  // up rows (gated only)
-  const bf16_t* xrow[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xrow[mt] = A + (long)min(mt * 16 + r, M - 1) * lda + q * 8;
-
-  const int steps = (K + 31) / 32;   // k-steps of 32
-  f32x4 acc[NG][MT];
-#pragma unroll
-  for (int g = 0; g < NG; ++g)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-
-  for (int s0 = wave; s0 < steps; s0 += NW * SK_UNROLL) {
-    bf16x8 wf[SK_UNROLL], uf[SK_UNROLL], xf[SK_UNROLL][MT];
-#pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u) {
-      const int k = (s0 + NW * u) * 32;
-      const bool ok = k + q * 8 < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
-      wf[u] = ok ? *(const bf16x8*)(wrow + k) : zero;
-      if (EPI == SK_GATED) uf[u] = ok ? *(const bf16x8*)(urow + k) : zero;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) xf[u][mt] = ok ? *(const bf16x8*)(xrow[mt] + k) : zero;
-    }
-#pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        acc[0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u][mt], acc[0][mt], 0, 0, 0);
-        if (EPI == SK_GATED) acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u], xf[u][mt], acc[1][mt], 0, 0, 0);
-      }
-    }
-  }
-
-  // the waves' partial tiles, summed in wave order by the wave that owns the tile
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int g = 0; g < NG; ++g)
 #pragma unroll
@@ -81,36 +161,329 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
     red[0][t][lane] = v;   // only this thread touches red[*][t][lane] before the barrier
   }
   __syncthreads();
-  // epilogue: lane holds C[mt*16 + r][n0 + 4q .. +3]
+
+  // epilogue: lane holds tile rows 4q .. 4q+3 (columns of C) of token mt*16 + r
   for (int mt = wave; mt < MT; mt += NW) {
     const int m = mt * 16 + r;
-    if (m >= M) continue;
+    const bool m_ok = m < M;
     f32x4 v = red[0][mt][lane];
+    f32x4 up = (EPI == SK_GATED) ? red[0][MT + mt][lane] : zero4;
+    if (XNORM) {
+      float ss = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) ss += sm_ssq[w][min(m, 63)];
+      const float rms = 1.0f / sqrtf(ss / (float)K + nrm.eps);
+      v *= rms;
+      up *= rms;
+    }
     if (EPI == SK_GATED) {
-      const f32x4 up = red[0][MT + mt][lane];
 #pragma unroll
       for (int c = 0; c < 4; ++c) v[c] = v[c] / (1.0f + __expf(-v[c])) * up[c];
     }
+    if (EPI == SK_QKV) {
+      const int hs = rp.head_dim;
+      const int pos = m_ok ? rp.positions[m] : 0;
+      int col = 16 * sub + 4 * q;          // first of this lane's 4 columns inside the head
+      if (rotated) {
+        const int half = hs / 2;
+        if (rp.adjacent) {
+          const int jj = (16 * sub + 4 * q) / 2;
+          const float c0 = rp.cos_tab[(long)pos * half + jj], s0 = rp.sin_tab[(long)pos * half + jj];
+          const float c1 = rp.cos_tab[(long)pos * half + jj + 1], s1 = rp.sin_tab[(long)pos * half + jj + 1];
+          const f32x4 o = v;
+          v[0] = o[0] * c0 - o[1] * s0;
+          v[1] = o[0] * s0 + o[1] * c0;
+          v[2] = o[2] * c1 - o[3] * s1;
+          v[3] = o[2] * s1 + o[3] * c1;
+        } else {
+          // quarters 0,1 hold the first elements of 8 pairs, quarters 2,3 their partners
+          const bool first = q < 2;
+          const int jj = 8 * sub + 4 * (q & 1);
+          col = (first ? 0 : half) + jj;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const float other = __shfl_xor(v[c], 32, 64);
+            const float co = rp.cos_tab[(long)pos * half + jj + c], si = rp.sin_tab[(long)pos * half + jj + c];
+            v[c] = first ? v[c] * co - other * si : other * si + v[c] * co;
+          }
+        }
+      }
+      if (m_ok) {
+        if (hd < rp.n_heads) {
+          bf16x4 o4;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) o4[c] = static_cast<bf16_t>(v[c]);
+          *(bf16x4*)((bf16_t*)C + (long)m * ldc + (long)hd * hs + col) = o4;
+        } else {
+          const long page = rp.block_table[(long)rp.seq_of_token[m] * rp.table_stride + pos / rp.page_size];
+          const int in_page = pos % rp.page_size;
+          if (hd < rp.n_heads + rp.n_kv) {
+            const int ch = hd - rp.n_heads;
+            bf16x4 o4;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) o4[c] = static_cast<bf16_t>(v[c]);
+            *(bf16x4*)(rp.k_cache + ((page * rp.n_kv + ch) * rp.page_size + in_page) * hs + col) = o4;
+          } else {
+            const int ch = hd - rp.n_heads - rp.n_kv;
+            bf16_t* vt = rp.v_cache + (page * rp.n_kv + ch) * (long)rp.page_size * hs + in_page;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) vt[(long)(col + c) * rp.page_size] = static_cast<bf16_t>(v[c]);
+          }
+        }
+      }
+      continue;
+    }
     const int n = n0 + 4 * q;
     TC* cp = C + (long)m * ldc + n;
+    float sq = 0.f;
+    if (m_ok) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      if (n + c < N) {
-        if (EPI == SK_ADD) cp[c] = from_f32<TC>(to_f32<TC>(cp[c]) + v[c]);
-        else cp[c] = from_f32<TC>(v[c]);
+      for (int c = 0; c < 4; ++c) {
+        if (n + c < N) {
+          float o = v[c];
+          if (EPI == SK_ADD) o += to_f32<TC>(cp[c]);
+          cp[c] = from_f32<TC>(o);
+          sq += o * o;
+        }
       }
+    }
+    if (SSQ) {
+      sq += __shfl_xor(sq, 16, 64);
+      sq += __shfl_xor(sq, 32, 64);
+      if (q == 0 && m_ok) ssq_out[(long)strip * 64 + m] = sq;
     }
   }
 }
 
-template <int MT, int EPI, typename TC>
-static int launch_skinny(int nw, const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw,
-                         long ldc, hipStream_t stream) {
+template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __restrict__ Av, const bf16_t* __restrict__ W,
+                                                              TC* __restrict__ C, int M, int N, int K, long lda,
+                                                              long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out,
+                                                              SkRope rp) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
-  dim3 grid((N + 15) / 16);
-#define GO(NW)                                                                                                       \
-  gemm_skinny_kernel<MT, NW, EPI, TC><<<grid, dim3(NW * 64), 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, (TC*)C, \
-                                                                          M, N, K, lda, ldw, ldc)
+  constexpr int UNROLL = XNORM ? 4 : 8;
+  __shared__ f32x4 red[NW][NG * MT][64];
+  __shared__ float sm_ssq[XNORM ? NW : 1][64];
+  const int strip = blockIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+  int hd, sub;
+  bool rotated;
+  const int wr = sk_strip_row<EPI>(strip, r, N, rp, hd, sub, rotated);
+  const bf16_t* wrow = W + (long)wr * ldw + q * 8;
+  const bf16_t* urow = wrow + (long)N * ldw;  // up rows (gated only)
+  const void* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = sk_x_row<XNORM>(Av, lda, min(mt * 16 + r, M - 1), nrm) ;
+  if (XNORM) sk_ssq_partials<NW>(sm_ssq, M, nrm);
+
+  const int steps = (K + 31) / 32;   // k-steps of 32
+  f32x4 acc[NG][MT];
+#pragma unroll
+  for (int g = 0; g < NG; ++g)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  for (int s0 = wave; s0 < steps; s0 += NW * UNROLL) {
+    bf16x8 wf[UNROLL], uf[UNROLL], xf[UNROLL][MT];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int k = (s0 + NW * u) * 32;
+      const bool ok = k + q * 8 < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
+      wf[u] = ok ? *(const bf16x8*)(wrow + k) : zero;
+      if (EPI == SK_GATED) uf[u] = ok ? *(const bf16x8*)(urow + k) : zero;
+      sk_load_x<MT, XNORM>(xf[u], xrow, k + q * 8, ok, nrm);
+    }
+    __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        acc[0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u][mt], acc[0][mt], 0, 0, 0);
+        if (EPI == SK_GATED) acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u], xf[u][mt], acc[1][mt], 0, 0, 0);
+      }
+    }
+  }
+  sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp);
+}
+
+// The resident kernel: K <= 32 * NW * KS. `n_strips` strips are shared out over the blocks.
+template <int MT, int NW, int KS, int EPI, typename TC, bool XNORM, bool SSQ>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
+    const void* __restrict__ Av, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N, int K, long lda,
+    long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out, SkRope rp, int n_strips) {
+  constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
+  __shared__ f32x4 red[NW][NG * MT][64];
+  __shared__ float sm_ssq[XNORM ? NW : 1][64];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // Everything the block needs first is asked for before anything is waited for, so that it all
+  // arrives in one trip to memory: the first strip's rows of W, the rows' partial sums of squares,
+  // and this wave's share of A (k-steps wave, wave + NW, ...).
+  int strip = blockIdx.x;
+  int hd, sub;
+  bool rotated;
+  bf16x8 wf[KS], uf[KS];
+  {
+    const int wr = sk_strip_row<EPI>(strip, r, N, rp, hd, sub, rotated);
+    const bf16_t* wrow = W + (long)wr * ldw + q * 8;
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      const int k = (wave + NW * i) * 32;
+      const bool ok = k + q * 8 < K;
+      wf[i] = ok ? *(const bf16x8*)(wrow + k) : zero;
+      if (EPI == SK_GATED) uf[i] = ok ? *(const bf16x8*)(wrow + (long)N * ldw + k) : zero;
+    }
+  }
+  float sq[16];
+  int sq_row = 0;
+  if (XNORM) {
+    sq_row = (lane < M && nrm.rows) ? nrm.rows[lane] : lane;   // the partial sums are stored by row of A
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int p = wave + NW * i;
+      sq[i] = (lane < M && p < nrm.n_partials) ? nrm.ssq[(long)p * 64 + sq_row] : 0.f;
+    }
+  }
+  bf16x8 xf[KS][MT];
+  f32x4 xr[XNORM ? KS : 1][MT][2], gr[XNORM ? KS : 1][2];
+  {
+    const void* xrow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xrow[mt] = sk_x_row<XNORM>(Av, lda, min(mt * 16 + r, M - 1), nrm);
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      const int k = (wave + NW * i) * 32 + q * 8;
+      const bool ok = k < K;
+      if (XNORM) {
+        const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+        const float* gp = (const float*)nrm.weight + k;
+        gr[i][0] = ok ? *(const f32x4*)gp : zero4;
+        gr[i][1] = ok ? *(const f32x4*)(gp + 4) : zero4;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const float* xp = (const float*)xrow[mt] + k;
+          xr[i][mt][0] = ok ? *(const f32x4*)xp : zero4;
+          xr[i][mt][1] = ok ? *(const f32x4*)(xp + 4) : zero4;
+        }
+      } else {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xf[i][mt] = ok ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
+      }
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  if (XNORM) {
+    float sp = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sp += sq[i];
+    if (lane < M)
+      for (int p = wave + NW * 16; p < nrm.n_partials; p += NW) sp += nrm.ssq[(long)p * 64 + sq_row];
+    sm_ssq[wave][lane] = sp;
+#pragma unroll
+    for (int i = 0; i < KS; ++i)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        bf16x8 h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          h[e] = static_cast<bf16_t>(gr[i][0][e] * xr[i][mt][0][e]);
+          h[4 + e] = static_cast<bf16_t>(gr[i][1][e] * xr[i][mt][1][e]);
+        }
+        xf[i][mt] = h;
+      }
+  }
+  while (strip < n_strips) {
+    // ask for the next strip's rows before this strip's are used
+    const int next = strip + gridDim.x;
+    bf16x8 wn[KS], un[KS];
+    int hd_n = 0, sub_n = 0;
+    bool rot_n = false;
+    if (next < n_strips) {
+      const int wr = sk_strip_row<EPI>(next, r, N, rp, hd_n, sub_n, rot_n);
+      const bf16_t* wrow = W + (long)wr * ldw + q * 8;
+#pragma unroll
+      for (int i = 0; i < KS; ++i) {
+        const int k = (wave + NW * i) * 32;
+        const bool ok = k + q * 8 < K;
+        wn[i] = ok ? *(const bf16x8*)(wrow + k) : zero;
+        if (EPI == SK_GATED) un[i] = ok ? *(const bf16x8*)(wrow + (long)N * ldw + k) : zero;
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);   // the next strip's loads are on their way before this strip's are used
+    f32x4 acc[NG][MT];
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        acc[0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], xf[i][mt], acc[0][mt], 0, 0, 0);
+        if (EPI == SK_GATED) acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[i], xf[i][mt], acc[1][mt], 0, 0, 0);
+      }
+    }
+    sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp);
+    if (next >= n_strips) break;
+    __syncthreads();   // the partial tiles in shared memory are free again
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      wf[i] = wn[i];
+      if (EPI == SK_GATED) uf[i] = un[i];
+    }
+    strip = next; hd = hd_n; sub = sub_n; rotated = rot_n;
+  }
+}
+
+struct SkCall {
+  const void* A; const void* W; void* C;
+  int M, N, K; long lda, ldw, ldc;
+  SkNorm nrm; float* ssq_out; SkRope rp;
+  hipStream_t stream;
+  bool resident = true;
+};
+
+// Blocks of the resident kernel: every strip its own block while that still leaves CUs idle, else
+// two blocks per CU that walk over the strips.
+static int resident_blocks(int n_strips, int nw) {
+  const int most = nw == 16 ? 256 : 512;
+  return n_strips < most ? n_strips : most;
+}
+
+template <int MT, int EPI, typename TC, bool XNORM, bool SSQ>
+static int launch_skinny(int nw, const SkCall& a) {
+  constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
+  dim3 grid((a.N + 15) / 16);
+  const int n_strips = (a.N + 15) / 16;
+  const int steps = (a.K + 31) / 32;
+#define RES(NW, KS)                                                                                               \
+  do {                                                                                                            \
+    gemm_skinny_resident_kernel<MT, NW, KS, EPI, TC, XNORM, SSQ>                                                  \
+        <<<dim3(resident_blocks(n_strips, NW)), dim3(NW * 64), 0, a.stream>>>(                                    \
+            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.rp, n_strips); \
+    GL3_LAUNCH_CHECK();                                                                                           \
+    return 0;                                                                                                     \
+  } while (0)
+  if (a.resident) {
+    // 16 waves a strip where their partial tiles fit, so that a strip's rows are asked for at once
+    if constexpr (NG * MT <= 2) {
+      if (steps <= 64) RES(16, 4);
+    }
+    // (variants whose registers would spill are left to the streaming kernel)
+    if constexpr (NG * MT <= 4 && !(XNORM && MT >= 3)) {
+      if (steps <= 64) RES(8, 8);
+    }
+    if constexpr (MT == 1 && !XNORM && EPI != SK_GATED) {
+      if (steps <= 128) RES(8, 16);
+    }
+  }
+#undef RES
+#define GO(NW)                                                                                                    \
+  gemm_skinny_kernel<MT, NW, EPI, TC, XNORM, SSQ><<<grid, dim3(NW * 64), 0, a.stream>>>(                          \
+      a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.rp)
   if constexpr (NG * MT <= 2) {
     if (nw >= 16) { GO(16); GL3_LAUNCH_CHECK(); return 0; }
   }
@@ -123,48 +496,115 @@ static int launch_skinny(int nw, const void* A, const void* W, void* C, int M, i
   return 0;
 }
 
-template <int EPI, typename TC>
-static int pick_mt(int mt, int nw, const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw,
-                   long ldc, hipStream_t stream) {
-  switch (mt) {
-    case 1: return launch_skinny<1, EPI, TC>(nw, A, W, C, M, N, K, lda, ldw, ldc, stream);
-    case 2: return launch_skinny<2, EPI, TC>(nw, A, W, C, M, N, K, lda, ldw, ldc, stream);
-    case 3: return launch_skinny<3, EPI, TC>(nw, A, W, C, M, N, K, lda, ldw, ldc, stream);
-    default: return launch_skinny<4, EPI, TC>(nw, A, W, C, M, N, K, lda, ldw, ldc, stream);
+template <int EPI, typename TC, bool XNORM, bool SSQ>
+static int pick_mt(int nw, const SkCall& a) {
+  switch ((a.M + 15) / 16) {
+    case 1: return launch_skinny<1, EPI, TC, XNORM, SSQ>(nw, a);
+    case 2: return launch_skinny<2, EPI, TC, XNORM, SSQ>(nw, a);
+    case 3: return launch_skinny<3, EPI, TC, XNORM, SSQ>(nw, a);
+    default: return launch_skinny<4, EPI, TC, XNORM, SSQ>(nw, a);
   }
 }
 
-// `waves`: waves per block wanted (4, 8, 16; 0 lets the library choose). Fewer are used when the
-// partial tiles of that many waves would not fit the block's shared memory.
-extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
-                               long ldw, long ldc, int epilogue, int waves, hipStream_t stream) {
-  if (M == 0 || N == 0) return 0;
-  GL3_REQUIRE(A && W && C, "gl3_gemm_skinny: null operand");
-  GL3_REQUIRE(M > 0 && M <= 64, "gl3_gemm_skinny: M=%d is outside 1..64", M);
+static int pick_waves(int waves, int N, int K) {
+  if (waves) return waves;
+  // enough waves to keep every CU's memory pipeline full, at least two k-steps each
+  const long strips = (N + 15) / 16, steps = (K + 31) / 32;
+  waves = 4;
+  while (waves < 16 && strips * waves < 4096 && steps / (waves * 2) >= 2) waves *= 2;
+  return waves;
+}
+
+static int check_common(const char* who, const void* A, const void* W, const void* C, int M, int N, int K, long lda,
+                        long ldw, int waves) {
+  GL3_REQUIRE(A && W && C, "%s: null operand", who);
+  GL3_REQUIRE(M > 0 && M <= 64, "%s: M=%d is outside 1..64", who, M);
   GL3_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0,
-              "gl3_gemm_skinny: K=%d, lda=%ld, ldw=%ld must be multiples of 8", K, lda, ldw);
-  GL3_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gl3_gemm_skinny: operands must be 16-byte aligned");
-  GL3_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gl3_gemm_skinny: leading dimensions too small");
+              "%s: K=%d, lda=%ld, ldw=%ld must be multiples of 8", who, K, lda, ldw);
+  GL3_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "%s: operands must be 16-byte aligned", who);
+  GL3_REQUIRE(lda >= K && ldw >= K, "%s: leading dimensions too small", who);
+  GL3_REQUIRE(waves == 0 || waves == 4 || waves == 8 || waves == 16, "%s: waves=%d", who, waves);
+  return 0;
+}
+
+// `waves`: 0 lets the library choose the kernel (the resident one where K allows) and its block size;
+// 4, 8 or 16 ask for the streaming kernel with that many waves per block (fewer are used when the
+// partial tiles of that many waves would not fit the block's shared memory).
+// ssq_out (may be null, add epilogue only, N % 16 == 0): [N/16][64] partial sums of squares of the
+// completed rows.
+extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
+                               long ldw, long ldc, int epilogue, int waves, float* ssq_out, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  if (check_common("gl3_gemm_skinny", A, W, C, M, N, K, lda, ldw, waves)) return -1;
+  GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny: ldc too small");
   GL3_REQUIRE(epilogue >= 0 && epilogue <= 2, "gl3_gemm_skinny: unknown epilogue %d", epilogue);
   GL3_REQUIRE(epilogue != SK_ADD || c_dtype == GL3_F32, "gl3_gemm_skinny: the add epilogue needs a float output");
-  GL3_REQUIRE(waves == 0 || waves == 4 || waves == 8 || waves == 16, "gl3_gemm_skinny: waves=%d", waves);
-  const int mt = (M + 15) / 16;
-  if (waves == 0) {
-    // enough waves to keep every CU's memory pipeline full, at least two k-steps each
-    const long strips = (N + 15) / 16, steps = (K + 31) / 32;
-    waves = 4;
-    while (waves < 16 && strips * waves < 4096 && steps / (waves * 2) >= 2) waves *= 2;
-  }
-#define GO(EPI, TC) return pick_mt<EPI, TC>(mt, waves, A, W, C, M, N, K, lda, ldw, ldc, stream)
+  GL3_REQUIRE(!ssq_out || (epilogue == SK_ADD && N % 16 == 0),
+              "gl3_gemm_skinny: sums of squares come with the add epilogue and N a multiple of 16");
+  const SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, ssq_out, SkRope{}, stream, waves == 0};
+  const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32) {
-    if (epilogue == SK_STORE) GO(SK_STORE, float);
-    if (epilogue == SK_ADD) GO(SK_ADD, float);
-    GO(SK_GATED, float);
+    if (epilogue == SK_STORE) return pick_mt<SK_STORE, float, false, false>(nw, a);
+    if (epilogue == SK_ADD) return ssq_out ? pick_mt<SK_ADD, float, false, true>(nw, a)
+                                           : pick_mt<SK_ADD, float, false, false>(nw, a);
+    return pick_mt<SK_GATED, float, false, false>(nw, a);
   } else if (c_dtype == GL3_BF16) {
-    if (epilogue == SK_STORE) GO(SK_STORE, bf16_t);
-    GO(SK_GATED, bf16_t);
+    if (epilogue == SK_STORE) return pick_mt<SK_STORE, bf16_t, false, false>(nw, a);
+    return pick_mt<SK_GATED, bf16_t, false, false>(nw, a);
   }
-#undef GO
   GL3_REQUIRE(false, "gl3_gemm_skinny: unknown output dtype %d", c_dtype);
   return 0;
+}
+
+// The product of RMSNorm(x) with W: x float [rows, K] (lda), norm weight [K], ssq [n_partials][64]
+// partial sums of squares of the rows of x (indexed by the row of x, so x has at most 64 rows).
+// Epilogues: store (float or bfloat16) and gated (bfloat16).
+extern "C" int gl3_gemm_skinny_norm(const float* x, const int* rows, const void* norm_weight, int norm_weight_dtype,
+                                    const float* ssq, int n_partials, float eps, const void* W, void* C, int c_dtype,
+                                    int M, int N, int K, long lda, long ldw, long ldc, int epilogue, int waves,
+                                    hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  if (check_common("gl3_gemm_skinny_norm", x, W, C, M, N, K, lda, ldw, waves)) return -1;
+  GL3_REQUIRE(norm_weight && ssq && n_partials > 0, "gl3_gemm_skinny_norm: norm arguments missing");
+  GL3_REQUIRE(norm_weight_dtype == GL3_F32, "gl3_gemm_skinny_norm: the norm weight must be float");
+  GL3_REQUIRE((uintptr_t)norm_weight % 16 == 0, "gl3_gemm_skinny_norm: norm weight must be 16-byte aligned");
+  GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny_norm: ldc too small");
+  GL3_REQUIRE(epilogue == SK_STORE || epilogue == SK_GATED, "gl3_gemm_skinny_norm: epilogue %d", epilogue);
+  const SkNorm nrm = {(const float*)norm_weight, ssq, n_partials, eps, rows};
+  const SkCall a = {x, W, C, M, N, K, lda, ldw, ldc, nrm, nullptr, SkRope{}, stream, waves == 0};
+  const int nw = pick_waves(waves, N, K);
+  if (c_dtype == GL3_F32 && epilogue == SK_STORE) return pick_mt<SK_STORE, float, true, false>(nw, a);
+  if (c_dtype == GL3_BF16 && epilogue == SK_STORE) return pick_mt<SK_STORE, bf16_t, true, false>(nw, a);
+  if (c_dtype == GL3_BF16 && epilogue == SK_GATED) return pick_mt<SK_GATED, bf16_t, true, false>(nw, a);
+  GL3_REQUIRE(false, "gl3_gemm_skinny_norm: output dtype %d with epilogue %d is not built", c_dtype, epilogue);
+  return 0;
+}
+
+// RMSNorm(x) . Wqkv^T, rotation of q and k, q to `q_out` [M, n_heads*head_dim] (ldq), k and v into
+// the paged cache (keys [page][kv head][position][head_dim], values transposed). One token per row;
+// cos/sin null: no rotation. head_dim a multiple of 16; the rotation covers the whole head.
+extern "C" int gl3_qkv_rope_cache(const float* x, const void* norm_weight, int norm_weight_dtype, const float* ssq,
+                                  int n_partials, float eps, const void* Wqkv, void* q_out, long ldq, int M, int K,
+                                  long lda, long ldw, const int* positions, const int* seq_of_token,
+                                  const int* block_table, int table_stride, const float* cos_tab,
+                                  const float* sin_tab, void* k_cache, void* v_cache, int n_heads, int n_kv,
+                                  int head_dim, int adjacent, int page_size, int waves, hipStream_t stream) {
+  if (M == 0) return 0;
+  const int N = (n_heads + 2 * n_kv) * head_dim;
+  if (check_common("gl3_qkv_rope_cache", x, Wqkv, q_out, M, N, K, lda, ldw, waves)) return -1;
+  GL3_REQUIRE(norm_weight && ssq && n_partials > 0 && (uintptr_t)norm_weight % 16 == 0,
+              "gl3_qkv_rope_cache: norm arguments missing or misaligned");
+  GL3_REQUIRE(norm_weight_dtype == GL3_F32, "gl3_qkv_rope_cache: the norm weight must be float");
+  GL3_REQUIRE(head_dim % 16 == 0 && n_heads > 0 && n_kv > 0, "gl3_qkv_rope_cache: head_dim %d must be a multiple of 16",
+              head_dim);
+  GL3_REQUIRE(positions && seq_of_token && block_table && k_cache && v_cache && page_size > 0 && table_stride > 0,
+              "gl3_qkv_rope_cache: cache arguments missing");
+  GL3_REQUIRE((cos_tab == nullptr) == (sin_tab == nullptr), "gl3_qkv_rope_cache: one table without the other");
+  GL3_REQUIRE(ldq >= (long)n_heads * head_dim && ldq % 4 == 0 && (uintptr_t)q_out % 8 == 0,
+              "gl3_qkv_rope_cache: q_out stride/alignment");
+  const SkNorm nrm = {(const float*)norm_weight, ssq, n_partials, eps, nullptr};
+  const SkRope rp = {positions, seq_of_token, block_table, table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
+                     (bf16_t*)v_cache, n_heads, n_kv, head_dim, adjacent, page_size};
+  const SkCall a = {x, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
+  return pick_mt<SK_QKV, bf16_t, true, false>(pick_waves(waves, N, K), a);
 }

@@ -47,13 +47,16 @@ def _declare(lib):
     sigs = {
         "gl3_abi_version": [],
         "gl3_fill_u32": [P, c_uint32, L, P],
-        "gl3_embed": [P, I, P, P, I, I, P],
+        "gl3_embed": [P, I, P, P, I, I, P, P],
         "gl3_rmsnorm": [P, P, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P],
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
-        "gl3_sample": [P, L, P, P, P, P, P, I, I, P],
-        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P],
+        "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
+        "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
+        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, P],
+        "gl3_gemm_skinny_norm": [P, P, P, I, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P],
+        "gl3_qkv_rope_cache": [P, P, I, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
@@ -119,13 +122,19 @@ def fill_u32(t, value):
     _check(library().gl3_fill_u32(_ptr(t), value, t.element_size() * t.numel() // 4, _stream()), "fill_u32")
 
 
-def embed(table, ids, out):
-    """out[t] = table[ids[t]] as float32. The caller has checked ids < rows."""
+def embed(table, ids, out, ssq=None):
+    """out[t] = table[ids[t]] as float32. The caller has checked ids < rows. ``ssq`` (at least 64
+    floats, at most 64 tokens) receives each row's sum of squares."""
     _dev(table, "table"); _dev(ids, "ids", torch.int32); _dev(out, "out", torch.float32)
     T, d = out.shape
     if table.dim() != 2 or table.shape[1] != d or ids.numel() != T:
         raise KernelError(f"embed: table {tuple(table.shape)}, ids {tuple(ids.shape)}, out {tuple(out.shape)}")
-    _check(library().gl3_embed(_ptr(table), _code(table, "table"), _ptr(ids), _ptr(out), T, d, _stream()), "embed")
+    if ssq is not None:
+        _dev(ssq, "ssq", torch.float32)
+        if ssq.numel() < 64 or T > 64:
+            raise KernelError("embed: sums of squares need 64 floats and at most 64 tokens")
+    _check(library().gl3_embed(_ptr(table), _code(table, "table"), _ptr(ids), _ptr(out), T, d, _ptr(ssq), _stream()),
+           "embed")
 
 
 def rmsnorm(x, weight, out, eps, rows=None):
@@ -212,7 +221,20 @@ def attention_generic(q, k_cache, v_cache, positions, seq_of_token, block_table,
         int(window or 0), float(scale), _stream()), "attention_generic")
 
 
-def sample(logits, work, temperature, top_p, uniform, out):
+def decode_advance(token_ids, positions, kv_before, sampled, history, step):
+    """Feed the sampled tokens back, move every sequence on by one, log the tokens in row step[0]
+    of ``history`` [rows, n], count the step."""
+    n = token_ids.numel()
+    for t, name in ((token_ids, "token_ids"), (positions, "positions"), (kv_before, "kv_before"),
+                    (sampled, "sampled"), (history, "history"), (step, "step")):
+        _dev(t, name, torch.int32)
+    if positions.numel() != n or kv_before.numel() != n or sampled.numel() < n or history.dim() != 2 or history.shape[1] < n:
+        raise KernelError("decode_advance: sizes")
+    _check(library().gl3_decode_advance(_ptr(token_ids), _ptr(positions), _ptr(kv_before), _ptr(sampled),
+                                        _ptr(history), history.stride(0), _ptr(step), n, _stream()), "decode_advance")
+
+
+def sample(logits, work, temperature, top_p, uniform, out, step=None, uniform_stride=0):
     _dev(logits, "logits", torch.float32, contiguous=False); _dev(work, "work", torch.float32)
     for t, n in ((temperature, "temperature"), (top_p, "top_p"), (uniform, "uniform")):
         _dev(t, n, torch.float32)
@@ -221,8 +243,10 @@ def sample(logits, work, temperature, top_p, uniform, out):
     if logits.stride(1) != 1 or work.numel() < R * V or min(temperature.numel(), top_p.numel(), uniform.numel(),
                                                               out.numel()) < R:
         raise KernelError("sample: argument sizes")
+    if step is not None:
+        _dev(step, "step", torch.int32)
     _check(library().gl3_sample(_ptr(logits), logits.stride(0), _ptr(work), _ptr(temperature), _ptr(top_p),
-                                _ptr(uniform), _ptr(out), R, V, _stream()), "sample")
+                                _ptr(uniform), _ptr(out), R, V, _ptr(step), int(uniform_stride), _stream()), "sample")
 
 
 # ------------------------------------------------------------------ bfloat16 product for few rows
@@ -234,8 +258,9 @@ def gemm_skinny_fits(a, w, out, epilogue):
             and (out.dtype == torch.float32 or (out.dtype == torch.bfloat16 and epilogue != EPI_ADD)))
 
 
-def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0):
-    """out (=, +=, gated) a @ w.T on the matrix cores for at most 64 rows of ``a``."""
+def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None):
+    """out (=, +=, gated) a @ w.T on the matrix cores for at most 64 rows of ``a``. ``ssq_out``
+    [N/16, 64] float32 (add epilogue): partial sums of squares of the completed rows."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
         raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
@@ -244,8 +269,80 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0):
     rows = 2 * N if epilogue == EPI_GATED else N
     if w.shape != (rows, K) or out.shape[0] != M:
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
+    if ssq_out is not None:
+        _dev(ssq_out, "ssq_out", torch.float32)
+        if epilogue != EPI_ADD or N % 16 or ssq_out.numel() < N // 16 * 64:
+            raise KernelError("gemm_skinny: sums of squares need the add epilogue, N % 16 == 0 and N/16*64 floats")
     _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
-                                     out.stride(0), epilogue, waves, _stream()), "gemm_skinny")
+                                     out.stride(0), epilogue, waves, _ptr(ssq_out), _stream()), "gemm_skinny")
+
+
+def _check_norm_args(x, norm_weight, ssq, n_partials, K):
+    _dev(x, "x", torch.float32, contiguous=False); _dev(norm_weight, "norm_weight"); _dev(ssq, "ssq", torch.float32)
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] != K or norm_weight.shape != (K,):
+        raise KernelError(f"fused norm: x {tuple(x.shape)}, weight {tuple(norm_weight.shape)} for K={K}")
+    if x.shape[0] > 64 or n_partials < 1 or ssq.numel() < n_partials * 64:
+        raise KernelError("fused norm: at most 64 rows of x, and n_partials * 64 partial sums")
+
+
+def gemm_skinny_norm_fits(x, w, out, epilogue):
+    K = x.shape[1]
+    return (x.shape[0] <= 64 and K % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and w.dtype == torch.bfloat16
+            and ((epilogue == EPI_STORE and out.dtype in (torch.float32, torch.bfloat16))
+                 or (epilogue == EPI_GATED and out.dtype == torch.bfloat16)))
+
+
+def gemm_skinny_norm(x, norm_weight, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=None, waves=0):
+    """out (=, gated) RMSNorm(x)[rows] @ w.T; the norm's sum of squares comes as partial sums."""
+    _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
+    K = w.shape[1]
+    _check_norm_args(x, norm_weight, ssq, n_partials, K)
+    M = x.shape[0]
+    if rows is not None:
+        _dev(rows, "rows", torch.int32)
+        M = rows.numel()
+    N = out.shape[1]
+    wrows = 2 * N if epilogue == EPI_GATED else N
+    if w.shape != (wrows, K) or out.shape[0] != M or out.stride(1) != 1 or M > 64:
+        raise KernelError(f"gemm: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
+    _check(library().gl3_gemm_skinny_norm(
+        _ptr(x), _ptr(rows), _ptr(norm_weight), _code(norm_weight, "norm_weight"), _ptr(ssq), n_partials, float(eps),
+        _ptr(w), _ptr(out), _code(out, "out"), M, N, K, x.stride(0), w.stride(0), out.stride(0), epilogue, waves,
+        _stream()), "gemm_skinny_norm")
+
+
+def qkv_rope_cache_fits(x, w_qkv, head_dim, rot_dim):
+    K = x.shape[1]
+    return (x.shape[0] <= 64 and K % 8 == 0 and x.stride(0) % 8 == 0 and w_qkv.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and w_qkv.data_ptr() % 16 == 0 and w_qkv.dtype == torch.bfloat16
+            and head_dim % 16 == 0 and rot_dim in (0, head_dim))
+
+
+def qkv_rope_cache(x, norm_weight, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_token, block_table, cos, sin,
+                   k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page_size, waves=0):
+    """RMSNorm(x) @ w_qkv.T, rotation, q into ``q_out`` [T, H*hs] bfloat16, k and v into the cache."""
+    _dev(w_qkv, "w_qkv", torch.bfloat16); _dev(q_out, "q_out", torch.bfloat16, contiguous=False)
+    K = w_qkv.shape[1]
+    _check_norm_args(x, norm_weight, ssq, n_partials, K)
+    T = x.shape[0]
+    _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
+    _dev(block_table, "block_table", torch.int32)
+    _dev(k_cache, "k_cache", torch.bfloat16); _dev(v_cache, "v_cache", torch.bfloat16)
+    _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "qkv_rope_cache")
+    if (w_qkv.shape[0] != (n_heads + 2 * n_kv) * head_dim or q_out.shape[0] != T or q_out.stride(1) != 1
+            or q_out.shape[1] < n_heads * head_dim or positions.numel() != T or seq_of_token.numel() != T
+            or block_table.dim() != 2):
+        raise KernelError("qkv_rope_cache: shapes")
+    if cos is not None:
+        _dev(cos, "cos", torch.float32); _dev(sin, "sin", torch.float32)
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != head_dim // 2:
+            raise KernelError(f"qkv_rope_cache: table {tuple(cos.shape)} for head_dim {head_dim}")
+    _check(library().gl3_qkv_rope_cache(
+        _ptr(x), _ptr(norm_weight), _code(norm_weight, "norm_weight"), _ptr(ssq), n_partials, float(eps), _ptr(w_qkv),
+        _ptr(q_out), q_out.stride(0), T, K, x.stride(0), w_qkv.stride(0), _ptr(positions), _ptr(seq_of_token),
+        _ptr(block_table), block_table.shape[1], _ptr(cos), _ptr(sin), _ptr(k_cache), _ptr(v_cache), n_heads, n_kv,
+        head_dim, int(adjacent), page_size, waves, _stream()), "qkv_rope_cache")
 
 
 # ------------------------------------------------------------------ bfloat16 attention of a decode step
@@ -254,11 +351,11 @@ def attention_decode_fits(head_dim, n_heads, n_kv, page_size):
 
 
 def decode_splits(n_tokens, n_heads, n_kv, kv_len):
-    """Blocks that share a sequence's keys: enough blocks for the chip, a wave keeps at least one
-    chunk of 32 keys."""
+    """Blocks that share a sequence's keys. A split costs a second kernel that merges the
+    parts, which is worth its few microseconds only when a block would otherwise walk
+    thousands of keys; there are never more blocks than cover the chip a few times."""
     blocks = n_tokens * n_kv * -(-(n_heads // n_kv) // 16)
-    most = max(1, kv_len // 128)
-    return int(max(1, min(most, -(-768 // blocks), 64)))
+    return int(max(1, min(kv_len // 1024, -(-2048 // blocks), 16)))
 
 
 def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,

@@ -59,7 +59,8 @@ __device__ uint32_t search_threshold(const float* p, int V, double thr, double* 
 __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ logits, long ld, float* __restrict__ work,
                                                     const float* __restrict__ temperature,
                                                     const float* __restrict__ top_p, const float* __restrict__ uniform,
-                                                    int* __restrict__ out, int V) {
+                                                    int* __restrict__ out, int V, const int* __restrict__ step,
+                                                    int uniform_stride) {
   __shared__ float fs[16];
   __shared__ int is[16];
   __shared__ double ds[16];
@@ -107,7 +108,8 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
   __syncthreads();
 
   const float tp = top_p[row];
-  const double u = (double)uniform[row];
+  // in a run of steps replayed from a graph the step's number is read from memory
+  const double u = (double)uniform[(step ? (long)step[0] * uniform_stride : 0) + row];
   const int chunk = (V + SB - 1) / SB;
   const int b = min(V, tid * chunk), e = min(V, (tid + 1) * chunk);
   if (tid == 0) winner = -1;
@@ -182,12 +184,15 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
 }
 
 // work: [n_rows, V] floats of scratch (probabilities); unused for greedy rows.
+// step (may be null): a counter in device memory; row r then takes uniform[step[0] * uniform_stride + r].
 extern "C" int gl3_sample(const float* logits, long ld, float* work, const float* temperature, const float* top_p,
-                          const float* uniform, int* out, int n_rows, int V, hipStream_t stream) {
+                          const float* uniform, int* out, int n_rows, int V, const int* step, int uniform_stride,
+                          hipStream_t stream) {
   if (n_rows == 0) return 0;
   GL3_REQUIRE(logits && work && temperature && top_p && uniform && out, "gl3_sample: null argument");
   GL3_REQUIRE(n_rows > 0 && V > 0 && ld >= V, "gl3_sample: bad sizes (rows=%d V=%d ld=%ld)", n_rows, V, ld);
-  sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, ld, work, temperature, top_p, uniform, out, V);
+  sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, ld, work, temperature, top_p, uniform, out, V, step,
+                                                       uniform_stride);
   GL3_LAUNCH_CHECK();
   return 0;
 }

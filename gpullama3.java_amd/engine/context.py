@@ -47,6 +47,8 @@ class StepContext:
         self.q_lens, self.kv_before_host, self.slots = q_lens, kv_before_host, slots
         self.decode = decode
         self.max_q_len, self.max_kv_len = max_q_len, max_kv_len
+        self.fuse = getattr(engine, "fuse", False)   # few-token steps fold norms and rotation into the products
+        self.ssq = None                    # (address of the residual stream, its partial sums of squares, how many)
         self.kv_len_hint = max_kv_len      # what launch shapes are sized for; a replayed graph keeps its own
         self.token_ids = self.positions = self.seq_of_token = self.cu_seqlens = self.kv_before = None
         self.slot_ids = None
@@ -57,6 +59,11 @@ class StepContext:
 
     def buffer(self, name, shape, dtype):
         return self.engine.workspace.get(name, shape, dtype)
+
+    def ssq_buffer(self, n_partials):
+        """[n_partials, 64] partial sums of squares; one buffer, as large as the widest writer needs."""
+        most = max(n_partials, -(-self.engine.spec.hidden // 16))
+        return self.buffer("ssq", (most, 64), torch.float32)[:n_partials]
 
     def logits_buffer(self, n_rows, vocab):
         return torch.empty((n_rows, vocab), dtype=torch.float32, device=self.device)

@@ -40,10 +40,14 @@ def _require_gpu(device):
     return torch.device(device)
 
 
+RUN_LENGTH = 16     # most decode steps that run on the device before the host looks at the tokens
+
+
 class _DecodeGraph:
-    """A captured decode step for one batch bucket: its fixed input buffer and its logits."""
-    graph = logits = host = dev = blank = None
-    width = off_before = off_slots = off_tables = 0
+    """A captured decode step for one batch bucket: its fixed input buffer and its logits; for runs
+    of steps also the sampling of the next tokens and their feeding back."""
+    graph = logits = host = dev = blank = fhost = fdev = copied = None
+    width = off_before = off_slots = off_tables = off_step = off_sampled = off_hist = 0
 
 
 class Engine:
@@ -76,6 +80,7 @@ class Engine:
         parts = [p for b in self.model.blocks for p in b.parts()]
         self.use_graphs = bool(use_graphs and not self.cache.state
                                and all(getattr(p, "graph_safe", False) for p in parts))
+        self.fuse = bool(self.dtype == torch.bfloat16 and all(getattr(p, "graph_safe", False) for p in parts))
         self._graphs = {}
         self._graphs_generation = 0
 
@@ -212,11 +217,49 @@ class Engine:
         return self.model.forward(ctx, rows)
 
     # ------------------------------------------------------------------ decode steps from captured graphs
-    def _step_graph(self, B, token_ids, positions, slots, max_kv):
-        """One token for each of B sequences: the step's index arrays go into a fixed buffer and
-        the captured launches are replayed. The batch is padded to a bucket; a padded entry is a
-        one-token sequence whose block table names the sink page only, so it reads and writes
-        nothing that a real sequence owns, and its logits are not returned."""
+    @property
+    def decode_run_length(self):
+        return RUN_LENGTH if self.use_graphs else 1
+
+    def decode_run(self, entries, n, temperatures, top_ps, uniforms):
+        """``n`` decode steps in a row for ``entries = [(slot, token), ...]``: every step samples
+        each sequence's next token on the device and feeds it back, the host waits once at the
+        end. ``uniforms[k][r]`` is step k's uniform number for entry r. Returns the sampled
+        tokens ``[n][len(entries)]``. The cache has all n positions reserved before the first
+        step, or ``CacheFull`` is raised and nothing has changed."""
+        B = len(entries)
+        if not self.use_graphs or not 1 <= n <= RUN_LENGTH:
+            raise ValueError(f"a run takes 1..{RUN_LENGTH} steps on an engine that replays graphs")
+        slots = [int(s) for s, _ in entries]
+        tokens = [int(t) for _, t in entries]
+        if len(set(slots)) != B:
+            raise ValueError("a slot appears twice in one step")
+        if any(not 0 <= t < self.spec.vocab_size for t in tokens):
+            raise ValueError("a token id is outside the vocabulary")
+        starts = [self.cache.length(s) for s in slots]
+        self.cache.reserve({s: n for s in slots})
+        with torch.cuda.device(self.device):
+            dg = self._graph_for(B, max(starts) + n, run=True)
+            self._fill_graph_input(dg, B, tokens, starts, slots)
+            B_pad = dg.B_pad
+            f = dg.fhost
+            f.zero_()
+            f[0:B] = torch.tensor(list(temperatures), dtype=torch.float32)
+            f[B_pad:B_pad + B] = torch.tensor(list(top_ps), dtype=torch.float32)
+            u = torch.tensor([list(row) for row in uniforms], dtype=torch.float32)        # [n, B]
+            f[2 * B_pad:2 * B_pad + RUN_LENGTH * B_pad].view(RUN_LENGTH, B_pad)[:n, :B] = u
+            dg.fdev.copy_(f, non_blocking=True)
+            dg.dev.copy_(dg.host, non_blocking=True)
+            dg.copied = torch.cuda.Event()
+            dg.copied.record()
+            for _ in range(n):
+                dg.graph.replay()
+            hist = dg.dev[dg.off_hist:dg.off_hist + RUN_LENGTH * B_pad].view(RUN_LENGTH, B_pad)[:n, :B].cpu()
+        for s in slots:
+            self.cache.advance(s, n)
+        return hist.tolist()
+
+    def _graph_for(self, B, max_kv, run):
         if self._graphs_generation != self.workspace.generation:
             self._graphs.clear()                 # a scratch buffer moved: the captured addresses are stale
             self._graphs_generation = self.workspace.generation
@@ -224,17 +267,21 @@ class Engine:
         kv_bucket = 256
         while kv_bucket < max_kv:
             kv_bucket *= 2
-        key = (B_pad, kv_bucket)
+        key = (B_pad, kv_bucket, run)
         dg = self._graphs.get(key)
         if dg is None:
-            dg = self._capture(B_pad, kv_bucket)
+            dg = self._capture(B_pad, kv_bucket, run)
             if self._graphs_generation != self.workspace.generation:    # the warm-up grew a buffer
                 self._graphs.clear()
                 self._graphs_generation = self.workspace.generation
-                dg = self._capture(B_pad, kv_bucket)
+                dg = self._capture(B_pad, kv_bucket, run)
             self._graphs[key] = dg
-        h = dg.host
-        W = dg.width
+        return dg
+
+    def _fill_graph_input(self, dg, B, token_ids, positions, slots):
+        h, W, B_pad = dg.host, dg.width, dg.B_pad
+        if dg.copied is not None:
+            dg.copied.synchronize()              # the last copy out of this pinned buffer has left it
         h[:] = dg.blank
         h[0:B] = torch.tensor(token_ids, dtype=torch.int32)
         h[B_pad:B_pad + B] = torch.tensor(positions, dtype=torch.int32)
@@ -244,21 +291,34 @@ class Engine:
             rows = torch.tensor(self.cache.block_rows(g, slots, W), dtype=torch.int32)
             o = dg.off_tables + g * B_pad * W
             h[o:o + B * W] = rows.view(-1)
-        dg.dev.copy_(h, non_blocking=True)
+
+    def _step_graph(self, B, token_ids, positions, slots, max_kv):
+        """One token for each of B sequences: the step's index arrays go into a fixed buffer and
+        the captured launches are replayed. The batch is padded to a bucket; a padded entry is a
+        one-token sequence whose block table names the sink page only, so it reads and writes
+        nothing that a real sequence owns, and its logits are not returned."""
+        dg = self._graph_for(B, max_kv, run=False)
+        self._fill_graph_input(dg, B, token_ids, positions, slots)
+        dg.dev.copy_(dg.host, non_blocking=True)
+        dg.copied = torch.cuda.Event()
+        dg.copied.record()
         dg.graph.replay()
         return dg.logits[:B]
 
-    def _capture(self, B_pad, kv_bucket):
+    def _capture(self, B_pad, kv_bucket, run=False):
         W = self.cache.max_pages_per_seq
         G = len(self.cache.groups)
         dg = _DecodeGraph()
-        dg.width = W
+        dg.width, dg.B_pad = W, B_pad
         # layout: tokens | positions | seq_of_token | cu_seqlens | kv_before | slots | rows | tables
         dg.off_before = 3 * B_pad + B_pad + 1
         dg.off_slots = dg.off_before + B_pad
         off_rows = dg.off_slots + B_pad
         dg.off_tables = off_rows + B_pad
-        n = dg.off_tables + G * B_pad * W
+        dg.off_step = dg.off_tables + G * B_pad * W          # for runs: step counter, sampled tokens, their history
+        dg.off_sampled = dg.off_step + 1
+        dg.off_hist = dg.off_sampled + B_pad
+        n = dg.off_hist + RUN_LENGTH * B_pad if run else dg.off_step
         blank = torch.zeros(n, dtype=torch.int32)
         ar = torch.arange(B_pad + 1, dtype=torch.int32)
         blank[2 * B_pad:3 * B_pad] = ar[:B_pad]                   # seq_of_token
@@ -280,18 +340,36 @@ class Engine:
         rows = d[off_rows:off_rows + B_pad]
         ctx._tables = [d[dg.off_tables + g * B_pad * W:dg.off_tables + (g + 1) * B_pad * W].view(B_pad, W)
                        for g in range(G)]
+        if run:
+            from ..csrc import lib as K
+            dg.fhost = torch.zeros((2 + RUN_LENGTH) * B_pad, dtype=torch.float32).pin_memory()
+            dg.fdev = torch.zeros((2 + RUN_LENGTH) * B_pad, dtype=torch.float32, device=self.device)
+            work = torch.empty(B_pad * self.spec.vocab_size, dtype=torch.float32, device=self.device)
+            step = d[dg.off_step:dg.off_step + 1]
+            sampled = d[dg.off_sampled:dg.off_sampled + B_pad]
+            hist = d[dg.off_hist:dg.off_hist + RUN_LENGTH * B_pad].view(RUN_LENGTH, B_pad)
+            temps, tops = dg.fdev[0:B_pad], dg.fdev[B_pad:2 * B_pad]
+            us = dg.fdev[2 * B_pad:]
+
+        def body():
+            logits = self.model.forward(ctx, rows)
+            if run:
+                K.sample(logits, work, temps, tops, us, sampled, step=step, uniform_stride=B_pad)
+                K.decode_advance(ctx.token_ids, ctx.positions, ctx.kv_before, sampled, hist, step)
+            return logits
+
         # once outside a capture: scratch buffers get their sizes, the library is loaded
         side = torch.cuda.Stream(device=self.device)
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            self.model.forward(ctx, rows)
+            body()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.workspace.frozen = True
         try:
             dg.graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(dg.graph):
-                dg.logits = self.model.forward(ctx, rows)
+                dg.logits = body()
         finally:
             self.workspace.frozen = False
         return dg

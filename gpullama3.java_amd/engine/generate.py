@@ -11,7 +11,9 @@ requests form the next one. Once a batch has started no request joins it.
 The loop only decides; the model is behind ``backend``:
 ``take_slot()``, ``give_back_slot(slot)``, ``step(entries) -> logits handle`` (last
 row of each entry), ``sample(logits, temperatures, top_ps, uniforms) -> ids``,
-``max_context``, ``page_size``, ``tokens_capacity()``, ``slots_free()``.
+``max_context``, ``page_size``, ``tokens_capacity()``, ``slots_free()``; optionally
+``decode_run_length`` and ``decode_run(entries, n, temperatures, top_ps, uniforms[n]) ->
+ids[n]``: n steps in a row, each feeding back what it sampled.
 """
 from __future__ import annotations
 
@@ -109,48 +111,71 @@ def _run_batch(backend, requests, results, ids, on_token, metrics):
         if not live:
             return
         held = {i: len(requests[i].prompt) for i, _ in live}
+
+        def take(i, slot, tok):
+            """Record a sampled token; true if the sequence goes on."""
+            r, out = requests[i], results[i]
+            out.tokens.append(int(tok))
+            metrics.generated_tokens += 1
+            if on_token is not None:
+                on_token(i, int(tok))
+            if int(tok) in r.stop_ids:
+                out.finish_reason = "stop"       # the stop token is part of the result
+            elif len(out.tokens) >= r.max_new_tokens or held[i] >= backend.max_context:
+                out.finish_reason = "length"     # no room to feed this token back
+            return out.finish_reason is None
+
+        def params(rows, k=0):
+            return ([requests[i].sampling.temperature for i in rows], [requests[i].sampling.top_p for i in rows],
+                    [uniform(requests[i].sampling.seed, i, len(results[i].tokens) + k) for i in rows])
+
+        # the prompts of the batch in one step, and each sequence's first token
         t0 = time.perf_counter()
         logits = backend.step([(slot, list(requests[i].prompt)) for i, slot in live])
-        step_no = 0
-        prefill = True
+        first = backend.sample(logits, *params([i for i, _ in live]))
+        metrics.prefill_seconds += time.perf_counter() - t0
+        metrics.prompt_tokens += sum(len(requests[i].prompt) for i, _ in live)
+        nxt = []
+        for (i, slot), tok in zip(live, first):
+            if take(i, slot, tok):
+                nxt.append((i, slot))
+            else:
+                backend.give_back_slot(slot)
+        live = nxt
+
+        # then one token per live sequence and step. A backend may run several steps before it
+        # reports (it feeds each sampled token back itself): then a sequence that ends inside
+        # such a run leaves the batch at the run's end, and what it sampled after its end is
+        # dropped. No run is longer than the shortest remaining budget of its sequences.
+        most = max(1, int(getattr(backend, "decode_run_length", 1)))
         while live:
             rows = [i for i, _ in live]
-            ids_out = backend.sample(
-                logits,
-                [requests[i].sampling.temperature for i in rows],
-                [requests[i].sampling.top_p for i in rows],
-                [uniform(requests[i].sampling.seed, i, len(results[i].tokens)) for i in rows])
-            dt = time.perf_counter() - t0
-            if prefill:
-                metrics.prefill_seconds += dt
-                metrics.prompt_tokens += sum(len(requests[i].prompt) for i in rows)
-                prefill = False
-            else:
-                metrics.decode_seconds += dt
-                metrics.decode_steps += 1
+            n = min([most] + [min(requests[i].max_new_tokens - len(results[i].tokens),
+                                  backend.max_context - held[i]) for i in rows])
             t0 = time.perf_counter()
+            if n <= 1 or not hasattr(backend, "decode_run"):
+                n = 1
+                logits = backend.step([(slot, [results[i].tokens[-1]]) for i, slot in live])
+                sampled = [backend.sample(logits, *params(rows))]
+            else:
+                temps, tops, _ = params(rows)
+                us = [params(rows, k)[2] for k in range(n)]
+                sampled = backend.decode_run([(slot, results[i].tokens[-1]) for i, slot in live], n, temps, tops, us)
+            metrics.decode_seconds += time.perf_counter() - t0
+            metrics.decode_steps += n
+            going = {i: True for i in rows}
+            for k in range(n):
+                for (i, slot), tok in zip(live, sampled[k]):
+                    held[i] += 1                      # step k fed this sequence's previous token
+                    if going[i]:
+                        going[i] = take(i, slot, tok)
             nxt = []
-            for (i, slot), tok in zip(live, ids_out):
-                r, out = requests[i], results[i]
-                out.tokens.append(int(tok))
-                metrics.generated_tokens += 1
-                if on_token is not None:
-                    on_token(i, int(tok))
-                if int(tok) in r.stop_ids:
-                    out.finish_reason = "stop"       # the stop token is part of the result
-                elif len(out.tokens) >= r.max_new_tokens or held[i] >= backend.max_context:
-                    out.finish_reason = "length"     # no room to feed this token back
-                if out.finish_reason is not None:
-                    backend.give_back_slot(slot)
-                else:
+            for i, slot in live:
+                if going[i]:
                     nxt.append((i, slot))
+                else:
+                    backend.give_back_slot(slot)
             live = nxt
-            if not live:
-                break
-            logits = backend.step([(slot, [results[i].tokens[-1]]) for i, slot in live])
-            for i, _ in live:
-                held[i] += 1
-            step_no += 1
     except BaseException:
         for _, slot in live:
             try:

@@ -12,7 +12,6 @@ import math
 import torch
 
 from ..cache import KVNeed
-from ..csrc import lib as K
 from ..weights.loader import TensorSpec
 from . import ops
 from .base import build_part, register_part
@@ -59,20 +58,11 @@ class GQAAttention:
         T, H, Kh, hs = h.shape[0], self.H, self.Kh, self.hs
         k_cache, v_cache = ctx.cache.layer_kv(run.kv_entry)
         table = ctx.block_table(ctx.cache.group_index(run.kv_entry))
-        pos = self.position
-        if run.writes_kv:
-            qkv = ctx.buffer("qkv", (T, (H + 2 * Kh) * hs), self.dtype)
-            ops.linear(h, self.w_qkv, qkv)
-        else:
-            qkv = ctx.buffer("qkv", (T, H * hs), self.dtype)
-            ops.linear(h, self.w_q, qkv)
-        K.rope_cache_write(qkv, ctx.positions, ctx.seq_of_token, table,
-                           pos.cos if pos else None, pos.sin if pos else None, k_cache, v_cache,
-                           H, Kh, hs, pos.rot_dim if pos else 0, pos.adjacent if pos else False,
-                           ctx.cache.page_size, write_kv=run.writes_kv)
+        q = ops.qkv_project(ctx, h, self.w_qkv, self.w_q, self.position, k_cache, v_cache, table, H, Kh, hs,
+                            self.dtype, run.writes_kv)
         att = ctx.buffer("attn_out", (T, H * hs), self.dtype)
-        ops.attention(ctx, qkv, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale)
-        ops.linear(att, self.w_o, x, ops.EPI_ADD)
+        ops.attention(ctx, q, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale)
+        ops.linear(att, self.w_o, x, ops.EPI_ADD, ctx)
 
 
 register_part("mixer", "attention", GQAAttention)

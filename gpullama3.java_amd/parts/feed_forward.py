@@ -34,8 +34,8 @@ class GatedFeedForward:
 
     def forward(self, ctx, h, x):
         act = ctx.buffer("ffn_act", (h.shape[0], self.F), self.dtype)
-        ops.linear(h, self.w_gate_up, act, ops.EPI_GATED)
-        ops.linear(act, self.w_down, x, ops.EPI_ADD)
+        ops.linear(h, self.w_gate_up, act, ops.EPI_GATED, ctx)
+        ops.linear(act, self.w_down, x, ops.EPI_ADD, ctx)
 
 
 register_part("ffn", "gated", GatedFeedForward)

@@ -78,12 +78,18 @@ class DecoderModel:
     def forward(self, ctx, want_rows):
         """Logits ``[len(want_rows), vocab]`` float32 at the wanted packed rows."""
         x = ctx.buffer("residual", (ctx.n_tokens, self.spec.hidden), torch.float32)
-        K.embed(self.embedding, ctx.token_ids, x)
+        if getattr(ctx, "fuse", False) and ctx.n_tokens <= ops.FUSE_ROWS:
+            ssq = ctx.ssq_buffer(1)                      # the first norm's sums of squares come with the rows
+            K.embed(self.embedding, ctx.token_ids, x, ssq)
+            ops.residual_written(ctx, x, ssq, 1)
+        else:
+            K.embed(self.embedding, ctx.token_ids, x)
+            ops.residual_written(ctx, x)
         for run, r in zip(self.runs, self.spec.run_order):
             self.blocks[r.layer].forward(ctx, x, run)
         n = want_rows.numel()
         logits = ctx.logits_buffer(n, self.spec.vocab_size)
         if n:
             h = self.final_norm(ctx, x, rows=want_rows, name="final_normed")
-            ops.linear(h, self.head, logits)
+            ops.linear(h, self.head, logits, ops.EPI_STORE, ctx)
         return logits

@@ -7,6 +7,8 @@ from ..csrc import lib as K
 from ..weights.loader import TensorSpec
 from .base import register_part
 
+FUSE_ROWS = 32      # a norm is folded into the next product for steps of at most this many tokens
+
 
 class RMSNorm:
     graph_safe = True      # kernel launches on the current stream only, sizes fixed by (T, B)
@@ -21,8 +23,17 @@ class RMSNorm:
 
     def load(self, weights):
         self.weight = weights[self.name]
+        # the products that fold the norm in read the weight as float (exact for 16-bit storage)
+        self.weight_f32 = self.weight if self.weight.dtype == torch.float32 else self.weight.float()
 
     def __call__(self, ctx, x, rows=None, name="normed"):
+        """The normalised rows, or a ``Normed`` when the next product can do the work itself (few
+        rows, and the sums of squares of exactly this tensor are at hand)."""
+        ssq = getattr(ctx, "ssq", None)
+        if (getattr(ctx, "fuse", False) and ssq is not None and ssq[0] == x.data_ptr() and x.shape[0] <= FUSE_ROWS
+                and self.dtype == torch.bfloat16):
+            from .ops import Normed
+            return Normed(ctx, x, self.weight, self.weight_f32, self.eps, self.dtype, ssq[1], ssq[2], rows, name)
         n = x.shape[0] if rows is None else rows.numel()
         out = ctx.buffer(name, (n, self.dim), self.dtype)
         K.rmsnorm(x, self.weight, out, self.eps, rows)

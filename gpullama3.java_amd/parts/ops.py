@@ -12,19 +12,97 @@ from ..csrc import lib as K
 
 EPI_STORE, EPI_ADD, EPI_GATED = K.EPI_STORE, K.EPI_ADD, K.EPI_GATED
 
+# a norm is folded into the next product for steps of at most this many tokens: beyond two token
+# tiles the folded kernels run out of registers
+FUSE_ROWS = 32
+
 # switches for tests and measurements: names of fast kernels that must not be used
 disabled = set()
 
 
-def linear(a, w, out, epilogue=EPI_STORE):
-    """out (=, +=, gated) a @ w.T."""
+class Normed:
+    """The RMSNorm of (rows of) the float residual stream, not computed yet.
+
+    A norm hands this out instead of a tensor when the step is small enough for the
+    product that follows to do the norm's work itself: the sum of squares of every row is
+    already there as partial sums, left by the kernel that last wrote the rows.
+    ``materialize`` runs the norm as a kernel of its own, for consumers that cannot."""
+
+    def __init__(self, ctx, x, weight, weight_f32, eps, dtype, ssq, n_partials, rows, name):
+        self.ctx, self.x, self.weight, self.eps, self.dtype = ctx, x, weight, eps, dtype
+        self.weight_f32 = weight_f32
+        self.ssq, self.n_partials, self.rows, self.name = ssq, n_partials, rows, name
+        self.shape = (x.shape[0] if rows is None else rows.numel(), x.shape[1])
+
+    def materialize(self):
+        out = self.ctx.buffer(self.name, self.shape, self.dtype)
+        K.rmsnorm(self.x, self.weight, out, self.eps, self.rows)
+        return out
+
+
+def residual_written(ctx, x, ssq=None, n_partials=0):
+    """Every writer of the residual stream says so: the partial sums of squares that a folded
+    norm would use are those of the last writer, or none."""
+    if ctx is not None:
+        ctx.ssq = (x.data_ptr(), ssq, n_partials) if ssq is not None else None
+
+
+def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
+    """out (=, +=, gated) a @ w.T. ``a`` may be a ``Normed``. With the add epilogue ``out`` is the
+    residual stream."""
+    if isinstance(a, Normed):
+        if ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.x, w, out, epilogue)
+                and a.x.shape[0] <= 64):
+            return K.gemm_skinny_norm(a.x, a.weight_f32, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows)
+        a = a.materialize()
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
-        M = a.shape[0]
-        if "skinny" not in disabled and K.has("gl3_gemm_skinny") and K.gemm_skinny_fits(a, w, out, epilogue):
-            return K.gemm_skinny(a, w, out, epilogue)
-        if "mfma" not in disabled and K.has("gl3_gemm_mfma") and K.gemm_mfma_fits(a, w, out, epilogue):
-            return K.gemm_mfma(a, w, out, epilogue)
-    return K.gemm_generic(a, w, out, epilogue)
+        if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
+            N = out.shape[1]
+            if (epilogue == EPI_ADD and ctx is not None and getattr(ctx, "fuse", False) and N % 16 == 0
+                    and "fused" not in disabled):
+                ssq = ctx.ssq_buffer(N // 16)
+                K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq)
+                return residual_written(ctx, out, ssq, N // 16)
+            K.gemm_skinny(a, w, out, epilogue)
+            if epilogue == EPI_ADD:
+                residual_written(ctx, out)
+            return
+        if "mfma" not in disabled and K.gemm_mfma_fits(a, w, out, epilogue):
+            K.gemm_mfma(a, w, out, epilogue)
+            if epilogue == EPI_ADD:
+                residual_written(ctx, out)
+            return
+    K.gemm_generic(a, w, out, epilogue)
+    if epilogue == EPI_ADD:
+        residual_written(ctx, out)
+
+
+def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_heads, n_kv, head_dim, dtype, writes_kv):
+    """Queries, keys and values of the step's tokens: q rotated into a buffer whose rows start
+    with the H*hs query columns (returned), k rotated and v into the cache. One kernel when
+    ``h`` is a ``Normed`` and the shapes allow, else product and rotation apart."""
+    T = h.shape[0]
+    page = k_cache.shape[2]
+    cos, sin = (rotary.cos, rotary.sin) if rotary is not None else (None, None)
+    rot = rotary.rot_dim if rotary is not None else 0
+    adjacent = rotary.adjacent if rotary is not None else False
+    if (isinstance(h, Normed) and writes_kv and h.rows is None and "fused" not in disabled
+            and K.qkv_rope_cache_fits(h.x, w_qkv, head_dim, rot)):
+        q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
+        K.qkv_rope_cache(h.x, h.weight_f32, h.ssq, h.n_partials, h.eps, w_qkv, q, ctx.positions, ctx.seq_of_token,
+                         block_table, cos, sin, k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page)
+        return q
+    if isinstance(h, Normed):
+        h = h.materialize()
+    if writes_kv:
+        qkv = ctx.buffer("qkv", (T, (n_heads + 2 * n_kv) * head_dim), dtype)
+        linear(h, w_qkv, qkv)
+    else:
+        qkv = ctx.buffer("qkv", (T, n_heads * head_dim), dtype)
+        linear(h, w_q, qkv)
+    K.rope_cache_write(qkv, ctx.positions, ctx.seq_of_token, block_table, cos, sin, k_cache, v_cache,
+                       n_heads, n_kv, head_dim, rot, adjacent, page, write_kv=writes_kv)
+    return qkv
 
 
 def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale):

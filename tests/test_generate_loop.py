@@ -58,6 +58,27 @@ class FakeBackend:
         return [sample_host(l, t, p, u) for l, t, p, u in zip(logits, temperatures, top_ps, uniforms)]
 
 
+class RunBackend(FakeBackend):
+    """Runs several decode steps before it reports, as an engine that samples on the device does."""
+    decode_run_length = 4
+
+    def decode_run(self, entries, n, temperatures, top_ps, uniforms):
+        assert 1 <= n <= self.decode_run_length
+        out = []
+        cur = list(entries)
+        self.runs.append(n)
+        for k in range(n):
+            logits = self.step([(s, [t]) for s, t in cur])
+            toks = self.sample(logits, temperatures, top_ps, uniforms[k])
+            out.append(toks)
+            cur = [(s, t) for (s, _), t in zip(cur, toks)]
+        return out
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self.runs = []
+
+
 def alone(prompt, n, sampling=SamplingParams(), stops=(), index=0, max_context=64):
     seq, out = list(prompt), []
     while len(out) < n:
@@ -175,3 +196,23 @@ def test_a_failing_step_gives_the_slots_back():
     with pytest.raises(CacheFull):
         generate(be, [Request([1] * 30, 2), Request([1] * 30, 2)])
     assert be.cache.slots.live == set() and be.cache.groups[0].pool.n_free == 2
+
+
+def test_runs_of_steps_give_the_same_tokens_and_respect_every_budget():
+    sp = SamplingParams(0.9, 0.9, seed=3)
+    ps = prompts([5, 11, 3, 8], seed=9)
+    news = [6, 13, 2, 9]
+    free = [alone(p, n, sp, index=i) for i, (p, n) in enumerate(zip(ps, news))]
+    stop = free[1][7]
+    reqs = [Request(p, n, sp, frozenset([stop])) for p, n in zip(ps, news)]
+    plain = generate(FakeBackend(), reqs)
+    be = RunBackend()
+    got = generate(be, reqs)
+    assert [r.tokens for r in got] == [r.tokens for r in plain]
+    assert [r.finish_reason for r in got] == [r.finish_reason for r in plain]
+    assert max(be.runs) == 4 and be.cache.slots.live == set()
+    # no sequence was stepped past its budget: the cache never held more than prompt + new - 1 tokens
+    tight = RunBackend(max_context=16)
+    p = prompts([10], seed=10)[0]
+    out = generate(tight, [Request(p, 50, sp)])[0]
+    assert len(out.tokens) == 7 and out.finish_reason == "length"         # 16 - 10 fed back, one more sampled

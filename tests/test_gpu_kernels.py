@@ -482,3 +482,94 @@ def test_attention_prefill_far_key_and_window_edge():
         got, ref = run_attention(prefill_fn([0], [n]), [k2], [v], [q], [0], [n], H, Kh, hs, "bfloat16", rng, window=w)
         np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
         assert (np.abs(got[-1, 2] - v[hot, 1]).max() < 4e-2) == inside
+
+
+# ------------------------------------------------------------------ norms and rotation folded into the products
+def ssq_partials(x, n_partials):
+    """Partial sums of squares as a producer leaves them: [n_partials, 64], rows of x in the columns."""
+    M, d = x.shape
+    out = np.zeros((n_partials, 64), np.float32)
+    for p, cols in enumerate(np.array_split(np.arange(d), n_partials)):
+        out[p, :M] = (x[:, cols] ** 2).sum(1)
+    return out
+
+
+@pytest.mark.parametrize("M", [1, 8, 33, 64])
+@pytest.mark.parametrize("N, Kd, P_", [(2048, 2048, 128), (130, 64, 1), (1000, 112, 7)])
+def test_gemm_skinny_with_folded_norm(M, N, Kd, P_, wdtype="float32"):
+    rng = np.random.default_rng(M + N)
+    extra = 3 if M + 3 <= 64 else 0
+    x = (rng.standard_normal((M + extra, Kd)) * 2).astype(np.float32)       # more rows than are used, where they fit
+    nw = rounded(1 + 0.2 * rng.standard_normal(Kd), wdtype)
+    w = rounded(rng.standard_normal((2 * N, Kd)) / math.sqrt(Kd), "bfloat16")
+    lib = K()
+    X, NW_, W = dev(x), dev(nw, TD[wdtype]), dev(w, torch.bfloat16)
+    ssq = dev(ssq_partials(x, P_))
+    h = P.rmsnorm(x, nw, 1e-5)
+    rows = np.arange(M)[::-1].copy() + extra                                 # a gather of rows
+    ref = P.linear(h[rows], w[:N])
+    out = torch.zeros(M, N, device=DEV)
+    lib.gemm_skinny_norm(X, NW_, ssq, P_, 1e-5, W[:N], out, lib.EPI_STORE, rows=dev(rows, torch.int32))
+    np.testing.assert_allclose(out.cpu().numpy(), ref, atol=1e-2 * np.abs(ref).max())   # x*w is rounded to bfloat16
+    refg = P.silu(P.linear(h[:M], w[:N])) * P.linear(h[:M], w[N:])
+    g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+    lib.gemm_skinny_norm(X[:M], NW_, ssq, P_, 1e-5, W, g_, lib.EPI_GATED)
+    np.testing.assert_allclose(g_.float().cpu().numpy(), refg, atol=1.5e-2 * max(np.abs(refg).max(), 1e-3))
+
+
+@pytest.mark.parametrize("M", [1, 8, 40])
+def test_gemm_skinny_leaves_sums_of_squares(M):
+    rng = np.random.default_rng(M)
+    N, Kd = 208, 96
+    a = rounded(rng.standard_normal((M, Kd)), "bfloat16")
+    w = rounded(rng.standard_normal((N, Kd)) / 10, "bfloat16")
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    x = dev(res)
+    ssq = torch.full((N // 16, 64), -1.0, device=DEV)
+    K().gemm_skinny(dev(a, torch.bfloat16), dev(w, torch.bfloat16), x, K().EPI_ADD, ssq_out=ssq)
+    new = res + P.linear(a, w)
+    np.testing.assert_allclose(x.cpu().numpy(), new, atol=1e-4)
+    got = ssq.cpu().numpy()
+    np.testing.assert_allclose(got[:, :M], ssq_partials(new, N // 16)[:, :M], rtol=1e-4)
+    assert np.all(got[:, M:] == -1.0)                                        # rows that do not exist are not written
+
+
+@pytest.mark.parametrize("pairing", ["adjacent", "half", None])
+@pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 16), (5, 5, 48), (8, 1, 128)])
+def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs):
+    rng = np.random.default_rng(hs + H)
+    d, page = 96, 64
+    lens_before = [70, 0, 129, 63, 64]
+    T = len(lens_before)
+    x = (rng.standard_normal((T, d)) * 2).astype(np.float32)
+    nw = rounded(1 + 0.2 * rng.standard_normal(d), "bfloat16")
+    w = rounded(rng.standard_normal(((H + 2 * Kh) * hs, d)) / math.sqrt(d), "bfloat16")
+    positions = np.array(lens_before)
+    seq_of = np.arange(T)
+    zk = [np.zeros((b + 1, Kh, hs), np.float32) for b in lens_before]
+    kc, vc, table = paged(zk, zk, Kh, hs, page, "bfloat16", rng)
+    before_k, before_v = kc.clone(), vc.clone()
+    cos, sin = P.rope_table(256, hs, 50000.0)
+    q_out = torch.zeros(T, H * hs, device=DEV, dtype=torch.bfloat16)
+    K().qkv_rope_cache(dev(x), dev(nw), dev(ssq_partials(x, 6)), 6, 1e-5, dev(w, torch.bfloat16), q_out,
+                       dev(positions, torch.int32), dev(seq_of, torch.int32), table,
+                       dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
+                       pairing == "adjacent", page)
+    qkv = P.linear(P.rmsnorm(x, nw, 1e-5), w)
+    q = qkv[:, :H * hs].reshape(T, H, hs)
+    k = qkv[:, H * hs:(H + Kh) * hs].reshape(T, Kh, hs)
+    v = qkv[:, (H + Kh) * hs:].reshape(T, Kh, hs)
+    if pairing:
+        q = P.rope_rotate(q, positions, cos, sin, pairing)
+        k = P.rope_rotate(k, positions, cos, sin, pairing)
+    tol_ = 1.5e-2 * np.abs(qkv).max()
+    np.testing.assert_allclose(q_out.float().cpu().numpy().reshape(T, H, hs), q, atol=tol_)
+    kcpu, vcpu, tab = kc.float().cpu().numpy(), vc.float().cpu().numpy(), table.cpu().numpy()
+    mk, mv = torch.ones_like(kc, dtype=torch.bool), torch.ones_like(vc, dtype=torch.bool)
+    for i in range(T):
+        pid = tab[i, positions[i] // page]
+        np.testing.assert_allclose(kcpu[pid, :, positions[i] % page], k[i], atol=tol_)
+        np.testing.assert_allclose(vcpu[pid, :, :, positions[i] % page], v[i], atol=tol_)
+        mk[pid, :, positions[i] % page] = False
+        mv[pid, :, :, positions[i] % page] = False
+    assert torch.equal(kc[mk], before_k[mk]) and torch.equal(vc[mv], before_v[mv])   # nothing else moved
