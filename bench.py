@@ -168,8 +168,8 @@ def main():
             "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "vocab_size": cfg.vocab_size, "tied_head": cfg.tie_word_embeddings, "rope_theta": cfg.rope_theta,
             "rope_scaling_factor": cfg.rope_scaling.factor, "rms_norm_eps": cfg.rms_norm_eps,
-            "global_batch": args.batch, "context_length": CONTEXT, "prompt_len": PROMPT,
-            "prefill_len": PREFILL, "parallelism": "single GPU", "sampling": "greedy on device",
+            "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPT, "prefill_len": PREFILL,
+            "parallelism": "single GPU", "sampling": "greedy on device",
         },
         "prefill": {"value": round(PREFILL / prefill_s, 1), "tokens": PREFILL, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / (PEAK_TFLOPS[short] * 1e12), 4)},
