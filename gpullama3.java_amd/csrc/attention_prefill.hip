@@ -12,9 +12,12 @@
 //   O^T[dim, query] += V^T[dim, key] . P^T[key, query]
 // which makes 16 bytes of a key row, and of a row of the transposed value page, the
 // operands as the instruction wants them, and leaves the probabilities in the register
-// order the second product takes. The four waves of a block take neighbouring query
-// tiles and share their keys and values through the caches only; they never wait for
-// each other.
+// order the second product takes (row i of the first score tile is key 8*(i/4) + i%4 of
+// the chunk, row i of the second the key 4 further, so a quarter of the lanes ends up with
+// 8 consecutive keys: one 16-byte load from a row of the transposed value page). The
+// operands of the next chunk are asked for before the current chunk is worked on. The four
+// waves of a block take neighbouring query tiles and share their keys and values through
+// the caches only; they never wait for each other.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -35,12 +38,14 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int qb = q_blocks - 1 - blockIdx.x;
   const int b = blockIdx.y;
   const int c = blockIdx.z / groups, hg = blockIdx.z % groups;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // scalar: what depends on the wave alone (chunk, page) lives in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int j = lane & 15, qd = lane >> 4;
-  const int tok0 = cu_seqlens[b], q_len = cu_seqlens[b + 1] - tok0;
+  const int tok0 = __builtin_amdgcn_readfirstlane(cu_seqlens[b]);
+  const int q_len = __builtin_amdgcn_readfirstlane(cu_seqlens[b + 1]) - tok0;
   const int qi0 = qb * 64 + wave * 16;   // first query of this wave, counted inside the step's tokens
   if (qi0 >= q_len) return;
-  const int before = kv_before[b];
+  const int before = __builtin_amdgcn_readfirstlane(kv_before[b]);
   const int heads_here = min(GH, g - hg * GH);
   const int h0 = c * g + hg * GH;
   const int* bt = block_table + (long)b * table_stride;
@@ -71,30 +76,33 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     for (int dt = 0; dt < DT; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int ck = lo_first / 32; ck * 32 <= p_last; ++ck) {
+  const int krow = 8 * (j >> 2) + (j & 3);   // which key of a chunk is row j of the first score tile
+  bf16x8 ka[KK], kb2[KK], vt[DT], ka_n[KK], kb2_n[KK], vt_n[DT];
+  auto load_chunk = [&](int ck, bf16x8 (&a)[KK], bf16x8 (&b2)[KK], bf16x8 (&v)[DT]) {
     const int key0 = ck * 32;
-    const long page = bt[key0 / page_size];
+    const long page = __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
     const int po = key0 % page_size;
     const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
     const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + po;
-    bf16x8 ka[KK], kb2[KK];
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      ka[kk] = *(const bf16x8*)(kb + (long)j * HS + kk * 32 + 8 * qd);
-      kb2[kk] = *(const bf16x8*)(kb + (long)(16 + j) * HS + kk * 32 + 8 * qd);
+      a[kk] = *(const bf16x8*)(kb + (long)krow * HS + kk * 32 + 8 * qd);
+      b2[kk] = *(const bf16x8*)(kb + (long)(krow + 4) * HS + kk * 32 + 8 * qd);
     }
-    bf16x8 vt[DT];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const bf16_t* vr = vb + (long)(dt * 16 + j) * page_size + 4 * qd;
-      const bf16x4 v0 = *(const bf16x4*)vr, v1 = *(const bf16x4*)(vr + 16);
-      vt[dt] = bf16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-    }
+    for (int dt = 0; dt < DT; ++dt) v[dt] = *(const bf16x8*)(vb + (long)(dt * 16 + j) * page_size + 8 * qd);
+  };
+  const int ck_first = lo_first / 32, ck_last = p_last / 32;
+  load_chunk(ck_first, ka, kb2, vt);
+  for (int ck = ck_first; ck <= ck_last; ++ck) {
+    const int key0 = ck * 32;
+    if (ck < ck_last) load_chunk(ck + 1, ka_n, kb2_n, vt_n);   // on its way while this chunk is worked on
+    __builtin_amdgcn_sched_barrier(0);
     // this lane's 8 keys of the chunk and whether its query may see them
     bool see[8];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const int k1 = key0 + 4 * qd + v, k2 = k1 + 16;
+      const int k1 = key0 + 8 * qd + v, k2 = k1 + 4;
       see[v] = k1 >= lo_mine && k1 <= p_mine;
       see[4 + v] = k2 >= lo_mine && k2 <= p_mine;
     }
@@ -134,6 +142,12 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
         o[hh][dt] *= alpha;
         o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt], pb, o[hh][dt], 0, 0, 0);
       }
+    }
+    if (ck < ck_last) {
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) { ka[kk] = ka_n[kk]; kb2[kk] = kb2_n[kk]; }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vt[dt] = vt_n[dt];
     }
   }
 
