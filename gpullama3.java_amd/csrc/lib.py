@@ -53,6 +53,7 @@ def _declare(lib):
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P],
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
+        "gl3_argmax": [P, L, P, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
         "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P],
@@ -232,6 +233,16 @@ def decode_advance(token_ids, positions, kv_before, sampled, history, step):
         raise KernelError("decode_advance: sizes")
     _check(library().gl3_decode_advance(_ptr(token_ids), _ptr(positions), _ptr(kv_before), _ptr(sampled),
                                         _ptr(history), history.stride(0), _ptr(step), n, _stream()), "decode_advance")
+
+
+def argmax(logits, work, out):
+    """Every row's first greatest logit; ``work``: at least 128 floats per row."""
+    _dev(logits, "logits", torch.float32, contiguous=False); _dev(work, "work", torch.float32)
+    _dev(out, "out", torch.int32)
+    R, V = logits.shape
+    if logits.stride(1) != 1 or work.numel() < 128 * R or out.numel() < R:
+        raise KernelError("argmax: argument sizes")
+    _check(library().gl3_argmax(_ptr(logits), logits.stride(0), _ptr(work), _ptr(out), R, V, _stream()), "argmax")
 
 
 def sample(logits, work, temperature, top_p, uniform, out, step=None, uniform_stride=0):

@@ -183,6 +183,67 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
   if (tid == 0) out[row] = winner >= 0 ? winner : V - 1;
 }
 
+// Greedy rows only, in two stages so that a row is read by many blocks at once: each block finds the
+// first greatest logit of its slice, a second kernel the first greatest of the slices' results.
+#define ARG_SLICES 64
+
+__global__ __launch_bounds__(256) void argmax_slice_kernel(const float* __restrict__ logits, long ld,
+                                                           float* __restrict__ part_val, int* __restrict__ part_idx,
+                                                           int V) {
+  __shared__ float fs[4];
+  __shared__ int is[4];
+  const int row = blockIdx.x, slice = blockIdx.y, tid = threadIdx.x;
+  const int per = (V + ARG_SLICES - 1) / ARG_SLICES;
+  const int lo = slice * per, hi = min(V, lo + per);
+  const float* lg = logits + (long)row * ld;
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = lo + tid; i < hi; i += 256) {
+    const float v = lg[i];
+    if (v > best) { best = v; idx = i; }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(idx, o, 64);
+    if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
+  }
+  if ((tid & 63) == 0) { fs[tid >> 6] = best; is[tid >> 6] = idx; }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (fs[w] > best || (fs[w] == best && is[w] < idx)) { best = fs[w]; idx = is[w]; }
+    part_val[row * ARG_SLICES + slice] = best;
+    part_idx[row * ARG_SLICES + slice] = idx;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ part_val,
+                                                          const int* __restrict__ part_idx, int* __restrict__ out) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  float best = part_val[row * ARG_SLICES + lane];
+  int idx = part_idx[row * ARG_SLICES + lane];
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(idx, o, 64);
+    if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
+  }
+  if (lane == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
+}
+
+// Every row greedy (J/inference/sampler/Sampler.java:144-157). work: at least 2 * n_rows * 64 floats.
+extern "C" int gl3_argmax(const float* logits, long ld, float* work, int* out, int n_rows, int V, hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  GL3_REQUIRE(logits && work && out && n_rows > 0 && V > 0 && ld >= V, "gl3_argmax: bad arguments");
+  GL3_REQUIRE(n_rows <= 65535, "gl3_argmax: too many rows");
+  float* pv = work;
+  int* pi = (int*)(work + (long)n_rows * ARG_SLICES);
+  argmax_slice_kernel<<<dim3(n_rows, ARG_SLICES), dim3(256), 0, stream>>>(logits, ld, pv, pi, V);
+  GL3_LAUNCH_CHECK();
+  argmax_final_kernel<<<dim3(n_rows), dim3(64), 0, stream>>>(pv, pi, out);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
 // work: [n_rows, V] floats of scratch (probabilities); unused for greedy rows.
 // step (may be null): a counter in device memory; row r then takes uniform[step[0] * uniform_stride + r].
 extern "C" int gl3_sample(const float* logits, long ld, float* work, const float* temperature, const float* top_p,

@@ -239,7 +239,8 @@ class Engine:
         starts = [self.cache.length(s) for s in slots]
         self.cache.reserve({s: n for s in slots})
         with torch.cuda.device(self.device):
-            dg = self._graph_for(B, max(starts) + n, run=True)
+            greedy = all(t == 0 for t in temperatures)
+            dg = self._graph_for(B, max(starts) + n, run="greedy" if greedy else "sampled")
             self._fill_graph_input(dg, B, tokens, starts, slots)
             B_pad = dg.B_pad
             f = dg.fhost
@@ -344,7 +345,7 @@ class Engine:
             from ..csrc import lib as K
             dg.fhost = torch.zeros((2 + RUN_LENGTH) * B_pad, dtype=torch.float32).pin_memory()
             dg.fdev = torch.zeros((2 + RUN_LENGTH) * B_pad, dtype=torch.float32, device=self.device)
-            work = torch.empty(B_pad * self.spec.vocab_size, dtype=torch.float32, device=self.device)
+            work = torch.empty(B_pad * max(self.spec.vocab_size, 128), dtype=torch.float32, device=self.device)
             step = d[dg.off_step:dg.off_step + 1]
             sampled = d[dg.off_sampled:dg.off_sampled + B_pad]
             hist = d[dg.off_hist:dg.off_hist + RUN_LENGTH * B_pad].view(RUN_LENGTH, B_pad)
@@ -353,8 +354,11 @@ class Engine:
 
         def body():
             logits = self.model.forward(ctx, rows)
-            if run:
+            if run == "greedy":
+                K.argmax(logits, work, sampled)
+            elif run:
                 K.sample(logits, work, temps, tops, us, sampled, step=step, uniform_stride=B_pad)
+            if run:
                 K.decode_advance(ctx.token_ids, ctx.positions, ctx.kv_before, sampled, hist, step)
             return logits
 

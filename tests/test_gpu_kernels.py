@@ -573,3 +573,19 @@ def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs):
         mk[pid, :, positions[i] % page] = False
         mv[pid, :, :, positions[i] % page] = False
     assert torch.equal(kc[mk], before_k[mk]) and torch.equal(vc[mv], before_v[mv])   # nothing else moved
+
+
+@pytest.mark.parametrize("V", [2, 63, 1000, 128256])
+def test_argmax_kernel_takes_the_first_of_the_greatest(V):
+    rng = np.random.default_rng(V)
+    R = 9
+    logits = rng.standard_normal((R, V)).astype(np.float32)
+    logits[2, [V // 3, V - 1]] = 50.0                       # ties: the lower index, across slices
+    logits[5, :] = -np.inf                                    # nothing greater than -inf: index 0
+    logits[6, 0] = 60.0
+    logits[7, V - 1] = 60.0
+    wide = torch.zeros(R, V + 5, device=DEV)                  # rows with a stride
+    wide[:, :V] = dev(logits)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    K().argmax(wide[:, :V], torch.empty(128 * R, device=DEV), out)
+    assert out.tolist() == [P.argmax(row) for row in logits]
