@@ -12,48 +12,139 @@
 // The uniform number u in [0,1) comes from the caller, one per row.
 //
 // No sort: the kept set is {p > v} plus the first k of {p == v}, where v is the
-// greatest threshold whose mass {p >= v} still exceeds top_p; v is found bit by
-// bit over the float's pattern (31 passes), and the walk to the drawn token is the
-// same search with u * mass in place of top_p. Masses are summed in 64-bit so that
-// the order of the sum cannot move a comparison.
+// greatest threshold whose mass {p >= v} still exceeds top_p; v is found digit by
+// digit over the float's bit pattern (four passes with histograms), and the walk to
+// the drawn token is the same search with u * mass in place of top_p. Masses are
+// summed as 64-bit integers (p * 2^62), so the order of a sum cannot move a comparison.
 #include "common.h"
 
 #define SB 1024
+#define SW 16          // waves of a block
+#define UN 16          // elements a thread asks for before it uses the first: a pass is bound by trips to memory
+#define QSCALE 4611686018427387904.0   // 2^62: probabilities as 64-bit integers, sums exact and in any order
 
-// inclusive scan of one double per thread over the block; result in cdf[SB]
-__device__ void block_scan_f64(double v, double* cdf, double* wave_tot) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  double x = v;
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    double y = __shfl_up(x, o, 64);
-    if (lane >= o) x += y;
-  }
-  __syncthreads();
-  if (lane == 63) wave_tot[wave] = x;
-  __syncthreads();
-  double off = 0.0;
-  for (int w = 0; w < wave; ++w) off += wave_tot[w];
-  cdf[threadIdx.x] = x + off;
-  __syncthreads();
+// A probability (0 <= p <= 1) as an integer: floor(p * 2^62), exact for p >= 2^-38, truncated below;
+// taken from the float's bits: mantissa shifted by its exponent.
+__device__ __forceinline__ unsigned long long to_q(float p) {
+  const uint32_t b = __float_as_uint(p);
+  const int e = (int)(b >> 23) - 127;                    // p = 1.m * 2^e (e = -127: zero or denormal, taken as 0)
+  if (e < -62) return 0ull;
+  const unsigned long long m = (unsigned long long)((b & 0x7fffffu) | 0x800000u);   // 24 bits, value m * 2^(e-23)
+  const int sh = 62 - 23 + e;                            // q = m * 2^sh
+  return sh >= 0 ? m << sh : m >> -sh;
 }
 
-// greatest v (as a bit pattern) with sum{p_i >= v} > thr
-__device__ uint32_t search_threshold(const float* p, int V, double thr, double* scratch) {
-  uint32_t cur = 0;
-  for (int bit = 30; bit >= 0; --bit) {
-    const uint32_t cand = cur | (1u << bit);
-    if (cand > 0x3f800000u) continue;  // above 1.0: no probability reaches it
-    const float v = __uint_as_float(cand);
-    double mass = 0.0;
-    for (int i = threadIdx.x; i < V; i += SB) {
-      const float pi = p[i];
-      if (pi >= v) mass += (double)pi;
+struct Found {
+  uint32_t bits;               // the threshold value's bit pattern
+  unsigned long long above;    // mass of the values greater than it
+  unsigned long long each;     // the value as an integer
+  int ties;                    // how many values equal it
+};
+
+// The greatest value v with mass{p >= v} > thr, found digit by digit over the float's bit pattern
+// (8, 8, 8 and 7 bits): per digit one pass builds a histogram of mass and count over the values that
+// share the digits found so far, in private per-wave tables (integer adds in shared memory), and
+// wave 0 walks the 256 bins from the top. If no prefix of the values exceeds thr (thr is not below
+// the total mass), the smallest value is returned.
+__device__ Found radix_search(const float* __restrict__ p, int V, unsigned long long thr,
+                              unsigned long long (*h_mass)[256], int (*h_cnt)[256], unsigned long long* t_mass,
+                              int* t_cnt, unsigned long long* res) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  uint32_t prefix = 0;
+  unsigned long long above = 0;
+  const int shifts[4] = {23, 15, 7, 0}, widths[4] = {8, 8, 8, 7};
+  for (int level = 0; level < 4; ++level) {
+    const int shift = shifts[level], width = widths[level];
+    const uint32_t mask = (1u << width) - 1u;
+    for (int i = tid; i < SW * 256; i += SB) { (&h_mass[0][0])[i] = 0; (&h_cnt[0][0])[i] = 0; }
+    __syncthreads();
+    for (int base = 0; base < V; base += UN * SB) {   // every lane stays in the loop: the wave votes below
+      const int i0 = base + tid;
+      float v[UN];
+#pragma unroll
+      for (int u = 0; u < UN; ++u) v[u] = (i0 + u * SB < V) ? p[i0 + u * SB] : -1.f;
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const uint32_t b = __float_as_uint(v[u]);
+        const bool in = v[u] >= 0.f && (b >> (shift + width)) == prefix;
+        const int bin = (b >> shift) & mask;
+        // a wave whose lanes all fall into one bin adds once
+        const int first = __builtin_amdgcn_readfirstlane(in ? bin : -1);
+        if (__all(in && bin == first)) {
+          unsigned long long q = to_q(v[u]);
+#pragma unroll
+          for (int o = 32; o > 0; o >>= 1) q += __shfl_xor(q, o, 64);
+          if (lane == 0) { atomicAdd(&h_mass[wave][bin], q); atomicAdd(&h_cnt[wave][bin], 64); }
+        } else if (in) {
+          atomicAdd(&h_mass[wave][bin], to_q(v[u]));
+          atomicAdd(&h_cnt[wave][bin], 1);
+        }
+      }
     }
-    mass = block_sum_f64(mass, scratch);
-    if (mass > thr) cur = cand;
+    __syncthreads();
+    if (tid < 256) {
+      unsigned long long m = 0;
+      int c = 0;
+      for (int w = 0; w < SW; ++w) { m += h_mass[w][tid]; c += h_cnt[w][tid]; }
+      t_mass[tid] = m;
+      t_cnt[tid] = c;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      // lane l owns bins 255-4l .. 252-4l, walked downwards
+      unsigned long long mine = 0;
+      int cnt_mine = 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) { mine += t_mass[255 - 4 * lane - k]; cnt_mine += t_cnt[255 - 4 * lane - k]; }
+      unsigned long long incl = mine;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const unsigned long long y = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += y;
+      }
+      const bool crosses = above + incl > thr;
+      const unsigned long long hit = __ballot(crosses);
+      const unsigned long long some = __ballot(cnt_mine > 0);
+      int who, bin = -1;
+      unsigned long long cum = above + incl - mine;
+      if (hit) {
+        who = __ffsll((long long)hit) - 1;
+        if (lane == who) {
+          for (int k = 0; k < 4; ++k) {
+            const int b = 255 - 4 * lane - k;
+            if (cum + t_mass[b] > thr) { bin = b; break; }
+            cum += t_mass[b];
+          }
+        }
+      } else {
+        who = 63 - __builtin_clzll(some);   // the lowest bins that hold anything
+        if (lane == who) {
+          for (int k = 3; k >= 0; --k) {
+            const int b = 255 - 4 * lane - k;
+            if (t_cnt[b] > 0) { bin = b; break; }
+          }
+          cum = above + incl;
+          for (int k = 3; 255 - 4 * lane - k <= bin; --k) cum -= t_mass[255 - 4 * lane - k];
+        }
+      }
+      if (lane == who) { res[0] = (unsigned long long)bin; res[1] = cum; }
+    }
+    __syncthreads();
+    const int bin = (int)res[0];
+    above = res[1];
+    prefix = (prefix << width) | (uint32_t)bin;
+    if (level == 3) {
+      Found f;
+      f.bits = prefix;
+      f.above = above;
+      f.ties = t_cnt[bin];
+      f.each = f.ties ? t_mass[bin] / (unsigned long long)f.ties : 0;
+      __syncthreads();
+      return f;
+    }
+    __syncthreads();
   }
-  return cur;
+  return Found{};
 }
 
 __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ logits, long ld, float* __restrict__ work,
@@ -64,9 +155,14 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
   __shared__ float fs[16];
   __shared__ int is[16];
   __shared__ double ds[16];
-  __shared__ double cdf[SB];
+  __shared__ unsigned long long h_mass[SW][256];
+  __shared__ int h_cnt[SW][256];
+  __shared__ unsigned long long t_mass[256];
+  __shared__ int t_cnt[256];
+  __shared__ unsigned long long res[2];
+  __shared__ unsigned long long w_tot[SW];
   __shared__ int winner;
-  const int row = blockIdx.x, tid = threadIdx.x;
+  const int row = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const float* lg = logits + (long)row * ld;
   const float T = temperature[row];
 
@@ -93,91 +189,145 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
     return;
   }
 
+  // p = softmax(logits / T), kept in `work`
   float* p = work + (long)row * V;
   float m = -INFINITY;
-  for (int i = tid; i < V; i += SB) m = fmaxf(m, lg[i] / T);
+  for (int i0 = tid; i0 < V; i0 += UN * SB) {
+    float v[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) v[u] = (i0 + u * SB < V) ? lg[i0 + u * SB] : -INFINITY;
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const float sc = v[u] / T;                          // the division of the reference, once per element
+      if (i0 + u * SB < V) p[i0 + u * SB] = sc;
+      m = fmaxf(m, sc);
+    }
+  }
   m = block_max(m, fs);
   double z = 0.0;
-  for (int i = tid; i < V; i += SB) {
-    const float e = expf(lg[i] / T - m);
-    p[i] = e;
-    z += (double)e;
+  for (int i0 = tid; i0 < V; i0 += UN * SB) {
+    float v[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) v[u] = (i0 + u * SB < V) ? p[i0 + u * SB] : 0.f;
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int i = i0 + u * SB;
+      if (i < V) {
+        const float e = expf(v[u] - m);
+        p[i] = e;
+        z += (double)e;
+      }
+    }
   }
   const float zf = (float)block_sum_f64(z, ds);
-  for (int i = tid; i < V; i += SB) p[i] = p[i] / zf;
+  for (int i0 = tid; i0 < V; i0 += UN * SB) {
+    float v[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) v[u] = (i0 + u * SB < V) ? p[i0 + u * SB] : 0.f;
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+      if (i0 + u * SB < V) p[i0 + u * SB] = v[u] / zf;
+  }
   __syncthreads();
 
   const float tp = top_p[row];
   // in a run of steps replayed from a graph the step's number is read from memory
   const double u = (double)uniform[(step ? (long)step[0] * uniform_stride : 0) + row];
-  const int chunk = (V + SB - 1) / SB;
-  const int b = min(V, tid * chunk), e = min(V, (tid + 1) * chunk);
+  // every wave owns a contiguous range of the row, a multiple of 64 long
+  const int per = ((V + SW - 1) / SW + 63) / 64 * 64;
+  const int lo = min(V, wave * per), hi = min(V, lo + per);
   if (tid == 0) winner = -1;
 
+  float want_value = 0.f;             // top-p: the drawn token is the `want_index`-th (from 0) with this probability
+  long want_index = 0;
   if (tp <= 0.f || tp >= 1.f) {
-    double mine = 0.0;
-    for (int i = b; i < e; ++i) mine += (double)p[i];
-    block_scan_f64(mine, cdf, ds);
-    const double before = tid ? cdf[tid - 1] : 0.0;
-    if (before <= u && u < cdf[tid]) {
-      double c = before;
-      int pick = e - 1;
-      for (int i = b; i < e; ++i) {
-        c += (double)p[i];
-        if (u < c) { pick = i; break; }
+    // the first index whose running sum in index order exceeds u
+    const unsigned long long uq = (unsigned long long)(u * QSCALE);   // u = k / 2^24: exact
+    unsigned long long mine = 0;
+    for (int i0 = lo + lane; i0 < hi; i0 += 8 * 64) {
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = (i0 + 64 * k < hi) ? p[i0 + 64 * k] : 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) mine += to_q(v[k]);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
+    if (lane == 0) w_tot[wave] = mine;
+    __syncthreads();
+    unsigned long long before = 0;
+    for (int w = 0; w < wave; ++w) before += w_tot[w];
+    if (before <= uq && uq < before + w_tot[wave]) {       // the crossing lies in this wave's range
+      for (int base = lo; base < hi; base += 64) {
+        const int i = base + lane;
+        const unsigned long long q = i < hi ? to_q(p[i]) : 0;
+        unsigned long long incl = q;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const unsigned long long y = __shfl_up(incl, o, 64);
+          if (lane >= o) incl += y;
+        }
+        const unsigned long long hit = __ballot(uq < before + incl);
+        if (hit) {
+          if (lane == 0) winner = base + __ffsll((long long)hit) - 1;
+          break;
+        }
+        before += __shfl(incl, 63, 64);
       }
-      winner = pick;
     }
     __syncthreads();
     if (tid == 0) out[row] = winner >= 0 ? winner : V - 1;
     return;
   }
 
-  // nucleus: threshold v1, the mass above it, and how many of the equal ones are kept
-  const float v1 = __uint_as_float(search_threshold(p, V, (double)tp, ds));
-  double gt = 0.0;
-  for (int i = tid; i < V; i += SB) if (p[i] > v1) gt += (double)p[i];
-  gt = block_sum_f64(gt, ds);
-  double ties = 0.0;
-  for (int i = tid; i < V; i += SB) if (p[i] == v1) ties += 1.0;
-  ties = block_sum_f64(ties, ds);
-  // smallest k >= 1 with gt + k * v1 > tp
-  double k1 = v1 > 0.f ? floor(((double)tp - gt) / (double)v1) + 1.0 : ties;
-  if (!(k1 >= 1.0)) k1 = 1.0;
-  while (k1 > 1.0 && gt + (k1 - 1.0) * (double)v1 > (double)tp) k1 -= 1.0;
-  while (k1 < ties && !(gt + k1 * (double)v1 > (double)tp)) k1 += 1.0;
-  if (k1 > ties) k1 = ties;
-  const double mass = gt + k1 * (double)v1;
-
+  // nucleus: the threshold value, the mass above it, and how many of the equal ones are kept
+  const unsigned long long tq = (unsigned long long)((double)tp * QSCALE);
+  const Found f1 = radix_search(p, V, tq, h_mass, h_cnt, t_mass, t_cnt, res);
+  long k1 = 1;
+  if (f1.each > 0 && tq >= f1.above) k1 = (long)((tq - f1.above) / f1.each) + 1;   // smallest k with above + k*each > tq
+  if (k1 > f1.ties) k1 = f1.ties;
+  if (k1 < 1) k1 = 1;
+  const unsigned long long mass = f1.above + (unsigned long long)k1 * f1.each;
   // the drawn token: first in the kept order whose running sum exceeds u * mass
-  const double target = u * mass;
-  const float v2 = __uint_as_float(search_threshold(p, V, target, ds));
-  double gt2 = 0.0;
-  for (int i = tid; i < V; i += SB) if (p[i] > v2) gt2 += (double)p[i];
-  gt2 = block_sum_f64(gt2, ds);
-  double ties2 = 0.0;
-  for (int i = tid; i < V; i += SB) if (p[i] == v2) ties2 += 1.0;
-  ties2 = block_sum_f64(ties2, ds);
-  double j = v2 > 0.f ? floor((target - gt2) / (double)v2) : 0.0;
-  if (!(j >= 0.0)) j = 0.0;
-  while (j > 0.0 && target < gt2 + j * (double)v2) j -= 1.0;
-  while (j + 1.0 < ties2 && !(target < gt2 + (j + 1.0) * (double)v2)) j += 1.0;
-  double limit = ties2;
-  if (v2 == v1) limit = k1;
-  if (j > limit - 1.0) j = limit - 1.0;
+  const unsigned long long target = (unsigned long long)(u * (double)mass);
+  const Found f2 = radix_search(p, V, target, h_mass, h_cnt, t_mass, t_cnt, res);
+  long j = (f2.each > 0 && target >= f2.above) ? (long)((target - f2.above) / f2.each) : 0;
+  const long limit = (f2.bits == f1.bits) ? k1 : (long)f2.ties;
+  if (j > limit - 1) j = limit - 1;
+  if (j < 0) j = 0;
+  want_value = __uint_as_float(f2.bits);
+  want_index = j;
 
-  // the j-th (from 0) index in ascending order with p == v2
-  double cnt = 0.0;
-  for (int i = b; i < e; ++i) if (p[i] == v2) cnt += 1.0;
-  block_scan_f64(cnt, cdf, ds);
-  const double before = tid ? cdf[tid - 1] : 0.0;
-  if (before <= j && j < cdf[tid]) {
-    double c = before;
-    for (int i = b; i < e; ++i)
-      if (p[i] == v2) {
-        if (c == j) { winner = i; break; }
-        c += 1.0;
+  // the want_index-th index, in ascending order, whose probability is want_value
+  int mine = 0;
+  for (int i0 = lo + lane; i0 < hi; i0 += 8 * 64) {
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = (i0 + 64 * k < hi) ? p[i0 + 64 * k] : -1.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) mine += (v[k] == want_value) ? 1 : 0;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
+  if (lane == 0) w_tot[wave] = (unsigned long long)mine;
+  __syncthreads();
+  long before = 0;
+  for (int w = 0; w < wave; ++w) before += (long)w_tot[w];
+  if (before <= want_index && want_index < before + (long)w_tot[wave]) {
+    for (int base = lo; base < hi; base += 64) {
+      const int i = base + lane;
+      const unsigned long long hit = __ballot(i < hi && p[i] == want_value);
+      const int n = __popcll(hit);
+      if (want_index < before + n) {
+        if (lane == 0) {
+          unsigned long long h = hit;
+          for (long skip = want_index - before; skip > 0; --skip) h &= h - 1;   // drop the lowest set bits
+          winner = base + __ffsll((long long)h) - 1;
+        }
+        break;
       }
+      before += n;
+    }
   }
   __syncthreads();
   if (tid == 0) out[row] = winner >= 0 ? winner : V - 1;
