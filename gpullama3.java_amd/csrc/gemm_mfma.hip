@@ -2,14 +2,13 @@
 // products of a prefill step. 32-bit accumulation; W is row-major [out, in]
 // (J/core/model/tensor/FloatTensor.java:98-100).
 //
-// A block of four waves computes a 128 x 128 tile of C (128 x 64 for the gated epilogue,
-// whose W tile holds 64 gate rows and the 64 matching up rows; 64 x 128 when the matrix
-// would otherwise give fewer tiles than two per CU). K advances in steps of
-// 64: the next step's operands travel from memory to registers while the matrix cores
-// work on the current step out of shared memory. Each wave owns 64 x 64 (or 32 x 64) of
-// the tile as 2 x 2 (1 x 2) tiles of the 32x32x16 instruction. Rows in shared memory are
-// padded by 16 bytes so that the 32 lanes that read one column of 16-byte operands hit
-// different banks.
+// A block is WM x WN waves; each wave owns 64 x 64 (or 32 x 64) of the block's tile of C as
+// 2 x 2 (1 x 2) tiles of the 32x32x16 instruction: sixteen waves on 256 x 256 for large products,
+// eight waves on 128 x 128 otherwise. For the gated epilogue a W tile holds the gate rows of
+// half as many output columns and the matching up rows. K advances in steps of 64: the next
+// step's operands travel from memory to registers while the matrix cores work on the current
+// step out of shared memory. Rows in shared memory are padded by 16 bytes so that the 32 lanes
+// that read one column of 16-byte operands hit different banks.
 // Blocks are numbered so that each XCD (whose second-level cache is its own) works on a
 // contiguous range of tiles, neighbouring tiles sharing their panel of W.
 //
@@ -21,22 +20,26 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 enum { MF_STORE = 0, MF_ADD = 1, MF_GATED = 2 };
 
-#define MF_BM 128
-#define MF_BN 128
 #define MF_BK 64
 #define MF_LD (MF_BK + 8)   // padded row, in elements
 
-template <int EPI, typename TC, int TM>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
-                                                        TC* __restrict__ C, int M, int N, int K, long lda, long ldw,
-                                                        long ldc, int tiles_m, int tiles_n) {
-  constexpr int NCOLS = (EPI == MF_GATED) ? 64 : 128;   // output columns of a block
-  constexpr int BM = 64 * TM;                            // rows of a block
-  constexpr int NA = BM / 32;                            // 16-byte chunks of A per thread and k-step
+// WM x WN waves; a wave owns (32*TM) x 64 of the tile.
+template <int EPI, typename TC, int TM, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* __restrict__ A,
+                                                                  const bf16_t* __restrict__ W, TC* __restrict__ C,
+                                                                  int M, int N, int K, long lda, long ldw, long ldc,
+                                                                  int tiles_m, int tiles_n) {
+  constexpr int NT = 64 * WM * WN;                       // threads
+  constexpr int BM = 32 * TM * WM;                       // rows of a block
+  constexpr int BN = 64 * WN;                            // rows of W of a block
+  constexpr int NCOLS = (EPI == MF_GATED) ? BN / 2 : BN; // output columns of a block
+  constexpr int NA = BM * 8 / NT;                        // 16-byte chunks of A per thread and k-step
+  constexpr int NWC = BN * 8 / NT;                       // and of W
+  static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile does not divide over the threads");
   __shared__ __attribute__((aligned(16))) bf16_t As[BM][MF_LD];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[MF_BN][MF_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[BN][MF_LD];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   const int lr = lane & 31, lh = lane >> 5;
 
   // block -> tile: 8 XCDs take turns on consecutive block ids; give each a contiguous range
@@ -47,29 +50,35 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   const int m0 = (tile % tiles_m) * BM;
   const int n0 = (tile / tiles_m) * NCOLS;
 
-  // global -> register staging: chunks of 16 bytes, NA of A and 4 of W per thread
+  // global -> register staging in chunks of 16 bytes
   const bf16_t* ap[NA];
-  const bf16_t* wp[4];
-  int srow[4], scol[4];
+  const bf16_t* wp[NWC];
+  int arow_s[NA], wrow_s[NWC];
+  const int scol = (tid & 7) * 8;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int c = tid + 256 * i;
-    srow[i] = c >> 3;
-    scol[i] = (c & 7) * 8;
-    if (i < NA) ap[i] = A + (long)min(m0 + srow[i], M - 1) * lda + scol[i];
+  for (int i = 0; i < NA; ++i) {
+    arow_s[i] = (tid + NT * i) >> 3;
+    ap[i] = A + (long)min(m0 + arow_s[i], M - 1) * lda + scol;
+  }
+#pragma unroll
+  for (int i = 0; i < NWC; ++i) {
+    const int r = (tid + NT * i) >> 3;
+    wrow_s[i] = r;
     int wr;
-    if (EPI == MF_GATED) wr = srow[i] < 64 ? min(n0 + srow[i], N - 1) : N + min(n0 + srow[i] - 64, N - 1);
-    else wr = min(n0 + srow[i], N - 1);
-    wp[i] = W + (long)wr * ldw + scol[i];
+    if (EPI == MF_GATED) wr = r < BN / 2 ? min(n0 + r, N - 1) : N + min(n0 + r - BN / 2, N - 1);
+    else wr = min(n0 + r, N - 1);
+    wp[i] = W + (long)wr * ldw + scol;
   }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  bf16x8 ra[NA], rw[4];
+  bf16x8 ra[NA], rw[NWC];
+  auto fetch = [&](int k0) {
+    const bool ok = k0 + scol < K;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const bool ok = scol[i] < K;
-    if (i < NA) ra[i] = ok ? *(const bf16x8*)ap[i] : zero;
-    rw[i] = ok ? *(const bf16x8*)wp[i] : zero;
-  }
+    for (int i = 0; i < NA; ++i) ra[i] = ok ? *(const bf16x8*)(ap[i] + k0) : zero;
+#pragma unroll
+    for (int i = 0; i < NWC; ++i) rw[i] = ok ? *(const bf16x8*)(wp[i] + k0) : zero;
+  };
+  fetch(0);
 
   f32x16 acc[TM][2];
 #pragma unroll
@@ -81,24 +90,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
 
   const int arow = wm * 32 * TM + lr;
   const int wrow0 = (EPI == MF_GATED) ? wn * 32 + lr : wn * 64 + lr;
-  const int wrow1 = (EPI == MF_GATED) ? 64 + wn * 32 + lr : wn * 64 + 32 + lr;
+  const int wrow1 = (EPI == MF_GATED) ? BN / 2 + wn * 32 + lr : wn * 64 + 32 + lr;
 
   for (int k0 = 0; k0 < K; k0 += MF_BK) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (i < NA) *(bf16x8*)&As[srow[i]][scol[i]] = ra[i];
-      *(bf16x8*)&Ws[srow[i]][scol[i]] = rw[i];
-    }
-    __syncthreads();
-    const int kn = k0 + MF_BK;
-    if (kn < K) {
+    for (int i = 0; i < NA; ++i) *(bf16x8*)&As[arow_s[i]][scol] = ra[i];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const bool ok = kn + scol[i] < K;
-        if (i < NA) ra[i] = ok ? *(const bf16x8*)(ap[i] + kn) : zero;
-        rw[i] = ok ? *(const bf16x8*)(wp[i] + kn) : zero;
-      }
-    }
+    for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[wrow_s[i]][scol] = rw[i];
+    __syncthreads();
+    if (k0 + MF_BK < K) fetch(k0 + MF_BK);
 #pragma unroll
     for (int kk = 0; kk < MF_BK / 16; ++kk) {
       const int kc = kk * 16 + lh * 8;
@@ -142,27 +142,32 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   }
 }
 
-template <int EPI, typename TC>
-static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                       hipStream_t stream) {
-  const int ncols = (EPI == MF_GATED) ? 64 : 128;
+template <int EPI, typename TC, int TM, int WM, int WN>
+static int launch_shape(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
+                        hipStream_t stream) {
+  const int bm = 32 * TM * WM;
+  const int ncols = (EPI == MF_GATED) ? 32 * WN : 64 * WN;
   const int tiles_n = (N + ncols - 1) / ncols;
-  // blocks of 128 rows unless that leaves fewer than two blocks per CU: then 64 rows, so that one
-  // block's loads overlap another's products
-  const bool tall = (long)((M + 127) / 128) * tiles_n >= 512;
-  const int bm = tall ? 128 : 64;
   const int tiles_m = (M + bm - 1) / bm;
   const long n_tiles = (long)tiles_m * tiles_n;
   const long blocks = ((n_tiles + 7) / 8) * 8;
   GL3_REQUIRE(blocks < (1L << 31), "gl3_gemm_mfma: too many tiles");
-  if (tall)
-    gemm_mfma_kernel<EPI, TC, 2><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
-        (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
-  else
-    gemm_mfma_kernel<EPI, TC, 1><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
-        (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
+  gemm_mfma_kernel<EPI, TC, TM, WM, WN><<<dim3((unsigned)blocks), dim3(64 * WM * WN), 0, stream>>>(
+      (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
   GL3_LAUNCH_CHECK();
   return 0;
+}
+
+template <int EPI, typename TC>
+static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
+                       hipStream_t stream) {
+  // 256 x 256 tiles of sixteen waves where they still give two blocks per CU: half the operand
+  // traffic per product, and that traffic is what bounds the large products. Otherwise 128 x 128
+  // tiles of eight waves, of which several fit a CU and overlap each other's waits.
+  const long big_n = (EPI == MF_GATED) ? (N + 127) / 128 : (N + 255) / 256;
+  if ((long)((M + 255) / 256) * big_n >= 512)
+    return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, stream);
+  return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, stream);
 }
 
 // N counts output columns: for the gated epilogue W has 2N rows (gate, then up).

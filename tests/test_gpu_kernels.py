@@ -413,7 +413,9 @@ def test_attention_decode_far_key_and_window_edge(splits):
 
 
 # ------------------------------------------------------------------ bfloat16 product for many rows (matrix cores)
-@pytest.mark.parametrize("M, N, Kd", [(65, 130, 64), (128, 128, 64), (200, 257, 136), (300, 64, 2048), (1000, 1000, 112)])
+# the last case is large enough for the 256 x 256 tiles, with edges in both directions
+@pytest.mark.parametrize("M, N, Kd", [(65, 130, 64), (128, 128, 64), (200, 257, 136), (300, 64, 2048), (1000, 1000, 112),
+                                      (4100, 8200, 72)])
 def test_gemm_mfma(M, N, Kd):
     rng = np.random.default_rng(M + N + Kd)
     a = rounded(rng.standard_normal((M, Kd)), "bfloat16")
