@@ -79,6 +79,63 @@ extern "C" int gl3_rmsnorm(const float* x, const int* rows, const void* w, int w
   return 0;
 }
 
+// ----------------------------------------------------------------- slices of a product + rmsnorm
+// A product whose K was cut into slices left its sums as P[slice][row][ldp] (float). Here they
+// are added to the residual rows in slice order, x[row] += P[0][row] + P[1][row] + ..., and the
+// rows' RMSNorm is written to `out` (null: the sums alone). With `rows` the listed rows are
+// normalised and x is left as it was (a row may be listed twice). One block per row.
+template <typename TW, typename TO>
+__global__ void add_slices_rmsnorm_kernel(float* __restrict__ x, const int* __restrict__ rows,
+                                          const float* __restrict__ P, int n_slices, long slice_stride, long ldp,
+                                          const TW* __restrict__ w, TO* __restrict__ out, int d, float eps) {
+  __shared__ float scratch[16];
+  const long r = blockIdx.x;
+  const long src = rows ? rows[r] : r;
+  float* xr = x + src * d;
+  const float* pr = P + src * ldp;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float v = xr[i];
+    for (int s = 0; s < n_slices; ++s) v += pr[s * slice_stride + i];
+    if (!rows) xr[i] = v;
+    ss += v * v;
+  }
+  if (!out) return;
+  ss = block_sum(ss, scratch);
+  ss = ss / (float)d;
+  ss = ss + eps;
+  ss = 1.0f / sqrtf(ss);
+  TO* o = out + r * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float v = xr[i];   // this thread's own store when the sums were written back
+    if (rows)
+      for (int s = 0; s < n_slices; ++s) v += pr[s * slice_stride + i];
+    o[i] = from_f32<TO>(to_f32<TW>(w[i]) * (ss * v));
+  }
+}
+
+extern "C" int gl3_add_slices_rmsnorm(float* x, const int* rows, const float* P, int n_slices, long slice_stride,
+                                      long ldp, const void* w, int w_dtype, void* out, int out_dtype, int n_rows,
+                                      int d, float eps, hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  GL3_REQUIRE(x && P && n_rows > 0 && d > 0 && n_slices > 0 && ldp >= d,
+              "gl3_add_slices_rmsnorm: bad arguments (rows=%d d=%d slices=%d)", n_rows, d, n_slices);
+  GL3_REQUIRE((w != nullptr) == (out != nullptr), "gl3_add_slices_rmsnorm: weight and output come together");
+  dim3 grid(n_rows), block(256);
+#define GO(TW, TO)                                                                                              \
+  add_slices_rmsnorm_kernel<TW, TO><<<grid, block, 0, stream>>>(x, rows, P, n_slices, slice_stride, ldp,       \
+                                                                 (const TW*)w, (TO*)out, d, eps)
+  if (!out) GO(float, float);
+  else if (w_dtype == GL3_F32 && out_dtype == GL3_F32) GO(float, float);
+  else if (w_dtype == GL3_F32 && out_dtype == GL3_BF16) GO(float, bf16_t);
+  else if (w_dtype == GL3_BF16 && out_dtype == GL3_F32) GO(bf16_t, float);
+  else if (w_dtype == GL3_BF16 && out_dtype == GL3_BF16) GO(bf16_t, bf16_t);
+  else GL3_REQUIRE(false, "gl3_add_slices_rmsnorm: unknown dtypes %d %d", w_dtype, out_dtype);
+#undef GO
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
 // ----------------------------------------------------------------- rotary + cache write
 // qkv[t] holds [n_heads q heads | n_kv k heads | n_kv v heads], each of head_dim.
 // Queries are rotated in place; keys are rotated and written to the paged key

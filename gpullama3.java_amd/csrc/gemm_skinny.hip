@@ -438,6 +438,87 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
   }
 }
 
+// The wide kernel, for steps of three or four token tiles: there a strip's share of A is as
+// large as the strip of W itself, and reading it again for every strip is what takes the time.
+// A block works on NS strips at once (NS pairs of gate and up strips for the gated epilogue), so
+// that A is read once for all of them, and on one slice of K only (blockIdx.y), so that the
+// chip still has blocks enough. With more than one slice the epilogue is a plain store of the
+// slice's sums into slice `blockIdx.y` of a float buffer [slices][M][ldc]: whoever reads the
+// result next adds the slices up in order, no block waits for another.
+template <int MT, int NS, int NW, int EPI, typename TC>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t* __restrict__ A,
+                                                                   const bf16_t* __restrict__ W, TC* __restrict__ C,
+                                                                   int M, int N, int K, long lda, long ldw, long ldc,
+                                                                   long slice_stride, int steps_per_slice, SkRope rp) {
+  constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
+  constexpr int UNROLL = 4;
+  __shared__ f32x4 red[NW][NG * MT][64];
+  __shared__ float sm_ssq[1][64];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const int n_strips = (N + 15) / 16;
+  const int strip0 = blockIdx.x * NS;
+  int hd[NS], sub[NS];
+  bool rotated[NS];
+  const bf16_t* wrow[NS];
+#pragma unroll
+  for (int g = 0; g < NS; ++g) {
+    const int wr = sk_strip_row<EPI>(min(strip0 + g, n_strips - 1), r, N, rp, hd[g], sub[g], rotated[g]);
+    wrow[g] = W + (long)wr * ldw + q * 8;
+  }
+  const bf16_t* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = A + (long)min(mt * 16 + r, M - 1) * lda + q * 8;
+
+  const int steps = (K + 31) / 32;
+  const int s_begin = blockIdx.y * steps_per_slice;
+  const int s_end = min(steps, s_begin + steps_per_slice);
+  f32x4 acc[NS][NG][MT];
+#pragma unroll
+  for (int g = 0; g < NS; ++g)
+#pragma unroll
+    for (int h = 0; h < NG; ++h)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[g][h][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  for (int s0 = s_begin + wave; s0 < s_end; s0 += NW * UNROLL) {
+    bf16x8 wf[UNROLL][NS], uf[UNROLL][NS], xf[UNROLL][MT];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int st = s0 + NW * u;
+      const int k = st * 32;
+      const bool ok = st < s_end && k + q * 8 < K;
+#pragma unroll
+      for (int g = 0; g < NS; ++g) {
+        wf[u][g] = ok ? *(const bf16x8*)(wrow[g] + k) : zero;
+        if (EPI == SK_GATED) uf[u][g] = ok ? *(const bf16x8*)(wrow[g] + (long)N * ldw + k) : zero;
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) xf[u][mt] = ok ? *(const bf16x8*)(xrow[mt] + k) : zero;
+    }
+    __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int g = 0; g < NS; ++g)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          acc[g][0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][g], xf[u][mt], acc[g][0][mt], 0, 0, 0);
+          if (EPI == SK_GATED)
+            acc[g][1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u][g], xf[u][mt], acc[g][1][mt], 0, 0, 0);
+        }
+  }
+  TC* out = C + (long)blockIdx.y * slice_stride;
+#pragma unroll
+  for (int g = 0; g < NS; ++g) {
+    if (g) __syncthreads();   // the partial tiles in shared memory are free again
+    if (strip0 + g < n_strips)   // the same for all threads of the block
+      sk_finish<MT, NW, EPI, TC, false, false>(red, sm_ssq, acc[g], strip0 + g, hd[g], sub[g], rotated[g], out, M, N, K,
+                                                ldc, SkNorm{}, nullptr, rp);
+  }
+}
+
 struct SkCall {
   const void* A; const void* W; void* C;
   int M, N, K; long lda, ldw, ldc;
@@ -556,6 +637,69 @@ extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtyp
   return 0;
 }
 
+template <int MT, int NS, int EPI, typename TC>
+static int launch_wide(const SkCall& a, int slices, long slice_stride) {
+  constexpr int NW = 8;
+  const int n_strips = (a.N + 15) / 16;
+  const int steps = (a.K + 31) / 32;
+  const int per_slice = (steps + slices - 1) / slices;
+  gemm_skinny_wide_kernel<MT, NS, NW, EPI, TC>
+      <<<dim3((n_strips + NS - 1) / NS, slices), dim3(NW * 64), 0, a.stream>>>(
+          (const bf16_t*)a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, slice_stride, per_slice,
+          a.rp);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int EPI, typename TC>
+static int pick_wide(const SkCall& a, int strips_per_block, int slices, long slice_stride) {
+  constexpr int BIG = (EPI == SK_GATED) ? 2 : 4;   // a gated strip is a pair of strips
+  const bool big = strips_per_block == BIG;
+  if ((a.M + 15) / 16 <= 3)
+    return big ? launch_wide<3, BIG, EPI, TC>(a, slices, slice_stride)
+               : launch_wide<3, BIG / 2, EPI, TC>(a, slices, slice_stride);
+  return big ? launch_wide<4, BIG, EPI, TC>(a, slices, slice_stride)
+             : launch_wide<4, BIG / 2, EPI, TC>(a, slices, slice_stride);
+}
+
+// How many strips a block of the wide kernel takes: as many as leave the chip enough blocks.
+static int wide_strips(int N, int slices, int epilogue) {
+  const int big = epilogue == SK_GATED ? 2 : 4;
+  const long n_strips = (N + 15) / 16;
+  return (n_strips / big) * slices >= 192 ? big : big / 2;
+}
+
+// The product for 33 to 64 rows of A (bfloat16). `slices` > 1 (store epilogue, float output only):
+// K is cut into that many slices and C is [slices][M][ldc] with `slice_stride` elements between
+// slices; the caller adds them up. `strips_per_block`: 0 lets the library choose.
+extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
+                                    long ldw, long ldc, int epilogue, int slices, long slice_stride,
+                                    int strips_per_block, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  if (check_common("gl3_gemm_skinny_wide", A, W, C, M, N, K, lda, ldw, 0)) return -1;
+  GL3_REQUIRE(M > 32, "gl3_gemm_skinny_wide: M=%d; up to 32 rows are gl3_gemm_skinny's", M);
+  GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny_wide: ldc too small");
+  GL3_REQUIRE(epilogue >= 0 && epilogue <= 2, "gl3_gemm_skinny_wide: unknown epilogue %d", epilogue);
+  GL3_REQUIRE(slices >= 1 && slices <= (K + 31) / 32, "gl3_gemm_skinny_wide: %d slices of K=%d", slices, K);
+  GL3_REQUIRE(slices == 1 || (epilogue == SK_STORE && c_dtype == GL3_F32 && slice_stride >= (long)(M - 1) * ldc + N),
+              "gl3_gemm_skinny_wide: slices need the store epilogue, a float output and room for M rows a slice");
+  GL3_REQUIRE(epilogue != SK_ADD || c_dtype == GL3_F32, "gl3_gemm_skinny_wide: the add epilogue needs a float output");
+  const int big = epilogue == SK_GATED ? 2 : 4;
+  if (strips_per_block == 0) strips_per_block = wide_strips(N, slices, epilogue);
+  GL3_REQUIRE(strips_per_block == big || strips_per_block == big / 2, "gl3_gemm_skinny_wide: %d strips per block",
+              strips_per_block);
+  const SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, nullptr, SkRope{}, stream, false};
+  if (c_dtype == GL3_F32) {
+    if (epilogue == SK_STORE) return pick_wide<SK_STORE, float>(a, strips_per_block, slices, slice_stride);
+    if (epilogue == SK_ADD) return pick_wide<SK_ADD, float>(a, strips_per_block, slices, slice_stride);
+  } else if (c_dtype == GL3_BF16) {
+    if (epilogue == SK_STORE) return pick_wide<SK_STORE, bf16_t>(a, strips_per_block, slices, slice_stride);
+    if (epilogue == SK_GATED) return pick_wide<SK_GATED, bf16_t>(a, strips_per_block, slices, slice_stride);
+  }
+  GL3_REQUIRE(false, "gl3_gemm_skinny_wide: output dtype %d with epilogue %d is not built", c_dtype, epilogue);
+  return 0;
+}
+
 // The product of RMSNorm(x) with W: x float [rows, K] (lda), norm weight [K], ssq [n_partials][64]
 // partial sums of squares of the rows of x (indexed by the row of x, so x has at most 64 rows).
 // Epilogues: store (float or bfloat16) and gated (bfloat16).
@@ -583,7 +727,9 @@ extern "C" int gl3_gemm_skinny_norm(const float* x, const int* rows, const void*
 // RMSNorm(x) . Wqkv^T, rotation of q and k, q to `q_out` [M, n_heads*head_dim] (ldq), k and v into
 // the paged cache (keys [page][kv head][position][head_dim], values transposed). One token per row;
 // cos/sin null: no rotation. head_dim a multiple of 16; the rotation covers the whole head.
-extern "C" int gl3_qkv_rope_cache(const float* x, const void* norm_weight, int norm_weight_dtype, const float* ssq,
+// With norm_weight null x is bfloat16 and already normalised: the product, rotation and cache
+// write alone.
+extern "C" int gl3_qkv_rope_cache(const void* x, const void* norm_weight, int norm_weight_dtype, const float* ssq,
                                   int n_partials, float eps, const void* Wqkv, void* q_out, long ldq, int M, int K,
                                   long lda, long ldw, const int* positions, const int* seq_of_token,
                                   const int* block_table, int table_stride, const float* cos_tab,
@@ -592,9 +738,11 @@ extern "C" int gl3_qkv_rope_cache(const float* x, const void* norm_weight, int n
   if (M == 0) return 0;
   const int N = (n_heads + 2 * n_kv) * head_dim;
   if (check_common("gl3_qkv_rope_cache", x, Wqkv, q_out, M, N, K, lda, ldw, waves)) return -1;
-  GL3_REQUIRE(norm_weight && ssq && n_partials > 0 && (uintptr_t)norm_weight % 16 == 0,
-              "gl3_qkv_rope_cache: norm arguments missing or misaligned");
-  GL3_REQUIRE(norm_weight_dtype == GL3_F32, "gl3_qkv_rope_cache: the norm weight must be float");
+  if (norm_weight) {
+    GL3_REQUIRE(ssq && n_partials > 0 && (uintptr_t)norm_weight % 16 == 0,
+                "gl3_qkv_rope_cache: norm arguments missing or misaligned");
+    GL3_REQUIRE(norm_weight_dtype == GL3_F32, "gl3_qkv_rope_cache: the norm weight must be float");
+  }
   GL3_REQUIRE(head_dim % 16 == 0 && n_heads > 0 && n_kv > 0, "gl3_qkv_rope_cache: head_dim %d must be a multiple of 16",
               head_dim);
   GL3_REQUIRE(positions && seq_of_token && block_table && k_cache && v_cache && page_size > 0 && table_stride > 0,
@@ -606,5 +754,6 @@ extern "C" int gl3_qkv_rope_cache(const float* x, const void* norm_weight, int n
   const SkRope rp = {positions, seq_of_token, block_table, table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
                      (bf16_t*)v_cache, n_heads, n_kv, head_dim, adjacent, page_size};
   const SkCall a = {x, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
+  if (!norm_weight) return pick_mt<SK_QKV, bf16_t, false, false>(pick_waves(waves, N, K), a);
   return pick_mt<SK_QKV, bf16_t, true, false>(pick_waves(waves, N, K), a);
 }

@@ -49,6 +49,7 @@ def _declare(lib):
         "gl3_fill_u32": [P, c_uint32, L, P],
         "gl3_embed": [P, I, P, P, I, I, P, P],
         "gl3_rmsnorm": [P, P, P, I, P, I, I, I, F, P],
+        "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P],
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
@@ -56,6 +57,7 @@ def _declare(lib):
         "gl3_argmax": [P, L, P, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
         "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, P],
+        "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P],
         "gl3_qkv_rope_cache": [P, P, I, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, P],
@@ -153,6 +155,33 @@ def rmsnorm(x, weight, out, eps, rows=None):
         raise KernelError(f"rmsnorm: {x.shape[0]} inputs for {n} outputs")
     _check(library().gl3_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _code(weight, "weight"), _ptr(out),
                                  _code(out, "out"), n, d, float(eps), _stream()), "rmsnorm")
+
+
+def add_slices_rmsnorm(x, slices, weight=None, out=None, eps=0.0, rows=None):
+    """x += slices[0] + slices[1] + ... (in that order; ``slices`` [S, rows of x, d] float32), and
+    out[r] = weight * x[r] / rms when ``out`` is given. With ``rows`` the listed rows are normalised
+    and x keeps its values."""
+    _dev(x, "x", torch.float32); _dev(slices, "slices", torch.float32, contiguous=False)
+    d = x.shape[-1]
+    if (x.dim() != 2 or slices.dim() != 3 or slices.shape[1:] != x.shape or slices.stride(2) != 1
+            or (weight is None) != (out is None)):
+        raise KernelError(f"add_slices_rmsnorm: x {tuple(x.shape)}, slices {tuple(slices.shape)}")
+    n = x.shape[0]
+    if out is not None:
+        _dev(weight, "weight"); _dev(out, "out")
+        n = out.shape[0]
+        if out.dim() != 2 or out.shape[1] != d or weight.shape != (d,):
+            raise KernelError(f"add_slices_rmsnorm: weight {tuple(weight.shape)}, out {tuple(out.shape)} for d={d}")
+    if rows is not None:
+        _dev(rows, "rows", torch.int32)
+        if out is None or rows.numel() != n:
+            raise KernelError("add_slices_rmsnorm: rows select the rows that are normalised, one per output row")
+    elif x.shape[0] != n:
+        raise KernelError(f"add_slices_rmsnorm: {x.shape[0]} inputs for {n} outputs")
+    _check(library().gl3_add_slices_rmsnorm(
+        _ptr(x), _ptr(rows), _ptr(slices), slices.shape[0], slices.stride(0), slices.stride(1), _ptr(weight),
+        _code(weight, "weight") if weight is not None else 0, _ptr(out), _code(out, "out") if out is not None else 0,
+        n, d, float(eps), _stream()), "add_slices_rmsnorm")
 
 
 def rope_cache_write(qkv, positions, seq_of_token, block_table, cos, sin, k_cache, v_cache, n_heads, n_kv,
@@ -288,6 +317,34 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None):
                                      out.stride(0), epilogue, waves, _ptr(ssq_out), _stream()), "gemm_skinny")
 
 
+def gemm_skinny_wide_fits(a, w, out, epilogue):
+    return 32 < a.shape[0] <= 64 and gemm_skinny_fits(a, w, out, epilogue)
+
+
+def wide_slices(N, K):
+    """Into how many slices of K the wide kernel's product [*, K] x [N, K] is cut: enough blocks for
+    the chip (a block takes 64 columns), at least two k-steps of 32 for each of a block's 8 waves."""
+    return max(1, min(8, 256 // -(-N // 64), K // 512))
+
+
+def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0):
+    """out (=, +=, gated) a @ w.T for 33 to 64 rows of ``a``. ``out`` with three axes [slices, M, N]
+    (float32, store epilogue) takes the sums of one slice of K each: the caller adds them up."""
+    _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
+    M, K = a.shape
+    slices, slice_stride = 1, 0
+    rows = out
+    if out.dim() == 3:
+        slices, slice_stride, rows = out.shape[0], out.stride(0), out[0]
+    N = rows.shape[1]
+    wrows = 2 * N if epilogue == EPI_GATED else N
+    if (w.shape != (wrows, K) or rows.shape[0] != M or rows.stride(1) != 1 or a.stride(1) != 1 or not 32 < M <= 64):
+        raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
+    _check(library().gl3_gemm_skinny_wide(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0),
+                                          w.stride(0), rows.stride(0), epilogue, slices, slice_stride, strips,
+                                          _stream()), "gemm_skinny_wide")
+
+
 def _check_norm_args(x, norm_weight, ssq, n_partials, K):
     _dev(x, "x", torch.float32, contiguous=False); _dev(norm_weight, "norm_weight"); _dev(ssq, "ssq", torch.float32)
     if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] != K or norm_weight.shape != (K,):
@@ -324,18 +381,26 @@ def gemm_skinny_norm(x, norm_weight, ssq, n_partials, eps, w, out, epilogue=EPI_
 
 
 def qkv_rope_cache_fits(x, w_qkv, head_dim, rot_dim):
+    """x: the float residual rows (with the norm's arguments) or normalised bfloat16 rows (without)."""
     K = x.shape[1]
-    return (x.shape[0] <= 64 and K % 8 == 0 and x.stride(0) % 8 == 0 and w_qkv.stride(0) % 8 == 0
+    return (x.shape[0] <= 64 and x.stride(1) == 1 and K % 8 == 0 and x.stride(0) % 8 == 0 and w_qkv.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w_qkv.data_ptr() % 16 == 0 and w_qkv.dtype == torch.bfloat16
             and head_dim % 16 == 0 and rot_dim in (0, head_dim))
 
 
 def qkv_rope_cache(x, norm_weight, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_token, block_table, cos, sin,
                    k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page_size, waves=0):
-    """RMSNorm(x) @ w_qkv.T, rotation, q into ``q_out`` [T, H*hs] bfloat16, k and v into the cache."""
+    """RMSNorm(x) @ w_qkv.T, rotation, q into ``q_out`` [T, H*hs] bfloat16, k and v into the cache.
+    ``norm_weight`` None: x is bfloat16, normalised already."""
     _dev(w_qkv, "w_qkv", torch.bfloat16); _dev(q_out, "q_out", torch.bfloat16, contiguous=False)
     K = w_qkv.shape[1]
-    _check_norm_args(x, norm_weight, ssq, n_partials, K)
+    if norm_weight is None:
+        _dev(x, "x", torch.bfloat16, contiguous=False)
+        if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] != K or x.shape[0] > 64:
+            raise KernelError(f"qkv_rope_cache: x {tuple(x.shape)} for K={K}")
+        ssq, n_partials = None, 0
+    else:
+        _check_norm_args(x, norm_weight, ssq, n_partials, K)
     T = x.shape[0]
     _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
     _dev(block_table, "block_table", torch.int32)
@@ -350,8 +415,8 @@ def qkv_rope_cache(x, norm_weight, ssq, n_partials, eps, w_qkv, q_out, positions
         if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != head_dim // 2:
             raise KernelError(f"qkv_rope_cache: table {tuple(cos.shape)} for head_dim {head_dim}")
     _check(library().gl3_qkv_rope_cache(
-        _ptr(x), _ptr(norm_weight), _code(norm_weight, "norm_weight"), _ptr(ssq), n_partials, float(eps), _ptr(w_qkv),
-        _ptr(q_out), q_out.stride(0), T, K, x.stride(0), w_qkv.stride(0), _ptr(positions), _ptr(seq_of_token),
+        _ptr(x), _ptr(norm_weight), _code(norm_weight, "norm_weight") if norm_weight is not None else 0, _ptr(ssq),
+        n_partials, float(eps), _ptr(w_qkv), _ptr(q_out), q_out.stride(0), T, K, x.stride(0), w_qkv.stride(0), _ptr(positions), _ptr(seq_of_token),
         _ptr(block_table), block_table.shape[1], _ptr(cos), _ptr(sin), _ptr(k_cache), _ptr(v_cache), n_heads, n_kv,
         head_dim, int(adjacent), page_size, waves, _stream()), "qkv_rope_cache")
 

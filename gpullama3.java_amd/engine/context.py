@@ -49,6 +49,7 @@ class StepContext:
         self.max_q_len, self.max_kv_len = max_q_len, max_kv_len
         self.fuse = getattr(engine, "fuse", False)   # few-token steps fold norms and rotation into the products
         self.ssq = None                    # (address of the residual stream, its partial sums of squares, how many)
+        self.pending = None                # (address of the residual stream, slices of a product still to be added to it)
         self.kv_len_hint = max_kv_len      # what launch shapes are sized for; a replayed graph keeps its own
         self.token_ids = self.positions = self.seq_of_token = self.cu_seqlens = self.kv_before = None
         self.slot_ids = None

@@ -36,6 +36,13 @@ class RMSNorm:
             return Normed(ctx, x, self.weight, self.weight_f32, self.eps, self.dtype, ssq[1], ssq[2], rows, name)
         n = x.shape[0] if rows is None else rows.numel()
         out = ctx.buffer(name, (n, self.dim), self.dtype)
+        pending = getattr(ctx, "pending", None)
+        if pending is not None and pending[0] == x.data_ptr():
+            # the product that last added to x left its sums in slices: add them up and normalise at once
+            K.add_slices_rmsnorm(x, pending[1], self.weight, out, self.eps, rows)
+            if rows is None:
+                ctx.pending = None
+            return out
         K.rmsnorm(x, self.weight, out, self.eps, rows)
         return out
 

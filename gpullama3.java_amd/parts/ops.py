@@ -40,6 +40,16 @@ class Normed:
         return out
 
 
+def settle_residual(ctx, x):
+    """A product of 33 to 64 rows into the residual stream may have left its sums as slices that the
+    next norm adds up. Whoever else wants to READ the rows (adding to them is always fine) calls
+    this first."""
+    pending = getattr(ctx, "pending", None)
+    if pending is not None and pending[0] == x.data_ptr():
+        K.add_slices_rmsnorm(x, pending[1])
+        ctx.pending = None
+
+
 def residual_written(ctx, x, ssq=None, n_partials=0):
     """Every writer of the residual stream says so: the partial sums of squares that a folded
     norm would use are those of the last writer, or none."""
@@ -56,6 +66,8 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
             return K.gemm_skinny_norm(a.x, a.weight_f32, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows)
         a = a.materialize()
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        if "wide" not in disabled and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx):
+            return
         if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
             N = out.shape[1]
             if (epilogue == EPI_ADD and ctx is not None and getattr(ctx, "fuse", False) and N % 16 == 0
@@ -77,6 +89,33 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
         residual_written(ctx, out)
 
 
+def _linear_wide(a, w, out, epilogue, ctx):
+    """Products of 33 to 64 rows where another kernel than the skinny one is faster. True when done."""
+    M, Kd = a.shape
+    N = out.shape[1]
+    if epilogue == EPI_GATED:
+        if N < 32 * 192:          # too few blocks of two strip pairs for the chip
+            return False
+        K.gemm_skinny_wide(a, w, out, epilogue)
+        return True
+    if epilogue == EPI_STORE:
+        # many columns (the head): the tiled kernel, whose blocks share their rows of a
+        if N >= 128 * 512 and "mfma" not in disabled and K.gemm_mfma_fits(a, w, out, epilogue):
+            K.gemm_mfma(a, w, out, epilogue)
+            return True
+        return False
+    # into the residual stream: K in slices, added up by the norm that follows
+    slices = K.wide_slices(N, Kd)
+    if slices < 2 or ctx is None or not getattr(ctx, "fuse", False) or "fused" in disabled:
+        return False
+    settle_residual(ctx, out)
+    part = ctx.buffer(f"slices{slices}", (slices, M, N), torch.float32)
+    K.gemm_skinny_wide(a, w, part, EPI_STORE)
+    residual_written(ctx, out)
+    ctx.pending = (out.data_ptr(), part)
+    return True
+
+
 def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_heads, n_kv, head_dim, dtype, writes_kv):
     """Queries, keys and values of the step's tokens: q rotated into a buffer whose rows start
     with the H*hs query columns (returned), k rotated and v into the cache. One kernel when
@@ -94,6 +133,12 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
         return q
     if isinstance(h, Normed):
         h = h.materialize()
+    if (writes_kv and h.dtype == torch.bfloat16 and "fused" not in disabled and "skinny" not in disabled
+            and K.qkv_rope_cache_fits(h, w_qkv, head_dim, rot)):
+        q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
+        K.qkv_rope_cache(h, None, None, 0, 0.0, w_qkv, q, ctx.positions, ctx.seq_of_token, block_table, cos, sin,
+                         k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page)
+        return q
     if writes_kv:
         qkv = ctx.buffer("qkv", (T, (n_heads + 2 * n_kv) * head_dim), dtype)
         linear(h, w_qkv, qkv)

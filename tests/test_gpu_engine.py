@@ -141,6 +141,26 @@ def test_batch_mates_order_and_slot_change_nothing(dtype):
     close(mixed, plain_logits(name, a), dtype)
 
 
+@pytest.mark.parametrize("name, dtype", [("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+@pytest.mark.parametrize("graphs", [False, True])
+def test_decode_steps_of_33_to_64_sequences(name, dtype, graphs):
+    """Between 33 and 64 tokens a step the products into the residual stream leave their sums in
+    slices of K that the next norm adds up, and rotation and cache write ride on the QKV product."""
+    B = 41
+    eng = engine(name, dtype, n_slots=64, max_tokens=64 * 64, use_graphs=graphs)
+    seqs = [rand_tokens(name, 200 + i, 2 + i % 5 + 6) for i in range(B)]
+    slots = [eng.take_slot() for _ in range(B)]
+    first = eng.step([(s, q[:2 + i % 5]) for i, (s, q) in enumerate(zip(slots, seqs))]).cpu().numpy()
+    rows = [[first[i]] for i in range(B)]
+    for k in range(5):
+        o = eng.step([(s, [q[2 + i % 5 + k]]) for i, (s, q) in enumerate(zip(slots, seqs))]).cpu().numpy()
+        for i in range(B):
+            rows[i].append(o[i])
+    for i in range(B):
+        n0 = 2 + i % 5
+        close(np.stack(rows[i]), plain_logits(name, seqs[i])[n0 - 1:n0 + 5], dtype, f"request {i}")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_wanted_places_and_errors(dtype):
     from gpullama3_java_amd.engine import CacheFull

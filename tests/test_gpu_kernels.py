@@ -536,12 +536,13 @@ def test_gemm_skinny_leaves_sums_of_squares(M):
     assert np.all(got[:, M:] == -1.0)                                        # rows that do not exist are not written
 
 
+@pytest.mark.parametrize("folded_norm", [True, False])
 @pytest.mark.parametrize("pairing", ["adjacent", "half", None])
 @pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 16), (5, 5, 48), (8, 1, 128)])
-def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs):
+def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs, folded_norm):
     rng = np.random.default_rng(hs + H)
     d, page = 96, 64
-    lens_before = [70, 0, 129, 63, 64]
+    lens_before = [70, 0, 129, 63, 64] if folded_norm else [70, 0, 129, 63, 64] + list(range(3, 48))   # 50 rows
     T = len(lens_before)
     x = (rng.standard_normal((T, d)) * 2).astype(np.float32)
     nw = rounded(1 + 0.2 * rng.standard_normal(d), "bfloat16")
@@ -553,11 +554,19 @@ def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs):
     before_k, before_v = kc.clone(), vc.clone()
     cos, sin = P.rope_table(256, hs, 50000.0)
     q_out = torch.zeros(T, H * hs, device=DEV, dtype=torch.bfloat16)
-    K().qkv_rope_cache(dev(x), dev(nw), dev(ssq_partials(x, 6)), 6, 1e-5, dev(w, torch.bfloat16), q_out,
-                       dev(positions, torch.int32), dev(seq_of, torch.int32), table,
-                       dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
-                       pairing == "adjacent", page)
-    qkv = P.linear(P.rmsnorm(x, nw, 1e-5), w)
+    if folded_norm:
+        K().qkv_rope_cache(dev(x), dev(nw), dev(ssq_partials(x, 6)), 6, 1e-5, dev(w, torch.bfloat16), q_out,
+                           dev(positions, torch.int32), dev(seq_of, torch.int32), table,
+                           dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
+                           pairing == "adjacent", page)
+        qkv = P.linear(P.rmsnorm(x, nw, 1e-5), w)
+    else:                                                                     # rows that are normalised already
+        h = rounded(x, "bfloat16")
+        K().qkv_rope_cache(dev(h, torch.bfloat16), None, None, 0, 0.0, dev(w, torch.bfloat16), q_out,
+                           dev(positions, torch.int32), dev(seq_of, torch.int32), table,
+                           dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
+                           pairing == "adjacent", page)
+        qkv = P.linear(h, w)
     q = qkv[:, :H * hs].reshape(T, H, hs)
     k = qkv[:, H * hs:(H + Kh) * hs].reshape(T, Kh, hs)
     v = qkv[:, (H + Kh) * hs:].reshape(T, Kh, hs)
@@ -575,6 +584,92 @@ def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs):
         mk[pid, :, positions[i] % page] = False
         mv[pid, :, :, positions[i] % page] = False
     assert torch.equal(kc[mk], before_k[mk]) and torch.equal(vc[mv], before_v[mv])   # nothing else moved
+
+
+# ------------------------------------------------------------------ the wide kernel for 33 to 64 rows, K in slices
+@pytest.mark.parametrize("M", [33, 48, 64])
+@pytest.mark.parametrize("N, Kd", [(2048, 2048), (130, 72), (40, 40), (1000, 1544), (6144, 256)])
+def test_gemm_skinny_wide(M, N, Kd):
+    rng = np.random.default_rng(M + N)
+    a = rounded(rng.standard_normal((M, Kd)), "bfloat16")
+    w = rounded(rng.standard_normal((2 * N, Kd)) / math.sqrt(Kd), "bfloat16")
+    A, W = dev(a, torch.bfloat16), dev(w, torch.bfloat16)
+    lib = K()
+    ref = P.linear(a, w[:N])
+    scale = np.abs(ref).max()
+    tol32 = 2e-5 * scale * math.sqrt(Kd / 64)
+    for strips in (0, 2, 4):
+        out = torch.full((M + 1, N + 3), -1.0, device=DEV)                  # a view with a row stride, a row beyond
+        lib.gemm_skinny_wide(A, W[:N], out[:M, :N], lib.EPI_STORE, strips=strips)
+        np.testing.assert_allclose(out[:M, :N].cpu().numpy(), ref, atol=tol32, err_msg=f"strips {strips}")
+        assert torch.all(out[M] == -1) and torch.all(out[:, N:] == -1)
+        for slices in sorted({s_ for s_ in (2, 3, 8) if s_ <= (Kd + 31) // 32}):
+            part = torch.full((slices, M, N), 7.0, device=DEV)
+            lib.gemm_skinny_wide(A, W[:N], part, lib.EPI_STORE, strips=strips)
+            np.testing.assert_allclose(part.sum(0).cpu().numpy(), ref, atol=tol32, err_msg=f"{slices} slices")
+            per = -(-((Kd + 31) // 32) // slices) * 32                        # each slice is its own range of K
+            for s_ in range(slices):
+                lo, hi = min(s_ * per, Kd), min((s_ + 1) * per, Kd)
+                np.testing.assert_allclose(part[s_].cpu().numpy(), P.linear(a[:, lo:hi], w[:N, lo:hi]) if hi > lo
+                                           else np.zeros((M, N), np.float32), atol=tol32)
+    ob = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+    lib.gemm_skinny_wide(A, W[:N], ob)
+    np.testing.assert_allclose(ob.float().cpu().numpy(), ref, atol=1e-2 * scale)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    x = dev(res)
+    lib.gemm_skinny_wide(A, W[:N], x, lib.EPI_ADD)
+    np.testing.assert_allclose(x.cpu().numpy(), res + ref, atol=tol32 + 1e-6)
+    refg = P.silu(P.linear(a, w[:N])) * P.linear(a, w[N:])
+    for strips in (0, 1, 2):
+        g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+        lib.gemm_skinny_wide(A, W, g_, lib.EPI_GATED, strips=strips)
+        np.testing.assert_allclose(g_.float().cpu().numpy(), refg, atol=1e-2 * max(np.abs(refg).max(), 1e-3))
+
+
+def test_gemm_skinny_wide_refuses_what_it_cannot_do():
+    lib = K()
+    a = torch.zeros(40, 64, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(32, 64, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(lib.KernelError):
+        lib.gemm_skinny_wide(a[:20], w, torch.zeros(20, 32, device=DEV))                       # the skinny kernel's rows
+    with pytest.raises(lib.KernelError, match="slices"):
+        lib.gemm_skinny_wide(a, w, torch.zeros(2, 40, 32, device=DEV), lib.EPI_ADD)            # slices are stored, not added
+    with pytest.raises(lib.KernelError, match="slices"):
+        lib.gemm_skinny_wide(a, w, torch.zeros(3, 40, 32, device=DEV))                         # more slices than k-steps
+    assert lib.wide_slices(2048, 8192) == 8 and lib.wide_slices(2048, 2048) == 4 and lib.wide_slices(128256, 2048) == 1
+
+
+@pytest.mark.parametrize("d, wdtype, odtype", [(2048, "bfloat16", "bfloat16"), (100, "float32", "float32"), (7, "float32", "bfloat16")])
+def test_add_slices_rmsnorm(d, wdtype, odtype):
+    rng = np.random.default_rng(d)
+    M, S = 37, 5
+    x = (rng.standard_normal((M, d)) * 3).astype(np.float32)
+    parts = rng.standard_normal((S, M, d)).astype(np.float32)
+    w = rounded(1 + 0.2 * rng.standard_normal(d), wdtype)
+    total = x.copy()
+    for s_ in range(S):
+        total = total + parts[s_]                                            # the kernel's order of summation
+    lib = K()
+    X = dev(x)
+    out = torch.empty(M, d, device=DEV, dtype=TD[odtype])
+    lib.add_slices_rmsnorm(X, dev(parts), dev(w, TD[wdtype]), out, 1e-6)
+    assert np.array_equal(X.cpu().numpy(), total)
+    plain = torch.empty(M, d, device=DEV, dtype=TD[odtype])
+    lib.rmsnorm(X, dev(w, TD[wdtype]), plain, 1e-6)
+    assert torch.equal(out, plain)                                           # the same norm as the kernel of its own
+    np.testing.assert_allclose(out.float().cpu().numpy(), P.rmsnorm(total, w, 1e-6),
+                               rtol=1e-5 if odtype == "float32" else 5e-3, atol=1e-6)
+    X2 = dev(x)
+    lib.add_slices_rmsnorm(X2, dev(parts))                                   # the sums alone
+    assert np.array_equal(X2.cpu().numpy(), total)
+    rows = np.array([7, 0, 7, 36])                                           # listed rows: x stays as it was
+    X3 = dev(x)
+    out3 = torch.empty(4, d, device=DEV, dtype=TD[odtype])
+    lib.add_slices_rmsnorm(X3, dev(parts), dev(w, TD[wdtype]), out3, 1e-6, dev(rows, torch.int32))
+    assert np.array_equal(X3.cpu().numpy(), x)
+    assert torch.equal(out3, out[torch.as_tensor(rows).to(DEV)])
+    with pytest.raises(lib.KernelError):
+        lib.add_slices_rmsnorm(X, dev(parts[:, :5]))
 
 
 @pytest.mark.parametrize("V", [2, 63, 1000, 128256])
