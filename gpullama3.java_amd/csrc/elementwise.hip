@@ -84,21 +84,45 @@ extern "C" int gl3_rmsnorm(const float* x, const int* rows, const void* w, int w
 // are added to the residual rows in slice order, x[row] += P[0][row] + P[1][row] + ..., and the
 // rows' RMSNorm is written to `out` (null: the sums alone). With `rows` the listed rows are
 // normalised and x is left as it was (a row may be listed twice). One block per row.
-template <typename TW, typename TO>
-__global__ void add_slices_rmsnorm_kernel(float* __restrict__ x, const int* __restrict__ rows,
-                                          const float* __restrict__ P, int n_slices, long slice_stride, long ldp,
-                                          const TW* __restrict__ w, TO* __restrict__ out, int d, float eps) {
+// A thread's first VEC elements stay in registers between the two passes, and the loads of up to
+// eight slices are all asked for before the first is added: for rows of up to 4096 floats the
+// kernel is two trips to memory.
+template <typename TW, typename TO, int VEC>
+__global__ __launch_bounds__(1024) void add_slices_rmsnorm_kernel(float* __restrict__ x, const int* __restrict__ rows,
+                                                                  const float* __restrict__ P, int n_slices,
+                                                                  long slice_stride, long ldp,
+                                                                  const TW* __restrict__ w, TO* __restrict__ out, int d,
+                                                                  float eps) {
+  typedef float vec_t __attribute__((ext_vector_type(VEC)));
   __shared__ float scratch[16];
   const long r = blockIdx.x;
   const long src = rows ? rows[r] : r;
   float* xr = x + src * d;
   const float* pr = P + src * ldp;
+  // the sum of the slices for elements i .. i+VEC-1, in slice order
+  auto summed = [&](int i) {
+    vec_t v = *(const vec_t*)(xr + i);
+    for (int s0 = 0; s0 < n_slices; s0 += 8) {
+      vec_t p[8];
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        p[s] = s0 + s < n_slices ? *(const vec_t*)(pr + (long)(s0 + s) * slice_stride + i) : vec_t(0.f);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        if (s0 + s < n_slices) v += p[s];
+    }
+    return v;
+  };
+  const int first = threadIdx.x * VEC, stride = blockDim.x * VEC;
+  vec_t kept = vec_t(0.f);
   float ss = 0.f;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    float v = xr[i];
-    for (int s = 0; s < n_slices; ++s) v += pr[s * slice_stride + i];
-    if (!rows) xr[i] = v;
-    ss += v * v;
+  for (int i = first; i < d; i += stride) {
+    const vec_t v = summed(i);
+    if (i == first) kept = v;
+    if (!rows) *(vec_t*)(xr + i) = v;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) ss += ((const float*)&v)[e] * ((const float*)&v)[e];
   }
   if (!out) return;
   ss = block_sum(ss, scratch);
@@ -106,11 +130,11 @@ __global__ void add_slices_rmsnorm_kernel(float* __restrict__ x, const int* __re
   ss = ss + eps;
   ss = 1.0f / sqrtf(ss);
   TO* o = out + r * d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    float v = xr[i];   // this thread's own store when the sums were written back
-    if (rows)
-      for (int s = 0; s < n_slices; ++s) v += pr[s * slice_stride + i];
-    o[i] = from_f32<TO>(to_f32<TW>(w[i]) * (ss * v));
+  for (int i = first; i < d; i += stride) {
+    // beyond the kept elements: this thread's own stores, or the sum again when x was not written
+    const vec_t v = i == first ? kept : (rows ? summed(i) : *(const vec_t*)(xr + i));
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o[i + e] = from_f32<TO>(to_f32<TW>(w[i + e]) * (ss * ((const float*)&v)[e]));
   }
 }
 
@@ -121,10 +145,19 @@ extern "C" int gl3_add_slices_rmsnorm(float* x, const int* rows, const float* P,
   GL3_REQUIRE(x && P && n_rows > 0 && d > 0 && n_slices > 0 && ldp >= d,
               "gl3_add_slices_rmsnorm: bad arguments (rows=%d d=%d slices=%d)", n_rows, d, n_slices);
   GL3_REQUIRE((w != nullptr) == (out != nullptr), "gl3_add_slices_rmsnorm: weight and output come together");
-  dim3 grid(n_rows), block(256);
+  const bool vec4 = d % 4 == 0 && ldp % 4 == 0 && slice_stride % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)P % 16 == 0;
+  const int per = vec4 ? 4 : 1;
+  const int threads = d / per >= 1024 ? 1024 : d / per > 256 ? 512 : 256;
+  dim3 grid(n_rows), block(threads);
 #define GO(TW, TO)                                                                                              \
-  add_slices_rmsnorm_kernel<TW, TO><<<grid, block, 0, stream>>>(x, rows, P, n_slices, slice_stride, ldp,       \
-                                                                 (const TW*)w, (TO*)out, d, eps)
+  do {                                                                                                          \
+    if (vec4)                                                                                                   \
+      add_slices_rmsnorm_kernel<TW, TO, 4><<<grid, block, 0, stream>>>(x, rows, P, n_slices, slice_stride, ldp, \
+                                                                       (const TW*)w, (TO*)out, d, eps);         \
+    else                                                                                                        \
+      add_slices_rmsnorm_kernel<TW, TO, 1><<<grid, block, 0, stream>>>(x, rows, P, n_slices, slice_stride, ldp, \
+                                                                       (const TW*)w, (TO*)out, d, eps);         \
+  } while (0)
   if (!out) GO(float, float);
   else if (w_dtype == GL3_F32 && out_dtype == GL3_F32) GO(float, float);
   else if (w_dtype == GL3_F32 && out_dtype == GL3_BF16) GO(float, bf16_t);

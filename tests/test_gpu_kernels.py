@@ -639,10 +639,11 @@ def test_gemm_skinny_wide_refuses_what_it_cannot_do():
     assert lib.wide_slices(2048, 8192) == 8 and lib.wide_slices(2048, 2048) == 4 and lib.wide_slices(128256, 2048) == 1
 
 
-@pytest.mark.parametrize("d, wdtype, odtype", [(2048, "bfloat16", "bfloat16"), (100, "float32", "float32"), (7, "float32", "bfloat16")])
-def test_add_slices_rmsnorm(d, wdtype, odtype):
+@pytest.mark.parametrize("d, wdtype, odtype, S", [(2048, "bfloat16", "bfloat16", 8), (100, "float32", "float32", 5),
+                                                  (7, "float32", "bfloat16", 3), (9000, "float32", "float32", 11)])
+def test_add_slices_rmsnorm(d, wdtype, odtype, S):
     rng = np.random.default_rng(d)
-    M, S = 37, 5
+    M = 37
     x = (rng.standard_normal((M, d)) * 3).astype(np.float32)
     parts = rng.standard_normal((S, M, d)).astype(np.float32)
     w = rounded(1 + 0.2 * rng.standard_normal(d), wdtype)
@@ -654,9 +655,6 @@ def test_add_slices_rmsnorm(d, wdtype, odtype):
     out = torch.empty(M, d, device=DEV, dtype=TD[odtype])
     lib.add_slices_rmsnorm(X, dev(parts), dev(w, TD[wdtype]), out, 1e-6)
     assert np.array_equal(X.cpu().numpy(), total)
-    plain = torch.empty(M, d, device=DEV, dtype=TD[odtype])
-    lib.rmsnorm(X, dev(w, TD[wdtype]), plain, 1e-6)
-    assert torch.equal(out, plain)                                           # the same norm as the kernel of its own
     np.testing.assert_allclose(out.float().cpu().numpy(), P.rmsnorm(total, w, 1e-6),
                                rtol=1e-5 if odtype == "float32" else 5e-3, atol=1e-6)
     X2 = dev(x)
