@@ -4,6 +4,7 @@ import json
 import math
 import os
 from dataclasses import dataclass, field
+from types import SimpleNamespace
 
 import numpy as np
 import pytest
@@ -147,6 +148,79 @@ def test_feed_forward_part(dtype):
     np.testing.assert_allclose(x.cpu().numpy() - 2, ref, atol=(2e-5 if dtype == "float32" else 2e-2) * np.abs(ref).max())
     with pytest.raises(ValueError, match="gelu"):
         build_part("ffn", GatedFeedForwardSpec(hidden=d, intermediate=F, activation="gelu"), dtype=TD[dtype], device=DEV)
+
+
+def test_rotary_part_tables():
+    """The position encoding alone: its tables are the plain implementation's, with and without the
+    llama3 rule; sizes chosen so that all three branches of the rule are taken."""
+    from gpullama3_java_amd.config import Llama3RopeScaling, RotarySpec
+    from gpullama3_java_amd.parts import build_part
+    for hs, theta, scaling in [(48, 10000.0, None), (64, 500000.0, (32.0, 1.0, 4.0, 8192)), (16, 1000.0, (8.0, 2.0, 3.0, 100))]:
+        sc = Llama3RopeScaling(*scaling) if scaling else None
+        part = build_part("position", RotarySpec(head_dim=hs, theta=theta, scaling=sc, pairing="adjacent", max_positions=300),
+                          device=torch.device(DEV))
+        plain_sc = None if not scaling else dict(zip(("factor", "low_freq_factor", "high_freq_factor",
+                                                      "original_max_position_embeddings"), scaling))
+        cos, sin = P.rope_table(300, hs, theta, plain_sc)
+        assert part.rot_dim == hs and part.adjacent and part.cos.shape == (300, hs // 2)
+        np.testing.assert_array_equal(part.cos.cpu().numpy(), cos)
+        np.testing.assert_array_equal(part.sin.cpu().numpy(), sin)
+        if scaling:
+            f0, f1 = P.rope_frequencies(hs, theta, None), P.rope_frequencies(hs, theta, plain_sc)
+            kinds = {"kept" if b == a else "divided" if b == np.float32(a / np.float32(scaling[0])) else "between"
+                     for a, b in zip(f0, f1)}
+            assert {"kept", "divided"} <= kinds
+    with pytest.raises(ValueError, match="even"):
+        build_part("position", RotarySpec(head_dim=15, max_positions=8), device=torch.device(DEV))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_tok", [9, 50, 150])
+def test_block_part(dtype, n_tok):
+    """The arrangement alone: x += mixer(norm(x)); x += ffn(norm(x)), at step sizes that take the
+    folded norms (few rows), the sliced products (33 to 64 rows) and the kernels of their own."""
+    from gpullama3_java_amd.config import AttentionSpec, BlockSpec, GatedFeedForwardSpec, NormSpec, RotarySpec
+    from gpullama3_java_amd.parts import RunInfo, build_part
+    rng = np.random.default_rng(n_tok)
+    d, H, Kh, hs, F = 80, 4, 2, 32, 144
+    spec = BlockSpec(kind="prenorm",
+                     mixer_norm=NormSpec(dim=d, eps=1e-4, names={"weight": "n1"}),
+                     mixer=AttentionSpec(hidden=d, n_heads=H, n_kv_heads=Kh, head_dim=hs, names={k: k for k in "qkvo"},
+                                         position=RotarySpec(head_dim=hs, theta=300.0, pairing="half", max_positions=512)),
+                     ffn_norm=NormSpec(dim=d, eps=1e-4, names={"weight": "n2"}),
+                     ffn=GatedFeedForwardSpec(hidden=d, intermediate=F, names={"gate": "g", "up": "u", "down": "dn"}))
+    block = build_part("block", spec, dtype=TD[dtype], device=torch.device(DEV))
+    shapes = {}
+    for p_ in block.parts():
+        shapes.update({n: t.shape for n, t in p_.tensors().items()})
+    assert set(shapes) == {"n1", "n2", "q", "k", "v", "o", "g", "u", "dn"}
+    W = {n: stored(1 + 0.2 * rng.standard_normal(sh) if n in ("n1", "n2") else rng.standard_normal(sh) * 0.15, dtype)
+         for n, sh in shapes.items()}
+    weights = {n: t.to(DEV) for n, t in W.items()}
+    for p_ in block.parts():
+        p_.load(weights)
+    Wn = {n: t.float().numpy() for n, t in W.items()}
+    x0 = rng.standard_normal((n_tok, d)).astype(np.float32)
+    cos, sin = P.rope_table(512, hs, 300.0)
+    pos = np.arange(n_tok)
+    h = P.rmsnorm(x0, Wn["n1"], 1e-4)
+    q = P.rope_rotate(P.linear(h, Wn["q"]).reshape(n_tok, H, hs), pos, cos, sin, "half")
+    k = P.rope_rotate(P.linear(h, Wn["k"]).reshape(n_tok, Kh, hs), pos, cos, sin, "half")
+    v = P.linear(h, Wn["v"]).reshape(n_tok, Kh, hs)
+    x1 = x0 + P.linear(P.attention(q, k, v).reshape(n_tok, H * hs), Wn["o"])
+    ref = x1 + P.feed_forward(P.rmsnorm(x1, Wn["n2"], 1e-4), Wn["g"], Wn["u"], Wn["dn"])
+    for fuse in ([False, True] if dtype == "bfloat16" else [False]):
+        harness = Harness([block.mixer.kv_need()], [None], dtype)
+        harness.fuse = fuse                                                  # as the engine sets it for known parts
+        harness.spec = SimpleNamespace(hidden=d)
+        ctx = harness.context([(harness.cache.take_slot(), n_tok)])
+        assert ctx.fuse == fuse
+        x = torch.as_tensor(x0).to(DEV)
+        block.forward(ctx, x, RunInfo(entry=0, kv_entry=0, writes_kv=True))
+        from gpullama3_java_amd.parts import ops
+        ops.settle_residual(ctx, x)                                          # sums still in slices, if any
+        t = (2e-5 if dtype == "float32" else 2e-2) * np.abs(ref).max()
+        np.testing.assert_allclose(x.cpu().numpy(), ref, atol=t, err_msg=f"fuse {fuse}")
 
 
 def test_unknown_part_kind_lists_the_known():
