@@ -137,13 +137,64 @@ __device__ __forceinline__ void sk_ssq_partials(float (*sm_ssq)[64], int M, cons
   sm_ssq[wave][lane] = sp;
 }
 
+// What a strip's epilogue reads besides the sums, asked for before the main loop so that the
+// epilogue does not wait for memory again: the residual values it adds to (add epilogue), the
+// token's position, its cache page and the rotation's cos and sin (SK_QKV). Wave `mt` finishes
+// token tile `mt`; a lane holds 4 columns of one token.
+struct SkPre {
+  f32x4 prev;
+  f32x4 co, si;
+  int pos;
+  int page;
+};
+
+template <int MT, int EPI, typename TC>
+__device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int N, long ldc, int strip, int hd, int sub,
+                                            bool rotated, const SkRope& rp) {
+  SkPre p;
+  p.prev = p.co = p.si = f32x4{0.f, 0.f, 0.f, 0.f};
+  p.pos = 0; p.page = 0;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const int m = wave * 16 + r;
+  if (wave >= MT || m >= M) return p;
+  if (EPI == SK_ADD) {
+    const int n = strip * 16 + 4 * q;
+    const TC* cp = C + (long)m * ldc + n;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      if (n + c < N) p.prev[c] = to_f32<TC>(cp[c]);
+  }
+  if (EPI == SK_QKV) {
+    p.pos = rp.positions[m];
+    if (hd >= rp.n_heads) p.page = rp.block_table[(long)rp.seq_of_token[m] * rp.table_stride + p.pos / rp.page_size];
+    if (rotated) {
+      const int half = rp.head_dim / 2;
+      if (rp.adjacent) {
+        const int jj = (16 * sub + 4 * q) / 2;
+        p.co[0] = rp.cos_tab[(long)p.pos * half + jj];     p.si[0] = rp.sin_tab[(long)p.pos * half + jj];
+        p.co[1] = rp.cos_tab[(long)p.pos * half + jj + 1]; p.si[1] = rp.sin_tab[(long)p.pos * half + jj + 1];
+      } else {
+        const int jj = 8 * sub + 4 * (q & 1);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          p.co[c] = rp.cos_tab[(long)p.pos * half + jj + c];
+          p.si[c] = rp.sin_tab[(long)p.pos * half + jj + c];
+        }
+      }
+    }
+  }
+  return p;
+}
+
 // The end of a strip: the waves' partial tiles are summed in wave order by the wave that owns
 // the tile, then the epilogue runs. `sub`, `hd`, `rotated` describe the strip for SK_QKV.
 template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ>
 __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 1) * MT][64], float (*sm_ssq)[64],
                                           const f32x4 (&acc)[(EPI == SK_GATED) ? 2 : 1][MT], int strip, int hd, int sub,
                                           bool rotated, TC* __restrict__ C, int M, int N, int K, long ldc,
-                                          const SkNorm& nrm, float* __restrict__ ssq_out, const SkRope& rp) {
+                                          const SkNorm& nrm, float* __restrict__ ssq_out, const SkRope& rp,
+                                          const SkPre& pre) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
@@ -182,14 +233,13 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
     }
     if (EPI == SK_QKV) {
       const int hs = rp.head_dim;
-      const int pos = m_ok ? rp.positions[m] : 0;
+      const int pos = pre.pos;
       int col = 16 * sub + 4 * q;          // first of this lane's 4 columns inside the head
       if (rotated) {
         const int half = hs / 2;
         if (rp.adjacent) {
-          const int jj = (16 * sub + 4 * q) / 2;
-          const float c0 = rp.cos_tab[(long)pos * half + jj], s0 = rp.sin_tab[(long)pos * half + jj];
-          const float c1 = rp.cos_tab[(long)pos * half + jj + 1], s1 = rp.sin_tab[(long)pos * half + jj + 1];
+          const float c0 = pre.co[0], s0 = pre.si[0];
+          const float c1 = pre.co[1], s1 = pre.si[1];
           const f32x4 o = v;
           v[0] = o[0] * c0 - o[1] * s0;
           v[1] = o[0] * s0 + o[1] * c0;
@@ -203,7 +253,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
             const float other = __shfl_xor(v[c], 32, 64);
-            const float co = rp.cos_tab[(long)pos * half + jj + c], si = rp.sin_tab[(long)pos * half + jj + c];
+            const float co = pre.co[c], si = pre.si[c];
             v[c] = first ? v[c] * co - other * si : other * si + v[c] * co;
           }
         }
@@ -215,7 +265,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
           for (int c = 0; c < 4; ++c) o4[c] = static_cast<bf16_t>(v[c]);
           *(bf16x4*)((bf16_t*)C + (long)m * ldc + (long)hd * hs + col) = o4;
         } else {
-          const long page = rp.block_table[(long)rp.seq_of_token[m] * rp.table_stride + pos / rp.page_size];
+          const long page = pre.page;
           const int in_page = pos % rp.page_size;
           if (hd < rp.n_heads + rp.n_kv) {
             const int ch = hd - rp.n_heads;
@@ -241,7 +291,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
       for (int c = 0; c < 4; ++c) {
         if (n + c < N) {
           float o = v[c];
-          if (EPI == SK_ADD) o += to_f32<TC>(cp[c]);
+          if (EPI == SK_ADD) o += pre.prev[c];
           cp[c] = from_f32<TC>(o);
           sq += o * o;
         }
@@ -276,6 +326,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) xrow[mt] = sk_x_row<XNORM>(Av, lda, min(mt * 16 + r, M - 1), nrm) ;
   if (XNORM) sk_ssq_partials<NW>(sm_ssq, M, nrm);
+  const SkPre pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp);
 
   const int steps = (K + 31) / 32;   // k-steps of 32
   f32x4 acc[NG][MT];
@@ -305,7 +356,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
       }
     }
   }
-  sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp);
+  sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp,
+                                         pre);
 }
 
 // The resident kernel: K <= 32 * NW * KS. `n_strips` strips are shared out over the blocks.
@@ -412,6 +464,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
         if (EPI == SK_GATED) un[i] = ok ? *(const bf16x8*)(wrow + (long)N * ldw + k) : zero;
       }
     }
+    const SkPre pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp);
     __builtin_amdgcn_sched_barrier(0);   // the next strip's loads are on their way before this strip's are used
     f32x4 acc[NG][MT];
 #pragma unroll
@@ -426,7 +479,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
         if (EPI == SK_GATED) acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[i], xf[i][mt], acc[1][mt], 0, 0, 0);
       }
     }
-    sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp);
+    sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp,
+                                           pre);
     if (next >= n_strips) break;
     __syncthreads();   // the partial tiles in shared memory are free again
 #pragma unroll
@@ -470,6 +524,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) xrow[mt] = A + (long)min(mt * 16 + r, M - 1) * lda + q * 8;
 
+  TC* out = C + (long)blockIdx.y * slice_stride;
+  SkPre pre[NS];
+#pragma unroll
+  for (int g = 0; g < NS; ++g)
+    pre[g] = sk_preload<MT, EPI, TC>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g], rotated[g], rp);
+
   const int steps = (K + 31) / 32;
   const int s_begin = blockIdx.y * steps_per_slice;
   const int s_end = min(steps, s_begin + steps_per_slice);
@@ -509,13 +569,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
             acc[g][1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u][g], xf[u][mt], acc[g][1][mt], 0, 0, 0);
         }
   }
-  TC* out = C + (long)blockIdx.y * slice_stride;
 #pragma unroll
   for (int g = 0; g < NS; ++g) {
     if (g) __syncthreads();   // the partial tiles in shared memory are free again
     if (strip0 + g < n_strips)   // the same for all threads of the block
       sk_finish<MT, NW, EPI, TC, false, false>(red, sm_ssq, acc[g], strip0 + g, hd[g], sub[g], rotated[g], out, M, N, K,
-                                                ldc, SkNorm{}, nullptr, rp);
+                                                ldc, SkNorm{}, nullptr, rp, pre[g]);
   }
 }
 
