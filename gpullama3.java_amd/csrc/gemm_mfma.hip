@@ -28,7 +28,8 @@ template <int EPI, typename TC, int TM, int WM, int WN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* __restrict__ A,
                                                                   const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                   int M, int N, int K, long lda, long ldw, long ldc,
-                                                                  int tiles_m, int tiles_n) {
+                                                                  int tiles_m, int tiles_n, int k_per_slice,
+                                                                  float* __restrict__ P, long p_stride, long ldp) {
   constexpr int NT = 64 * WM * WN;                       // threads
   constexpr int BM = 32 * TM * WM;                       // rows of a block
   constexpr int BN = 64 * WN;                            // rows of W of a block
@@ -69,6 +70,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
     else wr = min(n0 + r, N - 1);
     wp[i] = W + (long)wr * ldw + scol;
   }
+  // K in slices (blockIdx.y): slice 0 ends in the epilogue proper, the others store their sums
+  // as floats into P[slice - 1], for the reader to add up in slice order
+  const int slice = blockIdx.y;
+  const int k_begin = slice * k_per_slice;
+  K = min(K, k_begin + k_per_slice);
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   bf16x8 ra[NA], rw[NWC];
   auto fetch = [&](int k0) {
@@ -78,7 +84,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
 #pragma unroll
     for (int i = 0; i < NWC; ++i) rw[i] = ok ? *(const bf16x8*)(wp[i] + k0) : zero;
   };
-  fetch(0);
+  fetch(k_begin);
 
   f32x16 acc[TM][2];
 #pragma unroll
@@ -92,7 +98,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   const int wrow0 = (EPI == MF_GATED) ? wn * 32 + lr : wn * 64 + lr;
   const int wrow1 = (EPI == MF_GATED) ? BN / 2 + wn * 32 + lr : wn * 64 + 32 + lr;
 
-  for (int k0 = 0; k0 < K; k0 += MF_BK) {
+  for (int k0 = k_begin; k0 < K; k0 += MF_BK) {
 #pragma unroll
     for (int i = 0; i < NA; ++i) *(bf16x8*)&As[arow_s[i]][scol] = ra[i];
 #pragma unroll
@@ -121,6 +127,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
     for (int v = 0; v < 16; ++v) {
       const int m = m0 + wm * 32 * TM + tm * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
       if (m >= M) continue;
+      if (slice > 0) {
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) {
+          const int n = n0 + wn * 64 + tn * 32 + lr;
+          if (n < N) P[(long)(slice - 1) * p_stride + (long)m * ldp + n] = acc[tm][tn][v];
+        }
+        continue;
+      }
       if (EPI == MF_GATED) {
         const int n = n0 + wn * 32 + lr;
         if (n < N) {
@@ -144,7 +158,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
 
 template <int EPI, typename TC, int TM, int WM, int WN>
 static int launch_shape(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                        hipStream_t stream) {
+                        int slices, float* P, long p_stride, long ldp, hipStream_t stream) {
   const int bm = 32 * TM * WM;
   const int ncols = (EPI == MF_GATED) ? 32 * WN : 64 * WN;
   const int tiles_n = (N + ncols - 1) / ncols;
@@ -152,27 +166,33 @@ static int launch_shape(const void* A, const void* W, void* C, int M, int N, int
   const long n_tiles = (long)tiles_m * tiles_n;
   const long blocks = ((n_tiles + 7) / 8) * 8;
   GL3_REQUIRE(blocks < (1L << 31), "gl3_gemm_mfma: too many tiles");
-  gemm_mfma_kernel<EPI, TC, TM, WM, WN><<<dim3((unsigned)blocks), dim3(64 * WM * WN), 0, stream>>>(
-      (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
+  const int k_per_slice = ((K + MF_BK - 1) / MF_BK + slices - 1) / slices * MF_BK;
+  gemm_mfma_kernel<EPI, TC, TM, WM, WN><<<dim3((unsigned)blocks, slices), dim3(64 * WM * WN), 0, stream>>>(
+      (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n, k_per_slice, P, p_stride,
+      ldp);
   GL3_LAUNCH_CHECK();
   return 0;
 }
 
 template <int EPI, typename TC>
 static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                       hipStream_t stream) {
+                       int slices, float* P, long p_stride, long ldp, hipStream_t stream) {
   // 256 x 256 tiles of sixteen waves where they still give two blocks per CU: half the operand
   // traffic per product, and that traffic is what bounds the large products. Otherwise 128 x 128
   // tiles of eight waves, of which several fit a CU and overlap each other's waits.
   const long big_n = (EPI == MF_GATED) ? (N + 127) / 128 : (N + 255) / 256;
-  if ((long)((M + 255) / 256) * big_n >= 512)
-    return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, stream);
-  return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, stream);
+  if ((long)((M + 255) / 256) * big_n * slices >= 512)
+    return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, stream);
+  return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, stream);
 }
 
 // N counts output columns: for the gated epilogue W has 2N rows (gate, then up).
+// slices > 1 (not with the gated epilogue): K is cut into that many slices; the first ends in the
+// epilogue into C, slice s > 0 stores its sums into P[s - 1] ([slices - 1][M][ldp] floats,
+// p_stride elements apart), which the caller adds to C in that order.
 extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
-                             long ldc, int epilogue, hipStream_t stream) {
+                             long ldc, int epilogue, int slices, float* P, long p_stride, long ldp,
+                             hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_mfma: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gl3_gemm_mfma: K=%d, lda=%ld, ldw=%ld must be multiples of 8",
@@ -181,14 +201,20 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
   GL3_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gl3_gemm_mfma: leading dimensions too small");
   GL3_REQUIRE(epilogue >= 0 && epilogue <= 2, "gl3_gemm_mfma: unknown epilogue %d", epilogue);
   GL3_REQUIRE(epilogue != MF_ADD || c_dtype == GL3_F32, "gl3_gemm_mfma: the add epilogue needs a float output");
+  GL3_REQUIRE(slices >= 1 && slices <= 64 && slices <= (K + MF_BK - 1) / MF_BK, "gl3_gemm_mfma: %d slices of K=%d",
+              slices, K);
+  GL3_REQUIRE(slices == 1 || (epilogue != MF_GATED && P && ldp >= N && p_stride >= (long)(M - 1) * ldp + N),
+              "gl3_gemm_mfma: slices need a buffer for their sums and another epilogue than the gated one");
+#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, stream
   if (c_dtype == GL3_F32) {
-    if (epilogue == MF_STORE) return launch_mfma<MF_STORE, float>(A, W, C, M, N, K, lda, ldw, ldc, stream);
-    if (epilogue == MF_ADD) return launch_mfma<MF_ADD, float>(A, W, C, M, N, K, lda, ldw, ldc, stream);
-    return launch_mfma<MF_GATED, float>(A, W, C, M, N, K, lda, ldw, ldc, stream);
+    if (epilogue == MF_STORE) return launch_mfma<MF_STORE, float>(ARGS);
+    if (epilogue == MF_ADD) return launch_mfma<MF_ADD, float>(ARGS);
+    return launch_mfma<MF_GATED, float>(ARGS);
   } else if (c_dtype == GL3_BF16) {
-    if (epilogue == MF_STORE) return launch_mfma<MF_STORE, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, stream);
-    if (epilogue == MF_GATED) return launch_mfma<MF_GATED, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, stream);
+    if (epilogue == MF_STORE) return launch_mfma<MF_STORE, bf16_t>(ARGS);
+    if (epilogue == MF_GATED) return launch_mfma<MF_GATED, bf16_t>(ARGS);
   }
+#undef ARGS
   GL3_REQUIRE(false, "gl3_gemm_mfma: unsupported output dtype %d for epilogue %d", c_dtype, epilogue);
   return 0;
 }

@@ -61,7 +61,7 @@ def _declare(lib):
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P],
         "gl3_qkv_rope_cache": [P, P, I, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
-        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, P],
+        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
         "gl3_attention_prefill": [P, L, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, P],
@@ -478,9 +478,18 @@ def gemm_mfma_fits(a, w, out, epilogue):
             and (out.dtype == torch.float32 or (out.dtype == torch.bfloat16 and epilogue != EPI_ADD)))
 
 
-def gemm_mfma(a, w, out, epilogue=EPI_STORE):
-    """out (=, +=, gated) a @ w.T on the matrix cores, tiled for many rows of ``a``."""
+def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None):
+    """out (=, +=, gated) a @ w.T on the matrix cores, tiled for many rows of ``a``. With
+    ``more_slices`` [S, M, N] float32 K is cut into S + 1 slices: the first goes into ``out``, the
+    others' sums are stored there, for the caller to add to ``out`` in that order."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
+    slices, p_stride, ldp = 1, 0, 0
+    if more_slices is not None:
+        _dev(more_slices, "more_slices", torch.float32, contiguous=False)
+        if (more_slices.dim() != 3 or more_slices.shape[1:] != out.shape or more_slices.stride(2) != 1
+                or epilogue == EPI_GATED):
+            raise KernelError(f"gemm: slices {tuple(more_slices.shape)} for out {tuple(out.shape)}, epilogue {epilogue}")
+        slices, p_stride, ldp = more_slices.shape[0] + 1, more_slices.stride(0), more_slices.stride(1)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
         raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
     M, K = a.shape
@@ -489,7 +498,16 @@ def gemm_mfma(a, w, out, epilogue=EPI_STORE):
     if w.shape != (rows, K) or out.shape[0] != M:
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_mfma(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
-                                   out.stride(0), epilogue, _stream()), "gemm_mfma")
+                                   out.stride(0), epilogue, slices, _ptr(more_slices), p_stride, ldp, _stream()),
+           "gemm_mfma")
+
+
+def mfma_slices(M, N, K):
+    """Into how many slices of K the tiled product [M, K] x [N, K] into the residual stream is cut:
+    more than one only where the tiles of 128 x 128 are too few for the chip and K is long enough
+    for a slice to outweigh the extra pass over its sums."""
+    tiles = -(-M // 128) * -(-N // 128)
+    return max(1, min(4, 512 // tiles, K // 2048))
 
 
 # ------------------------------------------------------------------ bfloat16 attention of a prefill step

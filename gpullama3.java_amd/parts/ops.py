@@ -80,6 +80,17 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
                 residual_written(ctx, out)
             return
         if "mfma" not in disabled and K.gemm_mfma_fits(a, w, out, epilogue):
+            M, Kd = a.shape
+            slices = K.mfma_slices(M, out.shape[1], Kd) if epilogue == EPI_ADD else 1
+            if slices > 1 and ctx is not None and getattr(ctx, "fuse", False) and "fused" not in disabled:
+                # a long K over few tiles: the first slice adds into the rows, the norm that follows
+                # adds the others
+                settle_residual(ctx, out)
+                part = ctx.buffer(f"slices{slices - 1}", (slices - 1, M, out.shape[1]), torch.float32)
+                K.gemm_mfma(a, w, out, epilogue, more_slices=part)
+                residual_written(ctx, out)
+                ctx.pending = (out.data_ptr(), part)
+                return
             K.gemm_mfma(a, w, out, epilogue)
             if epilogue == EPI_ADD:
                 residual_written(ctx, out)

@@ -161,6 +161,27 @@ def test_decode_steps_of_33_to_64_sequences(name, dtype, graphs):
         close(np.stack(rows[i]), plain_logits(name, seqs[i])[n0 - 1:n0 + 5], dtype, f"request {i}")
 
 
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_prompt_products_cut_into_slices_of_k(name, monkeypatch):
+    """Products of a prompt into the residual stream cut K into slices when K is long and the tiles
+    are few; the tiny models' K is short, so the rule is replaced here by one that always cuts."""
+    from gpullama3_java_amd.csrc import lib
+    calls = []
+
+    def always(M, N, Kd):
+        n = 3 if Kd >= 192 else 2 if Kd >= 128 else 1
+        calls.append(n)
+        return n
+    monkeypatch.setattr(lib, "mfma_slices", always)
+    eng = engine(name, "bfloat16")
+    toks = rand_tokens(name, 77, 120)
+    s = eng.take_slot()
+    got = eng.step([(s, toks[:70])], want="all").cpu().numpy()
+    got2 = eng.step([(s, toks[70:])], want="all").cpu().numpy()
+    assert max(calls) > 1
+    close(np.concatenate([got, got2]), plain_logits(name, toks), "bfloat16", f"{name} in slices")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_wanted_places_and_errors(dtype):
     from gpullama3_java_amd.engine import CacheFull

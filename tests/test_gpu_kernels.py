@@ -438,6 +438,16 @@ def test_gemm_mfma(M, N, Kd):
     g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
     lib.gemm_mfma(A, W, g_, lib.EPI_GATED)
     np.testing.assert_allclose(g_.float().cpu().numpy(), refg, atol=1e-2 * max(np.abs(refg).max(), 1e-3))
+    if Kd > 64:                                                          # K in slices: the first adds, the others are stored
+        for extra in [e for e in (1, 2) if e + 1 <= -(-Kd // 64)]:
+            x2 = dev(res)
+            part = torch.full((extra, M, N), 7.0, device=DEV)
+            lib.gemm_mfma(A, W[:N], x2, lib.EPI_ADD, more_slices=part)
+            per = -(-(-(-Kd // 64)) // (extra + 1)) * 64
+            np.testing.assert_allclose(x2.cpu().numpy(), res + P.linear(a[:, :per], w[:N, :per]),
+                                       atol=2e-5 * scale * math.sqrt(Kd / 64) + 1e-6)
+            np.testing.assert_allclose((x2 + part.sum(0)).cpu().numpy(), res + ref,
+                                       atol=2e-5 * scale * math.sqrt(Kd / 64) + 1e-6, err_msg=f"{extra + 1} slices")
     wide = torch.zeros(M, N + 24, device=DEV, dtype=torch.bfloat16)      # a view with a row stride as output
     lib.gemm_mfma(A, W[:N], wide[:, 8:8 + N])
     assert torch.equal(wide[:, 8:8 + N], ob) and torch.all(wide[:, :8] == 0) and torch.all(wide[:, 8 + N:] == 0)
