@@ -4,34 +4,54 @@
 // head h / (H/K); score = q.k * scale over the keys lo..p of the query's own position
 // p; softmax; weighted sum of the values.
 //
-// A wave owns 16 consecutive queries of one sequence and up to GH query heads that
-// share one kv head, so a key or value operand that it loads serves GH heads. It walks
-// the keys in chunks of 32 with the running maximum and sum of the softmax in 32-bit.
-// Both products are transposed, as in the decode kernel:
+// A block is four waves on 64 consecutive queries of one sequence; a wave owns 16 of them
+// and up to GH query heads that share one kv head. The block walks the keys in chunks of
+// 32: its 256 threads bring a chunk of keys and of transposed values from the cache into
+// shared memory once (the next chunk travels to registers while the current one is
+// worked on, and goes into the other of two buffers), and every wave reads its operands
+// from there, so the first-level cache carries each key once per block and not once per
+// wave. Both products are transposed, as in the decode kernel:
 //   S^T[key, query]  = K[key, :] . Q[query, :]^T
 //   O^T[dim, query] += V^T[dim, key] . P^T[key, query]
 // which makes 16 bytes of a key row, and of a row of the transposed value page, the
 // operands as the instruction wants them, and leaves the probabilities in the register
 // order the second product takes (row i of the first score tile is key 8*(i/4) + i%4 of
 // the chunk, row i of the second the key 4 further, so a quarter of the lanes ends up with
-// 8 consecutive keys: one 16-byte load from a row of the transposed value page). The
-// operands of the next chunk are asked for before the current chunk is worked on. The four
-// waves of a block take neighbouring query tiles and share their keys and values through
-// the caches only; they never wait for each other.
+// 8 consecutive keys). The running maximum and sum of the softmax are kept in 32-bit, in
+// units of log2: p = 2^(s*scale*log2(e) - m) is one multiply-add and one exponential per
+// score; chunks that every query of the wave sees whole skip the mask, and the sums are
+// rescaled only when some maximum moved. Rows in shared memory are padded by 16 bytes, which
+// spreads the 16 rows that a quarter of the lanes reads over all banks.
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// max over the four lanes j, j+16, j+32, j+48 (which hold different keys of one query), by the
+// row-swap instructions: no trip through shared memory as a general shuffle makes
+__device__ __forceinline__ float max_over_quarters(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  const float m = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(m), __float_as_uint(m), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
 template <int HS, int GH>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(
+__global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
     int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
     float scale, int q_blocks) {
   constexpr int KK = HS / 32;
   constexpr int DT = HS / 16;
+  constexpr int KROW = HS + 8;            // a key row in shared memory, in elements
+  constexpr int VROW = 32 + 8;            // a row of the transposed value chunk
+  constexpr int UNITS = HS * 4;           // 16-byte units of a chunk of keys (and of values)
+  constexpr int NU = (UNITS + 255) / 256; // units per thread
+  __shared__ __attribute__((aligned(16))) bf16_t ks[2][32][KROW];
+  __shared__ __attribute__((aligned(16))) bf16_t vs[2][HS][VROW];
   const int g = n_heads / n_kv;
   const int groups = (g + GH - 1) / GH;
   // the longest query blocks first: blockIdx.x counts down through a sequence
@@ -39,22 +59,30 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int b = blockIdx.y;
   const int c = blockIdx.z / groups, hg = blockIdx.z % groups;
   // scalar: what depends on the wave alone (chunk, page) lives in scalar registers
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int j = lane & 15, qd = lane >> 4;
   const int tok0 = __builtin_amdgcn_readfirstlane(cu_seqlens[b]);
   const int q_len = __builtin_amdgcn_readfirstlane(cu_seqlens[b + 1]) - tok0;
-  const int qi0 = qb * 64 + wave * 16;   // first query of this wave, counted inside the step's tokens
-  if (qi0 >= q_len) return;
+  if (qb * 64 >= q_len) return;            // the whole block: no barrier has been passed yet
   const int before = __builtin_amdgcn_readfirstlane(kv_before[b]);
   const int heads_here = min(GH, g - hg * GH);
   const int h0 = c * g + hg * GH;
   const int* bt = block_table + (long)b * table_stride;
+  // the block's range of chunks, and the wave's own inside it
+  const int blk_first = before + qb * 64, blk_last = before + min(qb * 64 + 63, q_len - 1);
+  const int blk_lo = (window > 0 && blk_first + 1 > window) ? blk_first + 1 - window : 0;
+  const int ck0 = blk_lo / 32, ck1 = blk_last / 32;
+  const int qi0 = qb * 64 + wave * 16;     // first query of this wave, counted inside the step's tokens
+  const bool active = qi0 < q_len;
   const bool q_ok = qi0 + j < q_len;
   const int p_mine = before + qi0 + j;                           // position of this lane's query
   const int p_last = before + min(qi0 + 15, q_len - 1);          // last position of the wave
   const int p_first = before + qi0;
   const int lo_first = (window > 0 && p_first + 1 > window) ? p_first + 1 - window : 0;
+  const int lo_last = (window > 0 && p_last + 1 > window) ? p_last + 1 - window : 0;
   const int lo_mine = (window > 0 && p_mine + 1 > window) ? p_mine + 1 - window : 0;
+  const int ck_first = active ? lo_first / 32 : 1, ck_last = active ? p_last / 32 : 0;
 
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   bf16x8 qt[GH][KK];
@@ -76,78 +104,125 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     for (int dt = 0; dt < DT; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  const int krow = 8 * (j >> 2) + (j & 3);   // which key of a chunk is row j of the first score tile
-  bf16x8 ka[KK], kb2[KK], vt[DT], ka_n[KK], kb2_n[KK], vt_n[DT];
-  auto load_chunk = [&](int ck, bf16x8 (&a)[KK], bf16x8 (&b2)[KK], bf16x8 (&v)[DT]) {
+  // cache -> registers -> shared memory, 16 bytes a unit: a chunk's keys are 32 consecutive rows
+  // of a page, its values 32 consecutive positions of each of the HS rows of the transposed page.
+  // Three chunks are on their way in registers while one is worked on: a chunk's work takes a
+  // fraction of a trip to memory.
+  constexpr int AHEAD = 3;
+  bf16x8 rk[AHEAD][NU], rv[AHEAD][NU];
+  auto fetch = [&](int ck, bf16x8 (&fk)[NU], bf16x8 (&fv)[NU]) {
     const int key0 = ck * 32;
     const long page = __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
     const int po = key0 % page_size;
     const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
     const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + po;
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      a[kk] = *(const bf16x8*)(kb + (long)krow * HS + kk * 32 + 8 * qd);
-      b2[kk] = *(const bf16x8*)(kb + (long)(krow + 4) * HS + kk * 32 + 8 * qd);
+    for (int i = 0; i < NU; ++i) {
+      const int u = tid + 256 * i;
+      if (UNITS % 256 == 0 || u < UNITS) {
+        fk[i] = *(const bf16x8*)(kb + u * 8);
+        fv[i] = *(const bf16x8*)(vb + (long)(u >> 2) * page_size + (u & 3) * 8);
+      }
     }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) v[dt] = *(const bf16x8*)(vb + (long)(dt * 16 + j) * page_size + 8 * qd);
   };
-  const int ck_first = lo_first / 32, ck_last = p_last / 32;
-  load_chunk(ck_first, ka, kb2, vt);
-  for (int ck = ck_first; ck <= ck_last; ++ck) {
-    const int key0 = ck * 32;
-    if (ck < ck_last) load_chunk(ck + 1, ka_n, kb2_n, vt_n);   // on its way while this chunk is worked on
-    __builtin_amdgcn_sched_barrier(0);
-    // this lane's 8 keys of the chunk and whether its query may see them
-    bool see[8];
+  auto stage = [&](int buf, const bf16x8 (&fk)[NU], const bf16x8 (&fv)[NU]) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int u = tid + 256 * i;
+      if (UNITS % 256 == 0 || u < UNITS) {
+        *(bf16x8*)&ks[buf][(u * 8) / HS][(u * 8) % HS] = fk[i];
+        *(bf16x8*)&vs[buf][u >> 2][(u & 3) * 8] = fv[i];
+      }
+    }
+  };
+
+  const float c2 = scale * 1.4426950408889634f;   // scores in units of log2
+  const int krow = 8 * (j >> 2) + (j & 3);   // which key of a chunk is row j of the first score tile
+
+  // one chunk of one head: scores, running softmax, weighted values. MASKED: some query of the
+  // wave does not see some key of the chunk (the diagonal, a window's edge).
+  auto head_chunk = [&](int hh, const bf16x8 (&ka)[KK], const bf16x8 (&kb2)[KK], const bf16x8 (&vt)[DT], int key0,
+                        auto masked) {
+    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kk], qt[hh][kk], sa, 0, 0, 0);
+      sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb2[kk], qt[hh][kk], sb, 0, 0, 0);
+    }
+    float s[8];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const int k1 = key0 + 8 * qd + v, k2 = k1 + 4;
-      see[v] = k1 >= lo_mine && k1 <= p_mine;
-      see[4 + v] = k2 >= lo_mine && k2 <= p_mine;
+      s[v] = sa[v];
+      s[4 + v] = sb[v];
     }
-#pragma unroll
-    for (int hh = 0; hh < GH; ++hh) {
-      f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kk], qt[hh][kk], sa, 0, 0, 0);
-        sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb2[kk], qt[hh][kk], sb, 0, 0, 0);
-      }
-      float s[8];
-      float mx = -INFINITY;
+    if (decltype(masked)::value) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        s[v] = see[v] ? sa[v] * scale : -INFINITY;
-        s[4 + v] = see[4 + v] ? sb[v] * scale : -INFINITY;
-        mx = fmaxf(mx, fmaxf(s[v], s[4 + v]));
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run[hh], mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __expf(m_run[hh] - m_use);
-      float ps = 0.f;
-      bf16x8 pb;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float p = __expf(s[e] - m_use);
-        ps += p;
-        pb[e] = static_cast<bf16_t>(p);
-      }
-      l_run[hh] = l_run[hh] * alpha + ps;
-      m_run[hh] = m_new;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        o[hh][dt] *= alpha;
-        o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt], pb, o[hh][dt], 0, 0, 0);
+        const int k1 = key0 + 8 * qd + v, k2 = k1 + 4;
+        s[v] = (k1 >= lo_mine && k1 <= p_mine) ? s[v] : -INFINITY;
+        s[4 + v] = (k2 >= lo_mine && k2 <= p_mine) ? s[4 + v] : -INFINITY;
       }
     }
-    if (ck < ck_last) {
+    float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+    mx = max_over_quarters(mx);
+    mx *= c2;                                   // c2 > 0: the greatest score stays the greatest
+    const float m_new = fmaxf(m_run[hh], mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run[hh] - m_use);
+    float ps = 0.f;
+    bf16x8 pb;
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) { ka[kk] = ka_n[kk]; kb2[kk] = kb2_n[kk]; }
+    for (int e = 0; e < 8; ++e) {
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[e], c2, -m_use));
+      ps += p;
+      pb[e] = static_cast<bf16_t>(p);
+    }
+    l_run[hh] = l_run[hh] * alpha + ps;
+    m_run[hh] = m_new;
+    if (!__all(alpha == 1.0f)) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) vt[dt] = vt_n[dt];
+      for (int dt = 0; dt < DT; ++dt) o[hh][dt] *= alpha;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt], pb, o[hh][dt], 0, 0, 0);
+  };
+
+#pragma unroll
+  for (int r = 0; r < AHEAD; ++r)
+    if (ck0 + r <= ck1) fetch(ck0 + r, rk[r], rv[r]);
+  stage(0, rk[0], rv[0]);
+  __syncthreads();
+  int buf = 0;
+  for (int base = ck0; base <= ck1; base += AHEAD) {
+#pragma unroll
+    for (int r = 0; r < AHEAD; ++r) {
+      const int ck = base + r;
+      if (ck > ck1) break;
+      const int key0 = ck * 32;
+      // the registers of this chunk are free (it lies in shared memory): ask for the chunk three further
+      if (ck + AHEAD <= ck1) fetch(ck + AHEAD, rk[r], rv[r]);
+      if (ck >= ck_first && ck <= ck_last) {
+        bf16x8 ka[KK], kb2[KK], vt[DT];
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          ka[kk] = *(const bf16x8*)&ks[buf][krow][kk * 32 + 8 * qd];
+          kb2[kk] = *(const bf16x8*)&ks[buf][krow + 4][kk * 32 + 8 * qd];
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vt[dt] = *(const bf16x8*)&vs[buf][dt * 16 + j][8 * qd];
+        // every query of the wave sees the whole chunk: no mask (the same for the whole wave)
+        if (key0 + 31 <= p_first && key0 >= lo_last) {
+#pragma unroll
+          for (int hh = 0; hh < GH; ++hh) head_chunk(hh, ka, kb2, vt, key0, std::false_type{});
+        } else {
+#pragma unroll
+          for (int hh = 0; hh < GH; ++hh) head_chunk(hh, ka, kb2, vt, key0, std::true_type{});
+        }
+      }
+      if (ck < ck1) stage(buf ^ 1, rk[(r + 1) % AHEAD], rv[(r + 1) % AHEAD]);
+      __syncthreads();
+      buf ^= 1;
     }
   }
 
@@ -187,11 +262,13 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
               head_dim, page_size);
   GL3_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "gl3_attention_prefill: %d heads over %d kv heads",
               n_heads, n_kv);
+  GL3_REQUIRE(scale > 0.f, "gl3_attention_prefill: the score scale %g must be positive", (double)scale);
   GL3_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 && out_stride % 4 == 0 && (uintptr_t)out % 8 == 0,
               "gl3_attention_prefill: queries must be 16-byte aligned, outputs 8-byte aligned");
   const int g = n_heads / n_kv;
   const int q_blocks = (max_q_len + 63) / 64;
-  const int gh = head_dim > 64 ? 2 : 4;
+  // query heads per wave: as many as the registers hold with two blocks on a CU
+  const int gh = head_dim <= 32 ? 4 : head_dim <= 64 ? 2 : 1;
   const long z = (long)n_kv * ((g + gh - 1) / gh);
   GL3_REQUIRE(n_seqs <= 65535 && z <= 65535, "gl3_attention_prefill: %d sequences / %ld head groups exceed the grid",
               n_seqs, z);
@@ -202,9 +279,9 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
       table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks)
   switch (head_dim) {
     case 32: GO(32, 4); break;
-    case 64: GO(64, 4); break;
-    case 96: GO(96, 2); break;
-    default: GO(128, 2); break;
+    case 64: GO(64, 2); break;
+    case 96: GO(96, 1); break;
+    default: GO(128, 1); break;
   }
 #undef GO
   GL3_LAUNCH_CHECK();

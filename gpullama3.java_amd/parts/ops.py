@@ -174,7 +174,7 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
                 part_ml = ctx.buffer("attn_part_ml", (T, n_heads, splits, 2), torch.float32)
             return K.attention_decode(q, k_cache, v_cache, ctx.positions, ctx.seq_of_token, block_table, out, n_heads,
                                       n_kv, head_dim, page, window, scale, splits, part_o, part_ml)
-        if (not ctx.decode and "attn_prefill" not in disabled and K.has("gl3_attention_prefill")
+        if (not ctx.decode and "attn_prefill" not in disabled and K.has("gl3_attention_prefill") and scale > 0
                 and K.attention_prefill_fits(head_dim, n_heads, n_kv, page)):
             return K.attention_prefill(q, k_cache, v_cache, ctx.cu_seqlens, ctx.kv_before, block_table, out,
                                        ctx.max_q_len, n_heads, n_kv, head_dim, page, window, scale)
