@@ -224,6 +224,85 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const int* __restrict__ p
     for (int i = rot_dim + threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
 }
 
+// The same for bfloat16 rows in units of 8 elements (16 bytes): one block per token, a thread
+// takes a unit of 8 pairs (half pairing: 8 elements and the 8 half a head further; adjacent
+// pairing: 16 consecutive elements), of 8 elements that pass through, or of 8 elements of a value
+// head. head_dim and rot_dim / 2 are multiples of 8.
+typedef __bf16 rc_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float rc_f32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void rope_cache_vec_kernel(
+    bf16_t* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+    const int* __restrict__ block_table, int table_stride, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int n_heads, int n_kv,
+    int head_dim, int rot_dim, int adjacent, int page_size, int write_kv, long row_stride) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  bf16_t* row = qkv + (long)t * row_stride;
+  const int half = rot_dim / 2;
+  long page = 0;
+  if (write_kv) page = block_table[(long)seq_of_token[t] * table_stride + pos / page_size];
+  const int in_page = pos % page_size;
+  const bool rotate = cos_tab != nullptr;
+  const int rot_heads = write_kv ? n_heads + n_kv : n_heads;
+  const int pair_units = rotate ? half / 8 : 0;              // per head
+  const int plain_units = (head_dim - (rotate ? rot_dim : 0)) / 8;
+  const int per_head = pair_units + plain_units;
+  const int v_units = write_kv ? n_kv * (head_dim / 8) : 0;
+  const int total = rot_heads * per_head + v_units;
+  for (int w = threadIdx.x; w < total; w += blockDim.x) {
+    if (w >= rot_heads * per_head) {            // a unit of a value head: transposed into the cache
+      const int u = w - rot_heads * per_head;
+      const int ch = u / (head_dim / 8), e0 = (u % (head_dim / 8)) * 8;
+      const rc_bf16x8 v = *(const rc_bf16x8*)(row + (long)(n_heads + n_kv + ch) * head_dim + e0);
+      bf16_t* vt = v_cache + ((long)page * n_kv + ch) * page_size * head_dim + in_page;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vt[(long)(e0 + e) * page_size] = v[e];
+      continue;
+    }
+    const int head = w / per_head, u = w % per_head;
+    bf16_t* src = row + (long)head * head_dim;
+    bf16_t* dst = src;
+    if (head >= n_heads) dst = k_cache + (((long)page * n_kv + (head - n_heads)) * page_size + in_page) * head_dim;
+    if (u >= pair_units) {                      // elements beyond the rotation pass through
+      const int e0 = (rotate ? rot_dim : 0) + (u - pair_units) * 8;
+      if (dst != src) *(rc_bf16x8*)(dst + e0) = *(const rc_bf16x8*)(src + e0);
+      continue;
+    }
+    const int j0 = u * 8;                        // first of the unit's 8 pairs
+    const float* cp = cos_tab + (long)pos * half + j0;
+    const float* sp = sin_tab + (long)pos * half + j0;
+    const rc_f32x4 c0 = *(const rc_f32x4*)cp, c1 = *(const rc_f32x4*)(cp + 4);
+    const rc_f32x4 s0 = *(const rc_f32x4*)sp, s1 = *(const rc_f32x4*)(sp + 4);
+    const int ea = adjacent ? 2 * j0 : j0, eb = adjacent ? 2 * j0 + 8 : j0 + half;
+    const rc_bf16x8 a = *(const rc_bf16x8*)(src + ea), b = *(const rc_bf16x8*)(src + eb);
+    rc_bf16x8 oa, ob;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float c = e < 4 ? c0[e] : c1[e - 4], sn = e < 4 ? s0[e] : s1[e - 4];
+      // pair e of the unit: (a[e], b[e]) for half pairing; elements 2e, 2e+1 of the 16 for adjacent
+      float v0, v1;
+      if (adjacent) {
+        v0 = e < 4 ? (float)a[2 * e] : (float)b[2 * e - 8];
+        v1 = e < 4 ? (float)a[2 * e + 1] : (float)b[2 * e - 7];
+      } else {
+        v0 = (float)a[e];
+        v1 = (float)b[e];
+      }
+      const bf16_t r0 = static_cast<bf16_t>(v0 * c - v1 * sn), r1 = static_cast<bf16_t>(v0 * sn + v1 * c);
+      if (adjacent) {
+        if (e < 4) { oa[2 * e] = r0; oa[2 * e + 1] = r1; }
+        else { ob[2 * e - 8] = r0; ob[2 * e - 7] = r1; }
+      } else {
+        oa[e] = r0;
+        ob[e] = r1;
+      }
+    }
+    *(rc_bf16x8*)(dst + ea) = oa;
+    *(rc_bf16x8*)(dst + eb) = ob;
+  }
+}
+
 extern "C" int gl3_rope_cache_write(void* qkv, int dtype, const int* positions, const int* seq_of_token,
                                     const int* block_table, int table_stride, const float* cos_tab,
                                     const float* sin_tab, void* k_cache, void* v_cache, int n_tokens, int n_heads,
@@ -240,6 +319,17 @@ extern "C" int gl3_rope_cache_write(void* qkv, int dtype, const int* positions, 
                 "gl3_rope_cache_write: cache arguments missing");
   const int heads = write_kv ? n_heads + 2 * n_kv : n_heads;   // without the write a row holds queries only
   const long row_stride = (long)heads * head_dim;
+  // bfloat16 rows whose sizes allow 16-byte units take the kernel of one block per token
+  const bool units = dtype == GL3_BF16 && head_dim % 8 == 0 && rot_dim % 16 == 0 && (uintptr_t)qkv % 16 == 0 &&
+                     (!cos_tab || ((uintptr_t)cos_tab % 16 == 0 && (uintptr_t)sin_tab % 16 == 0)) &&
+                     (!write_kv || ((uintptr_t)k_cache % 16 == 0));
+  if (units) {
+    rope_cache_vec_kernel<<<dim3(n_tokens), dim3(256), 0, stream>>>(
+        (bf16_t*)qkv, positions, seq_of_token, block_table, table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
+        (bf16_t*)v_cache, n_heads, n_kv, head_dim, cos_tab ? rot_dim : 0, adjacent, page_size, write_kv, row_stride);
+    GL3_LAUNCH_CHECK();
+    return 0;
+  }
   GL3_REQUIRE(heads <= 65535, "gl3_rope_cache_write: %d heads exceed the grid", heads);
   dim3 grid(n_tokens, heads), block(64);
   if (dtype == GL3_F32)

@@ -180,6 +180,47 @@ def test_rope_cache_write(dtype, pairing, H, Kh, hs):
     assert torch.equal(kc[mask], before_k[mask])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("pairing", ["adjacent", "half"])
+def test_rope_of_a_part_of_the_head_and_of_queries_only(dtype, pairing):
+    """Elements beyond the rotated part pass through, into the cache too; without the cache write a
+    row holds queries only."""
+    rng = np.random.default_rng(3)
+    H, Kh, hs, rot, page = 3, 2, 64, 32, 64
+    positions = np.array([5, 70, 0, 64, 127])
+    T = len(positions)
+    seq_of = np.array([0, 1, 2, 3, 3])
+    zk = [np.zeros((6, Kh, hs), np.float32), np.zeros((71, Kh, hs), np.float32), np.zeros((1, Kh, hs), np.float32),
+          np.zeros((128, Kh, hs), np.float32)]
+    kc, vc, table = paged(zk, zk, Kh, hs, page, dtype, rng)
+    cos, sin = P.rope_table(256, rot, 10000.0)
+    qkv = rounded(rng.standard_normal((T, (H + 2 * Kh) * hs)), dtype)
+
+    def rotated(x):                                                          # [T, heads, hs]
+        out = x.copy()
+        out[..., :rot] = P.rope_rotate(x[..., :rot], positions, cos, sin, pairing)
+        return out
+    buf = dev(qkv, TD[dtype])
+    K().rope_cache_write(buf, dev(positions, torch.int32), dev(seq_of, torch.int32), table, dev(cos), dev(sin),
+                         kc, vc, H, Kh, hs, rot, pairing == "adjacent", page)
+    t = tol(dtype) * 4
+    np.testing.assert_allclose(buf.float().cpu().numpy()[:, :H * hs].reshape(T, H, hs),
+                               rotated(qkv[:, :H * hs].reshape(T, H, hs)), atol=t)
+    kr = rotated(qkv[:, H * hs:(H + Kh) * hs].reshape(T, Kh, hs))
+    kcpu, vcpu, tab = kc.float().cpu().numpy(), vc.float().cpu().numpy(), table.cpu().numpy()
+    for i in range(T):
+        pid = tab[seq_of[i], positions[i] // page]
+        np.testing.assert_allclose(kcpu[pid, :, positions[i] % page], kr[i], atol=t)
+        np.testing.assert_array_equal(vcpu[pid, :, :, positions[i] % page], qkv[i, (H + Kh) * hs:].reshape(Kh, hs))
+    q_only = dev(np.ascontiguousarray(qkv[:, :H * hs]), TD[dtype])
+    k_before = kc.clone()
+    K().rope_cache_write(q_only, dev(positions, torch.int32), dev(seq_of, torch.int32), table, dev(cos), dev(sin),
+                         kc, vc, H, Kh, hs, rot, pairing == "adjacent", page, write_kv=False)
+    np.testing.assert_allclose(q_only.float().cpu().numpy().reshape(T, H, hs),
+                               rotated(qkv[:, :H * hs].reshape(T, H, hs)), atol=t)
+    assert torch.equal(kc, k_before)
+
+
 def test_rope_position_zero_and_no_table():
     rng = np.random.default_rng(1)
     qkv = rng.standard_normal((2, 4 * 16)).astype(np.float32)
