@@ -389,3 +389,183 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     np.testing.assert_allclose(again, toy_plain(cfg, W, b), atol=2e-4)
     res = eng.generate([a[:4], b[:6]], max_new_tokens=5)                      # and the generation loop runs it
     assert [len(r.tokens) for r in res] == [5, 5]
+
+
+# ------------------------------------------------------------------ a toy feed-forward with routing, a toy position encoding
+@dataclass(frozen=True)
+class LinearAnglesSpec:
+    """Rotation of the first ``rot_dim`` elements of a head by pos * (pair + 1) * step, adjacent pairs."""
+    kind: str = "toy_linear_angles"
+    head_dim: int = 0
+    rot_dim: int = 0
+    step: float = 0.01
+    max_positions: int = 0
+
+
+def linear_angle_tables(spec):
+    pos = np.arange(spec.max_positions, dtype=np.float32)[:, None]
+    ang = (pos * ((np.arange(spec.rot_dim // 2, dtype=np.float32) + 1)[None, :] * np.float32(spec.step))).astype(np.float32)
+    return np.cos(ang.astype(np.float64)).astype(np.float32), np.sin(ang.astype(np.float64)).astype(np.float32)
+
+
+class LinearAngles:
+    """What the attention mixer asks of a position encoding: cos, sin [positions, rot_dim/2], rot_dim, adjacent."""
+
+    def __init__(self, spec, device):
+        cos, sin = linear_angle_tables(spec)
+        self.cos, self.sin = torch.from_numpy(cos).to(device), torch.from_numpy(sin).to(device)
+        self.rot_dim, self.adjacent, self.max_positions = spec.rot_dim, True, spec.max_positions
+
+
+@dataclass(frozen=True)
+class RoutedSpec:
+    """Each token goes to the one expert with the greatest router logit; the expert's output is
+    weighted with that logit's softmax probability."""
+    kind: str = "toy_routed"
+    hidden: int = 0
+    n_experts: int = 0
+    names: dict = field(default_factory=dict)
+
+
+class RoutedFeedForward:
+    def __init__(self, spec, dtype, device):
+        self.spec, self.dtype = spec, dtype
+
+    def tensors(self):
+        from gpullama3_java_amd.weights import TensorSpec
+        s = self.spec
+        return {s.names["router"]: TensorSpec((s.n_experts, s.hidden)),
+                s.names["experts"]: TensorSpec((s.n_experts, s.hidden, s.hidden))}
+
+    def load(self, weights):
+        self.router, self.experts = weights[self.spec.names["router"]], weights[self.spec.names["experts"]]
+
+    def forward(self, ctx, h, x):
+        hf = h.float()
+        p = torch.softmax(hf @ self.router.float().t(), dim=-1)              # router logits in 32-bit
+        choice = p.argmax(dim=-1)
+        for e in range(self.spec.n_experts):                                  # every token of an expert, no capacity
+            idx = (choice == e).nonzero().flatten()
+            if idx.numel():
+                x[idx] += p[idx, e, None] * (hf[idx] @ self.experts[e].float().t())
+
+
+def mixed_plain(cfg, W, toks, pos_spec):
+    d, H, Kh, hs = cfg["hidden"], cfg["heads"], cfg["kv_heads"], cfg["head_dim"]
+    T = len(toks)
+    cos, sin = linear_angle_tables(pos_spec)
+    x = W["emb"][toks].astype(np.float32)
+    # layer 0: attention with the toy position encoding, routed feed-forward
+    h = P.rmsnorm(x, W["l0.n1"], cfg["eps"])
+    q, k = P.linear(h, W["l0.q"]).reshape(T, H, hs), P.linear(h, W["l0.k"]).reshape(T, Kh, hs)
+    r = pos_spec.rot_dim
+    q[..., :r] = P.rope_rotate(q[..., :r], np.arange(T), cos, sin, "adjacent")
+    k[..., :r] = P.rope_rotate(k[..., :r], np.arange(T), cos, sin, "adjacent")
+    v = P.linear(h, W["l0.v"]).reshape(T, Kh, hs)
+    x = x + P.linear(P.attention(q, k, v).reshape(T, H * hs), W["l0.o"])
+    h = P.rmsnorm(x, W["l0.n2"], cfg["eps"])
+    p = P.softmax(h @ W["l0.router"].T)
+    out = np.zeros_like(x)
+    for t in range(T):
+        e = int(np.argmax(p[t]))
+        out[t] = p[t, e] * (h[t] @ W["l0.experts"][e].T)
+    x = x + out
+    # layer 1: the toy mixer with state, the framework's dense feed-forward
+    h = P.rmsnorm(x, W["l1.n1"], cfg["eps"])
+    s = np.zeros(d, np.float32)
+    out = np.zeros_like(x)
+    for t in range(T):
+        s = np.float32(cfg["decay"]) * s + h[t]
+        out[t] = s @ W["l1.w"].T
+    x = x + out
+    x = x + P.feed_forward(P.rmsnorm(x, W["l1.n2"], cfg["eps"]), W["l1.g"], W["l1.u"], W["l1.dn"])
+    return P.rmsnorm(x, W["final"], cfg["eps"]) @ W["head"].T
+
+
+def test_toy_routing_and_toy_position_in_a_model_with_different_layers(tmp_path):
+    """One model whose two layers differ in mixer and feed-forward: attention with a position
+    encoding defined here and a routed feed-forward defined here; then a mixer with state and the
+    framework's dense feed-forward. Registered, built, stepped in pieces and generated from, with no
+    change to the framework's files."""
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.config import AttentionSpec, BlockSpec, GatedFeedForwardSpec, ModelSpec, NormSpec, Run
+    from gpullama3_java_amd.engine import Engine
+    from gpullama3_java_amd.parts import register_part
+
+    register_part("mixer", "toy_decay", DecayMixer)
+    register_part("ffn", "toy_routed", RoutedFeedForward)
+    register_part("position", "toy_linear_angles", LinearAngles)
+    pos_spec = LinearAnglesSpec(head_dim=16, rot_dim=8, step=0.05, max_positions=128)
+
+    @dataclass(frozen=True)
+    class MixedConfig:
+        c: tuple
+        max_position_embeddings: int = 128
+        stop_ids: tuple = ()
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(tuple(sorted((k, v) for k, v in d.items() if k != "architectures")))
+
+        def with_context_length(self, n):
+            return self
+
+        def model_spec(self):
+            c = dict(self.c)
+            d, eps = c["hidden"], c["eps"]
+            norm = lambda name: NormSpec(dim=d, eps=eps, names={"weight": name})
+            layer0 = BlockSpec(kind="prenorm", mixer_norm=norm("l0.n1"),
+                               mixer=AttentionSpec(hidden=d, n_heads=c["heads"], n_kv_heads=c["kv_heads"],
+                                                   head_dim=c["head_dim"], position=pos_spec,
+                                                   names={k: f"l0.{k}" for k in "qkvo"}),
+                               ffn_norm=norm("l0.n2"),
+                               ffn=RoutedSpec(hidden=d, n_experts=c["experts"],
+                                              names={"router": "l0.router", "experts": "l0.experts"}))
+            layer1 = BlockSpec(kind="prenorm", mixer_norm=norm("l1.n1"),
+                               mixer=DecaySpec(hidden=d, decay=c["decay"], names={"w": "l1.w"}),
+                               ffn_norm=norm("l1.n2"),
+                               ffn=GatedFeedForwardSpec(hidden=d, intermediate=c["intermediate"],
+                                                        names={"gate": "l1.g", "up": "l1.u", "down": "l1.dn"}))
+            return ModelSpec(architecture="MixedToyForCausalLM", vocab_size=c["vocab"], hidden=d, layers=(layer0, layer1),
+                             run_order=(Run(0), Run(1)), final_norm=norm("final"), max_positions=128,
+                             tie_embeddings=False, embedding_name="emb", head_name="head")
+
+    g.register_architecture("MixedToyForCausalLM", MixedConfig)
+    cfg = {"architectures": ["MixedToyForCausalLM"], "hidden": 24, "heads": 3, "kv_heads": 1, "head_dim": 16,
+           "experts": 3, "intermediate": 40, "vocab": 50, "decay": 0.6, "eps": 1e-5}
+    rng = np.random.default_rng(5)
+    d, E, F, V = 24, 3, 40, 50
+    W = {"emb": rng.standard_normal((V, d)), "head": rng.standard_normal((V, d)) * 0.3, "final": np.ones(d),
+         "l0.q": rng.standard_normal((48, d)) * 0.3, "l0.k": rng.standard_normal((16, d)) * 0.3,
+         "l0.v": rng.standard_normal((16, d)) * 0.3, "l0.o": rng.standard_normal((d, 48)) * 0.2,
+         "l0.router": rng.standard_normal((E, d)), "l0.experts": rng.standard_normal((E, d, d)) * 0.2,
+         "l1.w": rng.standard_normal((d, d)) * 0.2, "l1.g": rng.standard_normal((F, d)) * 0.3,
+         "l1.u": rng.standard_normal((F, d)) * 0.3, "l1.dn": rng.standard_normal((d, F)) * 0.2}
+    for n in ("l0.n1", "l0.n2", "l1.n1", "l1.n2"):
+        W[n] = 1 + 0.1 * rng.standard_normal(d)
+    W = {k: v.astype(np.float32) for k, v in W.items()}
+    folder = str(tmp_path / "mixed")
+    os.makedirs(folder)
+    json.dump(cfg, open(os.path.join(folder, "config.json"), "w"))
+    save_file({k: torch.as_tensor(v) for k, v in W.items()}, os.path.join(folder, "model.safetensors"))
+
+    eng = Engine.from_folder(folder, dtype="float32", max_tokens=512, n_slots=3)
+    assert len(eng.cache.groups) == 1 and sorted(eng.cache.state) == [1]     # keys and values for layer 0, state for layer 1
+    a, b = rng.integers(0, V, 70).tolist(), rng.integers(0, V, 9).tolist()
+    ref_a, ref_b = mixed_plain(cfg, W, a, pos_spec), mixed_plain(cfg, W, b, pos_spec)
+    choices = {int(np.argmax(P.softmax(P.rmsnorm(W["emb"][a], W["l0.n2"], 1e-5) @ W["l0.router"].T)[t])) for t in range(70)}
+    assert len(choices) > 1                                                   # more than one expert is in use
+    sa, sb = eng.take_slot(), eng.take_slot()
+    out = eng.step([(sa, a[:40]), (sb, b[:3])], want="all").cpu().numpy()
+    got_a, got_b = [out[:40]], [out[40:]]
+    for i in range(6):
+        o = eng.step([(sa, [a[40 + i]]), (sb, [b[3 + i]])]).cpu().numpy()
+        got_a.append(o[:1]); got_b.append(o[1:])
+    eng.give_back_slot(sb)
+    got_a.append(eng.step([(sa, a[46:])], want="all").cpu().numpy())
+    scale = np.abs(ref_a).max()
+    np.testing.assert_allclose(np.concatenate(got_a), ref_a, atol=1e-4 * scale)
+    np.testing.assert_allclose(np.concatenate(got_b), ref_b, atol=1e-4 * scale)
+    res = eng.generate([a[:5], b[:4]], max_new_tokens=4)
+    assert [len(r.tokens) for r in res] == [4, 4]
+    assert res[0].tokens[0] == int(np.argmax(mixed_plain(cfg, W, a[:5], pos_spec)[-1]))
