@@ -63,9 +63,11 @@ struct SkRope {
 };
 
 // Which row of W is row r of a strip's tile, and for SK_QKV which head the strip belongs to.
-template <int EPI>
+// A strip is ROWS rows of W: 16, or 8 (then rows 8..15 of the tile repeat rows 0..7 and are not
+// written: half a tile is wasted for twice as many blocks where 16-row strips leave CUs idle).
+template <int EPI, int ROWS = 16>
 __device__ __forceinline__ int sk_strip_row(int strip, int r, int N, const SkRope& rp, int& hd, int& sub, bool& rotated) {
-  int wr = min(strip * 16 + r, N - 1);
+  int wr = min(strip * ROWS + (r % ROWS), N - 1);
   hd = 0; sub = 0; rotated = false;
   if (EPI == SK_QKV) {
     const int per_head = rp.head_dim / 16;
@@ -148,7 +150,7 @@ struct SkPre {
   int page;
 };
 
-template <int MT, int EPI, typename TC>
+template <int MT, int EPI, typename TC, int ROWS = 16>
 __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int N, long ldc, int strip, int hd, int sub,
                                             bool rotated, const SkRope& rp) {
   SkPre p;
@@ -157,9 +159,9 @@ __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
   const int m = wave * 16 + r;
-  if (wave >= MT || m >= M) return p;
+  if (wave >= MT || m >= M || 4 * q >= ROWS) return p;
   if (EPI == SK_ADD) {
-    const int n = strip * 16 + 4 * q;
+    const int n = strip * ROWS + 4 * q;
     const TC* cp = C + (long)m * ldc + n;
 #pragma unroll
     for (int c = 0; c < 4; ++c)
@@ -189,7 +191,7 @@ __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int
 
 // The end of a strip: the waves' partial tiles are summed in wave order by the wave that owns
 // the tile, then the epilogue runs. `sub`, `hd`, `rotated` describe the strip for SK_QKV.
-template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ>
+template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ, int ROWS = 16>
 __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 1) * MT][64], float (*sm_ssq)[64],
                                           const f32x4 (&acc)[(EPI == SK_GATED) ? 2 : 1][MT], int strip, int hd, int sub,
                                           bool rotated, TC* __restrict__ C, int M, int N, int K, long ldc,
@@ -198,7 +200,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
-  const int n0 = strip * 16;
+  const int n0 = strip * ROWS;
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int g = 0; g < NG; ++g)
@@ -286,7 +288,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
     const int n = n0 + 4 * q;
     TC* cp = C + (long)m * ldc + n;
     float sq = 0.f;
-    if (m_ok) {
+    if (m_ok && 4 * q < ROWS) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         if (n + c < N) {
@@ -305,7 +307,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
   }
 }
 
-template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ>
+template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ, int ROWS = 16>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __restrict__ Av, const bf16_t* __restrict__ W,
                                                               TC* __restrict__ C, int M, int N, int K, long lda,
                                                               long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out,
@@ -319,14 +321,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   const int r = lane & 15, q = lane >> 4;
   int hd, sub;
   bool rotated;
-  const int wr = sk_strip_row<EPI>(strip, r, N, rp, hd, sub, rotated);
+  const int wr = sk_strip_row<EPI, ROWS>(strip, r, N, rp, hd, sub, rotated);
   const bf16_t* wrow = W + (long)wr * ldw + q * 8;
   const bf16_t* urow = wrow + (long)N * ldw;  // up rows (gated only)
   const void* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) xrow[mt] = sk_x_row<XNORM>(Av, lda, min(mt * 16 + r, M - 1), nrm) ;
   if (XNORM) sk_ssq_partials<NW>(sm_ssq, M, nrm);
-  const SkPre pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp);
+  const SkPre pre = sk_preload<MT, EPI, TC, ROWS>(C, M, N, ldc, strip, hd, sub, rotated, rp);
 
   const int steps = (K + 31) / 32;   // k-steps of 32
   f32x4 acc[NG][MT];
@@ -336,11 +338,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
     for (int mt = 0; mt < MT; ++mt) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  for (int s0 = wave; s0 < steps; s0 += NW * UNROLL) {
+  // a wave takes pairs of neighbouring k-steps (the two halves of one 128-byte line of a row of W):
+  // pair wave, wave + NW, ...
+  for (int p0 = wave; 2 * p0 < steps; p0 += NW * (UNROLL / 2)) {
     bf16x8 wf[UNROLL], uf[UNROLL], xf[UNROLL][MT];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int k = (s0 + NW * u) * 32;
+      const int k = (2 * (p0 + NW * (u / 2)) + (u & 1)) * 32;
       const bool ok = k + q * 8 < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
       wf[u] = ok ? *(const bf16x8*)(wrow + k) : zero;
       if (EPI == SK_GATED) uf[u] = ok ? *(const bf16x8*)(urow + k) : zero;
@@ -356,7 +360,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
       }
     }
   }
-  sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp,
+  sk_finish<MT, NW, EPI, TC, XNORM, SSQ, ROWS>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp,
                                          pre);
 }
 
@@ -584,6 +588,7 @@ struct SkCall {
   SkNorm nrm; float* ssq_out; SkRope rp;
   hipStream_t stream;
   bool resident = true;
+  int strip_rows = 16;
 };
 
 // Blocks of the resident kernel: every strip its own block while that still leaves CUs idle, else
@@ -607,6 +612,15 @@ static int launch_skinny(int nw, const SkCall& a) {
     GL3_LAUNCH_CHECK();                                                                                           \
     return 0;                                                                                                     \
   } while (0)
+  if constexpr (MT == 1 && !XNORM && (EPI == SK_STORE || EPI == SK_ADD)) {
+    if (a.strip_rows == 8) {
+      // strips of 8 rows: twice the blocks, each with half the rows to stream
+      gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
+          a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.rp);
+      GL3_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   if (a.resident) {
     // 16 waves a strip where their partial tiles fit, so that a strip's rows are asked for at once
     if constexpr (NG * MT <= 2) {
@@ -672,8 +686,11 @@ static int check_common(const char* who, const void* A, const void* W, const voi
 // partial tiles of that many waves would not fit the block's shared memory).
 // ssq_out (may be null, add epilogue only, N % 16 == 0): [N/16][64] partial sums of squares of the
 // completed rows.
+// strip_rows: 16, or 8 (store and add epilogues, M <= 16): a block takes 8 rows of W, and ssq_out has a
+// row per 8 columns, [ceil(N/8)][64].
 extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
-                               long ldw, long ldc, int epilogue, int waves, float* ssq_out, hipStream_t stream) {
+                               long ldw, long ldc, int epilogue, int waves, float* ssq_out, int strip_rows,
+                               hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny", A, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny: ldc too small");
@@ -681,7 +698,9 @@ extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtyp
   GL3_REQUIRE(epilogue != SK_ADD || c_dtype == GL3_F32, "gl3_gemm_skinny: the add epilogue needs a float output");
   GL3_REQUIRE(!ssq_out || (epilogue == SK_ADD && N % 16 == 0),
               "gl3_gemm_skinny: sums of squares come with the add epilogue and N a multiple of 16");
-  const SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, ssq_out, SkRope{}, stream, waves == 0};
+  GL3_REQUIRE(strip_rows == 16 || (strip_rows == 8 && M <= 16 && epilogue != SK_GATED),
+              "gl3_gemm_skinny: strips of %d rows (M=%d, epilogue %d)", strip_rows, M, epilogue);
+  const SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, ssq_out, SkRope{}, stream, waves == 0, strip_rows};
   const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32) {
     if (epilogue == SK_STORE) return pick_mt<SK_STORE, float, false, false>(nw, a);

@@ -57,7 +57,7 @@ def _declare(lib):
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_argmax": [P, L, P, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
-        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, P],
+        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P],
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P],
         "gl3_qkv_rope_cache": [P, P, I, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
@@ -305,9 +305,16 @@ def gemm_skinny_fits(a, w, out, epilogue):
             and (out.dtype == torch.float32 or (out.dtype == torch.bfloat16 and epilogue != EPI_ADD)))
 
 
-def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None):
+def skinny_strip_rows(M, N, K, epilogue):
+    """Rows of w that a block of the skinny kernel takes: 8 where strips of 16 would leave more than a
+    third of the CUs without a block and K is too long for the kernel that keeps its rows of ``a`` in
+    registers (measured: 17.0 -> 15.8 us at N=2048, K=8192; slower where that kernel applies), else 16."""
+    return 8 if M <= 16 and epilogue != EPI_GATED and -(-N // 16) <= 160 and K > 4096 else 16
+
+
+def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows=16):
     """out (=, +=, gated) a @ w.T on the matrix cores for at most 64 rows of ``a``. ``ssq_out``
-    [N/16, 64] float32 (add epilogue): partial sums of squares of the completed rows."""
+    [N/strip_rows, 64] float32 (add epilogue): partial sums of squares of the completed rows."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
         raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
@@ -318,10 +325,11 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None):
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     if ssq_out is not None:
         _dev(ssq_out, "ssq_out", torch.float32)
-        if epilogue != EPI_ADD or N % 16 or ssq_out.numel() < N // 16 * 64:
-            raise KernelError("gemm_skinny: sums of squares need the add epilogue, N % 16 == 0 and N/16*64 floats")
+        if epilogue != EPI_ADD or N % 16 or ssq_out.numel() < N // strip_rows * 64:
+            raise KernelError("gemm_skinny: sums of squares need the add epilogue, N % 16 == 0 and 64 floats a strip")
     _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
-                                     out.stride(0), epilogue, waves, _ptr(ssq_out), _stream()), "gemm_skinny")
+                                     out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _stream()),
+           "gemm_skinny")
 
 
 def gemm_skinny_wide_fits(a, w, out, epilogue):

@@ -63,7 +63,7 @@ class StepContext:
 
     def ssq_buffer(self, n_partials):
         """[n_partials, 64] partial sums of squares; one buffer, as large as the widest writer needs."""
-        most = max(n_partials, -(-self.engine.spec.hidden // 16))
+        most = max(n_partials, -(-self.engine.spec.hidden // 8))
         return self.buffer("ssq", (most, 64), torch.float32)[:n_partials]
 
     def logits_buffer(self, n_rows, vocab):

@@ -72,9 +72,10 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
             N = out.shape[1]
             if (epilogue == EPI_ADD and ctx is not None and getattr(ctx, "fuse", False) and N % 16 == 0
                     and "fused" not in disabled):
-                ssq = ctx.ssq_buffer(N // 16)
-                K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq)
-                return residual_written(ctx, out, ssq, N // 16)
+                rows = K.skinny_strip_rows(a.shape[0], N, a.shape[1], epilogue)
+                ssq = ctx.ssq_buffer(N // rows)
+                K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq, strip_rows=rows)
+                return residual_written(ctx, out, ssq, N // rows)
             K.gemm_skinny(a, w, out, epilogue)
             if epilogue == EPI_ADD:
                 residual_written(ctx, out)

@@ -388,6 +388,19 @@ def test_gemm_skinny(M, N, Kd):
     x = dev(res)
     lib.gemm_skinny(A, W[:N], x, lib.EPI_ADD)
     np.testing.assert_allclose(x.cpu().numpy(), res + ref, atol=2e-5 * scale * math.sqrt(Kd / 64) + 1e-6)
+    if M <= 16:                                                              # strips of 8 rows of w
+        x8 = dev(res)
+        ssq = torch.full((-(-N // 8), 64), -1.0, device=DEV) if N % 16 == 0 else None
+        lib.gemm_skinny(A, W[:N], x8, lib.EPI_ADD, ssq_out=ssq, strip_rows=8)
+        np.testing.assert_allclose(x8.cpu().numpy(), res + ref, atol=2e-5 * scale * math.sqrt(Kd / 64) + 1e-6)
+        if ssq is not None:
+            want = (x8.cpu().numpy().astype(np.float64) ** 2).reshape(M, N // 8, 8).sum(-1).T
+            np.testing.assert_allclose(ssq[:, :M].cpu().numpy(), want, rtol=1e-5)
+            assert torch.all(ssq[:, M:] == -1)
+        o8 = torch.full((M, N + 2), -1.0, device=DEV)
+        lib.gemm_skinny(A, W[:N], o8[:, :N], lib.EPI_STORE, strip_rows=8)
+        np.testing.assert_allclose(o8[:, :N].cpu().numpy(), ref, atol=2e-5 * scale * math.sqrt(Kd / 64))
+        assert torch.all(o8[:, N:] == -1)
     refg = P.silu(P.linear(a, w[:N])) * P.linear(a, w[N:])
     for waves in (0, 8):
         g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
