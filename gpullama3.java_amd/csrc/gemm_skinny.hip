@@ -97,13 +97,15 @@ __device__ __forceinline__ void sk_load_x(bf16x8 (&xf)[MT], const void* const (&
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
   if (XNORM) {
     const float* gp = (const float*)nrm.weight + k;
-    const f32x4 g0 = ok ? *(const f32x4*)gp : zero4;
-    const f32x4 g1 = ok ? *(const f32x4*)(gp + 4) : zero4;
+    const bool any = ok && xrow[0] != nullptr;   // a lane without a row in the first tile has none at all
+    const f32x4 g0 = any ? *(const f32x4*)gp : zero4;
+    const f32x4 g1 = any ? *(const f32x4*)(gp + 4) : zero4;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const float* xp = (const float*)xrow[mt] + k;
-      const f32x4 x0 = ok ? *(const f32x4*)xp : zero4;
-      const f32x4 x1 = ok ? *(const f32x4*)(xp + 4) : zero4;
+      const bool here = ok && xrow[mt] != nullptr;
+      const f32x4 x0 = here ? *(const f32x4*)xp : zero4;
+      const f32x4 x1 = here ? *(const f32x4*)(xp + 4) : zero4;
       bf16x8 h;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -114,7 +116,8 @@ __device__ __forceinline__ void sk_load_x(bf16x8 (&xf)[MT], const void* const (&
     }
   } else {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) xf[mt] = ok ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
+    for (int mt = 0; mt < MT; ++mt)
+      xf[mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
   }
 }
 
@@ -326,7 +329,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   const bf16_t* urow = wrow + (long)N * ldw;  // up rows (gated only)
   const void* xrow[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xrow[mt] = sk_x_row<XNORM>(Av, lda, min(mt * 16 + r, M - 1), nrm) ;
+  for (int mt = 0; mt < MT; ++mt)   // null for rows that do not exist: their lanes ask for nothing
+    xrow[mt] = mt * 16 + r < M ? sk_x_row<XNORM>(Av, lda, mt * 16 + r, nrm) : nullptr;
   if (XNORM) sk_ssq_partials<NW>(sm_ssq, M, nrm);
   const SkPre pre = sk_preload<MT, EPI, TC, ROWS>(C, M, N, ldc, strip, hd, sub, rotated, rp);
 
@@ -346,7 +350,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
     for (int u = 0; u < UNROLL; ++u) {
       const int k = (2 * (p0 + NW * (u / 2)) + (u & 1)) * 32;
       const bool ok = k + q * 8 < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
-      wf[u] = ok ? *(const bf16x8*)(wrow + k) : zero;
+      wf[u] = (ok && r < ROWS) ? *(const bf16x8*)(wrow + k) : zero;   // rows of the tile beyond the strip stay zero
       if (EPI == SK_GATED) uf[u] = ok ? *(const bf16x8*)(urow + k) : zero;
       sk_load_x<MT, XNORM>(xf[u], xrow, k + q * 8, ok, nrm);
     }
@@ -408,7 +412,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
   {
     const void* xrow[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) xrow[mt] = sk_x_row<XNORM>(Av, lda, min(mt * 16 + r, M - 1), nrm);
+    for (int mt = 0; mt < MT; ++mt)   // null for rows that do not exist: their lanes ask for nothing
+      xrow[mt] = mt * 16 + r < M ? sk_x_row<XNORM>(Av, lda, mt * 16 + r, nrm) : nullptr;
 #pragma unroll
     for (int i = 0; i < KS; ++i) {
       const int k = (wave + NW * i) * 32 + q * 8;
@@ -416,17 +421,20 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
       if (XNORM) {
         const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
         const float* gp = (const float*)nrm.weight + k;
-        gr[i][0] = ok ? *(const f32x4*)gp : zero4;
-        gr[i][1] = ok ? *(const f32x4*)(gp + 4) : zero4;
+        const bool any = ok && xrow[0] != nullptr;   // a lane without a row in the first tile has none at all
+        gr[i][0] = any ? *(const f32x4*)gp : zero4;
+        gr[i][1] = any ? *(const f32x4*)(gp + 4) : zero4;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const float* xp = (const float*)xrow[mt] + k;
-          xr[i][mt][0] = ok ? *(const f32x4*)xp : zero4;
-          xr[i][mt][1] = ok ? *(const f32x4*)(xp + 4) : zero4;
+          const bool here = ok && xrow[mt] != nullptr;
+          xr[i][mt][0] = here ? *(const f32x4*)xp : zero4;
+          xr[i][mt][1] = here ? *(const f32x4*)(xp + 4) : zero4;
         }
       } else {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xf[i][mt] = ok ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
+        for (int mt = 0; mt < MT; ++mt)
+          xf[i][mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
       }
     }
   }
@@ -526,7 +534,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   }
   const bf16_t* xrow[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xrow[mt] = A + (long)min(mt * 16 + r, M - 1) * lda + q * 8;
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = mt * 16 + r < M ? A + (long)(mt * 16 + r) * lda + q * 8 : nullptr;
 
   TC* out = C + (long)blockIdx.y * slice_stride;
   SkPre pre[NS];
@@ -559,7 +567,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
         if (EPI == SK_GATED) uf[u][g] = ok ? *(const bf16x8*)(wrow[g] + (long)N * ldw + k) : zero;
       }
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) xf[u][mt] = ok ? *(const bf16x8*)(xrow[mt] + k) : zero;
+      for (int mt = 0; mt < MT; ++mt) xf[u][mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)(xrow[mt] + k) : zero;
     }
     __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
 #pragma unroll
