@@ -16,12 +16,20 @@
 // digit over the float's bit pattern (four passes with histograms), and the walk to
 // the drawn token is the same search with u * mass in place of top_p. Masses are
 // summed as 64-bit integers (p * 2^62), so the order of a sum cannot move a comparison.
+//
+// At most 2^13 probabilities are 2^-13 or more. They are gathered in shared memory while the row
+// is normalised; when their mass alone exceeds top_p, the threshold and the drawn token lie among
+// them and both searches walk that short list instead of the row: three passes over the row in
+// place of twelve. A flat distribution, whose nucleus reaches further down, takes the passes over
+// the whole row.
 #include "common.h"
 
 #define SB 1024
 #define SW 16          // waves of a block
 #define UN 16          // elements a thread asks for before it uses the first: a pass is bound by trips to memory
 #define QSCALE 4611686018427387904.0   // 2^62: probabilities as 64-bit integers, sums exact and in any order
+#define CAND_MAX 8192  // candidates kept in shared memory: the probabilities of at least CAND_CUT
+#define CAND_CUT 0.0001220703125f      // 2^-13
 
 // A probability (0 <= p <= 1) as an integer: floor(p * 2^62), exact for p >= 2^-38, truncated below;
 // taken from the float's bits: mantissa shifted by its exponent.
@@ -46,7 +54,8 @@ struct Found {
 // share the digits found so far, in private per-wave tables (integer adds in shared memory), and
 // wave 0 walks the 256 bins from the top. If no prefix of the values exceeds thr (thr is not below
 // the total mass), the smallest value is returned.
-__device__ Found radix_search(const float* __restrict__ p, int V, unsigned long long thr,
+template <typename Src>
+__device__ Found radix_search(Src p, int V, unsigned long long thr,
                               unsigned long long (*h_mass)[256], int (*h_cnt)[256], unsigned long long* t_mass,
                               int* t_cnt, unsigned long long* res) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -162,6 +171,10 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
   __shared__ unsigned long long res[2];
   __shared__ unsigned long long w_tot[SW];
   __shared__ int winner;
+  __shared__ float cand_p[CAND_MAX];
+  __shared__ int cand_i[CAND_MAX];
+  __shared__ int n_cand;
+  __shared__ unsigned long long cand_mass;
   const int row = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const float* lg = logits + (long)row * ld;
   const float T = temperature[row];
@@ -220,17 +233,32 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
     }
   }
   const float zf = (float)block_sum_f64(z, ds);
+  const float tp = top_p[row];
+  const bool nucleus = tp > 0.f && tp < 1.f;
+  if (tid == 0) { n_cand = 0; cand_mass = 0ull; }
+  __syncthreads();
+  unsigned long long my_mass = 0;
   for (int i0 = tid; i0 < V; i0 += UN * SB) {
     float v[UN];
 #pragma unroll
     for (int u = 0; u < UN; ++u) v[u] = (i0 + u * SB < V) ? p[i0 + u * SB] : 0.f;
 #pragma unroll
-    for (int u = 0; u < UN; ++u)
-      if (i0 + u * SB < V) p[i0 + u * SB] = v[u] / zf;
+    for (int u = 0; u < UN; ++u) {
+      const int i = i0 + u * SB;
+      if (i < V) {
+        const float pv = v[u] / zf;
+        p[i] = pv;
+        if (nucleus && pv >= CAND_CUT) {
+          const int slot = atomicAdd(&n_cand, 1);
+          if (slot < CAND_MAX) { cand_p[slot] = pv; cand_i[slot] = i; }
+          my_mass += to_q(pv);
+        }
+      }
+    }
   }
+  if (nucleus && my_mass) atomicAdd(&cand_mass, my_mass);   // integers: the order does not matter
   __syncthreads();
 
-  const float tp = top_p[row];
   // in a run of steps replayed from a graph the step's number is read from memory
   const double u = (double)uniform[(step ? (long)step[0] * uniform_stride : 0) + row];
   // every wave owns a contiguous range of the row, a multiple of 64 long
@@ -282,6 +310,34 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
 
   // nucleus: the threshold value, the mass above it, and how many of the equal ones are kept
   const unsigned long long tq = (unsigned long long)((double)tp * QSCALE);
+  if (n_cand <= CAND_MAX && cand_mass > tq) {
+    // the candidates alone exceed top_p: every probability from the threshold upwards is among them
+    const int n = n_cand;
+    const Found f1 = radix_search(cand_p, n, tq, h_mass, h_cnt, t_mass, t_cnt, res);
+    long k1 = 1;
+    if (f1.each > 0 && tq >= f1.above) k1 = (long)((tq - f1.above) / f1.each) + 1;
+    if (k1 > f1.ties) k1 = f1.ties;
+    if (k1 < 1) k1 = 1;
+    const unsigned long long mass = f1.above + (unsigned long long)k1 * f1.each;
+    const unsigned long long target = (unsigned long long)(u * (double)mass);
+    const Found f2 = radix_search(cand_p, n, target, h_mass, h_cnt, t_mass, t_cnt, res);
+    long j = (f2.each > 0 && target >= f2.above) ? (long)((target - f2.above) / f2.each) : 0;
+    const long limit = (f2.bits == f1.bits) ? k1 : (long)f2.ties;
+    if (j > limit - 1) j = limit - 1;
+    if (j < 0) j = 0;
+    const float want = __uint_as_float(f2.bits);
+    // the candidate with this probability that has exactly j equal ones of smaller index before it
+    for (int a = tid; a < n; a += SB) {
+      if (cand_p[a] != want) continue;
+      const int ia = cand_i[a];
+      long rank = 0;
+      for (int b = 0; b < n; ++b) rank += (cand_p[b] == want && cand_i[b] < ia) ? 1 : 0;
+      if (rank == j) winner = ia;
+    }
+    __syncthreads();
+    if (tid == 0) out[row] = winner >= 0 ? winner : V - 1;
+    return;
+  }
   const Found f1 = radix_search(p, V, tq, h_mass, h_cnt, t_mass, t_cnt, res);
   long k1 = 1;
   if (f1.each > 0 && tq >= f1.above) k1 = (long)((tq - f1.above) / f1.each) + 1;   // smallest k with above + k*each > tq

@@ -341,6 +341,44 @@ def test_sample_kernel(V):
     assert out[3].item() == 0 if temps[3] == 0 else True
 
 
+def test_sample_kernel_nucleus_from_the_short_list_and_from_the_whole_row():
+    """A peaked row's nucleus lies among the few probabilities of 2^-13 or more, which the kernel
+    gathers; a flat row's does not. Both must give the twin's token, with equal probabilities spread
+    over the row, at the list's capacity and just beyond it."""
+    rng = np.random.default_rng(8)
+    V = 128256
+    rows, temps, tops = [], [], []
+    peaked = (rng.standard_normal(V) * 3).astype(np.float32)
+    hot = rng.choice(V, 9, replace=False)
+    peaked[hot] = peaked.max() + 2.0                                       # nine equal ones on top, anywhere in the row
+    for tp in (0.3, 0.9, 0.999):
+        rows.append(peaked); temps.append(0.5); tops.append(tp)
+    flat = (rng.standard_normal(V) * 0.5).astype(np.float32)               # no probability reaches 2^-13
+    rows.append(flat); temps.append(1.0); tops.append(0.9)
+    for n_equal in (8192, 8193, 100):                                       # the list full, one more than it holds, few
+        r = np.full(V, -np.inf, np.float32)
+        r[rng.choice(V, n_equal, replace=False)] = 1.5
+        rows.append(r); temps.append(1.0); tops.append(0.7)
+    mixed = flat.copy()
+    mixed[hot] += 9.0                                                       # most of the mass in nine, a long flat tail
+    for tp in (0.5, 0.99):
+        rows.append(mixed); temps.append(1.0); tops.append(tp)
+    logits = np.stack(rows)
+    R = len(rows)
+    lib = K()
+    for trial in range(6):
+        us = rng.random(R).astype(np.float32)
+        if trial == 0:
+            us[:] = 0.0
+        if trial == 1:
+            us[:] = np.float32(0.99999994)
+        out = torch.empty(R, dtype=torch.int32, device=DEV)
+        lib.sample(dev(logits), torch.empty(R * V, device=DEV), dev(np.array(temps, np.float32)),
+                   dev(np.array(tops, np.float32)), dev(us), out)
+        for r, tok in enumerate(out.tolist()):
+            check_draw(logits[r], temps[r], tops[r], float(us[r]), tok)
+
+
 def test_sample_kernel_frequencies_and_rules():
     rng = np.random.default_rng(5)
     V, R = 12, 4000
