@@ -14,9 +14,9 @@ from safetensors.torch import load_file
 
 import gpullama3_java_amd as g
 import plain_llama as P
-from tiny import TINY_A, TINY_B, TINY_C
+from tiny import TINY_A, TINY_B, TINY_C, TINY_D
 
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 DTYPES = ["float32", "bfloat16"]
 
 # Largest allowed |engine - plain| as a fraction of the largest |plain| logit of the

@@ -7,7 +7,7 @@ from gpu_helpers import CONFIGS, DTYPES, close, first_bad_row, model, plain_logi
 
 pytestmark = pytest.mark.gpu
 
-CASES = [(n, d) for n in ("A", "B", "C") for d in DTYPES]
+CASES = [(n, d) for n in ("A", "B", "C", "D") for d in DTYPES]
 
 
 def engine(name, dtype, **kw):
@@ -18,7 +18,7 @@ def engine(name, dtype, **kw):
 
 
 def lengths(name):
-    return {"A": [5, 11, 64, 100], "B": [3, 17, 40, 129, 200], "C": [1, 63, 65, 300]}[name]
+    return {"A": [5, 11, 64, 100], "B": [3, 17, 40, 129, 200], "C": [1, 63, 65, 300], "D": [2, 33, 70, 257]}[name]
 
 
 @pytest.mark.parametrize("name, dtype", CASES)
@@ -91,9 +91,10 @@ def test_unequal_batches_one_after_another_reuse_slots(name, dtype):
     assert eng.cache.slots.live == set()
 
 
-@pytest.mark.parametrize("name, dtype", [("B", "float32"), ("B", "bfloat16"), ("C", "float32"), ("C", "bfloat16")])
+@pytest.mark.parametrize("name, dtype", [("B", "float32"), ("B", "bfloat16"), ("C", "float32"), ("C", "bfloat16"),
+                                         ("D", "bfloat16")])
 def test_long_decoding(name, dtype):
-    n = {"B": 250, "C": 400}[name]
+    n = {"B": 250, "C": 400, "D": 330}[name]
     toks = rand_tokens(name, 77, n)
     ref = plain_logits(name, toks)
     eng = engine(name, dtype)
@@ -141,7 +142,8 @@ def test_batch_mates_order_and_slot_change_nothing(dtype):
     close(mixed, plain_logits(name, a), dtype)
 
 
-@pytest.mark.parametrize("name, dtype", [("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+@pytest.mark.parametrize("name, dtype", [("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16"),
+                                         ("D", "bfloat16")])
 @pytest.mark.parametrize("graphs", [False, True])
 def test_decode_steps_of_33_to_64_sequences(name, dtype, graphs):
     """Between 33 and 64 tokens a step the products into the residual stream leave their sums in
@@ -234,7 +236,7 @@ def test_no_gpu_library_no_engine(monkeypatch):
                     torch.zeros(1, 8, device="cuda"), 1e-5)
 
 
-@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+@pytest.mark.parametrize("name, dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "bfloat16"), ("D", "bfloat16")])
 def test_replayed_graphs_equal_plain_launches(name, dtype):
     """Decode steps replayed from captured graphs, with the batch padded to its bucket and other
     work of the same engine between the replays, give what the same kernels give when launched

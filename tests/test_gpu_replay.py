@@ -42,7 +42,7 @@ class Replay:
         assert self.p.wait(timeout=60) == 0
 
 
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "D"])
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_replay_cuts(name, dtype, tmp_path):
     folder, cfgd, _ = model(name)

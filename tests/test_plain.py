@@ -12,7 +12,7 @@ import pytest
 import torch
 
 import plain_llama as P
-from tiny import TINY_A, TINY_B, TINY_C, dims, make_weights, tokens
+from tiny import TINY_A, TINY_B, TINY_C, TINY_D, dims, make_weights, tokens
 
 
 # ------------------------------------------------------------------ rmsnorm
@@ -193,7 +193,7 @@ def test_silu_glu():
 
 
 # ------------------------------------------------------------------ whole model
-@pytest.mark.parametrize("cfg", [TINY_A, TINY_B, TINY_C], ids=["A", "B", "C"])
+@pytest.mark.parametrize("cfg", [TINY_A, TINY_B, TINY_C, TINY_D], ids=["A", "B", "C", "D"])
 def test_zero_output_projections_leave_the_embedding(cfg):
     W = make_weights(cfg, 7, norm_std=0.1)
     for i in range(cfg["num_hidden_layers"]):

@@ -49,6 +49,32 @@ TINY_B = {
     "hidden_act": "silu",
 }
 
+# The head size and grouping of the shape that bench.py measures (head_dim 64, four query heads to
+# a kv head), so that the kernels built for it are also checked inside a whole model; tied head,
+# a width and a vocabulary that no tile divides.
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"],
+    "hidden_size": 136,
+    "intermediate_size": 264,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 8,
+    "num_key_value_heads": 2,
+    "head_dim": 64,
+    "vocab_size": 515,
+    "max_position_embeddings": 512,
+    "rms_norm_eps": 2e-5,
+    "rope_theta": 500000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 32.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 4.0,
+        "original_max_position_embeddings": 128,
+    },
+    "tie_word_embeddings": True,
+    "hidden_act": "silu",
+}
+
 # Sizes that are no power of two anywhere: head_dim 48 with heads*head_dim != hidden,
 # as many kv heads as heads, a vocabulary that no tile divides, a longer context.
 TINY_C = {
