@@ -78,6 +78,7 @@ class DecoderModel:
     def forward(self, ctx, want_rows):
         """Logits ``[len(want_rows), vocab]`` float32 at the wanted packed rows."""
         x = ctx.buffer("residual", (ctx.n_tokens, self.spec.hidden), torch.float32)
+        ctx.ssq = ctx.pending = None       # a context may run more than one forward pass: nothing is left over
         if getattr(ctx, "fuse", False) and ctx.n_tokens <= ops.FUSE_ROWS:
             ssq = ctx.ssq_buffer(1)                      # the first norm's sums of squares come with the rows
             K.embed(self.embedding, ctx.token_ids, x, ssq)

@@ -145,9 +145,19 @@ def test_batch_mates_order_and_slot_change_nothing(dtype):
 @pytest.mark.parametrize("name, dtype", [("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16"),
                                          ("D", "bfloat16")])
 @pytest.mark.parametrize("graphs", [False, True])
-def test_decode_steps_of_33_to_64_sequences(name, dtype, graphs):
+def test_decode_steps_of_33_to_64_sequences(name, dtype, graphs, monkeypatch):
     """Between 33 and 64 tokens a step the products into the residual stream leave their sums in
-    slices of K that the next norm adds up, and rotation and cache write ride on the QKV product."""
+    slices of K that the next norm adds up, and rotation and cache write ride on the QKV product.
+    The tiny models' K is too short for the rule that cuts it, so the rule is replaced by one that
+    always cuts."""
+    from gpullama3_java_amd.csrc import lib
+    cut = []
+
+    def always(N, Kd):
+        n = 3 if Kd >= 192 else 2 if Kd >= 64 else 1
+        cut.append(n)
+        return n
+    monkeypatch.setattr(lib, "wide_slices", always)
     B = 41
     eng = engine(name, dtype, n_slots=64, max_tokens=64 * 64, use_graphs=graphs)
     seqs = [rand_tokens(name, 200 + i, 2 + i % 5 + 6) for i in range(B)]
@@ -158,6 +168,7 @@ def test_decode_steps_of_33_to_64_sequences(name, dtype, graphs):
         o = eng.step([(s, [q[2 + i % 5 + k]]) for i, (s, q) in enumerate(zip(slots, seqs))]).cpu().numpy()
         for i in range(B):
             rows[i].append(o[i])
+    assert dtype == "float32" or max(cut) > 1
     for i in range(B):
         n0 = 2 + i % 5
         close(np.stack(rows[i]), plain_logits(name, seqs[i])[n0 - 1:n0 + 5], dtype, f"request {i}")
