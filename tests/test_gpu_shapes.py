@@ -1,0 +1,77 @@
+"""The bfloat16 engine against the float32 engine at the layer sizes of real models.
+
+The tiny configurations of the other tests are too small for several choices that the
+product path makes by size: products of a prompt cut into slices of K, tiles of 256 x 256,
+strips of 8 rows, the kernels for 33 to 64 rows with their slices, the tiled kernel for the
+head. Here the layers have the sizes of Llama-3.2-1B (what bench.py measures) and of Llama-3.1-8B
+(two layers each, to keep the test short),
+and every kind of step is run on both engines with the same weights. The float32 engine is
+the reference: it uses one size-generic kernel per operation, and the other tests compare it
+with the plain implementation."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_helpers import TOL
+
+pytestmark = pytest.mark.gpu
+
+COMMON = {"architectures": ["LlamaForCausalLM"], "num_hidden_layers": 2, "vocab_size": 128256,
+          "max_position_embeddings": 4096, "rms_norm_eps": 1e-5, "rope_theta": 500000.0, "hidden_act": "silu"}
+SHAPES = {
+    # the layers of Llama-3.2-1B: head size 64, tied head
+    "1B": {**COMMON, "hidden_size": 2048, "intermediate_size": 8192, "num_attention_heads": 32, "num_key_value_heads": 8,
+           "head_dim": 64, "tie_word_embeddings": True,
+           "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                            "original_max_position_embeddings": 8192}},
+    # the layers of Llama-3.1-8B: head size 128, longer rows, a head of its own
+    "8B": {**COMMON, "hidden_size": 4096, "intermediate_size": 14336, "num_attention_heads": 32, "num_key_value_heads": 8,
+           "head_dim": 128, "tie_word_embeddings": False,
+           "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                            "original_max_position_embeddings": 8192}},
+}
+
+
+def steps(eng, vocab):
+    """Logits of every kind of step: a long prompt, single tokens after it, batches of 8, 20 and 40
+    sequences (short prompts, then decode steps that are replayed from graphs), prompts of 50."""
+    rng = np.random.default_rng(0)
+    out = []
+    s = eng.take_slot()
+    toks = rng.integers(0, vocab, 603).tolist()
+    out.append(eng.step([(s, toks[:600])]).cpu().numpy())
+    for t in toks[600:]:
+        out.append(eng.step([(s, [t])]).cpu().numpy())
+    eng.give_back_slot(s)
+    for B in (8, 20, 40):
+        slots = [eng.take_slot() for _ in range(B)]
+        seqs = [rng.integers(0, vocab, 7).tolist() for _ in range(B)]
+        out.append(eng.step([(sl, q[:4]) for sl, q in zip(slots, seqs)]).cpu().numpy())
+        for k in (4, 5, 6):
+            out.append(eng.step([(sl, [q[k]]) for sl, q in zip(slots, seqs)]).cpu().numpy())
+        for sl in slots:
+            eng.give_back_slot(sl)
+    five = [eng.take_slot() for _ in range(5)]
+    out.append(eng.step([(sl, rng.integers(0, vocab, 50).tolist()) for sl in five]).cpu().numpy())
+    return out
+
+
+@pytest.mark.parametrize("shape", ["1B", "8B"])
+def test_real_layer_sizes_bfloat16_against_float32(tmp_path, shape):
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.engine import Engine
+    cfg = g.config_from_dict(SHAPES[shape])
+    folder = str(tmp_path / "shape")
+    g.write_random_model(folder, cfg, 11, std=0.02, norm_std=0.1)
+    results = {}
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine.from_folder(folder, dtype=dtype, max_context=1024, max_tokens=4096, n_slots=48)
+        results[dtype] = steps(eng, cfg.vocab_size)
+        if dtype == "bfloat16":
+            assert eng._graphs, "the decode steps were not replayed from graphs"
+        del eng
+        torch.cuda.empty_cache()
+    for i, (ref, got) in enumerate(zip(results["float32"], results["bfloat16"])):
+        scale = float(np.abs(ref).max())
+        err = float(np.abs(ref - got).max())
+        assert err <= TOL["bfloat16"] * scale, f"step {i} ({ref.shape[0]} rows): {err / scale:.4f} of the logit scale"
