@@ -34,7 +34,8 @@ SHAPES = {
 
 def steps(eng, vocab):
     """Logits of every kind of step: a long prompt, single tokens after it, batches of 8, 20 and 40
-    sequences (short prompts, then decode steps that are replayed from graphs), prompts of 50."""
+    sequences (short prompts, then decode steps that are replayed from graphs), prompts of 50, a prompt
+    of 2,600 tokens and single tokens after it."""
     rng = np.random.default_rng(0)
     out = []
     s = eng.take_slot()
@@ -53,6 +54,14 @@ def steps(eng, vocab):
             eng.give_back_slot(sl)
     five = [eng.take_slot() for _ in range(5)]
     out.append(eng.step([(sl, rng.integers(0, vocab, 50).tolist()) for sl in five]).cpu().numpy())
+    for sl in five:
+        eng.give_back_slot(sl)
+    # a long prompt (the largest tiles), then tokens whose attention is split over the keys
+    s = eng.take_slot()
+    toks = rng.integers(0, vocab, 2603).tolist()
+    out.append(eng.step([(s, toks[:2600])]).cpu().numpy())
+    for t in toks[2600:]:
+        out.append(eng.step([(s, [t])]).cpu().numpy())
     return out
 
 
@@ -65,7 +74,7 @@ def test_real_layer_sizes_bfloat16_against_float32(tmp_path, shape):
     g.write_random_model(folder, cfg, 11, std=0.02, norm_std=0.1)
     results = {}
     for dtype in ("float32", "bfloat16"):
-        eng = Engine.from_folder(folder, dtype=dtype, max_context=1024, max_tokens=4096, n_slots=48)
+        eng = Engine.from_folder(folder, dtype=dtype, max_context=4096, max_tokens=4096, n_slots=48)
         results[dtype] = steps(eng, cfg.vocab_size)
         if dtype == "bfloat16":
             assert eng._graphs, "the decode steps were not replayed from graphs"
@@ -75,3 +84,31 @@ def test_real_layer_sizes_bfloat16_against_float32(tmp_path, shape):
         scale = float(np.abs(ref).max())
         err = float(np.abs(ref - got).max())
         assert err <= TOL["bfloat16"] * scale, f"step {i} ({ref.shape[0]} rows): {err / scale:.4f} of the logit scale"
+
+
+def test_runs_of_decode_steps_at_real_layer_sizes_pick_the_tokens_of_single_steps(tmp_path):
+    """Generation runs several decode steps on the device with one wait at the end; the tokens must
+    be those that single steps with a host-side argmax give, for 40 sequences (the kernels for 33 to
+    64 rows) and for 3."""
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.engine import Engine
+    cfg = g.config_from_dict(SHAPES["1B"])
+    folder = str(tmp_path / "shape")
+    g.write_random_model(folder, cfg, 12, std=0.02, norm_std=0.1)
+    eng = Engine.from_folder(folder, dtype="bfloat16", max_context=256, max_tokens=64 * 64, n_slots=64)
+    rng = np.random.default_rng(1)
+    for B in (40, 3):
+        prompts = [rng.integers(0, cfg.vocab_size, 3 + i % 4).tolist() for i in range(B)]
+        res = eng.generate(prompts, max_new_tokens=21, temperature=0.0, stop_ids=())
+        slots = [eng.take_slot() for _ in range(B)]
+        logits = eng.step(list(zip(slots, prompts)))
+        want = [[] for _ in range(B)]
+        for _ in range(21):
+            toks = logits.argmax(-1).tolist()
+            for i, t in enumerate(toks):
+                want[i].append(t)
+            logits = eng.step([(sl, [t]) for sl, t in zip(slots, toks)])
+        for sl in slots:
+            eng.give_back_slot(sl)
+        for i in range(B):
+            assert res[i].tokens == want[i], f"batch {B}, request {i}"
