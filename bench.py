@@ -23,7 +23,7 @@ sys.path.insert(0, ROOT)
 HBM_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 
-# BASELINE.json configs[2]: the Llama-3.2-1B shape
+# the Llama-3.2-1B shape: every size as the model's own config.json gives it
 SHAPE = {
     "architectures": ["LlamaForCausalLM"], "hidden_size": 2048, "intermediate_size": 8192,
     "num_hidden_layers": 16, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
