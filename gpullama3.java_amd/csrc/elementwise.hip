@@ -5,10 +5,11 @@
 // ----------------------------------------------------------------- embedding
 // out[t, :] = table[ids[t], :] as float (J/inference/InferenceCore.java:69).
 // ssq (may be null; then n_tokens <= 64): ssq[t] = sum of squares of row t, for a norm that is
-// folded into the product that follows.
+// folded into the product that follows; with it next_weight [d] (float) and xg [n_tokens][d]
+// (may be null): xg = bfloat16(next_weight * row), the rows as that product reads them.
 template <typename TW>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out, int d,
-                             float* __restrict__ ssq) {
+                             float* __restrict__ ssq, const float* __restrict__ next_weight, bf16_t* __restrict__ xg) {
   __shared__ float scratch[16];
   const long t = blockIdx.x;
   const TW* row = table + (long)ids[t] * d;
@@ -18,6 +19,7 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
     const float v = to_f32<TW>(row[i]);
     o[i] = v;
     ss += v * v;
+    if (xg) xg[t * d + i] = static_cast<bf16_t>(next_weight[i] * v);
   }
   if (ssq) {
     ss = block_sum(ss, scratch);
@@ -26,13 +28,17 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
 }
 
 extern "C" int gl3_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens, int d,
-                         float* ssq, hipStream_t stream) {
+                         float* ssq, const float* next_weight, void* xg, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(table && ids && out && n_tokens > 0 && d > 0, "gl3_embed: bad arguments (T=%d d=%d)", n_tokens, d);
   GL3_REQUIRE(!ssq || n_tokens <= 64, "gl3_embed: sums of squares are kept for at most 64 rows");
+  GL3_REQUIRE((next_weight == nullptr) == (xg == nullptr) && (!xg || ssq),
+              "gl3_embed: the next norm's weight and its rows come together, with the sums of squares");
   dim3 grid(n_tokens), block(256);
-  if (table_dtype == GL3_F32) embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, ids, out, d, ssq);
-  else if (table_dtype == GL3_BF16) embed_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)table, ids, out, d, ssq);
+  if (table_dtype == GL3_F32)
+    embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, ids, out, d, ssq, next_weight, (bf16_t*)xg);
+  else if (table_dtype == GL3_BF16)
+    embed_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)table, ids, out, d, ssq, next_weight, (bf16_t*)xg);
   else GL3_REQUIRE(false, "gl3_embed: unknown dtype %d", table_dtype);
   GL3_LAUNCH_CHECK();
   return 0;

@@ -14,14 +14,13 @@
 // A decode step is a chain of small kernels, each of which costs a few microseconds
 // before it does any work, so what would be kernels of their own is folded into the
 // products' ends:
-//  * XNORM: A is the float residual stream and the product is that of its RMSNorm
-//    (J/inference/InferenceCore.java:47-56): a lane multiplies x by the norm's weight as
-//    it loads it, and the row's 1/rms, which is a factor of the whole row, is applied to
-//    the sums at the end. The sum of squares of a row arrives as partial sums (one per
-//    16 columns of the row, written by the kernel that produced the row), added up here
-//    in a fixed order.
-//  * SSQ: the add epilogue also writes those partial sums of squares of the rows it
-//    completes, for the norm that follows.
+//  * XNORM: the product is that of an RMSNorm (J/inference/InferenceCore.java:47-56). Its rows
+//    arrive as bfloat16(weight * x), written by the kernel that completed the row of x (below),
+//    and the row's 1/rms, which is a factor of the whole row, is applied to the sums at the end.
+//    The sum of squares of a row arrives as partial sums (one per strip of the row's producer),
+//    added up here in a fixed order.
+//  * SSQ: the add epilogue also writes those partial sums of squares of the rows it completes,
+//    and bfloat16(next norm's weight * x) of its columns, for the product that follows the norm.
 //  * SK_QKV: the rows of W are [q heads | k heads | v heads]; the end rotates q and k by
 //    the token's position and writes q to its buffer, k and v into the paged cache
 //    (J/inference/InferenceCore.java:83-101). For half-split pairing a strip is made of 8
@@ -43,11 +42,17 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 enum { SK_STORE = 0, SK_ADD = 1, SK_GATED = 2, SK_QKV = 3 };
 
 struct SkNorm {
-  const float* weight;    // [K] norm weight, float
-  const float* ssq;       // [n_partials][64] partial sums of squares of the rows of A
+  const float* ssq;       // [n_partials][64] partial sums of squares of the rows of x
   int n_partials;
   float eps;
   const int* rows;        // may be null: row m of the product reads row rows[m] of A
+};
+
+// For the norm that follows an add epilogue: its weight, and where bfloat16(weight * x) goes.
+struct SkNext {
+  const float* weight;    // [N] float; null: nothing is written
+  bf16_t* xg;             // [M][ld]
+  long ld;
 };
 
 struct SkRope {
@@ -82,10 +87,7 @@ __device__ __forceinline__ int sk_strip_row(int strip, int r, int N, const SkRop
 
 template <bool XNORM>
 __device__ __forceinline__ const void* sk_x_row(const void* Av, long lda, int m, const SkNorm& nrm) {
-  if (XNORM) {
-    if (nrm.rows) m = nrm.rows[m];
-    return (const float*)Av + (long)m * lda;
-  }
+  if (XNORM && nrm.rows) m = nrm.rows[m];
   return (const bf16_t*)Av + (long)m * lda;
 }
 
@@ -94,31 +96,9 @@ template <int MT, bool XNORM>
 __device__ __forceinline__ void sk_load_x(bf16x8 (&xf)[MT], const void* const (&xrow)[MT], int k, bool ok,
                                           const SkNorm& nrm) {
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-  if (XNORM) {
-    const float* gp = (const float*)nrm.weight + k;
-    const bool any = ok && xrow[0] != nullptr;   // a lane without a row in the first tile has none at all
-    const f32x4 g0 = any ? *(const f32x4*)gp : zero4;
-    const f32x4 g1 = any ? *(const f32x4*)(gp + 4) : zero4;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const float* xp = (const float*)xrow[mt] + k;
-      const bool here = ok && xrow[mt] != nullptr;
-      const f32x4 x0 = here ? *(const f32x4*)xp : zero4;
-      const f32x4 x1 = here ? *(const f32x4*)(xp + 4) : zero4;
-      bf16x8 h;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        h[e] = static_cast<bf16_t>(g0[e] * x0[e]);
-        h[4 + e] = static_cast<bf16_t>(g1[e] * x1[e]);
-      }
-      xf[mt] = h;
-    }
-  } else {
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-      xf[mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
-  }
+  for (int mt = 0; mt < MT; ++mt)
+    xf[mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
 }
 
 // Partial sums of squares of the rows: wave w adds the partials w, w+NW, ... of row `lane`.
@@ -148,6 +128,7 @@ __device__ __forceinline__ void sk_ssq_partials(float (*sm_ssq)[64], int M, cons
 // token tile `mt`; a lane holds 4 columns of one token.
 struct SkPre {
   f32x4 prev;
+  f32x4 next_w;     // the next norm's weight at this lane's columns
   f32x4 co, si;
   int pos;
   int page;
@@ -155,9 +136,9 @@ struct SkPre {
 
 template <int MT, int EPI, typename TC, int ROWS = 16>
 __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int N, long ldc, int strip, int hd, int sub,
-                                            bool rotated, const SkRope& rp) {
+                                            bool rotated, const SkRope& rp, const SkNext& nx = SkNext{}) {
   SkPre p;
-  p.prev = p.co = p.si = f32x4{0.f, 0.f, 0.f, 0.f};
+  p.prev = p.next_w = p.co = p.si = f32x4{0.f, 0.f, 0.f, 0.f};
   p.pos = 0; p.page = 0;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
@@ -168,7 +149,10 @@ __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int
     const TC* cp = C + (long)m * ldc + n;
 #pragma unroll
     for (int c = 0; c < 4; ++c)
-      if (n + c < N) p.prev[c] = to_f32<TC>(cp[c]);
+      if (n + c < N) {
+        p.prev[c] = to_f32<TC>(cp[c]);
+        if (nx.weight) p.next_w[c] = nx.weight[n + c];
+      }
   }
   if (EPI == SK_QKV) {
     p.pos = rp.positions[m];
@@ -199,7 +183,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
                                           const f32x4 (&acc)[(EPI == SK_GATED) ? 2 : 1][MT], int strip, int hd, int sub,
                                           bool rotated, TC* __restrict__ C, int M, int N, int K, long ldc,
                                           const SkNorm& nrm, float* __restrict__ ssq_out, const SkRope& rp,
-                                          const SkPre& pre) {
+                                          const SkNext& nx, const SkPre& pre) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
@@ -299,6 +283,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
           if (EPI == SK_ADD) o += pre.prev[c];
           cp[c] = from_f32<TC>(o);
           sq += o * o;
+          if (SSQ && nx.weight) nx.xg[(long)m * nx.ld + n + c] = static_cast<bf16_t>(pre.next_w[c] * o);
         }
       }
     }
@@ -314,9 +299,9 @@ template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ, int ROWS =
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __restrict__ Av, const bf16_t* __restrict__ W,
                                                               TC* __restrict__ C, int M, int N, int K, long lda,
                                                               long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out,
-                                                              SkRope rp) {
+                                                              SkNext nx, SkRope rp) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
-  constexpr int UNROLL = XNORM ? 4 : 8;
+  constexpr int UNROLL = 8;
   __shared__ f32x4 red[NW][NG * MT][64];
   __shared__ float sm_ssq[XNORM ? NW : 1][64];
   const int strip = blockIdx.x;
@@ -332,7 +317,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   for (int mt = 0; mt < MT; ++mt)   // null for rows that do not exist: their lanes ask for nothing
     xrow[mt] = mt * 16 + r < M ? sk_x_row<XNORM>(Av, lda, mt * 16 + r, nrm) : nullptr;
   if (XNORM) sk_ssq_partials<NW>(sm_ssq, M, nrm);
-  const SkPre pre = sk_preload<MT, EPI, TC, ROWS>(C, M, N, ldc, strip, hd, sub, rotated, rp);
+  const SkPre pre = sk_preload<MT, EPI, TC, ROWS>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx);
 
   const int steps = (K + 31) / 32;   // k-steps of 32
   f32x4 acc[NG][MT];
@@ -365,14 +350,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
     }
   }
   sk_finish<MT, NW, EPI, TC, XNORM, SSQ, ROWS>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp,
-                                         pre);
+                                               nx, pre);
 }
 
 // The resident kernel: K <= 32 * NW * KS. `n_strips` strips are shared out over the blocks.
 template <int MT, int NW, int KS, int EPI, typename TC, bool XNORM, bool SSQ>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
     const void* __restrict__ Av, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N, int K, long lda,
-    long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out, SkRope rp, int n_strips) {
+    long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out, SkNext nx, SkRope rp, int n_strips) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   __shared__ f32x4 red[NW][NG * MT][64];
   __shared__ float sm_ssq[XNORM ? NW : 1][64];
@@ -408,7 +393,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
     }
   }
   bf16x8 xf[KS][MT];
-  f32x4 xr[XNORM ? KS : 1][MT][2], gr[XNORM ? KS : 1][2];
   {
     const void* xrow[MT];
 #pragma unroll
@@ -418,47 +402,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
     for (int i = 0; i < KS; ++i) {
       const int k = (wave + NW * i) * 32 + q * 8;
       const bool ok = k < K;
-      if (XNORM) {
-        const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-        const float* gp = (const float*)nrm.weight + k;
-        const bool any = ok && xrow[0] != nullptr;   // a lane without a row in the first tile has none at all
-        gr[i][0] = any ? *(const f32x4*)gp : zero4;
-        gr[i][1] = any ? *(const f32x4*)(gp + 4) : zero4;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const float* xp = (const float*)xrow[mt] + k;
-          const bool here = ok && xrow[mt] != nullptr;
-          xr[i][mt][0] = here ? *(const f32x4*)xp : zero4;
-          xr[i][mt][1] = here ? *(const f32x4*)(xp + 4) : zero4;
-        }
-      } else {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          xf[i][mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
-      }
+      for (int mt = 0; mt < MT; ++mt)
+        xf[i][mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
     }
   }
-  __builtin_amdgcn_sched_barrier(0);
-  if (XNORM) {
-    float sp = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) sp += sq[i];
-    if (lane < M)
-      for (int p = wave + NW * 16; p < nrm.n_partials; p += NW) sp += nrm.ssq[(long)p * 64 + sq_row];
-    sm_ssq[wave][lane] = sp;
-#pragma unroll
-    for (int i = 0; i < KS; ++i)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        bf16x8 h;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          h[e] = static_cast<bf16_t>(gr[i][0][e] * xr[i][mt][0][e]);
-          h[4 + e] = static_cast<bf16_t>(gr[i][1][e] * xr[i][mt][1][e]);
-        }
-        xf[i][mt] = h;
-      }
-  }
+  bool first_strip = true;
   while (strip < n_strips) {
     // ask for the next strip's rows before this strip's are used
     const int next = strip + gridDim.x;
@@ -476,7 +425,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
         if (EPI == SK_GATED) un[i] = ok ? *(const bf16x8*)(wrow + (long)N * ldw + k) : zero;
       }
     }
-    const SkPre pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp);
+    const SkPre pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx);
     __builtin_amdgcn_sched_barrier(0);   // the next strip's loads are on their way before this strip's are used
     f32x4 acc[NG][MT];
 #pragma unroll
@@ -491,8 +440,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
         if (EPI == SK_GATED) acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[i], xf[i][mt], acc[1][mt], 0, 0, 0);
       }
     }
+    if (XNORM && first_strip) {
+      // (waited for only now: the second strip's rows of W were asked for in the same trip)
+      float sp = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sp += sq[i];
+      if (lane < M)
+        for (int p = wave + NW * 16; p < nrm.n_partials; p += NW) sp += nrm.ssq[(long)p * 64 + sq_row];
+      sm_ssq[wave][lane] = sp;
+      first_strip = false;
+    }
     sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp,
-                                           pre);
+                                           nx, pre);
     if (next >= n_strips) break;
     __syncthreads();   // the partial tiles in shared memory are free again
 #pragma unroll
@@ -586,7 +545,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
     if (g) __syncthreads();   // the partial tiles in shared memory are free again
     if (strip0 + g < n_strips)   // the same for all threads of the block
       sk_finish<MT, NW, EPI, TC, false, false>(red, sm_ssq, acc[g], strip0 + g, hd[g], sub[g], rotated[g], out, M, N, K,
-                                                ldc, SkNorm{}, nullptr, rp, pre[g]);
+                                                ldc, SkNorm{}, nullptr, rp, SkNext{}, pre[g]);
   }
 }
 
@@ -597,6 +556,7 @@ struct SkCall {
   hipStream_t stream;
   bool resident = true;
   int strip_rows = 16;
+  SkNext nx = SkNext{};
 };
 
 // Blocks of the resident kernel: every strip its own block while that still leaves CUs idle, else
@@ -616,7 +576,7 @@ static int launch_skinny(int nw, const SkCall& a) {
   do {                                                                                                            \
     gemm_skinny_resident_kernel<MT, NW, KS, EPI, TC, XNORM, SSQ>                                                  \
         <<<dim3(resident_blocks(n_strips, NW)), dim3(NW * 64), 0, a.stream>>>(                                    \
-            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.rp, n_strips); \
+            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp, n_strips); \
     GL3_LAUNCH_CHECK();                                                                                           \
     return 0;                                                                                                     \
   } while (0)
@@ -624,7 +584,7 @@ static int launch_skinny(int nw, const SkCall& a) {
     if (a.strip_rows == 8) {
       // strips of 8 rows: twice the blocks, each with half the rows to stream
       gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
-          a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.rp);
+          a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp);
       GL3_LAUNCH_CHECK();
       return 0;
     }
@@ -634,18 +594,17 @@ static int launch_skinny(int nw, const SkCall& a) {
     if constexpr (NG * MT <= 2) {
       if (steps <= 64) RES(16, 4);
     }
-    // (variants whose registers would spill are left to the streaming kernel)
-    if constexpr (NG * MT <= 4 && !(XNORM && MT >= 3)) {
+    if constexpr (NG * MT <= 4) {
       if (steps <= 64) RES(8, 8);
     }
-    if constexpr (MT == 1 && !XNORM && EPI != SK_GATED) {
+    if constexpr (MT == 1 && EPI != SK_GATED) {
       if (steps <= 128) RES(8, 16);
     }
   }
 #undef RES
 #define GO(NW)                                                                                                    \
   gemm_skinny_kernel<MT, NW, EPI, TC, XNORM, SSQ><<<grid, dim3(NW * 64), 0, a.stream>>>(                          \
-      a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.rp)
+      a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp)
   if constexpr (NG * MT <= 2) {
     if (nw >= 16) { GO(16); GL3_LAUNCH_CHECK(); return 0; }
   }
@@ -696,9 +655,11 @@ static int check_common(const char* who, const void* A, const void* W, const voi
 // completed rows.
 // strip_rows: 16, or 8 (store and add epilogues, M <= 16): a block takes 8 rows of W, and ssq_out has a
 // row per 8 columns, [ceil(N/8)][64].
+// next_weight, xg (may be null; with ssq_out): the weight [N] (float) of the norm that follows, and
+// where bfloat16(weight * x) of the completed rows goes, [M][ldxg].
 extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                long ldw, long ldc, int epilogue, int waves, float* ssq_out, int strip_rows,
-                               hipStream_t stream) {
+                               const float* next_weight, void* xg, long ldxg, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny", A, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny: ldc too small");
@@ -708,7 +669,10 @@ extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtyp
               "gl3_gemm_skinny: sums of squares come with the add epilogue and N a multiple of 16");
   GL3_REQUIRE(strip_rows == 16 || (strip_rows == 8 && M <= 16 && epilogue != SK_GATED),
               "gl3_gemm_skinny: strips of %d rows (M=%d, epilogue %d)", strip_rows, M, epilogue);
-  const SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, ssq_out, SkRope{}, stream, waves == 0, strip_rows};
+  GL3_REQUIRE((next_weight == nullptr) == (xg == nullptr) && (!xg || (ssq_out && ldxg >= N)),
+              "gl3_gemm_skinny: the next norm's weight and its rows come together, with the sums of squares");
+  SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, ssq_out, SkRope{}, stream, waves == 0, strip_rows};
+  a.nx = SkNext{next_weight, (bf16_t*)xg, ldxg};
   const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32) {
     if (epilogue == SK_STORE) return pick_mt<SK_STORE, float, false, false>(nw, a);
@@ -786,22 +750,20 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
   return 0;
 }
 
-// The product of RMSNorm(x) with W: x float [rows, K] (lda), norm weight [K], ssq [n_partials][64]
-// partial sums of squares of the rows of x (indexed by the row of x, so x has at most 64 rows).
+// The product of RMSNorm(x) with W. xg: bfloat16(norm weight * x), [rows of x, K] (lda); ssq:
+// [n_partials][64] partial sums of squares of the rows of x (indexed by the row of x, so x has at
+// most 64 rows); `rows` (may be null) picks the rows of x that the product's rows read.
 // Epilogues: store (float or bfloat16) and gated (bfloat16).
-extern "C" int gl3_gemm_skinny_norm(const float* x, const int* rows, const void* norm_weight, int norm_weight_dtype,
-                                    const float* ssq, int n_partials, float eps, const void* W, void* C, int c_dtype,
-                                    int M, int N, int K, long lda, long ldw, long ldc, int epilogue, int waves,
-                                    hipStream_t stream) {
+extern "C" int gl3_gemm_skinny_norm(const void* xg, const int* rows, const float* ssq, int n_partials, float eps,
+                                    const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
+                                    long ldc, int epilogue, int waves, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
-  if (check_common("gl3_gemm_skinny_norm", x, W, C, M, N, K, lda, ldw, waves)) return -1;
-  GL3_REQUIRE(norm_weight && ssq && n_partials > 0, "gl3_gemm_skinny_norm: norm arguments missing");
-  GL3_REQUIRE(norm_weight_dtype == GL3_F32, "gl3_gemm_skinny_norm: the norm weight must be float");
-  GL3_REQUIRE((uintptr_t)norm_weight % 16 == 0, "gl3_gemm_skinny_norm: norm weight must be 16-byte aligned");
+  if (check_common("gl3_gemm_skinny_norm", xg, W, C, M, N, K, lda, ldw, waves)) return -1;
+  GL3_REQUIRE(ssq && n_partials > 0, "gl3_gemm_skinny_norm: norm arguments missing");
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny_norm: ldc too small");
   GL3_REQUIRE(epilogue == SK_STORE || epilogue == SK_GATED, "gl3_gemm_skinny_norm: epilogue %d", epilogue);
-  const SkNorm nrm = {(const float*)norm_weight, ssq, n_partials, eps, rows};
-  const SkCall a = {x, W, C, M, N, K, lda, ldw, ldc, nrm, nullptr, SkRope{}, stream, waves == 0};
+  const SkNorm nrm = {ssq, n_partials, eps, rows};
+  const SkCall a = {xg, W, C, M, N, K, lda, ldw, ldc, nrm, nullptr, SkRope{}, stream, waves == 0};
   const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32 && epilogue == SK_STORE) return pick_mt<SK_STORE, float, true, false>(nw, a);
   if (c_dtype == GL3_BF16 && epilogue == SK_STORE) return pick_mt<SK_STORE, bf16_t, true, false>(nw, a);
@@ -810,25 +772,21 @@ extern "C" int gl3_gemm_skinny_norm(const float* x, const int* rows, const void*
   return 0;
 }
 
-// RMSNorm(x) . Wqkv^T, rotation of q and k, q to `q_out` [M, n_heads*head_dim] (ldq), k and v into
-// the paged cache (keys [page][kv head][position][head_dim], values transposed). One token per row;
-// cos/sin null: no rotation. head_dim a multiple of 16; the rotation covers the whole head.
-// With norm_weight null x is bfloat16 and already normalised: the product, rotation and cache
-// write alone.
-extern "C" int gl3_qkv_rope_cache(const void* x, const void* norm_weight, int norm_weight_dtype, const float* ssq,
-                                  int n_partials, float eps, const void* Wqkv, void* q_out, long ldq, int M, int K,
-                                  long lda, long ldw, const int* positions, const int* seq_of_token,
-                                  const int* block_table, int table_stride, const float* cos_tab,
-                                  const float* sin_tab, void* k_cache, void* v_cache, int n_heads, int n_kv,
-                                  int head_dim, int adjacent, int page_size, int waves, hipStream_t stream) {
+// a . Wqkv^T, rotation of q and k, q to `q_out` [M, n_heads*head_dim] (ldq), k and v into the paged
+// cache (keys [page][kv head][position][head_dim], values transposed). One token per row; cos/sin
+// null: no rotation. head_dim a multiple of 16; the rotation covers the whole head.
+// ssq null: `a` holds the rows as they are. Else `a` is bfloat16(norm weight * x) and the product
+// is that of RMSNorm(x), with the rows' sums of squares in `ssq` [n_partials][64].
+extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_partials, float eps, const void* Wqkv,
+                                  void* q_out, long ldq, int M, int K, long lda, long ldw, const int* positions,
+                                  const int* seq_of_token, const int* block_table, int table_stride,
+                                  const float* cos_tab, const float* sin_tab, void* k_cache, void* v_cache,
+                                  int n_heads, int n_kv, int head_dim, int adjacent, int page_size, int waves,
+                                  hipStream_t stream) {
   if (M == 0) return 0;
   const int N = (n_heads + 2 * n_kv) * head_dim;
-  if (check_common("gl3_qkv_rope_cache", x, Wqkv, q_out, M, N, K, lda, ldw, waves)) return -1;
-  if (norm_weight) {
-    GL3_REQUIRE(ssq && n_partials > 0 && (uintptr_t)norm_weight % 16 == 0,
-                "gl3_qkv_rope_cache: norm arguments missing or misaligned");
-    GL3_REQUIRE(norm_weight_dtype == GL3_F32, "gl3_qkv_rope_cache: the norm weight must be float");
-  }
+  if (check_common("gl3_qkv_rope_cache", a_rows, Wqkv, q_out, M, N, K, lda, ldw, waves)) return -1;
+  GL3_REQUIRE(!ssq || n_partials > 0, "gl3_qkv_rope_cache: sums of squares without their count");
   GL3_REQUIRE(head_dim % 16 == 0 && n_heads > 0 && n_kv > 0, "gl3_qkv_rope_cache: head_dim %d must be a multiple of 16",
               head_dim);
   GL3_REQUIRE(positions && seq_of_token && block_table && k_cache && v_cache && page_size > 0 && table_stride > 0,
@@ -836,10 +794,10 @@ extern "C" int gl3_qkv_rope_cache(const void* x, const void* norm_weight, int no
   GL3_REQUIRE((cos_tab == nullptr) == (sin_tab == nullptr), "gl3_qkv_rope_cache: one table without the other");
   GL3_REQUIRE(ldq >= (long)n_heads * head_dim && ldq % 4 == 0 && (uintptr_t)q_out % 8 == 0,
               "gl3_qkv_rope_cache: q_out stride/alignment");
-  const SkNorm nrm = {(const float*)norm_weight, ssq, n_partials, eps, nullptr};
+  const SkNorm nrm = {ssq, n_partials, eps, nullptr};
   const SkRope rp = {positions, seq_of_token, block_table, table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
                      (bf16_t*)v_cache, n_heads, n_kv, head_dim, adjacent, page_size};
-  const SkCall a = {x, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
-  if (!norm_weight) return pick_mt<SK_QKV, bf16_t, false, false>(pick_waves(waves, N, K), a);
+  const SkCall a = {a_rows, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
+  if (!ssq) return pick_mt<SK_QKV, bf16_t, false, false>(pick_waves(waves, N, K), a);
   return pick_mt<SK_QKV, bf16_t, true, false>(pick_waves(waves, N, K), a);
 }

@@ -47,7 +47,7 @@ def _declare(lib):
     sigs = {
         "gl3_abi_version": [],
         "gl3_fill_u32": [P, c_uint32, L, P],
-        "gl3_embed": [P, I, P, P, I, I, P, P],
+        "gl3_embed": [P, I, P, P, I, I, P, P, P, P],
         "gl3_touch": [P, L, I, P, P],
         "gl3_rmsnorm": [P, P, P, I, P, I, I, I, F, P],
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
@@ -57,10 +57,10 @@ def _declare(lib):
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_argmax": [P, L, P, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
-        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P],
+        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P],
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P],
-        "gl3_gemm_skinny_norm": [P, P, P, I, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P],
-        "gl3_qkv_rope_cache": [P, P, I, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
+        "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P],
+        "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
@@ -126,9 +126,20 @@ def fill_u32(t, value):
     _check(library().gl3_fill_u32(_ptr(t), value, t.element_size() * t.numel() // 4, _stream()), "fill_u32")
 
 
-def embed(table, ids, out, ssq=None):
+def _check_next(next_weight, xg, rows, d, who):
+    """The next norm's float weight [d] and the bfloat16 rows [rows, d] that receive weight * x."""
+    if (next_weight is None) != (xg is None):
+        raise KernelError(f"{who}: the next norm's weight and its rows come together")
+    if xg is not None:
+        _dev(next_weight, "next_weight", torch.float32); _dev(xg, "xg", torch.bfloat16, contiguous=False)
+        if next_weight.shape != (d,) or xg.dim() != 2 or xg.shape != (rows, d) or xg.stride(1) != 1:
+            raise KernelError(f"{who}: next weight {tuple(next_weight.shape)}, rows {tuple(xg.shape)} for [{rows}, {d}]")
+
+
+def embed(table, ids, out, ssq=None, next_weight=None, xg=None):
     """out[t] = table[ids[t]] as float32. The caller has checked ids < rows. ``ssq`` (at least 64
-    floats, at most 64 tokens) receives each row's sum of squares."""
+    floats, at most 64 tokens) receives each row's sum of squares; with it ``xg`` [T, d] bfloat16
+    may receive ``next_weight * out``, the rows as the product after the next norm reads them."""
     _dev(table, "table"); _dev(ids, "ids", torch.int32); _dev(out, "out", torch.float32)
     T, d = out.shape
     if table.dim() != 2 or table.shape[1] != d or ids.numel() != T:
@@ -137,8 +148,11 @@ def embed(table, ids, out, ssq=None):
         _dev(ssq, "ssq", torch.float32)
         if ssq.numel() < 64 or T > 64:
             raise KernelError("embed: sums of squares need 64 floats and at most 64 tokens")
-    _check(library().gl3_embed(_ptr(table), _code(table, "table"), _ptr(ids), _ptr(out), T, d, _ptr(ssq), _stream()),
-           "embed")
+    _check_next(next_weight, xg, T, d, "embed")
+    if xg is not None and (ssq is None or not xg.is_contiguous()):
+        raise KernelError("embed: the next norm's rows come with the sums of squares, contiguous")
+    _check(library().gl3_embed(_ptr(table), _code(table, "table"), _ptr(ids), _ptr(out), T, d, _ptr(ssq),
+                               _ptr(next_weight), _ptr(xg), _stream()), "embed")
 
 
 def rmsnorm(x, weight, out, eps, rows=None):
@@ -312,9 +326,11 @@ def skinny_strip_rows(M, N, K, epilogue):
     return 8 if M <= 16 and epilogue != EPI_GATED and -(-N // 16) <= 160 and K > 4096 else 16
 
 
-def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows=16):
+def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows=16, next_weight=None, xg=None):
     """out (=, +=, gated) a @ w.T on the matrix cores for at most 64 rows of ``a``. ``ssq_out``
-    [N/strip_rows, 64] float32 (add epilogue): partial sums of squares of the completed rows."""
+    [N/strip_rows, 64] float32 (add epilogue): partial sums of squares of the completed rows; with it
+    ``xg`` [M, N] bfloat16 may receive ``next_weight * out``, the rows as the product after the next
+    norm reads them."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
         raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
@@ -327,9 +343,12 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows
         _dev(ssq_out, "ssq_out", torch.float32)
         if epilogue != EPI_ADD or N % 16 or ssq_out.numel() < N // strip_rows * 64:
             raise KernelError("gemm_skinny: sums of squares need the add epilogue, N % 16 == 0 and 64 floats a strip")
+    _check_next(next_weight, xg, M, N, "gemm_skinny")
+    if xg is not None and ssq_out is None:
+        raise KernelError("gemm_skinny: the next norm's rows come with the sums of squares")
     _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
-                                     out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _stream()),
-           "gemm_skinny")
+                                     out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _ptr(next_weight),
+                                     _ptr(xg), xg.stride(0) if xg is not None else 0, _stream()), "gemm_skinny")
 
 
 def gemm_skinny_wide_fits(a, w, out, epilogue):
@@ -360,63 +379,65 @@ def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0):
                                           _stream()), "gemm_skinny_wide")
 
 
-def _check_norm_args(x, norm_weight, ssq, n_partials, K):
-    _dev(x, "x", torch.float32, contiguous=False); _dev(norm_weight, "norm_weight"); _dev(ssq, "ssq", torch.float32)
-    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] != K or norm_weight.shape != (K,):
-        raise KernelError(f"fused norm: x {tuple(x.shape)}, weight {tuple(norm_weight.shape)} for K={K}")
-    if x.shape[0] > 64 or n_partials < 1 or ssq.numel() < n_partials * 64:
-        raise KernelError("fused norm: at most 64 rows of x, and n_partials * 64 partial sums")
+def _check_norm_args(xg, ssq, n_partials, K):
+    _dev(xg, "xg", torch.bfloat16, contiguous=False); _dev(ssq, "ssq", torch.float32)
+    if xg.dim() != 2 or xg.stride(1) != 1 or xg.shape[1] != K:
+        raise KernelError(f"folded norm: rows {tuple(xg.shape)} for K={K}")
+    if xg.shape[0] > 64 or n_partials < 1 or ssq.numel() < n_partials * 64:
+        raise KernelError("folded norm: at most 64 rows, and n_partials * 64 partial sums")
 
 
-def gemm_skinny_norm_fits(x, w, out, epilogue):
-    K = x.shape[1]
-    return (x.shape[0] <= 64 and K % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
-            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and w.dtype == torch.bfloat16
+def gemm_skinny_norm_fits(xg, w, out, epilogue):
+    K = xg.shape[1]
+    return (xg.shape[0] <= 64 and K % 8 == 0 and xg.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+            and xg.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and w.dtype == torch.bfloat16
             and ((epilogue == EPI_STORE and out.dtype in (torch.float32, torch.bfloat16))
                  or (epilogue == EPI_GATED and out.dtype == torch.bfloat16)))
 
 
-def gemm_skinny_norm(x, norm_weight, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=None, waves=0):
-    """out (=, gated) RMSNorm(x)[rows] @ w.T; the norm's sum of squares comes as partial sums."""
+def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=None, waves=0):
+    """out (=, gated) RMSNorm(x)[rows] @ w.T, where ``xg`` = bfloat16(norm weight * x) was left by the
+    kernel that completed the rows of x, together with their sums of squares as partial sums."""
     _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
     K = w.shape[1]
-    _check_norm_args(x, norm_weight, ssq, n_partials, K)
-    M = x.shape[0]
+    _check_norm_args(xg, ssq, n_partials, K)
+    M = xg.shape[0]
     if rows is not None:
         _dev(rows, "rows", torch.int32)
         M = rows.numel()
     N = out.shape[1]
     wrows = 2 * N if epilogue == EPI_GATED else N
     if w.shape != (wrows, K) or out.shape[0] != M or out.stride(1) != 1 or M > 64:
-        raise KernelError(f"gemm: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
+        raise KernelError(f"gemm: rows {tuple(xg.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_skinny_norm(
-        _ptr(x), _ptr(rows), _ptr(norm_weight), _code(norm_weight, "norm_weight"), _ptr(ssq), n_partials, float(eps),
-        _ptr(w), _ptr(out), _code(out, "out"), M, N, K, x.stride(0), w.stride(0), out.stride(0), epilogue, waves,
-        _stream()), "gemm_skinny_norm")
+        _ptr(xg), _ptr(rows), _ptr(ssq), n_partials, float(eps), _ptr(w), _ptr(out), _code(out, "out"), M, N, K,
+        xg.stride(0), w.stride(0), out.stride(0), epilogue, waves, _stream()), "gemm_skinny_norm")
 
 
-def qkv_rope_cache_fits(x, w_qkv, head_dim, rot_dim):
-    """x: the float residual rows (with the norm's arguments) or normalised bfloat16 rows (without)."""
-    K = x.shape[1]
-    return (x.shape[0] <= 64 and x.stride(1) == 1 and K % 8 == 0 and x.stride(0) % 8 == 0 and w_qkv.stride(0) % 8 == 0
-            and x.data_ptr() % 16 == 0 and w_qkv.data_ptr() % 16 == 0 and w_qkv.dtype == torch.bfloat16
+def qkv_rope_cache_fits(a, w_qkv, head_dim, rot_dim):
+    """a: normalised bfloat16 rows, or bfloat16(norm weight * x) with the sums of squares."""
+    K = a.shape[1]
+    return (a.shape[0] <= 64 and a.stride(1) == 1 and a.dtype == torch.bfloat16 and K % 8 == 0
+            and a.stride(0) % 8 == 0 and w_qkv.stride(0) % 8 == 0
+            and a.data_ptr() % 16 == 0 and w_qkv.data_ptr() % 16 == 0 and w_qkv.dtype == torch.bfloat16
             and head_dim % 16 == 0 and rot_dim in (0, head_dim))
 
 
-def qkv_rope_cache(x, norm_weight, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_token, block_table, cos, sin,
+def qkv_rope_cache(a, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_token, block_table, cos, sin,
                    k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page_size, waves=0):
-    """RMSNorm(x) @ w_qkv.T, rotation, q into ``q_out`` [T, H*hs] bfloat16, k and v into the cache.
-    ``norm_weight`` None: x is bfloat16, normalised already."""
+    """a @ w_qkv.T, rotation, q into ``q_out`` [T, H*hs] bfloat16, k and v into the cache. ``ssq`` None:
+    ``a`` holds the rows as they are; else ``a`` = bfloat16(norm weight * x) and the product is that
+    of RMSNorm(x), the rows' sums of squares coming as partial sums."""
     _dev(w_qkv, "w_qkv", torch.bfloat16); _dev(q_out, "q_out", torch.bfloat16, contiguous=False)
     K = w_qkv.shape[1]
-    if norm_weight is None:
-        _dev(x, "x", torch.bfloat16, contiguous=False)
-        if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] != K or x.shape[0] > 64:
-            raise KernelError(f"qkv_rope_cache: x {tuple(x.shape)} for K={K}")
-        ssq, n_partials = None, 0
+    if ssq is None:
+        _dev(a, "a", torch.bfloat16, contiguous=False)
+        if a.dim() != 2 or a.stride(1) != 1 or a.shape[1] != K or a.shape[0] > 64:
+            raise KernelError(f"qkv_rope_cache: rows {tuple(a.shape)} for K={K}")
+        n_partials = 0
     else:
-        _check_norm_args(x, norm_weight, ssq, n_partials, K)
-    T = x.shape[0]
+        _check_norm_args(a, ssq, n_partials, K)
+    T = a.shape[0]
     _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
     _dev(block_table, "block_table", torch.int32)
     _dev(k_cache, "k_cache", torch.bfloat16); _dev(v_cache, "v_cache", torch.bfloat16)
@@ -430,10 +451,10 @@ def qkv_rope_cache(x, norm_weight, ssq, n_partials, eps, w_qkv, q_out, positions
         if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != head_dim // 2:
             raise KernelError(f"qkv_rope_cache: table {tuple(cos.shape)} for head_dim {head_dim}")
     _check(library().gl3_qkv_rope_cache(
-        _ptr(x), _ptr(norm_weight), _code(norm_weight, "norm_weight") if norm_weight is not None else 0, _ptr(ssq),
-        n_partials, float(eps), _ptr(w_qkv), _ptr(q_out), q_out.stride(0), T, K, x.stride(0), w_qkv.stride(0), _ptr(positions), _ptr(seq_of_token),
-        _ptr(block_table), block_table.shape[1], _ptr(cos), _ptr(sin), _ptr(k_cache), _ptr(v_cache), n_heads, n_kv,
-        head_dim, int(adjacent), page_size, waves, _stream()), "qkv_rope_cache")
+        _ptr(a), _ptr(ssq), n_partials, float(eps), _ptr(w_qkv), _ptr(q_out), q_out.stride(0), T, K, a.stride(0),
+        w_qkv.stride(0), _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], _ptr(cos),
+        _ptr(sin), _ptr(k_cache), _ptr(v_cache), n_heads, n_kv, head_dim, int(adjacent), page_size, waves, _stream()),
+        "qkv_rope_cache")
 
 
 # ------------------------------------------------------------------ bfloat16 attention of a decode step

@@ -18,12 +18,20 @@ class PreNormBlock:
     def parts(self):
         return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
 
-    def forward(self, ctx, x, run):
+    def first_norm(self):
+        """The norm that reads the residual rows first: the block before this one may prepare its rows."""
+        return self.mixer_norm
+
+    def forward(self, ctx, x, run, norm_after=None):
+        """``norm_after``: the norm that reads the residual rows after this block, if known."""
         h = self.mixer_norm(ctx, x)
+        ctx.next_norm = self.ffn_norm if self.ffn is not None else norm_after
         self.mixer.forward(ctx, h, x, run)
         if self.ffn is not None:
             h = self.ffn_norm(ctx, x)
+            ctx.next_norm = norm_after
             self.ffn.forward(ctx, h, x)
+        ctx.next_norm = None
 
 
 register_part("block", "prenorm", PreNormBlock)

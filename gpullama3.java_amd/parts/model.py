@@ -78,16 +78,24 @@ class DecoderModel:
     def forward(self, ctx, want_rows):
         """Logits ``[len(want_rows), vocab]`` float32 at the wanted packed rows."""
         x = ctx.buffer("residual", (ctx.n_tokens, self.spec.hidden), torch.float32)
-        ctx.ssq = ctx.pending = None       # a context may run more than one forward pass: nothing is left over
-        if getattr(ctx, "fuse", False) and ctx.n_tokens <= ops.FUSE_ROWS:
-            ssq = ctx.ssq_buffer(1)                      # the first norm's sums of squares come with the rows
-            K.embed(self.embedding, ctx.token_ids, x, ssq)
-            ops.residual_written(ctx, x, ssq, 1)
+        ctx.ssq = ctx.pending = ctx.next_norm = None   # a context may run more than one forward pass: nothing is left over
+        order = [self.blocks[r.layer] for r in self.spec.run_order]
+        # the norm that reads the residual rows after entry i of the run order, where the block says which
+        firsts = [getattr(b, "first_norm", lambda: None)() for b in order] + [self.final_norm]
+        if getattr(ctx, "fuse", False) and ctx.n_tokens <= ops.FUSE_ROWS and getattr(firsts[0], "folds", False):
+            # the first norm's sums of squares, and its rows times its weight, come with the embedding
+            ssq = ctx.ssq_buffer(1)
+            xg = ctx.buffer("rows_times_norm_weight", (ctx.n_tokens, self.spec.hidden), torch.bfloat16)
+            K.embed(self.embedding, ctx.token_ids, x, ssq, firsts[0].weight_f32, xg)
+            ops.residual_written(ctx, x, ssq, 1, xg, firsts[0])
         else:
             K.embed(self.embedding, ctx.token_ids, x)
             ops.residual_written(ctx, x)
-        for run, r in zip(self.runs, self.spec.run_order):
-            self.blocks[r.layer].forward(ctx, x, run)
+        for i, (run, block) in enumerate(zip(self.runs, order)):
+            if hasattr(block, "first_norm"):
+                block.forward(ctx, x, run, norm_after=firsts[i + 1])
+            else:
+                block.forward(ctx, x, run)
         n = want_rows.numel()
         logits = ctx.logits_buffer(n, self.spec.vocab_size)
         if n:

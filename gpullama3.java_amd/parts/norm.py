@@ -12,6 +12,7 @@ FUSE_ROWS = 32      # a norm is folded into the next product for steps of at mos
 
 class RMSNorm:
     graph_safe = True      # kernel launches on the current stream only, sizes fixed by (T, B)
+    folds = True           # a product can take over this norm's work (see ``ops.Normed``)
 
     def __init__(self, spec, dtype):
         self.dim, self.eps, self.dtype = spec.dim, spec.eps, dtype
@@ -23,17 +24,17 @@ class RMSNorm:
 
     def load(self, weights):
         self.weight = weights[self.name]
-        # the products that fold the norm in read the weight as float (exact for 16-bit storage)
+        # the kernels that prepare a folded norm's rows read the weight as float (exact for 16-bit storage)
         self.weight_f32 = self.weight if self.weight.dtype == torch.float32 else self.weight.float()
 
     def __call__(self, ctx, x, rows=None, name="normed"):
         """The normalised rows, or a ``Normed`` when the next product can do the work itself (few
-        rows, and the sums of squares of exactly this tensor are at hand)."""
-        ssq = getattr(ctx, "ssq", None)
-        if (getattr(ctx, "fuse", False) and ssq is not None and ssq[0] == x.data_ptr() and x.shape[0] <= FUSE_ROWS
-                and self.dtype == torch.bfloat16):
+        rows, and the kernel that last wrote exactly this tensor prepared the rows for this norm)."""
+        rec = getattr(ctx, "ssq", None)
+        if (getattr(ctx, "fuse", False) and rec is not None and rec[0] == x.data_ptr() and rec[4] is self
+                and x.shape[0] <= FUSE_ROWS and self.dtype == torch.bfloat16):
             from .ops import Normed
-            return Normed(ctx, x, self.weight, self.weight_f32, self.eps, self.dtype, ssq[1], ssq[2], rows, name)
+            return Normed(ctx, x, self.weight, self.eps, self.dtype, rec[3], rec[1], rec[2], rows, name)
         n = x.shape[0] if rows is None else rows.numel()
         out = ctx.buffer(name, (n, self.dim), self.dtype)
         pending = getattr(ctx, "pending", None)

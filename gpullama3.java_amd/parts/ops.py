@@ -24,14 +24,14 @@ class Normed:
     """The RMSNorm of (rows of) the float residual stream, not computed yet.
 
     A norm hands this out instead of a tensor when the step is small enough for the
-    product that follows to do the norm's work itself: the sum of squares of every row is
-    already there as partial sums, left by the kernel that last wrote the rows.
+    product that follows to do the norm's work itself. The kernel that last wrote the rows
+    left what that takes: the rows times this norm's weight in bfloat16 (``xg``), and the
+    sum of squares of every row as partial sums; the product applies 1/rms to its sums.
     ``materialize`` runs the norm as a kernel of its own, for consumers that cannot."""
 
-    def __init__(self, ctx, x, weight, weight_f32, eps, dtype, ssq, n_partials, rows, name):
+    def __init__(self, ctx, x, weight, eps, dtype, xg, ssq, n_partials, rows, name):
         self.ctx, self.x, self.weight, self.eps, self.dtype = ctx, x, weight, eps, dtype
-        self.weight_f32 = weight_f32
-        self.ssq, self.n_partials, self.rows, self.name = ssq, n_partials, rows, name
+        self.xg, self.ssq, self.n_partials, self.rows, self.name = xg, ssq, n_partials, rows, name
         self.shape = (x.shape[0] if rows is None else rows.numel(), x.shape[1])
 
     def materialize(self):
@@ -50,33 +50,47 @@ def settle_residual(ctx, x):
         ctx.pending = None
 
 
-def residual_written(ctx, x, ssq=None, n_partials=0):
-    """Every writer of the residual stream says so: the partial sums of squares that a folded
-    norm would use are those of the last writer, or none."""
+def residual_written(ctx, x, ssq=None, n_partials=0, xg=None, norm=None):
+    """Every writer of the residual stream says so: what a folded norm would use (the partial sums
+    of squares of the rows, and the rows times the weight of ``norm``) is the last writer's, or
+    nothing."""
     if ctx is not None:
-        ctx.ssq = (x.data_ptr(), ssq, n_partials) if ssq is not None else None
+        ctx.ssq = (x.data_ptr(), ssq, n_partials, xg, norm) if ssq is not None and xg is not None else None
+
+
+def _next_norm(ctx, N):
+    """The norm that reads the residual rows next, if it is one whose work a product can take over:
+    (its float weight, a buffer for the rows times that weight), else (None, None)."""
+    norm = getattr(ctx, "next_norm", None)
+    w = getattr(norm, "weight_f32", None)
+    if norm is None or w is None or w.shape != (N,) or not getattr(norm, "folds", False):
+        return None, None
+    return norm, ctx.buffer("rows_times_norm_weight", (ctx.n_tokens, N), torch.bfloat16)
 
 
 def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
     """out (=, +=, gated) a @ w.T. ``a`` may be a ``Normed``. With the add epilogue ``out`` is the
     residual stream."""
     if isinstance(a, Normed):
-        if ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.x, w, out, epilogue)
-                and a.x.shape[0] <= 64):
-            return K.gemm_skinny_norm(a.x, a.weight_f32, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows)
+        if ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
+                and a.xg.shape[0] <= 64):
+            return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows)
         a = a.materialize()
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         if "wide" not in disabled and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx):
             return
         if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
             N = out.shape[1]
+            rows = K.skinny_strip_rows(a.shape[0], N, a.shape[1], epilogue)
             if (epilogue == EPI_ADD and ctx is not None and getattr(ctx, "fuse", False) and N % 16 == 0
-                    and "fused" not in disabled):
-                rows = K.skinny_strip_rows(a.shape[0], N, a.shape[1], epilogue)
-                ssq = ctx.ssq_buffer(N // rows)
-                K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq, strip_rows=rows)
-                return residual_written(ctx, out, ssq, N // rows)
-            K.gemm_skinny(a, w, out, epilogue)
+                    and "fused" not in disabled and out.shape[0] == ctx.n_tokens <= FUSE_ROWS):
+                # the rows are complete after this product: leave what the norm that follows needs
+                norm, xg = _next_norm(ctx, N)
+                if norm is not None:
+                    ssq = ctx.ssq_buffer(N // rows)
+                    K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq, strip_rows=rows, next_weight=norm.weight_f32, xg=xg)
+                    return residual_written(ctx, out, ssq, N // rows, xg, norm)
+            K.gemm_skinny(a, w, out, epilogue, strip_rows=rows)
             if epilogue == EPI_ADD:
                 residual_written(ctx, out)
             return
@@ -138,9 +152,9 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
     rot = rotary.rot_dim if rotary is not None else 0
     adjacent = rotary.adjacent if rotary is not None else False
     if (isinstance(h, Normed) and writes_kv and h.rows is None and "fused" not in disabled
-            and K.qkv_rope_cache_fits(h.x, w_qkv, head_dim, rot)):
+            and K.qkv_rope_cache_fits(h.xg, w_qkv, head_dim, rot)):
         q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
-        K.qkv_rope_cache(h.x, h.weight_f32, h.ssq, h.n_partials, h.eps, w_qkv, q, ctx.positions, ctx.seq_of_token,
+        K.qkv_rope_cache(h.xg, h.ssq, h.n_partials, h.eps, w_qkv, q, ctx.positions, ctx.seq_of_token,
                          block_table, cos, sin, k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page)
         return q
     if isinstance(h, Normed):
@@ -148,7 +162,7 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
     if (writes_kv and h.dtype == torch.bfloat16 and "fused" not in disabled and "skinny" not in disabled
             and K.qkv_rope_cache_fits(h, w_qkv, head_dim, rot)):
         q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
-        K.qkv_rope_cache(h, None, None, 0, 0.0, w_qkv, q, ctx.positions, ctx.seq_of_token, block_table, cos, sin,
+        K.qkv_rope_cache(h, None, 0, 0.0, w_qkv, q, ctx.positions, ctx.seq_of_token, block_table, cos, sin,
                          k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page)
         return q
     if writes_kv:

@@ -40,6 +40,18 @@ def test_embed(dtype):
     out = torch.empty(37, 70, device=DEV)
     K().embed(dev(table, TD[dtype]), dev(ids, torch.int32), out)
     np.testing.assert_array_equal(out.cpu().numpy(), table[ids])
+    # with the sums of squares and the rows times the next norm's weight, for a norm folded into a product
+    nw = (1 + 0.2 * rng.standard_normal(70)).astype(np.float32)
+    out2 = torch.empty(37, 70, device=DEV)
+    ssq = torch.full((64,), -1.0, device=DEV)
+    xg = torch.empty(37, 70, device=DEV, dtype=torch.bfloat16)
+    K().embed(dev(table, TD[dtype]), dev(ids, torch.int32), out2, ssq, dev(nw), xg)
+    assert torch.equal(out2, out)
+    np.testing.assert_allclose(ssq[:37].cpu().numpy(), (table[ids].astype(np.float64) ** 2).sum(1), rtol=1e-5)
+    assert torch.all(ssq[37:] == -1)
+    assert torch.equal(xg, (dev(nw)[None, :] * out).to(torch.bfloat16))
+    with pytest.raises(K().KernelError):
+        K().embed(dev(table, TD[dtype]), dev(ids, torch.int32), out2, None, dev(nw), xg)
 
 
 @pytest.mark.parametrize("d", [70, 2048, 5000])
@@ -598,26 +610,31 @@ def ssq_partials(x, n_partials):
     return out
 
 
+def times_weight(x, nw):
+    """The rows as a folded norm's product reads them: bfloat16(weight * x), computed in float."""
+    return (torch.as_tensor(nw.astype(np.float32))[None, :] * torch.as_tensor(x)).to(torch.bfloat16)
+
+
 @pytest.mark.parametrize("M", [1, 8, 33, 64])
-@pytest.mark.parametrize("N, Kd, P_", [(2048, 2048, 128), (130, 64, 1), (1000, 112, 7)])
-def test_gemm_skinny_with_folded_norm(M, N, Kd, P_, wdtype="float32"):
+@pytest.mark.parametrize("N, Kd, P_", [(2048, 2048, 128), (130, 64, 1), (1000, 112, 7), (96, 4096, 256), (64, 8192, 300)])
+def test_gemm_skinny_with_folded_norm(M, N, Kd, P_):
     rng = np.random.default_rng(M + N)
     extra = 3 if M + 3 <= 64 else 0
     x = (rng.standard_normal((M + extra, Kd)) * 2).astype(np.float32)       # more rows than are used, where they fit
-    nw = rounded(1 + 0.2 * rng.standard_normal(Kd), wdtype)
+    nw = rounded(1 + 0.2 * rng.standard_normal(Kd), "float32")
     w = rounded(rng.standard_normal((2 * N, Kd)) / math.sqrt(Kd), "bfloat16")
     lib = K()
-    X, NW_, W = dev(x), dev(nw, TD[wdtype]), dev(w, torch.bfloat16)
+    XG, W = times_weight(x, nw).to(DEV), dev(w, torch.bfloat16)
     ssq = dev(ssq_partials(x, P_))
     h = P.rmsnorm(x, nw, 1e-5)
     rows = np.arange(M)[::-1].copy() + extra                                 # a gather of rows
     ref = P.linear(h[rows], w[:N])
     out = torch.zeros(M, N, device=DEV)
-    lib.gemm_skinny_norm(X, NW_, ssq, P_, 1e-5, W[:N], out, lib.EPI_STORE, rows=dev(rows, torch.int32))
+    lib.gemm_skinny_norm(XG, ssq, P_, 1e-5, W[:N], out, lib.EPI_STORE, rows=dev(rows, torch.int32))
     np.testing.assert_allclose(out.cpu().numpy(), ref, atol=1e-2 * np.abs(ref).max())   # x*w is rounded to bfloat16
     refg = P.silu(P.linear(h[:M], w[:N])) * P.linear(h[:M], w[N:])
     g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
-    lib.gemm_skinny_norm(X[:M], NW_, ssq, P_, 1e-5, W, g_, lib.EPI_GATED)
+    lib.gemm_skinny_norm(XG[:M], ssq, P_, 1e-5, W, g_, lib.EPI_GATED)
     np.testing.assert_allclose(g_.float().cpu().numpy(), refg, atol=1.5e-2 * max(np.abs(refg).max(), 1e-3))
 
 
@@ -636,6 +653,20 @@ def test_gemm_skinny_leaves_sums_of_squares(M):
     got = ssq.cpu().numpy()
     np.testing.assert_allclose(got[:, :M], ssq_partials(new, N // 16)[:, :M], rtol=1e-4)
     assert np.all(got[:, M:] == -1.0)                                        # rows that do not exist are not written
+    # the same with the rows times the next norm's weight, in strips of 16 and (few rows) of 8
+    nw = (1 + 0.2 * rng.standard_normal(N)).astype(np.float32)
+    for strip in ((16, 8) if M <= 16 else (16,)):
+        x2 = dev(res)
+        ssq2 = torch.full((N // strip, 64), -1.0, device=DEV)
+        xg = torch.full((M, N + 8), 9.0, device=DEV, dtype=torch.bfloat16)   # a view with a row stride
+        K().gemm_skinny(dev(a, torch.bfloat16), dev(w, torch.bfloat16), x2, K().EPI_ADD, ssq_out=ssq2, strip_rows=strip,
+                        next_weight=dev(nw), xg=xg[:, :N])
+        np.testing.assert_allclose(x2.cpu().numpy(), new, atol=1e-4)         # (another order of summation per strip size)
+        assert torch.equal(xg[:, :N], (dev(nw)[None, :] * x2).to(torch.bfloat16)) and torch.all(xg[:, N:] == 9.0)
+        np.testing.assert_allclose(ssq2[:, :M].cpu().numpy(), ssq_partials(new, N // strip)[:, :M], rtol=1e-4)
+    with pytest.raises(K().KernelError):
+        K().gemm_skinny(dev(a, torch.bfloat16), dev(w, torch.bfloat16), x, K().EPI_ADD, next_weight=dev(nw),
+                        xg=torch.empty(M, N, device=DEV, dtype=torch.bfloat16))          # not without the sums of squares
 
 
 @pytest.mark.parametrize("folded_norm", [True, False])
@@ -657,14 +688,14 @@ def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs, folded_norm):
     cos, sin = P.rope_table(256, hs, 50000.0)
     q_out = torch.zeros(T, H * hs, device=DEV, dtype=torch.bfloat16)
     if folded_norm:
-        K().qkv_rope_cache(dev(x), dev(nw), dev(ssq_partials(x, 6)), 6, 1e-5, dev(w, torch.bfloat16), q_out,
+        K().qkv_rope_cache(times_weight(x, nw).to(DEV), dev(ssq_partials(x, 6)), 6, 1e-5, dev(w, torch.bfloat16), q_out,
                            dev(positions, torch.int32), dev(seq_of, torch.int32), table,
                            dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
                            pairing == "adjacent", page)
         qkv = P.linear(P.rmsnorm(x, nw, 1e-5), w)
     else:                                                                     # rows that are normalised already
         h = rounded(x, "bfloat16")
-        K().qkv_rope_cache(dev(h, torch.bfloat16), None, None, 0, 0.0, dev(w, torch.bfloat16), q_out,
+        K().qkv_rope_cache(dev(h, torch.bfloat16), None, 0, 0.0, dev(w, torch.bfloat16), q_out,
                            dev(positions, torch.int32), dev(seq_of, torch.int32), table,
                            dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
                            pairing == "adjacent", page)
