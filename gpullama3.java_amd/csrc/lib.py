@@ -48,7 +48,6 @@ def _declare(lib):
         "gl3_abi_version": [],
         "gl3_fill_u32": [P, c_uint32, L, P],
         "gl3_embed": [P, I, P, P, I, I, P, P, P, P],
-        "gl3_touch": [P, L, I, P, P],
         "gl3_rmsnorm": [P, P, P, I, P, I, I, I, F, P],
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
@@ -170,12 +169,6 @@ def rmsnorm(x, weight, out, eps, rows=None):
         raise KernelError(f"rmsnorm: {x.shape[0]} inputs for {n} outputs")
     _check(library().gl3_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _code(weight, "weight"), _ptr(out),
                                  _code(out, "out"), n, d, float(eps), _stream()), "rmsnorm")
-
-
-def touch(t, sink, blocks=64):
-    """Reads the whole of ``t`` and keeps nothing: afterwards it lies in the memory-side cache."""
-    _dev(t, "t"); _dev(sink, "sink", torch.int32)
-    _check(library().gl3_touch(_ptr(t), t.numel() * t.element_size(), blocks, _ptr(sink), _stream()), "touch")
 
 
 def add_slices_rmsnorm(x, slices, weight=None, out=None, eps=0.0, rows=None):
