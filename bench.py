@@ -1,13 +1,15 @@
 """Decode and prefill throughput of the Llama-3.2-1B shape with random weights on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 1b|3b|8b]
+                    [--prompt-len P] [--prefill-len T]
 
 A step is one decode step of the generation loop: the engine's step for B sequences (one
 token each, from the cache left by 512-token prompts) and the greedy pick of the next
 token on the device. ``value`` is decoded tokens a second at the default batch of 8.
 The same line carries the prefill of one 2,048-token prompt, the decode step's share of
 the memory roofline, and decode at batch 1 and 64. Peaks are the published ones of the
-MI355X: 8 TB/s HBM3E, 2.5 PFLOP/s dense bf16 matrix throughput.
+MI355X: 8 TB/s HBM3E, 2.5 PFLOP/s dense bf16 matrix throughput. Other layer sizes (--shape) and
+lengths are for looking further; the default run is the one that is reported.
 """
 import argparse
 import json
@@ -23,15 +25,31 @@ sys.path.insert(0, ROOT)
 HBM_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 
-# the Llama-3.2-1B shape: every size as the model's own config.json gives it
-SHAPE = {
-    "architectures": ["LlamaForCausalLM"], "hidden_size": 2048, "intermediate_size": 8192,
-    "num_hidden_layers": 16, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
-    "vocab_size": 128256, "max_position_embeddings": 4096, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
-    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
-                     "original_max_position_embeddings": 8192},
-    "tie_word_embeddings": True, "hidden_act": "silu",
+# every size as the model's own config.json gives it; "1b" is the shape that the default run measures
+_COMMON = {"architectures": ["LlamaForCausalLM"], "vocab_size": 128256, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+           "hidden_act": "silu"}
+
+
+def _scaling(factor):
+    return {"rope_type": "llama3", "factor": factor, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+            "original_max_position_embeddings": 8192}
+
+
+SHAPES = {
+    "1b": ("Llama-3.2-1B shape", {**_COMMON, "hidden_size": 2048, "intermediate_size": 8192, "num_hidden_layers": 16,
+                                  "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
+                                  "max_position_embeddings": 4096, "rope_scaling": _scaling(32.0),
+                                  "tie_word_embeddings": True}),
+    "3b": ("Llama-3.2-3B shape", {**_COMMON, "hidden_size": 3072, "intermediate_size": 8192, "num_hidden_layers": 28,
+                                  "num_attention_heads": 24, "num_key_value_heads": 8, "head_dim": 128,
+                                  "max_position_embeddings": 4096, "rope_scaling": _scaling(32.0),
+                                  "tie_word_embeddings": True}),
+    "8b": ("Llama-3.1-8B shape", {**_COMMON, "hidden_size": 4096, "intermediate_size": 14336, "num_hidden_layers": 32,
+                                  "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+                                  "max_position_embeddings": 8192, "rope_scaling": _scaling(8.0),
+                                  "tie_word_embeddings": False}),
 }
+SHAPE = SHAPES["1b"][1]
 CONTEXT = 4096
 PROMPT = 512
 PREFILL = 2048
@@ -64,8 +82,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
+    ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes; the default is what is reported")
+    ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the shape has (reported as such); never smaller layers")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT, help="tokens every sequence holds before the decode steps")
+    ap.add_argument("--prefill-len", type=int, default=PREFILL, help="tokens of the prompt whose prefill is timed")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma-separated")
@@ -80,20 +101,25 @@ def main():
     import gpullama3_java_amd as g
     from gpullama3_java_amd.engine import Engine
 
-    cfg = g.config_from_dict({**SHAPE, "num_hidden_layers": args.layers})
+    shape_name, shape = SHAPES[args.shape]
+    context = shape["max_position_embeddings"]
+    prompt_len, prefill_len = args.prompt_len, args.prefill_len
+    if args.layers is None:
+        args.layers = shape["num_hidden_layers"]
+    cfg = g.config_from_dict({**shape, "num_hidden_layers": args.layers})
     esize = 2 if args.dtype == "bfloat16" else 4
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     K, W = args.steps, args.warmup
     points = [int(b) for b in args.points.split(",") if b]
     biggest = max([args.batch] + points)
-    per_seq = -(-(PROMPT + K + W + 1) // 64) * 64
+    per_seq = -(-(prompt_len + K + W + 1) // 64) * 64
     tmp = tempfile.mkdtemp(prefix="gl3-bench-")
     try:
         t0 = time.time()
         g.write_random_model(tmp, cfg, args.seed)
         print(f"[bench] random {args.layers}-layer model written in {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
-        eng = Engine.from_folder(tmp, dtype=args.dtype, max_context=CONTEXT,
-                                 max_tokens=max(biggest * per_seq, PREFILL + 64), n_slots=biggest)
+        eng = Engine.from_folder(tmp, dtype=args.dtype, max_context=context,
+                                 max_tokens=max(biggest * per_seq, prefill_len + 64), n_slots=biggest)
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
     rng = np.random.default_rng(args.seed)
@@ -102,10 +128,10 @@ def main():
     def sync():
         torch.cuda.synchronize()
 
-    # ---- prefill: one prompt of 2,048 tokens, logits at its last token
+    # ---- prefill: one prompt (2,048 tokens unless told otherwise), logits at its last token
     def prefill_once():
         s = eng.take_slot()
-        toks = rng.integers(0, V, PREFILL).tolist()
+        toks = rng.integers(0, V, prefill_len).tolist()
         sync(); t = time.perf_counter()
         eng.step([(s, toks)])
         sync(); dt = time.perf_counter() - t
@@ -113,13 +139,13 @@ def main():
         return dt
     prefill_once()
     prefill_s = min(prefill_once() for _ in range(3))
-    print(f"[bench] prefill {PREFILL} tokens: {prefill_s * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    print(f"[bench] prefill {prefill_len} tokens: {prefill_s * 1e3:.2f} ms", file=sys.stderr, flush=True)
 
-    # ---- decode at batch B after 512-token prompts
+    # ---- decode at batch B after prompts of prompt_len tokens
     def decode(B):
         slots = [eng.take_slot() for _ in range(B)]
         for lo in range(0, B, 8):                              # prompts in groups of 8 to bound the step's memory
-            eng.step([(s, rng.integers(0, V, PROMPT).tolist()) for s in slots[lo:lo + 8]], want="none")
+            eng.step([(s, rng.integers(0, V, prompt_len).tolist()) for s in slots[lo:lo + 8]], want="none")
         temps, tops = [0.0] * B, [1.0] * B
         toks = rng.integers(0, V, B).tolist()
         run = eng.decode_run_length
@@ -155,23 +181,22 @@ def main():
     dt, nbytes = results[args.batch]
     ms = dt / K * 1e3
     achieved = nbytes / (dt / K) / 1e9
-    flops = prefill_flops(cfg, PREFILL)
+    flops = prefill_flops(cfg, prefill_len)
     line = {
-        "metric": "decode tok/s at batch 8 (Llama-3.2-1B shape, 512-token prompts)" if args.batch == 8
-        else f"decode tok/s at batch {args.batch} (Llama-3.2-1B shape, 512-token prompts)",
+        "metric": f"decode tok/s at batch {args.batch} ({shape_name}, {prompt_len}-token prompts)",
         "value": round(args.batch * K / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": short, "data": "synthetic: random N(0,0.02) weights, uniform random token ids",
         "config": {
-            "model": "Llama-3.2-1B shape", "layers": args.layers, "layers_of_shape": SHAPE["num_hidden_layers"],
+            "model": shape_name, "layers": args.layers, "layers_of_shape": shape["num_hidden_layers"],
             "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
             "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "vocab_size": cfg.vocab_size, "tied_head": cfg.tie_word_embeddings, "rope_theta": cfg.rope_theta,
             "rope_scaling_factor": cfg.rope_scaling.factor, "rms_norm_eps": cfg.rms_norm_eps,
-            "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPT, "prefill_len": PREFILL,
+            "global_batch": args.batch, "seq_len": context, "prompt_len": prompt_len, "prefill_len": prefill_len,
             "parallelism": "single GPU", "sampling": "greedy on device",
         },
-        "prefill": {"value": round(PREFILL / prefill_s, 1), "tokens": PREFILL, "ms": round(prefill_s * 1e3, 3),
+        "prefill": {"value": round(prefill_len / prefill_s, 1), "tokens": prefill_len, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / (PEAK_TFLOPS[short] * 1e12), 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},

@@ -3,7 +3,7 @@
 The tiny configurations of the other tests are too small for several choices that the
 product path makes by size: products of a prompt cut into slices of K, tiles of 256 x 256,
 strips of 8 rows, the kernels for 33 to 64 rows with their slices, the tiled kernel for the
-head. Here the layers have the sizes of Llama-3.2-1B (what bench.py measures) and of Llama-3.1-8B
+head. Here the layers have the sizes of Llama-3.2-1B (what bench.py measures), Llama-3.2-3B and Llama-3.1-8B
 (two layers each, to keep the test short),
 and every kind of step is run on both engines with the same weights. The float32 engine is
 the reference: it uses one size-generic kernel per operation, and the other tests compare it
@@ -22,6 +22,11 @@ SHAPES = {
     # the layers of Llama-3.2-1B: head size 64, tied head
     "1B": {**COMMON, "hidden_size": 2048, "intermediate_size": 8192, "num_attention_heads": 32, "num_key_value_heads": 8,
            "head_dim": 64, "tie_word_embeddings": True,
+           "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                            "original_max_position_embeddings": 8192}},
+    # the layers of Llama-3.2-3B: three query heads to a kv head, head size 128, a width of 3072
+    "3B": {**COMMON, "hidden_size": 3072, "intermediate_size": 8192, "num_attention_heads": 24, "num_key_value_heads": 8,
+           "head_dim": 128, "tie_word_embeddings": True,
            "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
                             "original_max_position_embeddings": 8192}},
     # the layers of Llama-3.1-8B: head size 128, longer rows, a head of its own
@@ -65,7 +70,7 @@ def steps(eng, vocab):
     return out
 
 
-@pytest.mark.parametrize("shape", ["1B", "8B"])
+@pytest.mark.parametrize("shape", ["1B", "3B", "8B"])
 def test_real_layer_sizes_bfloat16_against_float32(tmp_path, shape):
     import gpullama3_java_amd as g
     from gpullama3_java_amd.engine import Engine
