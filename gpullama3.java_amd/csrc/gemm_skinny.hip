@@ -445,8 +445,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
       float sp = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) sp += sq[i];
-      if (lane < M)
-        for (int p = wave + NW * 16; p < nrm.n_partials; p += NW) sp += nrm.ssq[(long)p * 64 + sq_row];
+      for (int p0 = wave + NW * 16; p0 < nrm.n_partials; p0 += NW * 16) {   // further partial sums, sixteen at a time
+        float more[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int p = p0 + NW * i;
+          more[i] = (lane < M && p < nrm.n_partials) ? nrm.ssq[(long)p * 64 + sq_row] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sp += more[i];
+      }
       sm_ssq[wave][lane] = sp;
       first_strip = false;
     }
@@ -594,10 +602,15 @@ static int launch_skinny(int nw, const SkCall& a) {
     if constexpr (NG * MT <= 2) {
       if (steps <= 64) RES(16, 4);
     }
+    // (more token tiles, the gated epilogue or the rotation's operands would not fit the registers with
+    // this many k-steps a wave: those take the streaming kernel for a longer K)
+    if constexpr (NG * MT == 1 && EPI != SK_QKV) {
+      if (steps <= 128) RES(16, 8);
+    }
     if constexpr (NG * MT <= 4) {
       if (steps <= 64) RES(8, 8);
     }
-    if constexpr (MT == 1 && EPI != SK_GATED) {
+    if constexpr (MT == 1 && EPI != SK_GATED && EPI != SK_QKV) {
       if (steps <= 128) RES(8, 16);
     }
   }
