@@ -811,6 +811,10 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
   const SkRope rp = {positions, seq_of_token, block_table, table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
                      (bf16_t*)v_cache, n_heads, n_kv, head_dim, adjacent, page_size};
   const SkCall a = {a_rows, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
+  if (!ssq && waves == 0 && M > 32 && (N + 15) / 16 / 2 >= 160) {
+    // many rows and many strips: two strips a block, so that the rows are read half as often
+    return (M + 15) / 16 <= 3 ? launch_wide<3, 2, SK_QKV, bf16_t>(a, 1, 0) : launch_wide<4, 2, SK_QKV, bf16_t>(a, 1, 0);
+  }
   if (!ssq) return pick_mt<SK_QKV, bf16_t, false, false>(pick_waves(waves, N, K), a);
   return pick_mt<SK_QKV, bf16_t, true, false>(pick_waves(waves, N, K), a);
 }

@@ -671,7 +671,7 @@ def test_gemm_skinny_leaves_sums_of_squares(M):
 
 @pytest.mark.parametrize("folded_norm", [True, False])
 @pytest.mark.parametrize("pairing", ["adjacent", "half", None])
-@pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 16), (5, 5, 48), (8, 1, 128)])
+@pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 16), (5, 5, 48), (8, 1, 128), (32, 8, 128), (21, 7, 112)])
 def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs, folded_norm):
     rng = np.random.default_rng(hs + H)
     d, page = 96, 64
