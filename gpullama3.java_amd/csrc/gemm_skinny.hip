@@ -4,12 +4,15 @@
 // Matrix cores, 16x16x32 tiles: the 16 rows of a strip of W are the tile's rows, up to
 // 64 tokens (MT tiles of 16) its columns, so a lane's 16-byte load from W (8 consecutive
 // k of one row) is the operand as the instruction wants it: W goes from memory to
-// registers and nowhere else. A block is NW waves (4, 8 or 16) on one strip; wave w
-// takes the k-steps w, w+NW, ... so that a strip's whole row range is in flight at
-// once, and the NW partial tiles are summed through shared memory in wave order: the
-// result has one fixed order of summation. K is never split across blocks: on this
-// chip a block that waits for another block's stores has to push them through the
-// per-XCD second-level caches, which costs more than the product itself.
+// registers and nowhere else. A block is NW waves (4, 8 or 16) on one strip; the waves
+// share out the k-steps so that a strip's whole row range is in flight at once, and the
+// NW partial tiles are summed through shared memory in wave order: the result has one
+// fixed order of summation. No block ever waits for another: on this chip a block that
+// waits for another block's stores has to push them through the per-XCD second-level
+// caches, which costs more than the product itself. Where K is cut across blocks (the
+// wide kernel) each slice's sums are stored apart and the next kernel adds them up.
+// Lanes whose token row does not exist ask for nothing: a CU draws a bounded number of
+// bytes a second through its first-level cache, whatever they are.
 //
 // A decode step is a chain of small kernels, each of which costs a few microseconds
 // before it does any work, so what would be kernels of their own is folded into the
@@ -27,12 +30,13 @@
 //    rows and the 8 rows half a head further, so both elements of a pair are in one tile.
 // Other epilogues as in gemm_generic.hip: store, add into a float matrix, gated.
 //
-// Two kernels share the strip's end. The streaming one reloads its share of A for every
-// strip and takes any K. The resident one is for K up to 32*NW*KS: a wave keeps the A
-// operands of its own k-steps in registers (with the norm's weight already applied) and
-// the block walks over several strips with them, asking for the next strip's rows of W
-// before it finishes the current strip; then the first-level cache carries W and nothing
-// else, which is what limits the streaming kernel when the same A is read for every strip.
+// Three kernels share the strip's end. The streaming one reloads its share of A for every
+// strip and takes any K (with strips of 16 rows of W, or of 8 where 16 leave CUs idle). The
+// resident one is for K up to 32*NW*KS: a wave keeps the A operands of its own k-steps in
+// registers and the block walks over several strips with them, asking for the next strip's
+// rows of W before it finishes the current strip; then the first-level cache carries W and
+// nothing else, which is what limits the streaming kernel when the same A is read for every
+// strip. The wide one, for 33 to 64 rows, takes several strips at once (see there).
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
