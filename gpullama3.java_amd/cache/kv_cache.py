@@ -1,7 +1,8 @@
 """The cache on the device: keys and values per run-order entry, per-slot state.
 
 Entries of the run order with the same needs (kv heads, head size, window, dtype)
-form a group; each group has storage, a page pool and block tables of its own:
+form a group; each group has storage, a page pool and block tables of its own (a group
+with a window holds only the pages its window still reaches):
 ``K: [entry in group, page, kv head, position in page, head_dim]``, ``V`` the same with its
 last two axes exchanged. A page is
 ``page_size`` positions of one sequence for every entry of the group. Beside it
@@ -90,7 +91,7 @@ class Cache:
     def give_back_slot(self, s):
         self.slots.check(s)
         for g, group in enumerate(self.groups):
-            group.pool.give_back(self.slots.pages[s][g])
+            group.pool.give_back([p for p in self.slots.pages[s][g] if p])   # (0: a page given back earlier)
             self.slots.pages[s][g] = []
         self.slots.give_back(s)
 
@@ -119,7 +120,22 @@ class Cache:
                 self.slots.pages[s][g].extend(self.groups[g].pool.take(extra))
 
     def advance(self, s, n):
+        """The sequence of slot ``s`` has ``n`` more tokens. A group with a window gives back the
+        pages that no later token can see: the next token, at position ``length``, reads the keys
+        from ``length + 1 - window`` on. Their places in the slot's list of pages become the sink
+        page, which nobody reads."""
         self.slots.length[s] += n
+        for g, group in enumerate(self.groups):
+            window = group.need.window
+            if not window:
+                continue
+            pages = self.slots.pages[s][g]
+            first_seen = max(0, self.slots.length[s] + 1 - window) // self.page_size
+            gone = [i for i in range(min(first_seen, len(pages))) if pages[i]]
+            if gone:
+                group.pool.give_back([pages[i] for i in gone])
+                for i in gone:
+                    pages[i] = 0
 
     # ---- what the kernels read
     def layer_kv(self, entry):

@@ -105,10 +105,15 @@ def test_random_traffic_keeps_the_books():
                 c.give_back_slot(s)
         # the books: every page is free or held by exactly one live slot; lengths fit their pages
         for g, group in enumerate(c.groups):
-            held = [p for s in live for p in c.slots.pages[s][g]]
-            assert len(held) == len(set(held)) and 0 not in held
+            held = [p for s in live for p in c.slots.pages[s][g] if p]
+            assert len(held) == len(set(held))
             assert len(held) + group.pool.n_free == total_pages[g]
             assert set(held) == group.pool._held
+            for s, n in live.items():
+                # a group without a window holds every page; with one, exactly the pages from the one
+                # with the first key that the next token sees
+                first = max(0, n + 1 - group.need.window) // 64 if group.need.window else 0
+                assert [bool(p) for p in c.slots.pages[s][g]] == [i >= first for i in range(-(-n // 64))]
         for s, n in live.items():
             assert c.length(s) == n and all(len(c.slots.pages[s][g]) == -(-n // 64) for g in range(2))
         assert set(live) == c.slots.live and len(live) + len(c.slots._free) == 5
@@ -123,3 +128,19 @@ def test_block_rows_pad_with_the_sink():
     c.reserve({a: 70})
     rows = c.block_rows(0, [a], 4)
     assert rows[0][:2] == c.slots.pages[a][0] and rows[0][2:] == [0, 0]
+
+
+def test_a_group_with_a_window_gives_back_the_pages_behind_it():
+    c = make(max_tokens=64 * 8, max_context=400, n_slots=2, needs=[KVNeed(2, 16), KVNeed(1, 32, window=70)], state=[None, None])
+    s = c.take_slot()
+    full, windowed = c.groups[0].pool, c.groups[1].pool
+    c.reserve({s: 130}); c.advance(s, 130)                      # the next token sees keys from 61 on: page 0 still
+    assert full.n_free == 8 - 3 and windowed.n_free == 8 - 3
+    c.reserve({s: 4}); c.advance(s, 4)                          # from 65 on: page 0 is out of reach
+    assert c.slots.pages[s][1][0] == 0 and all(c.slots.pages[s][1][1:]) and windowed.n_free == 8 - 2
+    assert all(c.slots.pages[s][0]) and full.n_free == 8 - 3    # the group without a window keeps everything
+    c.reserve({s: 200}); c.advance(s, 200)                      # 334 tokens: from 265 on, pages 4 and 5 of 6
+    assert [bool(p) for p in c.slots.pages[s][1]] == [False] * 4 + [True] * 2 and windowed.n_free == 8 - 2
+    assert c.block_rows(1, [s], 7)[0][:4] == [0, 0, 0, 0]       # the places of the pages given back point at the sink
+    c.give_back_slot(s)
+    assert full.n_free == 8 and windowed.n_free == 8

@@ -129,6 +129,43 @@ def test_attention_part_whole_and_in_pieces(dtype, H, Kh, hs, d, pairing, window
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_with_a_window_after_its_first_pages_were_given_back(dtype):
+    """A group with a window gives back the pages that lie behind it; the attention of later tokens,
+    in chunks and one by one, is that of the plain implementation over the whole sequence, and the
+    sequence holds two or three pages however long it grows."""
+    from gpullama3_java_amd.config import AttentionSpec, RotarySpec
+    from gpullama3_java_amd.parts import RunInfo, build_part
+    rng = np.random.default_rng(4)
+    H, Kh, hs, d, window, n = 4, 2, 32, 64, 50, 420
+    spec = AttentionSpec(hidden=d, n_heads=H, n_kv_heads=Kh, head_dim=hs, window=window, names={k: k for k in "qkvo"},
+                         position=RotarySpec(head_dim=hs, theta=1000.0, pairing="half", max_positions=512))
+    part = build_part("mixer", spec, dtype=TD[dtype], device=torch.device(DEV))
+    W = {k: stored(rng.standard_normal(s_.shape) * 0.3, dtype) for k, s_ in part.tensors().items()}
+    part.load({k: t.to(DEV) for k, t in W.items()})
+    Wn = {k: t.float().numpy() for k, t in W.items()}
+    h = stored(rng.standard_normal((n, d)), dtype)
+    hn = h.float().numpy()
+    cos, sin = P.rope_table(512, hs, 1000.0)
+    pos = np.arange(n)
+    q = P.rope_rotate(P.linear(hn, Wn["q"]).reshape(n, H, hs), pos, cos, sin, "half")
+    k = P.rope_rotate(P.linear(hn, Wn["k"]).reshape(n, Kh, hs), pos, cos, sin, "half")
+    v = P.linear(hn, Wn["v"]).reshape(n, Kh, hs)
+    ref = P.linear(P.attention(q, k, v, window=window).reshape(n, H * hs), Wn["o"])
+    harness = Harness([part.kv_need()], [None], dtype, max_tokens=64 * 5)    # five pages for 420 tokens
+    slot = harness.cache.take_slot()
+    run = RunInfo(entry=0, kv_entry=0, writes_kv=True)
+    outs, held = [], []
+    cuts = [0, 100, 101, 102, 190, 260, 261, 300, 301, 302, 303, 420]       # chunks, and tokens one by one
+    for lo, hi in zip(cuts[:-1], cuts[1:]):
+        x = torch.zeros(hi - lo, d, device=DEV)
+        part.forward(harness.context([(slot, hi - lo)]), h[lo:hi].to(DEV), x, run)
+        outs.append(x.cpu().numpy())
+        held.append(sum(1 for p_ in harness.cache.slots.pages[slot][0] if p_))
+    assert max(held) <= 3 and harness.cache.slots.pages[slot][0][0] == 0
+    np.testing.assert_allclose(np.concatenate(outs), ref, atol=(2e-5 if dtype == "float32" else 2e-2) * np.abs(ref).max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_feed_forward_part(dtype):
     from gpullama3_java_amd.config import GatedFeedForwardSpec
     from gpullama3_java_amd.parts import build_part
