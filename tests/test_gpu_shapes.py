@@ -38,7 +38,7 @@ SHAPES = {
 
 
 def steps(eng, vocab):
-    """Logits of every kind of step: a long prompt, single tokens after it, batches of 8, 20 and 40
+    """Logits of every kind of step: a long prompt, single tokens after it, batches of 8, 20, 40 and 100
     sequences (short prompts, then decode steps that are replayed from graphs), prompts of 50, a prompt
     of 2,600 tokens and single tokens after it."""
     rng = np.random.default_rng(0)
@@ -49,7 +49,7 @@ def steps(eng, vocab):
     for t in toks[600:]:
         out.append(eng.step([(s, [t])]).cpu().numpy())
     eng.give_back_slot(s)
-    for B in (8, 20, 40):
+    for B in (8, 20, 40, 100):
         slots = [eng.take_slot() for _ in range(B)]
         seqs = [rng.integers(0, vocab, 7).tolist() for _ in range(B)]
         out.append(eng.step([(sl, q[:4]) for sl, q in zip(slots, seqs)]).cpu().numpy())
@@ -79,7 +79,7 @@ def test_real_layer_sizes_bfloat16_against_float32(tmp_path, shape):
     g.write_random_model(folder, cfg, 11, std=0.02, norm_std=0.1)
     results = {}
     for dtype in ("float32", "bfloat16"):
-        eng = Engine.from_folder(folder, dtype=dtype, max_context=4096, max_tokens=4096, n_slots=48)
+        eng = Engine.from_folder(folder, dtype=dtype, max_context=4096, max_tokens=128 * 64, n_slots=128)
         results[dtype] = steps(eng, cfg.vocab_size)
         if dtype == "bfloat16":
             assert eng._graphs, "the decode steps were not replayed from graphs"
