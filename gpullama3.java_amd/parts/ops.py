@@ -68,6 +68,38 @@ def _next_norm(ctx, N):
     return norm, ctx.buffer("rows_times_norm_weight", (ctx.n_tokens, N), torch.bfloat16)
 
 
+def row_chunks(M):
+    """Steps of 66 to 192 rows are worked on in two or three pieces of 33 to 64 rows: the kernels for
+    so few rows stream the weights at several times the rate of the tiled kernel, whose tiles of
+    128 rows are too few for the chip at these sizes, and the pieces after the first find the
+    weights in the memory-side cache. None: no pieces."""
+    if not 65 < M <= 192:
+        return None
+    n = -(-M // 64)
+    size = -(-M // n)
+    return [(lo, min(M, lo + size)) for lo in range(0, M, size)]
+
+
+def _linear_in_chunks(a, w, out, epilogue, ctx, chunks):
+    M, Kd = a.shape
+    N = out.shape[1]
+    if epilogue != EPI_ADD:
+        for lo, hi in chunks:
+            linear(a[lo:hi], w, out[lo:hi], epilogue)
+        return
+    slices = K.wide_slices(N, Kd)
+    if slices < 2:
+        for lo, hi in chunks:
+            K.gemm_skinny(a[lo:hi], w, out[lo:hi], EPI_ADD)
+        return residual_written(ctx, out)
+    settle_residual(ctx, out)
+    part = ctx.buffer(f"slices{slices}", (slices, M, N), torch.float32)
+    for lo, hi in chunks:
+        K.gemm_skinny_wide(a[lo:hi], w, part[:, lo:hi], EPI_STORE)
+    residual_written(ctx, out)
+    ctx.pending = (out.data_ptr(), part)
+
+
 def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
     """out (=, +=, gated) a @ w.T. ``a`` may be a ``Normed``. With the add epilogue ``out`` is the
     residual stream."""
@@ -77,6 +109,11 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
             return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows)
         a = a.materialize()
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        chunks = row_chunks(a.shape[0])
+        if (chunks and ctx is not None and getattr(ctx, "fuse", False) and not disabled & {"wide", "fused", "skinny"}
+                and K.gemm_skinny_fits(a[:1], w, out[:1], epilogue)
+                and not (epilogue == EPI_STORE and out.shape[1] >= 128 * 512)):     # (the head: the tiled kernel)
+            return _linear_in_chunks(a, w, out, epilogue, ctx, chunks)
         if "wide" not in disabled and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx):
             return
         if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
@@ -159,11 +196,13 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
         return q
     if isinstance(h, Normed):
         h = h.materialize()
+    chunks = row_chunks(T) if getattr(ctx, "fuse", False) and "wide" not in disabled else None
     if (writes_kv and h.dtype == torch.bfloat16 and "fused" not in disabled and "skinny" not in disabled
-            and K.qkv_rope_cache_fits(h, w_qkv, head_dim, rot)):
+            and K.qkv_rope_cache_fits(h[:64], w_qkv, head_dim, rot) and (T <= 64 or chunks)):
         q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
-        K.qkv_rope_cache(h, None, 0, 0.0, w_qkv, q, ctx.positions, ctx.seq_of_token, block_table, cos, sin,
-                         k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page)
+        for lo, hi in (chunks or [(0, T)]):
+            K.qkv_rope_cache(h[lo:hi], None, 0, 0.0, w_qkv, q[lo:hi], ctx.positions[lo:hi], ctx.seq_of_token[lo:hi],
+                             block_table, cos, sin, k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page)
         return q
     if writes_kv:
         qkv = ctx.buffer("qkv", (T, (n_heads + 2 * n_kv) * head_dim), dtype)
