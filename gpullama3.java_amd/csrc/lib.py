@@ -84,7 +84,15 @@ def _check(rc, name):
         raise KernelError(f"{name}: {library().gl3_last_error().decode()}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    """The current stream of the current device (asked for at every launch: a graph capture changes it).
+    The raw handle where this torch offers it: building a stream object costs as much as a launch."""
+    if _raw_stream is not None and _raw_device is not None:
+        return c_void_p(_raw_stream(_raw_device()))
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 

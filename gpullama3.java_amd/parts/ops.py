@@ -68,12 +68,14 @@ def _next_norm(ctx, N):
     return norm, ctx.buffer("rows_times_norm_weight", (ctx.n_tokens, N), torch.bfloat16)
 
 
-def row_chunks(M):
+def row_chunks(M, ctx=None):
     """Steps of 66 to 192 rows are worked on in two or three pieces of 33 to 64 rows: the kernels for
     so few rows stream the weights at several times the rate of the tiled kernel, whose tiles of
     128 rows are too few for the chip at these sizes, and the pieces after the first find the
-    weights in the memory-side cache. None: no pieces."""
-    if not 65 < M <= 192:
+    weights in the memory-side cache. A step that is not replayed from a graph pays for every
+    launch on the host: there three pieces cost more than they gain (measured: 128 rows 2.9 ms
+    in pieces, 192 rows 3.6 ms in pieces against 3.2 ms tiled). None: no pieces."""
+    if not 65 < M <= (192 if ctx is None or getattr(ctx, "decode", False) else 128):
         return None
     n = -(-M // 64)
     size = -(-M // n)
@@ -109,7 +111,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
             return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows)
         a = a.materialize()
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
-        chunks = row_chunks(a.shape[0])
+        chunks = row_chunks(a.shape[0], ctx)
         if (chunks and ctx is not None and getattr(ctx, "fuse", False) and not disabled & {"wide", "fused", "skinny"}
                 and K.gemm_skinny_fits(a[:1], w, out[:1], epilogue)
                 and not (epilogue == EPI_STORE and out.shape[1] >= 128 * 512)):     # (the head: the tiled kernel)
@@ -196,7 +198,7 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
         return q
     if isinstance(h, Normed):
         h = h.materialize()
-    chunks = row_chunks(T) if getattr(ctx, "fuse", False) and "wide" not in disabled else None
+    chunks = row_chunks(T, ctx) if getattr(ctx, "fuse", False) and "wide" not in disabled else None
     if (writes_kv and h.dtype == torch.bfloat16 and "fused" not in disabled and "skinny" not in disabled
             and K.qkv_rope_cache_fits(h[:64], w_qkv, head_dim, rot) and (T <= 64 or chunks)):
         q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
