@@ -6,8 +6,8 @@ import torch
 from ..csrc import lib as K
 from ..weights.loader import TensorSpec
 from .base import register_part
+from .ops import FUSE_ROWS, Normed
 
-FUSE_ROWS = 32      # a norm is folded into the next product for steps of at most this many tokens
 
 
 class RMSNorm:
@@ -33,7 +33,6 @@ class RMSNorm:
         rec = getattr(ctx, "ssq", None)
         if (getattr(ctx, "fuse", False) and rec is not None and rec[0] == x.data_ptr() and rec[4] is self
                 and x.shape[0] <= FUSE_ROWS and self.dtype == torch.bfloat16):
-            from .ops import Normed
             return Normed(ctx, x, self.weight, self.eps, self.dtype, rec[3], rec[1], rec[2], rows, name)
         n = x.shape[0] if rows is None else rows.numel()
         out = ctx.buffer(name, (n, self.dim), self.dtype)

@@ -12,8 +12,8 @@ from ..csrc import lib as K
 
 EPI_STORE, EPI_ADD, EPI_GATED = K.EPI_STORE, K.EPI_ADD, K.EPI_GATED
 
-# a norm is folded into the next product for steps of at most this many tokens: beyond two token
-# tiles the folded kernels run out of registers
+# a norm is folded into the next product for steps of at most this many tokens (two token tiles);
+# larger steps take the kernels for 33 to 64 rows or the tiled ones, with a norm kernel of its own
 FUSE_ROWS = 32
 
 # switches for tests and measurements: names of fast kernels that must not be used
