@@ -54,6 +54,7 @@ def _declare(lib):
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P],
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
+        "gl3_sample_work_floats": [I, I],
         "gl3_argmax": [P, L, P, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
         "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P],
@@ -72,6 +73,7 @@ def _declare(lib):
             continue
         fn.argtypes = args
         fn.restype = c_int
+    lib.gl3_sample_work_floats.restype = ctypes.c_long
     lib._optional = set()
 
 
@@ -296,13 +298,18 @@ def argmax(logits, work, out):
     _check(library().gl3_argmax(_ptr(logits), logits.stride(0), _ptr(work), _ptr(out), R, V, _stream()), "argmax")
 
 
+def sample_work_size(rows, vocab):
+    """Floats of scratch that `sample` and `argmax` need for `rows` rows."""
+    return max(int(library().gl3_sample_work_floats(int(rows), int(vocab))), 128 * rows)
+
+
 def sample(logits, work, temperature, top_p, uniform, out, step=None, uniform_stride=0):
     _dev(logits, "logits", torch.float32, contiguous=False); _dev(work, "work", torch.float32)
     for t, n in ((temperature, "temperature"), (top_p, "top_p"), (uniform, "uniform")):
         _dev(t, n, torch.float32)
     _dev(out, "out", torch.int32)
     R, V = logits.shape
-    if logits.stride(1) != 1 or work.numel() < R * V or min(temperature.numel(), top_p.numel(), uniform.numel(),
+    if logits.stride(1) != 1 or work.numel() < sample_work_size(R, V) or min(temperature.numel(), top_p.numel(), uniform.numel(),
                                                               out.numel()) < R:
         raise KernelError("sample: argument sizes")
     if step is not None:

@@ -1,4 +1,4 @@
-// Token selection on the device: one block per row of logits.
+// Token selection on the device: a row's softmax by many blocks, its choice by one.
 //
 // temperature == 0: the first index of the strictly greatest logit
 //   (J/inference/sampler/Sampler.java:144-157).
@@ -17,11 +17,10 @@
 // the drawn token is the same search with u * mass in place of top_p. Masses are
 // summed as 64-bit integers (p * 2^62), so the order of a sum cannot move a comparison.
 //
-// At most 2^13 probabilities are 2^-13 or more. They are gathered in shared memory while the row
-// is normalised; when their mass alone exceeds top_p, the threshold and the drawn token lie among
-// them and both searches walk that short list instead of the row: three passes over the row in
-// place of twelve. A flat distribution, whose nucleus reaches further down, takes the passes over
-// the whole row.
+// At most 2^13 probabilities are 2^-13 or more. They are gathered while the row is normalised; when
+// their mass alone exceeds top_p, the threshold and the drawn token lie among them and both searches
+// walk that short list, in shared memory, instead of the row. A flat distribution, whose nucleus
+// reaches further down, takes eight passes over the whole row.
 #include "common.h"
 
 #define SB 1024
@@ -156,14 +155,159 @@ __device__ Found radix_search(Src p, int V, unsigned long long thr,
   return Found{};
 }
 
-__global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ logits, long ld, float* __restrict__ work,
+// A row's softmax is made by many blocks, ST_SLICES slices a row, in three kernels (the maximum, the
+// sum, the probabilities), before the row's one block picks the token: a single CU draws too few
+// bytes a second, and has too little arithmetic, for a row of a hundred thousand logits. Rows with
+// temperature 0 are left alone by the three.
+#define ST_SLICES 64
+
+// Scratch of a call, for every row: the probabilities; per slice the maximum, the sum of the
+// exponentials and the mass as an integer; the candidates (probabilities of at least CAND_CUT) with
+// their number and mass.
+struct SampleWork {
+  float* p;                        // [rows, V]
+  double* slice_sum;               // [rows, ST_SLICES]
+  unsigned long long* slice_mass;  // [rows, ST_SLICES]
+  unsigned long long* cand_mass;   // [rows]
+  float* slice_max;                // [rows, ST_SLICES]
+  int* cand_count;                 // [rows]
+  float* cand_p;                   // [rows, CAND_MAX]
+  int* cand_i;                     // [rows, CAND_MAX]
+};
+#define SAMPLE_ROW_FLOATS (ST_SLICES * 5 + 4 + CAND_MAX * 2)   // beside the probabilities, 8-byte units kept whole
+
+static SampleWork carve_sample_work(float* work, int n_rows, int V) {
+  SampleWork w;
+  w.p = work;
+  w.slice_sum = (double*)(work + (((long)n_rows * V + 1) & ~1L));
+  w.slice_mass = (unsigned long long*)(w.slice_sum + (long)n_rows * ST_SLICES);
+  w.cand_mass = w.slice_mass + (long)n_rows * ST_SLICES;
+  w.slice_max = (float*)(w.cand_mass + n_rows);
+  w.cand_count = (int*)(w.slice_max + (long)n_rows * ST_SLICES);
+  w.cand_p = (float*)(w.cand_count + n_rows);
+  w.cand_i = (int*)(w.cand_p + (long)n_rows * CAND_MAX);
+  return w;
+}
+
+__device__ __forceinline__ float row_max_of_slices(const float* slice_max, int row) {
+  float m = slice_max[row * ST_SLICES + (threadIdx.x & (ST_SLICES - 1))];   // every wave holds all 64 slices
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  return m;
+}
+
+__global__ __launch_bounds__(256) void softmax_max_kernel(const float* __restrict__ logits, long ld,
+                                                          const float* __restrict__ temperature, SampleWork w, int V) {
+  __shared__ float fs[16];
+  const int row = blockIdx.x, slice = blockIdx.y, tid = threadIdx.x;
+  const float T = temperature[row];
+  if (T == 0.f) return;
+  if (slice == 0 && tid == 0) { w.cand_count[row] = 0; w.cand_mass[row] = 0ull; }   // for the third kernel
+  const int per = (V + ST_SLICES - 1) / ST_SLICES;
+  const int lo = min(V, slice * per), hi = min(V, lo + per);
+  const float* lg = logits + (long)row * ld;
+  float m = -INFINITY;
+  for (int i = lo + tid; i < hi; i += 256) m = fmaxf(m, lg[i] / T);   // the division of the reference, per element
+  m = block_max(m, fs);
+  if (tid == 0) w.slice_max[row * ST_SLICES + slice] = m;
+}
+
+__global__ __launch_bounds__(256) void softmax_sum_kernel(const float* __restrict__ logits, long ld,
+                                                          const float* __restrict__ temperature, SampleWork w, int V) {
+  __shared__ double ds[16];
+  const int row = blockIdx.x, slice = blockIdx.y, tid = threadIdx.x;
+  const float T = temperature[row];
+  if (T == 0.f) return;
+  const float m = row_max_of_slices(w.slice_max, row);
+  const int per = (V + ST_SLICES - 1) / ST_SLICES;
+  const int lo = min(V, slice * per), hi = min(V, lo + per);
+  const float* lg = logits + (long)row * ld;
+  double z = 0.0;
+  for (int i = lo + tid; i < hi; i += 256) z += (double)expf(lg[i] / T - m);
+  z = block_sum_f64(z, ds);
+  if (tid == 0) w.slice_sum[row * ST_SLICES + slice] = z;
+}
+
+// p = softmax(logits / T) into the scratch, each slice's mass as an integer, and the candidates.
+__global__ __launch_bounds__(256) void softmax_prob_kernel(const float* __restrict__ logits, long ld,
+                                                           const float* __restrict__ temperature,
+                                                           const float* __restrict__ top_p, SampleWork w, int V) {
+  __shared__ unsigned long long qs[2][4];
+  __shared__ float bc_p[8 * 256];
+  __shared__ int bc_i[8 * 256];
+  __shared__ int bc_n, bc_base;
+  const int row = blockIdx.x, slice = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
+  const float T = temperature[row];
+  if (T == 0.f) return;
+  const float m = row_max_of_slices(w.slice_max, row);
+  double z = 0.0;
+  for (int k = 0; k < ST_SLICES; ++k) z += w.slice_sum[row * ST_SLICES + k];   // one order for every thread
+  const float zf = (float)z;
+  const float tp = top_p[row];
+  const bool nucleus = tp > 0.f && tp < 1.f;
+  const int per = (V + ST_SLICES - 1) / ST_SLICES;
+  const int lo = min(V, slice * per), hi = min(V, lo + per);
+  const float* lg = logits + (long)row * ld;
+  float* p = w.p + (long)row * V;
+  unsigned long long mass = 0, cmass = 0;
+  for (int base = lo; base < hi; base += 8 * 256) {
+    if (nucleus) {
+      if (tid == 0) bc_n = 0;
+      __syncthreads();
+    }
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) { const int i = base + u * 256 + tid; v[u] = i < hi ? lg[i] : 0.f; }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = base + u * 256 + tid;
+      if (i < hi) {
+        const float pv = expf(v[u] / T - m) / zf;
+        const unsigned long long q = to_q(pv);
+        p[i] = pv;
+        mass += q;
+        if (nucleus && pv >= CAND_CUT) {
+          const int slot = atomicAdd(&bc_n, 1);   // at most 8 * 256 of them
+          bc_p[slot] = pv;
+          bc_i[slot] = i;
+          cmass += q;
+        }
+      }
+    }
+    if (nucleus) {
+      // the block's candidates of this stretch go to the row's list with one addition to its counter
+      __syncthreads();
+      const int n = bc_n;
+      if (tid == 0 && n > 0) bc_base = atomicAdd(&w.cand_count[row], n);
+      __syncthreads();
+      for (int k = tid; k < n; k += 256) {
+        const int slot = bc_base + k;
+        if (slot < CAND_MAX) {
+          w.cand_p[(long)row * CAND_MAX + slot] = bc_p[k];
+          w.cand_i[(long)row * CAND_MAX + slot] = bc_i[k];
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { mass += __shfl_xor(mass, o, 64); cmass += __shfl_xor(cmass, o, 64); }
+  if (lane == 0) { qs[0][tid >> 6] = mass; qs[1][tid >> 6] = cmass; }
+  __syncthreads();
+  if (tid == 0) {
+    w.slice_mass[row * ST_SLICES + slice] = qs[0][0] + qs[0][1] + qs[0][2] + qs[0][3];
+    const unsigned long long c = qs[1][0] + qs[1][1] + qs[1][2] + qs[1][3];
+    if (c) atomicAdd(&w.cand_mass[row], c);   // integers: the order does not matter
+  }
+}
+
+// The choice, one block a row.
+__global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ logits, long ld, SampleWork w,
                                                     const float* __restrict__ temperature,
                                                     const float* __restrict__ top_p, const float* __restrict__ uniform,
                                                     int* __restrict__ out, int V, const int* __restrict__ step,
                                                     int uniform_stride) {
   __shared__ float fs[16];
   __shared__ int is[16];
-  __shared__ double ds[16];
   __shared__ unsigned long long h_mass[SW][256];
   __shared__ int h_cnt[SW][256];
   __shared__ unsigned long long t_mass[256];
@@ -173,8 +317,7 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
   __shared__ int winner;
   __shared__ float cand_p[CAND_MAX];
   __shared__ int cand_i[CAND_MAX];
-  __shared__ int n_cand;
-  __shared__ unsigned long long cand_mass;
+  __shared__ unsigned long long t_q[SB];
   const int row = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const float* lg = logits + (long)row * ld;
   const float T = temperature[row];
@@ -195,82 +338,42 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
     if ((tid & 63) == 0) { fs[tid >> 6] = best; is[tid >> 6] = idx; }
     __syncthreads();
     if (tid == 0) {
-      for (int w = 1; w < SB / 64; ++w)
-        if (fs[w] > best || (fs[w] == best && is[w] < idx)) { best = fs[w]; idx = is[w]; }
+      for (int w2 = 1; w2 < SB / 64; ++w2)
+        if (fs[w2] > best || (fs[w2] == best && is[w2] < idx)) { best = fs[w2]; idx = is[w2]; }
       out[row] = idx == 0x7fffffff ? 0 : idx;   // all -inf or NaN: index 0, as the reference's loop leaves it
     }
     return;
   }
 
-  // p = softmax(logits / T), kept in `work`
-  float* p = work + (long)row * V;
-  float m = -INFINITY;
-  for (int i0 = tid; i0 < V; i0 += UN * SB) {
-    float v[UN];
-#pragma unroll
-    for (int u = 0; u < UN; ++u) v[u] = (i0 + u * SB < V) ? lg[i0 + u * SB] : -INFINITY;
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const float sc = v[u] / T;                          // the division of the reference, once per element
-      if (i0 + u * SB < V) p[i0 + u * SB] = sc;
-      m = fmaxf(m, sc);
-    }
-  }
-  m = block_max(m, fs);
-  double z = 0.0;
-  for (int i0 = tid; i0 < V; i0 += UN * SB) {
-    float v[UN];
-#pragma unroll
-    for (int u = 0; u < UN; ++u) v[u] = (i0 + u * SB < V) ? p[i0 + u * SB] : 0.f;
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int i = i0 + u * SB;
-      if (i < V) {
-        const float e = expf(v[u] - m);
-        p[i] = e;
-        z += (double)e;
-      }
-    }
-  }
-  const float zf = (float)block_sum_f64(z, ds);
+  const float* p = w.p + (long)row * V;
   const float tp = top_p[row];
-  const bool nucleus = tp > 0.f && tp < 1.f;
-  if (tid == 0) { n_cand = 0; cand_mass = 0ull; }
-  __syncthreads();
-  unsigned long long my_mass = 0;
-  for (int i0 = tid; i0 < V; i0 += UN * SB) {
-    float v[UN];
-#pragma unroll
-    for (int u = 0; u < UN; ++u) v[u] = (i0 + u * SB < V) ? p[i0 + u * SB] : 0.f;
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int i = i0 + u * SB;
-      if (i < V) {
-        const float pv = v[u] / zf;
-        p[i] = pv;
-        if (nucleus && pv >= CAND_CUT) {
-          const int slot = atomicAdd(&n_cand, 1);
-          if (slot < CAND_MAX) { cand_p[slot] = pv; cand_i[slot] = i; }
-          my_mass += to_q(pv);
-        }
-      }
-    }
-  }
-  if (nucleus && my_mass) atomicAdd(&cand_mass, my_mass);   // integers: the order does not matter
-  __syncthreads();
-
   // in a run of steps replayed from a graph the step's number is read from memory
   const double u = (double)uniform[(step ? (long)step[0] * uniform_stride : 0) + row];
-  // every wave owns a contiguous range of the row, a multiple of 64 long
-  const int per = ((V + SW - 1) / SW + 63) / 64 * 64;
-  const int lo = min(V, wave * per), hi = min(V, lo + per);
   if (tid == 0) winner = -1;
+  __syncthreads();
 
-  float want_value = 0.f;             // top-p: the drawn token is the `want_index`-th (from 0) with this probability
-  long want_index = 0;
   if (tp <= 0.f || tp >= 1.f) {
-    // the first index whose running sum in index order exceeds u
+    // the first index whose running sum in index order exceeds u: first the slice, by the slices' masses
     const unsigned long long uq = (unsigned long long)(u * QSCALE);   // u = k / 2^24: exact
+    const unsigned long long sm = w.slice_mass[row * ST_SLICES + lane];
+    unsigned long long sincl = sm;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const unsigned long long y = __shfl_up(sincl, o, 64);
+      if (lane >= o) sincl += y;
+    }
+    const unsigned long long shit = __ballot(uq < sincl);
+    if (!shit) {                      // u lies beyond the whole mass: the last index
+      if (tid == 0) out[row] = V - 1;
+      return;
+    }
+    const int slice = __ffsll((long long)shit) - 1;
+    const unsigned long long before_slice = __shfl(sincl - sm, slice, 64);
+    const int sper = (V + ST_SLICES - 1) / ST_SLICES;
+    const int r_lo = min(V, slice * sper), r_hi = min(V, r_lo + sper);
+    // every wave owns a contiguous part of the slice, a multiple of 64 long
+    const int per = ((r_hi - r_lo + SW - 1) / SW + 63) / 64 * 64;
+    const int lo = min(r_hi, r_lo + wave * per), hi = min(r_hi, lo + per);
     unsigned long long mine = 0;
     for (int i0 = lo + lane; i0 < hi; i0 += 8 * 64) {
       float v[8];
@@ -283,9 +386,9 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
     for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
     if (lane == 0) w_tot[wave] = mine;
     __syncthreads();
-    unsigned long long before = 0;
-    for (int w = 0; w < wave; ++w) before += w_tot[w];
-    if (before <= uq && uq < before + w_tot[wave]) {       // the crossing lies in this wave's range
+    unsigned long long before = before_slice;
+    for (int w2 = 0; w2 < wave; ++w2) before += w_tot[w2];
+    if (before <= uq && uq < before + w_tot[wave]) {       // the crossing lies in this wave's part
       for (int base = lo; base < hi; base += 64) {
         const int i = base + lane;
         const unsigned long long q = i < hi ? to_q(p[i]) : 0;
@@ -310,9 +413,40 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
 
   // nucleus: the threshold value, the mass above it, and how many of the equal ones are kept
   const unsigned long long tq = (unsigned long long)((double)tp * QSCALE);
-  if (n_cand <= CAND_MAX && cand_mass > tq) {
+  const int n_cand = w.cand_count[row];
+  if (n_cand <= CAND_MAX && w.cand_mass[row] > tq) {
     // the candidates alone exceed top_p: every probability from the threshold upwards is among them
     const int n = n_cand;
+    for (int a = tid; a < n; a += SB) {
+      cand_p[a] = w.cand_p[(long)row * CAND_MAX + a];
+      cand_i[a] = w.cand_i[(long)row * CAND_MAX + a];
+    }
+    __syncthreads();
+    if (n <= SB) {
+      // few candidates, one a thread: the mass that stands before each in the kept order (descending
+      // probability, equal ones by ascending index) is summed directly. A candidate is kept if the
+      // mass before it does not exceed top_p; the drawn one is that whose stretch holds u * kept mass.
+      float pa = 0.f;
+      int ia = 0;
+      unsigned long long qa = 0;
+      if (tid < n) { pa = cand_p[tid]; ia = cand_i[tid]; qa = to_q(pa); }
+      if (tid < n) t_q[tid] = qa;
+      if (tid == 0) res[0] = w.cand_mass[row];
+      __syncthreads();
+      unsigned long long excl = 0;
+      if (tid < n)
+        for (int b = 0; b < n; ++b) {
+          const float pb = cand_p[b];
+          excl += (pb > pa || (pb == pa && cand_i[b] < ia)) ? t_q[b] : 0ull;
+        }
+      if (tid < n && excl <= tq && tq < excl + qa) res[0] = excl + qa;   // the last kept one: the kept mass
+      __syncthreads();
+      const unsigned long long target = (unsigned long long)(u * (double)res[0]);
+      if (tid < n && excl <= target && target < excl + qa) winner = ia;
+      __syncthreads();
+      if (tid == 0) out[row] = winner >= 0 ? winner : V - 1;
+      return;
+    }
     const Found f1 = radix_search(cand_p, n, tq, h_mass, h_cnt, t_mass, t_cnt, res);
     long k1 = 1;
     if (f1.each > 0 && tq >= f1.above) k1 = (long)((tq - f1.above) / f1.each) + 1;
@@ -351,10 +485,12 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
   const long limit = (f2.bits == f1.bits) ? k1 : (long)f2.ties;
   if (j > limit - 1) j = limit - 1;
   if (j < 0) j = 0;
-  want_value = __uint_as_float(f2.bits);
-  want_index = j;
+  const float want_value = __uint_as_float(f2.bits);   // the drawn token is the `want_index`-th (from 0) with this
+  const long want_index = j;                           // probability, in ascending order of index
 
-  // the want_index-th index, in ascending order, whose probability is want_value
+  // every wave owns a contiguous range of the row, a multiple of 64 long
+  const int per = ((V + SW - 1) / SW + 63) / 64 * 64;
+  const int lo = min(V, wave * per), hi = min(V, lo + per);
   int mine = 0;
   for (int i0 = lo + lane; i0 < hi; i0 += 8 * 64) {
     float v[8];
@@ -368,7 +504,7 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
   if (lane == 0) w_tot[wave] = (unsigned long long)mine;
   __syncthreads();
   long before = 0;
-  for (int w = 0; w < wave; ++w) before += (long)w_tot[w];
+  for (int w2 = 0; w2 < wave; ++w2) before += (long)w_tot[w2];
   if (before <= want_index && want_index < before + (long)w_tot[wave]) {
     for (int base = lo; base < hi; base += 64) {
       const int i = base + lane;
@@ -450,15 +586,31 @@ extern "C" int gl3_argmax(const float* logits, long ld, float* work, int* out, i
   return 0;
 }
 
-// work: [n_rows, V] floats of scratch (probabilities); unused for greedy rows.
+// Floats of scratch that gl3_sample needs: the rows' probabilities and, per row, what the kernels
+// hand to each other.
+extern "C" long gl3_sample_work_floats(int n_rows, int V) {
+  return (((long)n_rows * V + 1) & ~1L) + (long)n_rows * SAMPLE_ROW_FLOATS;
+}
+
+// work: gl3_sample_work_floats(n_rows, V) floats of scratch, 8-byte aligned.
 // step (may be null): a counter in device memory; row r then takes uniform[step[0] * uniform_stride + r].
 extern "C" int gl3_sample(const float* logits, long ld, float* work, const float* temperature, const float* top_p,
                           const float* uniform, int* out, int n_rows, int V, const int* step, int uniform_stride,
                           hipStream_t stream) {
   if (n_rows == 0) return 0;
   GL3_REQUIRE(logits && work && temperature && top_p && uniform && out, "gl3_sample: null argument");
-  GL3_REQUIRE(n_rows > 0 && V > 0 && ld >= V, "gl3_sample: bad sizes (rows=%d V=%d ld=%ld)", n_rows, V, ld);
-  sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, ld, work, temperature, top_p, uniform, out, V, step,
+  GL3_REQUIRE(n_rows > 0 && n_rows <= 65535 && V > 0 && ld >= V, "gl3_sample: bad sizes (rows=%d V=%d ld=%ld)", n_rows, V,
+              ld);
+  GL3_REQUIRE((uintptr_t)work % 8 == 0, "gl3_sample: the scratch must be 8-byte aligned");
+  const SampleWork w = carve_sample_work(work, n_rows, V);
+  const dim3 slices(n_rows, ST_SLICES);
+  softmax_max_kernel<<<slices, dim3(256), 0, stream>>>(logits, ld, temperature, w, V);
+  GL3_LAUNCH_CHECK();
+  softmax_sum_kernel<<<slices, dim3(256), 0, stream>>>(logits, ld, temperature, w, V);
+  GL3_LAUNCH_CHECK();
+  softmax_prob_kernel<<<slices, dim3(256), 0, stream>>>(logits, ld, temperature, top_p, w, V);
+  GL3_LAUNCH_CHECK();
+  sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, ld, w, temperature, top_p, uniform, out, V, step,
                                                        uniform_stride);
   GL3_LAUNCH_CHECK();
   return 0;

@@ -345,7 +345,7 @@ class Engine:
             from ..csrc import lib as K
             dg.fhost = torch.zeros((2 + RUN_LENGTH) * B_pad, dtype=torch.float32).pin_memory()
             dg.fdev = torch.zeros((2 + RUN_LENGTH) * B_pad, dtype=torch.float32, device=self.device)
-            work = torch.empty(B_pad * max(self.spec.vocab_size, 128), dtype=torch.float32, device=self.device)
+            work = torch.empty(K.sample_work_size(B_pad, self.spec.vocab_size), dtype=torch.float32, device=self.device)
             step = d[dg.off_step:dg.off_step + 1]
             sampled = d[dg.off_sampled:dg.off_sampled + B_pad]
             hist = d[dg.off_hist:dg.off_hist + RUN_LENGTH * B_pad].view(RUN_LENGTH, B_pad)

@@ -92,8 +92,8 @@ class DeviceSampler:
         R, V = logits.shape
         if R == 0:
             return []
-        if self._work is None or self._work.numel() < max(R * V, 128 * R):
-            self._work = torch.empty(max(R * V, 128 * R), dtype=torch.float32, device=self.device)
+        if self._work is None or self._work.numel() < K.sample_work_size(R, V):
+            self._work = torch.empty(K.sample_work_size(R, V), dtype=torch.float32, device=self.device)
         out = torch.empty(R, dtype=torch.int32, device=self.device)
         if all(t == 0 for t in temperatures):           # every row greedy: the rows are read by many blocks at once
             K.argmax(logits, self._work, out)

@@ -346,7 +346,7 @@ def test_sample_kernel(V):
     us = rng.random(R).astype(np.float32)
     us[4] = 0.0; us[6] = np.float32(0.99999994)
     out = torch.empty(R, dtype=torch.int32, device=DEV)
-    K().sample(dev(logits), torch.empty(R * V, device=DEV), dev(temps), dev(tops), dev(us), out)
+    K().sample(dev(logits), torch.empty(K().sample_work_size(R, V), device=DEV), dev(temps), dev(tops), dev(us), out)
     for r, tok in enumerate(out.tolist()):
         assert 0 <= tok < V
         check_draw(logits[r], float(temps[r]), float(tops[r]), float(us[r]), tok)
@@ -367,7 +367,8 @@ def test_sample_kernel_nucleus_from_the_short_list_and_from_the_whole_row():
         rows.append(peaked); temps.append(0.5); tops.append(tp)
     flat = (rng.standard_normal(V) * 0.5).astype(np.float32)               # no probability reaches 2^-13
     rows.append(flat); temps.append(1.0); tops.append(0.9)
-    for n_equal in (8192, 8193, 100):                                       # the list full, one more than it holds, few
+    # the list full, one more than it holds, few, and as many as the choosing block has threads, and one more
+    for n_equal in (8192, 8193, 100, 1024, 1025):
         r = np.full(V, -np.inf, np.float32)
         r[rng.choice(V, n_equal, replace=False)] = 1.5
         rows.append(r); temps.append(1.0); tops.append(0.7)
@@ -385,7 +386,7 @@ def test_sample_kernel_nucleus_from_the_short_list_and_from_the_whole_row():
         if trial == 1:
             us[:] = np.float32(0.99999994)
         out = torch.empty(R, dtype=torch.int32, device=DEV)
-        lib.sample(dev(logits), torch.empty(R * V, device=DEV), dev(np.array(temps, np.float32)),
+        lib.sample(dev(logits), torch.empty(lib.sample_work_size(R, V), device=DEV), dev(np.array(temps, np.float32)),
                    dev(np.array(tops, np.float32)), dev(us), out)
         for r, tok in enumerate(out.tolist()):
             check_draw(logits[r], temps[r], tops[r], float(us[r]), tok)
@@ -399,7 +400,7 @@ def test_sample_kernel_frequencies_and_rules():
     us = rng.random(R).astype(np.float32)
     out = torch.empty(R, dtype=torch.int32, device=DEV)
     lib = K()
-    work = torch.empty(R * V, device=DEV)
+    work = torch.empty(lib.sample_work_size(R, V), device=DEV)
     lib.sample(dev(logits), work, dev(np.full(R, 1.0)), dev(np.full(R, 1.0)), dev(us), out)
     p = P.probabilities(row, 1.0)
     counts = np.bincount(out.cpu().numpy(), minlength=V)
