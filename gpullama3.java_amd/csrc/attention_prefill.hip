@@ -200,8 +200,9 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
       const int ck = base + r;
       if (ck > ck1) break;
       const int key0 = ck * 32;
-      // the registers of this chunk are free (it lies in shared memory): ask for the chunk three further
-      if (ck + AHEAD <= ck1) fetch(ck + AHEAD, rk[r], rv[r]);
+      // the registers of this chunk are free (it lies in shared memory): ask for the chunk three further;
+      fetch(min(ck + AHEAD, ck1), rk[r], rv[r]);   // unconditional (the last chunk again at the end): a branch
+                                                   // around the loads makes the compiler wait for all of them at once
       if (ck >= ck_first && ck <= ck_last) {
         bf16x8 ka[KK], kb2[KK], vt[DT];
 #pragma unroll

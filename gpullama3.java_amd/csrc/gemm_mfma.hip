@@ -51,24 +51,31 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   const int m0 = (tile % tiles_m) * BM;
   const int n0 = (tile / tiles_m) * NCOLS;
 
-  // global -> register staging in chunks of 16 bytes
-  const bf16_t* ap[NA];
-  const bf16_t* wp[NWC];
+  // global -> register staging in chunks of 16 bytes. An address is a base that the whole block
+  // shares (it lives in scalar registers and takes the k-step) plus a 32-bit offset of the thread
+  // inside the tile, and every load is unconditional (rows and columns beyond the matrix are
+  // clamped to its last ones and their values dropped): no branch around a load, whose registers
+  // the compiler would then wait for at once.
+  const bf16_t* a_tile = A + (long)m0 * lda;
+  const bf16_t* w_tile[2];
+  w_tile[0] = W + (long)n0 * ldw;
+  w_tile[1] = (EPI == MF_GATED) ? W + ((long)N + n0) * ldw : w_tile[0];
+  static_assert(EPI != MF_GATED || (NWC % 2 == 0 && (NT / 8) * (NWC / 2) == BN / 2),
+                "gate rows and up rows must fall to different loads of a thread");
+  unsigned aoff[NA], woff[NWC];
   int arow_s[NA], wrow_s[NWC];
   const int scol = (tid & 7) * 8;
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
     arow_s[i] = (tid + NT * i) >> 3;
-    ap[i] = A + (long)min(m0 + arow_s[i], M - 1) * lda + scol;
+    aoff[i] = (unsigned)(min(m0 + arow_s[i], M - 1) - m0) * (unsigned)lda;
   }
 #pragma unroll
   for (int i = 0; i < NWC; ++i) {
     const int r = (tid + NT * i) >> 3;
     wrow_s[i] = r;
-    int wr;
-    if (EPI == MF_GATED) wr = r < BN / 2 ? min(n0 + r, N - 1) : N + min(n0 + r - BN / 2, N - 1);
-    else wr = min(n0 + r, N - 1);
-    wp[i] = W + (long)wr * ldw + scol;
+    const int rel = (EPI == MF_GATED && i >= NWC / 2) ? r - BN / 2 : r;
+    woff[i] = (unsigned)(min(n0 + rel, N - 1) - n0) * (unsigned)ldw;
   }
   // K in slices (blockIdx.y): slice 0 ends in the epilogue proper, the others store their sums
   // as floats into P[slice - 1], for the reader to add up in slice order
@@ -77,12 +84,19 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   K = min(K, k_begin + k_per_slice);
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   bf16x8 ra[NA], rw[NWC];
+  bool r_ok = false;                                   // whether the registers hold columns inside K
   auto fetch = [&](int k0) {
-    const bool ok = k0 + scol < K;
+    const int kf = min(k0, K - 8);                     // the step after the last one reads the last again
+    r_ok = k0 + scol < K;
+    const unsigned col = (unsigned)min(scol, K - 8 - kf);
+    const bf16_t* ak = a_tile + kf;
 #pragma unroll
-    for (int i = 0; i < NA; ++i) ra[i] = ok ? *(const bf16x8*)(ap[i] + k0) : zero;
+    for (int i = 0; i < NA; ++i) ra[i] = *(const bf16x8*)(ak + (aoff[i] + col));
 #pragma unroll
-    for (int i = 0; i < NWC; ++i) rw[i] = ok ? *(const bf16x8*)(wp[i] + k0) : zero;
+    for (int i = 0; i < NWC; ++i) {
+      const bf16_t* wk = w_tile[(EPI == MF_GATED && i >= NWC / 2) ? 1 : 0] + kf;
+      rw[i] = *(const bf16x8*)(wk + (woff[i] + col));
+    }
   };
   fetch(k_begin);
 
@@ -99,12 +113,18 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   const int wrow1 = (EPI == MF_GATED) ? BN / 2 + wn * 32 + lr : wn * 64 + 32 + lr;
 
   for (int k0 = k_begin; k0 < K; k0 += MF_BK) {
+    if (k0 + MF_BK <= K) {   // a whole step (the same for the whole block): nothing to drop
 #pragma unroll
-    for (int i = 0; i < NA; ++i) *(bf16x8*)&As[arow_s[i]][scol] = ra[i];
+      for (int i = 0; i < NA; ++i) *(bf16x8*)&As[arow_s[i]][scol] = ra[i];
 #pragma unroll
-    for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[wrow_s[i]][scol] = rw[i];
+      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[wrow_s[i]][scol] = rw[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < NA; ++i) *(bf16x8*)&As[arow_s[i]][scol] = r_ok ? ra[i] : zero;
+#pragma unroll
+      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[wrow_s[i]][scol] = r_ok ? rw[i] : zero;
+    }
     __syncthreads();
-    if (k0 + MF_BK < K) fetch(k0 + MF_BK);
 #pragma unroll
     for (int kk = 0; kk < MF_BK / 16; ++kk) {
       const int kc = kk * 16 + lh * 8;
@@ -115,6 +135,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
         const bf16x8 a = *(const bf16x8*)&As[arow + 32 * tm][kc];
         acc[tm][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, acc[tm][0], 0, 0, 0);
         acc[tm][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, acc[tm][1], 0, 0, 0);
+      }
+      if (kk == 0) {
+        // the next step's loads go out behind the first products (which cover the address
+        // arithmetic), and their values are first looked at when they are written to shared
+        // memory: the scheduler may not move either across the fences
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(k0 + MF_BK);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     __syncthreads();
@@ -177,11 +205,11 @@ static int launch_shape(const void* A, const void* W, void* C, int M, int N, int
 template <int EPI, typename TC>
 static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
                        int slices, float* P, long p_stride, long ldp, hipStream_t stream) {
-  // 256 x 256 tiles of sixteen waves where they still give two blocks per CU: half the operand
+  // 256 x 256 tiles of sixteen waves where there is at least one for every CU: half the operand
   // traffic per product, and that traffic is what bounds the large products. Otherwise 128 x 128
   // tiles of eight waves, of which several fit a CU and overlap each other's waits.
   const long big_n = (EPI == MF_GATED) ? (N + 127) / 128 : (N + 255) / 256;
-  if ((long)((M + 255) / 256) * big_n * slices >= 512)
+  if ((long)((M + 255) / 256) * big_n * slices >= 256)
     return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, stream);
   return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, stream);
 }
@@ -197,6 +225,9 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_mfma: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gl3_gemm_mfma: K=%d, lda=%ld, ldw=%ld must be multiples of 8",
               K, lda, ldw);
+  GL3_REQUIRE(lda > 0 && ldw > 0 && lda < (1L << 22) && ldw < (1L << 22),
+              "gl3_gemm_mfma: lda=%ld, ldw=%ld: rows of 2^22 elements or more are not built (32-bit offsets in a tile)",
+              lda, ldw);
   GL3_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gl3_gemm_mfma: operands must be 16-byte aligned");
   GL3_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gl3_gemm_mfma: leading dimensions too small");
   GL3_REQUIRE(epilogue >= 0 && epilogue <= 2, "gl3_gemm_mfma: unknown epilogue %d", epilogue);
