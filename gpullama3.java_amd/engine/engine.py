@@ -397,14 +397,37 @@ class Engine:
         self.metrics = RunMetrics()
         return generate(self, reqs, on_token=on_token, max_batch=max_batch, metrics=self.metrics)
 
-    def generate_tokens(self, prompt_tokens, stop_tokens, max_tokens, sampler, echo=False, on_token_generated=None):
+    def create_new_state(self):
+        """A sequence that outlives a call of ``generate_tokens``: it holds a slot of the cache
+        until ``close`` (the reference's ``createNewState``, J/model/Model.java:78; there the state
+        is the cache itself)."""
+        return SequenceState(self, self.take_slot())
+
+    def generate_tokens(self, prompt_tokens, stop_tokens, max_tokens, sampler, echo=False, on_token_generated=None,
+                        state=None, start_position=0):
         """One sequence, in the reference's own terms (J/model/Model.java:66,
         J/inference/InferenceEngine.java:67-141): ``max_tokens`` bounds the position
         (prompt and generated together; negative: the context length), the returned
-        list holds the generated tokens only, a stop token included."""
+        list holds the generated tokens only, a stop token included.
+
+        With a ``state`` the sequence goes on in that state's slot: ``prompt_tokens`` follow the
+        ``start_position`` tokens that the slot holds already (the reference's chat loop,
+        Model.java:136). The token sampled last is not in the cache when the call returns, as in
+        the reference; ``state.length`` says how many are, and the next call's tokens start there."""
         limit = self.max_context if max_tokens is None or max_tokens < 0 else min(max_tokens, self.max_context)
-        new = limit - len(prompt_tokens) + 1
-        req = Request(list(prompt_tokens), new, sampler, frozenset(stop_tokens or ()))
+        if state is None:
+            if start_position:
+                raise ValueError("a start position needs the state that holds the tokens before it")
+            slot = None
+        else:
+            if state.closed:
+                raise ValueError("the state has been closed")
+            if start_position != state.length:
+                raise ValueError(f"the state holds {state.length} tokens; the next tokens start there, "
+                                 f"not at {start_position}")
+            slot = state.slot
+        new = limit - start_position - len(prompt_tokens) + 1
+        req = Request(list(prompt_tokens), new, sampler, frozenset(stop_tokens or ()), slot=slot, cached=start_position)
 
         def seen(_, tok):
             if echo:
@@ -417,4 +440,27 @@ class Engine:
         return generate(self, [req], on_token=seen, metrics=self.metrics)[0].tokens
 
 
-__all__ = ["Engine", "CacheFull", "Generated", "Request", "RunMetrics"]
+class SequenceState:
+    """The slot of a sequence that goes on over several calls."""
+
+    def __init__(self, engine, slot):
+        self.engine, self.slot, self.closed = engine, slot, False
+
+    @property
+    def length(self):
+        """Tokens of the sequence that the cache holds."""
+        return self.engine.cache.length(self.slot)
+
+    def close(self):
+        if not self.closed:
+            self.engine.give_back_slot(self.slot)
+            self.closed = True
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+
+__all__ = ["Engine", "SequenceState", "CacheFull", "Generated", "Request", "RunMetrics"]

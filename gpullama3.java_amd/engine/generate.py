@@ -31,6 +31,10 @@ class Request:
     max_new_tokens: int
     sampling: SamplingParams = SamplingParams()
     stop_ids: frozenset = frozenset()
+    # a sequence that goes on: the slot that holds its earlier tokens (kept when the request ends)
+    # and how many they are; ``prompt`` then holds the tokens that follow them
+    slot: Optional[int] = None
+    cached: int = 0
 
 
 @dataclass
@@ -83,11 +87,19 @@ def generate(backend, requests, on_token: Optional[Callable[[int, int], None]] =
     for i, r in enumerate(requests):
         if len(r.prompt) == 0:
             raise ValueError(f"request {i} has an empty prompt")
-        if len(r.prompt) > backend.max_context:
-            raise ValueError(f"request {i}: a prompt of {len(r.prompt)} tokens exceeds the context of "
+        if r.cached + len(r.prompt) > backend.max_context:
+            raise ValueError(f"request {i}: a prompt of {r.cached + len(r.prompt)} tokens exceeds the context of "
                              f"{backend.max_context}")
+        if r.slot is None and r.cached:
+            raise ValueError(f"request {i} names earlier tokens but no slot that holds them")
     results = [Generated() for _ in requests]
     metrics = metrics if metrics is not None else RunMetrics()
+    if any(r.slot is not None for r in requests):
+        # sequences that go on hold their slots already: they form one batch as they are
+        if len({r.slot for r in requests}) != len(requests) or any(r.slot is None for r in requests):
+            raise ValueError("sequences that go on must each name a slot of their own, and all of a call must go on")
+        _run_batch(backend, requests, results, range(len(requests)), on_token, metrics)
+        return results
     first = 0
     while first < len(requests):
         slots = backend.slots_free()
@@ -107,10 +119,14 @@ def _run_batch(backend, requests, results, ids, on_token, metrics):
             if requests[i].max_new_tokens <= 0:
                 results[i].finish_reason = "length"
                 continue
-            live.append((i, backend.take_slot()))
+            live.append((i, requests[i].slot if requests[i].slot is not None else backend.take_slot()))
         if not live:
             return
-        held = {i: len(requests[i].prompt) for i, _ in live}
+        held = {i: requests[i].cached + len(requests[i].prompt) for i, _ in live}
+
+        def leave(i, slot):
+            if requests[i].slot is None:         # a slot that the caller holds stays the caller's
+                backend.give_back_slot(slot)
 
         def take(i, slot, tok):
             """Record a sampled token; true if the sequence goes on."""
@@ -140,7 +156,7 @@ def _run_batch(backend, requests, results, ids, on_token, metrics):
             if take(i, slot, tok):
                 nxt.append((i, slot))
             else:
-                backend.give_back_slot(slot)
+                leave(i, slot)
         live = nxt
 
         # then one token per live sequence and step. A backend may run several steps before it
@@ -148,6 +164,8 @@ def _run_batch(backend, requests, results, ids, on_token, metrics):
         # such a run leaves the batch at the run's end, and what it sampled after its end is
         # dropped. No run is longer than the shortest remaining budget of its sequences.
         most = max(1, int(getattr(backend, "decode_run_length", 1)))
+        if any(requests[i].slot is not None for i, _ in live):
+            most = 1     # a slot that is kept must hold the sequence's own tokens only, none sampled after its end
         while live:
             rows = [i for i, _ in live]
             n = min([most] + [min(requests[i].max_new_tokens - len(results[i].tokens),
@@ -174,12 +192,12 @@ def _run_batch(backend, requests, results, ids, on_token, metrics):
                 if going[i]:
                     nxt.append((i, slot))
                 else:
-                    backend.give_back_slot(slot)
+                    leave(i, slot)
             live = nxt
     except BaseException:
-        for _, slot in live:
+        for i, slot in live:
             try:
-                backend.give_back_slot(slot)
+                leave(i, slot)
             except Exception:
                 pass
         raise

@@ -216,3 +216,24 @@ def test_runs_of_steps_give_the_same_tokens_and_respect_every_budget():
     p = prompts([10], seed=10)[0]
     out = generate(tight, [Request(p, 50, sp)])[0]
     assert len(out.tokens) == 7 and out.finish_reason == "length"         # 16 - 10 fed back, one more sampled
+
+
+def test_a_sequence_that_goes_on_keeps_its_slot_and_runs_single_steps():
+    """A request that names a slot continues that slot's sequence: the slot is neither taken nor
+    given back, its steps are single ones (no token sampled after the sequence's end may reach a
+    slot that is kept), and the result is the one of the whole sequence in one request."""
+    be = RunBackend()
+    prompt = [5, 9, 2, 7]
+    whole = generate(RunBackend(), [Request(prompt, 9, SamplingParams())])[0].tokens
+    s = be.take_slot()
+    first = generate(be, [Request(prompt, 4, SamplingParams(), slot=s, cached=0)])[0].tokens
+    assert first == whole[:4] and be.runs == [] and s in be.seqs
+    assert be.cache.length(s) == len(prompt) + 3            # the last sampled token has not been fed
+    rest = generate(be, [Request([first[-1]], 5, SamplingParams(), slot=s, cached=be.cache.length(s))])[0].tokens
+    # the draw's index restarts with a request, greedy does not care
+    assert first + rest == whole and be.cache.slots.n_free == be.n_slots - 1
+    be.give_back_slot(s)
+    with pytest.raises(ValueError, match="no slot"):
+        generate(be, [Request([1], 2, SamplingParams(), cached=3)])
+    with pytest.raises(ValueError, match="slot of their own"):
+        generate(be, [Request([1], 2, SamplingParams(), slot=0, cached=0), Request([1], 2, SamplingParams())])

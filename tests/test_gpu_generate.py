@@ -114,3 +114,74 @@ def test_command_line(tmp_path):
     assert bad.returncode != 0 and "--top-p must be within [0, 1]" in bad.stderr
     noprompt = subprocess.run(cmd[:4] + ["--prompt", "hello"], capture_output=True, text=True, timeout=300)
     assert noprompt.returncode != 0 and "tokenizer.json" in noprompt.stderr
+
+
+def test_a_sequence_goes_on_in_its_state():
+    """Two calls on one state give what one sequence gives: the second call's tokens follow those
+    that the slot holds (the reference's chat loop, J/model/Model.java:136), the slot is kept
+    between the calls and given back at the end."""
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.sampling import SamplingParams
+    folder, _, _ = model("B")
+    eng = g.load_model(folder, dtype="float32", max_tokens=1024)
+    free = eng.slots_free()
+    first = rand_tokens("B", 60, 9)
+    with eng.create_new_state() as state:
+        assert eng.slots_free() == free - 1 and state.length == 0
+        a = eng.generate_tokens(first, (), len(first) + 5, SamplingParams(), state=state, start_position=0)
+        assert a == plain_greedy("B", first, len(a)) and len(a) == 6
+        assert state.length == len(first) + len(a) - 1            # the token sampled last has not been fed
+        with pytest.raises(ValueError, match="start there"):
+            eng.generate_tokens([1], (), 64, SamplingParams(), state=state, start_position=3)
+        more = rand_tokens("B", 61, 4)
+        seq = first + a + more
+        start = state.length
+        b = eng.generate_tokens(seq[start:], (), len(seq) + 4, SamplingParams(), state=state, start_position=start)
+        assert b == plain_greedy("B", seq, len(b)) and len(b) == 5
+        assert eng.slots_free() == free - 1
+    assert eng.slots_free() == free
+    with pytest.raises(ValueError, match="closed"):
+        eng.generate_tokens([1], (), 64, SamplingParams(), state=state, start_position=0)
+
+
+def test_chat_loop_keeps_the_dialogue_in_the_cache():
+    """The interactive loop with a toy tokenizer over a tiny model: every turn's answer is the plain
+    implementation's greedy continuation of the whole dialogue so far. A random model never emits the
+    end-of-turn id on purpose, so the toy format stops at a class of ordinary ids as well, chosen so
+    that both turns end by it."""
+    import argparse
+    import io
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd import cli
+    from gpullama3_java_amd.chat import ASSISTANT, USER, SYSTEM, LlamaChatFormat, Message
+    from test_chat_format import ToyTokenizer
+    folder, cfgd, _ = model("B")       # its head is its own: a tied one repeats the last token
+    limit = 100
+    lines = ["hi", "more", "quit", "never read"]
+    tok = ToyTokenizer()
+    chosen = None
+    for modulus, rest in ((2, 0), (2, 1), (3, 0), (3, 1), (3, 2)):
+        chat = LlamaChatFormat(tok)
+        chat.stop_tokens = frozenset(chat.stop_tokens) | frozenset(t for t in range(200) if t % modulus == rest)
+        conv = [chat.begin_of_text] + chat.encode_message(Message(SYSTEM, "s"))
+        ok = True
+        for line in lines[:2]:
+            conv += chat.encode_message(Message(USER, line)) + chat.encode_header(Message(ASSISTANT, ""))
+            gen = plain_greedy("B", conv, 12)
+            ends = [k for k, t in enumerate(gen) if t in chat.stop_tokens]
+            if not ends or ends[0] == 0:          # an answer of at least one token before the stop
+                ok = False
+                break
+            conv += gen[:ends[0] + 1]
+        if ok and len(conv) < limit:
+            chosen = (chat, conv)
+            break
+    assert chosen is not None, "no class of ids ends both turns; change the lines"
+    chat, want = chosen
+    eng = g.load_model(folder, dtype="float32", max_tokens=1024)
+    args = argparse.Namespace(system_prompt="s", stream=True, echo=False, max_tokens=limit)
+    out = io.StringIO()
+    free = eng.slots_free()
+    got = cli.run_interactive(eng, chat, tok, g.select_sampler(cfgd["vocab_size"], 0.0, 1.0, 1), args, lines=lines, out=out)
+    assert got == want
+    assert out.getvalue().count("> ") == 3 and eng.slots_free() == free
