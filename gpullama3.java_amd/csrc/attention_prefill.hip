@@ -245,6 +245,206 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   }
 }
 
+// The same attention with 32 queries of one head to a wave (128 to a block) on the 32x32x16 instruction, for
+// steps that bring enough queries to fill such blocks: a wave reads the chunk's keys and values out
+// of shared memory once for twice as many queries, and a block brings a chunk from the cache once
+// for twice as many, which is what bounds the kernel above. Tiles as there, transposed:
+//   S^T[key, query]  = K[key, :] . Q[query, :]^T     one 32 x 32 tile per chunk of 32 keys
+//   O^T[dim, query] += V^T[dim, key] . P^T[key, query]
+// A lane holds, of the score tile, query lane % 32 and the rows 8a + 4h + b (h = lane / 32, register
+// 4a + b); row r of the tile is made key 16*(a/2) + 8h + 4*(a%2) + b of the chunk by the order in
+// which the key rows are read, so that registers 0..7 hold the keys 8h..8h+7 of the chunk's first
+// half and registers 8..15 those of its second half: the order in which the second product takes
+// its 16 keys a step.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int HS, int AHEAD, int OCC>
+__global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
+    const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
+    int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
+    float scale, int q_blocks) {
+  constexpr int KS = HS / 16;             // steps of the score product
+  constexpr int DT = HS / 32;             // tiles of 32 dims of the output
+  constexpr int KROW = HS + 8;
+  constexpr int VROW = 32 + 8;
+  constexpr int UNITS = HS * 4;
+  constexpr int NU = (UNITS + 255) / 256;
+  constexpr int QB = 128;                 // queries of a block
+  __shared__ __attribute__((aligned(16))) bf16_t ks[2][32][KROW];
+  __shared__ __attribute__((aligned(16))) bf16_t vs[2][HS][VROW];
+  const int g = n_heads / n_kv;
+  const int qb = q_blocks - 1 - blockIdx.x;
+  const int b = blockIdx.y;
+  const int head = blockIdx.z, c = head / g;   // one query head to a block
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int n = lane & 31, h = lane >> 5;
+  const int tok0 = __builtin_amdgcn_readfirstlane(cu_seqlens[b]);
+  const int q_len = __builtin_amdgcn_readfirstlane(cu_seqlens[b + 1]) - tok0;
+  if (qb * QB >= q_len) return;            // the whole block: no barrier has been passed yet
+  const int before = __builtin_amdgcn_readfirstlane(kv_before[b]);
+  const int* bt = block_table + (long)b * table_stride;
+  const int blk_first = before + qb * QB, blk_last = before + min(qb * QB + QB - 1, q_len - 1);
+  const int blk_lo = (window > 0 && blk_first + 1 > window) ? blk_first + 1 - window : 0;
+  const int ck0 = blk_lo / 32, ck1 = blk_last / 32;
+  const int qi0 = qb * QB + wave * 32;
+  const bool active = qi0 < q_len;
+  const bool q_ok = qi0 + n < q_len;
+  const int p_mine = before + qi0 + n;
+  const int p_last = before + min(qi0 + 31, q_len - 1);
+  const int p_first = before + qi0;
+  const int lo_first = (window > 0 && p_first + 1 > window) ? p_first + 1 - window : 0;
+  const int lo_last = (window > 0 && p_last + 1 > window) ? p_last + 1 - window : 0;
+  const int lo_mine = (window > 0 && p_mine + 1 > window) ? p_mine + 1 - window : 0;
+  const int ck_first = active ? lo_first / 32 : 1, ck_last = active ? p_last / 32 : 0;
+
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8 qt[KS];
+#pragma unroll
+  for (int kk = 0; kk < KS; ++kk)
+    qt[kk] = q_ok ? *(const bf16x8*)(q + (long)(tok0 + qi0 + n) * q_stride + (long)head * HS + kk * 16 + 8 * h) : zero8;
+
+  float m_run = -INFINITY, l_run = 0.f;
+  f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[dt][v] = 0.f;
+
+  bf16x8 rk[AHEAD][NU], rv[AHEAD][NU];
+  auto fetch = [&](int ck, bf16x8 (&fk)[NU], bf16x8 (&fv)[NU]) {
+    const int key0 = ck * 32;
+    const long page = __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
+    const int po = key0 % page_size;
+    const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
+    const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + po;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int u = tid + 256 * i;
+      if (UNITS % 256 == 0 || u < UNITS) {
+        fk[i] = *(const bf16x8*)(kb + u * 8);
+        fv[i] = *(const bf16x8*)(vb + (long)(u >> 2) * page_size + (u & 3) * 8);
+      }
+    }
+  };
+  auto stage = [&](int buf, const bf16x8 (&fk)[NU], const bf16x8 (&fv)[NU]) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int u = tid + 256 * i;
+      if (UNITS % 256 == 0 || u < UNITS) {
+        *(bf16x8*)&ks[buf][(u * 8) / HS][(u * 8) % HS] = fk[i];
+        *(bf16x8*)&vs[buf][u >> 2][(u & 3) * 8] = fv[i];
+      }
+    }
+  };
+
+  const float c2 = scale * 1.4426950408889634f;   // scores in units of log2
+  // which key of a chunk is row n of the score tile
+  const int krow = 16 * (n >> 4) + 8 * ((n >> 2) & 1) + 4 * ((n >> 3) & 1) + (n & 3);
+
+  // One chunk: scores, running softmax, weighted values. The operands are read from shared memory
+  // where they are used, no more than four ahead of their products (the scheduler would read them
+  // all first, and they do not fit into the registers beside the sums). MASKED: some query of the
+  // wave does not see some key of the chunk (the diagonal, a window's edge).
+  auto chunk = [&](int buf, int key0, auto masked) {
+    f32x16 s;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) {
+      const bf16x8 a = *(const bf16x8*)&ks[buf][krow][kk * 16 + 8 * h];
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qt[kk], s, 0, 0, 0);
+      if (kk % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+    }
+    if (decltype(masked)::value) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = key0 + 16 * (v >> 3) + 8 * h + (v & 7);
+        s[v] = (key >= lo_mine && key <= p_mine) ? s[v] : -INFINITY;
+      }
+    }
+    float mx = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+    {   // the other half of the keys of this query sits 32 lanes away
+      auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+      mx = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    }
+    mx *= c2;                                   // c2 > 0: the greatest score stays the greatest
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    float ps = 0.f;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[e], c2, -m_use));
+      ps += p;
+      pb[e >> 3][e & 7] = static_cast<bf16_t>(p);
+    }
+    l_run = l_run * alpha + ps;
+    m_run = m_new;
+    if (!__all(alpha == 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt] *= alpha;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const bf16x8 v0 = *(const bf16x8*)&vs[buf][dt * 32 + n][8 * h];
+      const bf16x8 v1 = *(const bf16x8*)&vs[buf][dt * 32 + n][16 + 8 * h];
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, pb[0], o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, pb[1], o[dt], 0, 0, 0);
+      if (dt % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+#pragma unroll
+  for (int r = 0; r < AHEAD; ++r) fetch(min(ck0 + r, ck1), rk[r], rv[r]);
+  stage(0, rk[0], rv[0]);
+  __syncthreads();
+  int buf = 0;
+  for (int base = ck0; base <= ck1; base += AHEAD) {
+#pragma unroll
+    for (int r = 0; r < AHEAD; ++r) {
+      const int ck = base + r;
+      if (ck > ck1) break;
+      const int key0 = ck * 32;
+      // the registers of this chunk are free (it lies in shared memory): ask for the chunk AHEAD further;
+      // unconditional (the last chunk again at the end): a branch around the loads makes the compiler
+      // wait for all of them at once
+      fetch(min(ck + AHEAD, ck1), rk[r], rv[r]);
+      if (ck >= ck_first && ck <= ck_last) {
+        // every query of the wave sees the whole chunk: no mask (the same for the whole wave)
+        if (key0 + 31 <= p_first && key0 >= lo_last) chunk(buf, key0, std::false_type{});
+        else chunk(buf, key0, std::true_type{});
+      }
+      if (ck < ck1) stage(buf ^ 1, rk[(r + 1) % AHEAD], rv[(r + 1) % AHEAD]);
+      __syncthreads();
+      buf ^= 1;
+    }
+  }
+
+  float l = l_run;
+  l += __shfl_xor(l, 32, 64);
+  if (!q_ok) return;
+  const float inv = 1.0f / l;
+  bf16_t* op = out + (long)(tok0 + qi0 + n) * out_stride + (long)head * HS + 4 * h;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      bf16x4 r;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) r[v] = static_cast<bf16_t>(o[dt][4 * a + v] * inv);
+      *(bf16x4*)(op + dt * 32 + 8 * a) = r;
+    }
+}
+
+// From how many tokens of the longest sequence of a step on the kernel with 128 queries a block is
+// taken (settable: tests run both kernels on the same inputs).
+extern "C" int gl3_attention_prefill_wide_from = 256;
+
 extern "C" int gl3_attention_prefill_supports(int head_dim, int page_size) {
   return (head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128) && page_size % 32 == 0;
 }
@@ -267,13 +467,30 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
   GL3_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 && out_stride % 4 == 0 && (uintptr_t)out % 8 == 0,
               "gl3_attention_prefill: queries must be 16-byte aligned, outputs 8-byte aligned");
   const int g = n_heads / n_kv;
-  const int q_blocks = (max_q_len + 63) / 64;
   // query heads per wave: as many as the registers hold with two blocks on a CU
-  const int gh = head_dim <= 32 ? 4 : head_dim <= 64 ? 2 : 1;
+  const bool wide = max_q_len >= gl3_attention_prefill_wide_from;
+  // query heads per wave: as many as the registers hold with two blocks on a CU; one with 32 queries a wave
+  const int gh = wide ? 1 : head_dim <= 32 ? 4 : head_dim <= 64 ? 2 : 1;
   const long z = (long)n_kv * ((g + gh - 1) / gh);
   GL3_REQUIRE(n_seqs <= 65535 && z <= 65535, "gl3_attention_prefill: %d sequences / %ld head groups exceed the grid",
               n_seqs, z);
+  const int q_blocks = wide ? (max_q_len + 127) / 128 : (max_q_len + 63) / 64;
   dim3 grid(q_blocks, n_seqs, (unsigned)z), block(256);
+  if (wide) {
+#define GOW(HS, AH, OCC)                                                                                            \
+  attention_prefill_wide_kernel<HS, AH, OCC><<<grid, block, 0, stream>>>(                                           \
+      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table, \
+      table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks)
+    switch (head_dim) {
+      case 32: GOW(32, 2, 3); break;
+      case 64: GOW(64, 2, 3); break;
+      case 96: GOW(96, 2, 2); break;
+      default: GOW(128, 1, 2); break;
+    }
+#undef GOW
+    GL3_LAUNCH_CHECK();
+    return 0;
+  }
 #define GO(HS, GH)                                                                                                  \
   attention_prefill_kernel<HS, GH><<<grid, block, 0, stream>>>(                                                     \
       (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table, \

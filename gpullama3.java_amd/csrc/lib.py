@@ -552,6 +552,15 @@ def attention_prefill_fits(head_dim, n_heads, n_kv, page_size):
     return bool(library().gl3_attention_prefill_supports(head_dim, page_size)) and n_heads % n_kv == 0
 
 
+def attention_prefill_wide_from(tokens=None):
+    """From how many tokens of a step's longest sequence on the prefill attention takes its kernel
+    with 128 queries a block; with an argument, sets it (tests run both kernels on the same inputs)."""
+    var = ctypes.c_int.in_dll(library(), "gl3_attention_prefill_wide_from")
+    if tokens is not None:
+        var.value = int(tokens)
+    return var.value
+
+
 def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, out, max_q_len, n_heads, n_kv,
                       head_dim, page_size, window, scale):
     """Any number of tokens per sequence; ``cu_seqlens`` [B+1] and ``kv_before`` [B] say which tokens

@@ -569,8 +569,18 @@ def prefill_fn(lens_before, new):
     return fn
 
 
-@pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 32), (5, 5, 96), (8, 1, 128), (12, 2, 64)])
-def test_attention_prefill(H, Kh, hs):
+@pytest.fixture(params=["64 queries a block", "128 queries a block"])
+def prefill_kernel(request):
+    """Both kernels of the prefill attention on the same inputs, whatever the step's length."""
+    lib = K()
+    usual = lib.attention_prefill_wide_from()
+    lib.attention_prefill_wide_from(1 if request.param.startswith("128") else 1 << 30)
+    yield request.param
+    lib.attention_prefill_wide_from(usual)
+
+
+@pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 32), (5, 5, 96), (8, 1, 128), (12, 2, 64), (3, 1, 128)])
+def test_attention_prefill(H, Kh, hs, prefill_kernel):
     rng = np.random.default_rng(H * hs)
     lens_before, new = [0, 70, 0, 130, 5], [33, 1, 200, 17, 64]      # prompts, chunks after a prefix, one token
     sk, sv, qs = attention_case(rng, H, Kh, hs, lens_before, new, "bfloat16")
@@ -578,7 +588,7 @@ def test_attention_prefill(H, Kh, hs):
     np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
 
 
-def test_attention_prefill_far_key_and_window_edge():
+def test_attention_prefill_far_key_and_window_edge(prefill_kernel):
     rng = np.random.default_rng(29)
     H, Kh, hs, n = 4, 2, 64, 700
     k = rng.standard_normal((n, Kh, hs)).astype(np.float32) * 0.1
