@@ -5,10 +5,11 @@
 // A block is WM x WN waves; each wave owns 64 x 64 (or 32 x 64) of the block's tile of C as
 // 2 x 2 (1 x 2) tiles of the 32x32x16 instruction: sixteen waves on 256 x 256 for large products,
 // eight waves on 128 x 128 otherwise. For the gated epilogue a W tile holds the gate rows of
-// half as many output columns and the matching up rows. K advances in steps of 64: the next
-// step's operands travel from memory to registers while the matrix cores work on the current
-// step out of shared memory. Rows in shared memory are padded by 16 bytes so that the 32 lanes
-// that read one column of 16-byte operands hit different banks.
+// half as many output columns and the matching up rows. K advances in steps of 64 through two
+// buffers in shared memory: while a step's products run out of one, the next step's operands go
+// from registers into the other and the step after that travels from memory to registers; one
+// barrier a step. Rows in shared memory are padded by 16 bytes so that the 32 lanes that read one
+// column of 16-byte operands hit different banks.
 // Blocks are numbered so that each XCD (whose second-level cache is its own) works on a
 // contiguous range of tiles, neighbouring tiles sharing their panel of W.
 //
@@ -37,8 +38,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   constexpr int NA = BM * 8 / NT;                        // 16-byte chunks of A per thread and k-step
   constexpr int NWC = BN * 8 / NT;                       // and of W
   static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile does not divide over the threads");
-  __shared__ __attribute__((aligned(16))) bf16_t As[BM][MF_LD];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[BN][MF_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][BM][MF_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN][MF_LD];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wm = wave / WN, wn = wave % WN;
   const int lr = lane & 31, lh = lane >> 5;
@@ -112,36 +113,48 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   const int wrow0 = (EPI == MF_GATED) ? wn * 32 + lr : wn * 64 + lr;
   const int wrow1 = (EPI == MF_GATED) ? BN / 2 + wn * 32 + lr : wn * 64 + 32 + lr;
 
-  for (int k0 = k_begin; k0 < K; k0 += MF_BK) {
+  // registers -> shared memory; a step that reaches beyond K drops the columns from K on
+  auto store = [&](int buf, int k0) {
     if (k0 + MF_BK <= K) {   // a whole step (the same for the whole block): nothing to drop
 #pragma unroll
-      for (int i = 0; i < NA; ++i) *(bf16x8*)&As[arow_s[i]][scol] = ra[i];
+      for (int i = 0; i < NA; ++i) *(bf16x8*)&As[buf][arow_s[i]][scol] = ra[i];
 #pragma unroll
-      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[wrow_s[i]][scol] = rw[i];
+      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[buf][wrow_s[i]][scol] = rw[i];
     } else {
 #pragma unroll
-      for (int i = 0; i < NA; ++i) *(bf16x8*)&As[arow_s[i]][scol] = r_ok ? ra[i] : zero;
+      for (int i = 0; i < NA; ++i) *(bf16x8*)&As[buf][arow_s[i]][scol] = r_ok ? ra[i] : zero;
 #pragma unroll
-      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[wrow_s[i]][scol] = r_ok ? rw[i] : zero;
+      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[buf][wrow_s[i]][scol] = r_ok ? rw[i] : zero;
     }
-    __syncthreads();
+  };
+  auto products = [&](int buf, int kk) {
+    const int kc = kk * 16 + lh * 8;
+    const bf16x8 b0 = *(const bf16x8*)&Ws[buf][wrow0][kc];
+    const bf16x8 b1 = *(const bf16x8*)&Ws[buf][wrow1][kc];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const bf16x8 a = *(const bf16x8*)&As[buf][arow + 32 * tm][kc];
+      acc[tm][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, acc[tm][0], 0, 0, 0);
+      acc[tm][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, acc[tm][1], 0, 0, 0);
+    }
+  };
+  // Two buffers in shared memory: while a step's products run out of one, the next step's operands
+  // (in registers since the step before) are written to the other and the step after that is asked
+  // for; one barrier a step.
+  store(0, k_begin);
+  fetch(k_begin + MF_BK);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = k_begin; k0 < K; k0 += MF_BK, buf ^= 1) {
 #pragma unroll
     for (int kk = 0; kk < MF_BK / 16; ++kk) {
-      const int kc = kk * 16 + lh * 8;
-      const bf16x8 b0 = *(const bf16x8*)&Ws[wrow0][kc];
-      const bf16x8 b1 = *(const bf16x8*)&Ws[wrow1][kc];
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm) {
-        const bf16x8 a = *(const bf16x8*)&As[arow + 32 * tm][kc];
-        acc[tm][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, acc[tm][0], 0, 0, 0);
-        acc[tm][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, acc[tm][1], 0, 0, 0);
-      }
+      products(buf, kk);
       if (kk == 0) {
-        // the next step's loads go out behind the first products (which cover the address
-        // arithmetic), and their values are first looked at when they are written to shared
-        // memory: the scheduler may not move either across the fences
+        // behind the first products (which cover the wait for the registers and the address
+        // arithmetic); the scheduler may not move the loads or the writes across the fences
         __builtin_amdgcn_sched_barrier(0);
-        fetch(k0 + MF_BK);
+        if (k0 + MF_BK < K) store(buf ^ 1, k0 + MF_BK);
+        fetch(k0 + 2 * MF_BK);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
