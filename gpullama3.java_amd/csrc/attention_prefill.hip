@@ -258,7 +258,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 // its 16 keys a step.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-template <int HS, int AHEAD, int OCC>
+template <int HS, int CK, int AHEAD, int OCC>
 __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
@@ -266,12 +266,14 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     float scale, int q_blocks) {
   constexpr int KS = HS / 16;             // steps of the score product
   constexpr int DT = HS / 32;             // tiles of 32 dims of the output
+  constexpr int NT = CK / 32;             // score tiles of a chunk of CK keys
   constexpr int KROW = HS + 8;
-  constexpr int VROW = 32 + 8;
-  constexpr int UNITS = HS * 4;
+  constexpr int VROW = CK + 8;
+  constexpr int VU = CK / 8;              // 16-byte units of a row of the transposed value chunk
+  constexpr int UNITS = HS * CK / 8;      // 16-byte units of a chunk of keys (and of values)
   constexpr int NU = (UNITS + 255) / 256;
   constexpr int QB = 128;                 // queries of a block
-  __shared__ __attribute__((aligned(16))) bf16_t ks[2][32][KROW];
+  __shared__ __attribute__((aligned(16))) bf16_t ks[2][CK][KROW];
   __shared__ __attribute__((aligned(16))) bf16_t vs[2][HS][VROW];
   const int g = n_heads / n_kv;
   const int qb = q_blocks - 1 - blockIdx.x;
@@ -287,7 +289,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   const int* bt = block_table + (long)b * table_stride;
   const int blk_first = before + qb * QB, blk_last = before + min(qb * QB + QB - 1, q_len - 1);
   const int blk_lo = (window > 0 && blk_first + 1 > window) ? blk_first + 1 - window : 0;
-  const int ck0 = blk_lo / 32, ck1 = blk_last / 32;
+  const int ck0 = blk_lo / CK, ck1 = blk_last / CK;
   const int qi0 = qb * QB + wave * 32;
   const bool active = qi0 < q_len;
   const bool q_ok = qi0 + n < q_len;
@@ -297,7 +299,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   const int lo_first = (window > 0 && p_first + 1 > window) ? p_first + 1 - window : 0;
   const int lo_last = (window > 0 && p_last + 1 > window) ? p_last + 1 - window : 0;
   const int lo_mine = (window > 0 && p_mine + 1 > window) ? p_mine + 1 - window : 0;
-  const int ck_first = active ? lo_first / 32 : 1, ck_last = active ? p_last / 32 : 0;
+  const int ck_first = active ? lo_first / CK : 1, ck_last = active ? p_last / CK : 0;
 
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   bf16x8 qt[KS];
@@ -314,7 +316,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
 
   bf16x8 rk[AHEAD][NU], rv[AHEAD][NU];
   auto fetch = [&](int ck, bf16x8 (&fk)[NU], bf16x8 (&fv)[NU]) {
-    const int key0 = ck * 32;
+    const int key0 = ck * CK;
     const long page = __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
     const int po = key0 % page_size;
     const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
@@ -324,7 +326,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
       const int u = tid + 256 * i;
       if (UNITS % 256 == 0 || u < UNITS) {
         fk[i] = *(const bf16x8*)(kb + u * 8);
-        fv[i] = *(const bf16x8*)(vb + (long)(u >> 2) * page_size + (u & 3) * 8);
+        fv[i] = *(const bf16x8*)(vb + (long)(u / VU) * page_size + (u % VU) * 8);
       }
     }
   };
@@ -334,7 +336,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
       const int u = tid + 256 * i;
       if (UNITS % 256 == 0 || u < UNITS) {
         *(bf16x8*)&ks[buf][(u * 8) / HS][(u * 8) % HS] = fk[i];
-        *(bf16x8*)&vs[buf][u >> 2][(u & 3) * 8] = fv[i];
+        *(bf16x8*)&vs[buf][u / VU][(u % VU) * 8] = fv[i];
       }
     }
   };
@@ -348,25 +350,34 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   // all first, and they do not fit into the registers beside the sums). MASKED: some query of the
   // wave does not see some key of the chunk (the diagonal, a window's edge).
   auto chunk = [&](int buf, int key0, auto masked) {
-    f32x16 s;
+    f32x16 s[NT];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[t][v] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk) {
-      const bf16x8 a = *(const bf16x8*)&ks[buf][krow][kk * 16 + 8 * h];
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qt[kk], s, 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {      // the tiles' sums do not depend on each other: the matrix cores stay busy
+        const bf16x8 a = *(const bf16x8*)&ks[buf][32 * t + krow][kk * 16 + 8 * h];
+        s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qt[kk], s[t], 0, 0, 0);
+      }
       if (kk % 4 == 3) __builtin_amdgcn_sched_barrier(0);
     }
     if (decltype(masked)::value) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int key = key0 + 16 * (v >> 3) + 8 * h + (v & 7);
-        s[v] = (key >= lo_mine && key <= p_mine) ? s[v] : -INFINITY;
-      }
-    }
-    float mx = s[0];
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+        for (int v = 0; v < 16; ++v) {
+          const int key = key0 + 32 * t + 16 * (v >> 3) + 8 * h + (v & 7);
+          s[t][v] = (key >= lo_mine && key <= p_mine) ? s[t][v] : -INFINITY;
+        }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[t][v]);
     {   // the other half of the keys of this query sits 32 lanes away
       auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
       mx = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
@@ -376,13 +387,15 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
     float ps = 0.f;
-    bf16x8 pb[2];
+    bf16x8 pb[NT][2];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const float p = __builtin_amdgcn_exp2f(fmaf(s[e], c2, -m_use));
-      ps += p;
-      pb[e >> 3][e & 7] = static_cast<bf16_t>(p);
-    }
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[t][e], c2, -m_use));
+        ps += p;
+        pb[t][e >> 3][e & 7] = static_cast<bf16_t>(p);
+      }
     l_run = l_run * alpha + ps;
     m_run = m_new;
     if (!__all(alpha == 1.0f)) {
@@ -390,12 +403,15 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
       for (int dt = 0; dt < DT; ++dt) o[dt] *= alpha;
     }
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const bf16x8 v0 = *(const bf16x8*)&vs[buf][dt * 32 + n][8 * h];
-      const bf16x8 v1 = *(const bf16x8*)&vs[buf][dt * 32 + n][16 + 8 * h];
-      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, pb[0], o[dt], 0, 0, 0);
-      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, pb[1], o[dt], 0, 0, 0);
-      if (dt % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const bf16x8 v0 = *(const bf16x8*)&vs[buf][dt * 32 + n][32 * t + 8 * h];
+        const bf16x8 v1 = *(const bf16x8*)&vs[buf][dt * 32 + n][32 * t + 16 + 8 * h];
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, pb[t][0], o[dt], 0, 0, 0);
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, pb[t][1], o[dt], 0, 0, 0);
+        if (dt % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+      }
     }
   };
 
@@ -409,14 +425,14 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     for (int r = 0; r < AHEAD; ++r) {
       const int ck = base + r;
       if (ck > ck1) break;
-      const int key0 = ck * 32;
+      const int key0 = ck * CK;
       // the registers of this chunk are free (it lies in shared memory): ask for the chunk AHEAD further;
       // unconditional (the last chunk again at the end): a branch around the loads makes the compiler
       // wait for all of them at once
       fetch(min(ck + AHEAD, ck1), rk[r], rv[r]);
       if (ck >= ck_first && ck <= ck_last) {
         // every query of the wave sees the whole chunk: no mask (the same for the whole wave)
-        if (key0 + 31 <= p_first && key0 >= lo_last) chunk(buf, key0, std::false_type{});
+        if (key0 + CK - 1 <= p_first && key0 >= lo_last) chunk(buf, key0, std::false_type{});
         else chunk(buf, key0, std::true_type{});
       }
       if (ck < ck1) stage(buf ^ 1, rk[(r + 1) % AHEAD], rv[(r + 1) % AHEAD]);
@@ -477,15 +493,18 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
   const int q_blocks = wide ? (max_q_len + 127) / 128 : (max_q_len + 63) / 64;
   dim3 grid(q_blocks, n_seqs, (unsigned)z), block(256);
   if (wide) {
-#define GOW(HS, AH, OCC)                                                                                            \
-  attention_prefill_wide_kernel<HS, AH, OCC><<<grid, block, 0, stream>>>(                                           \
+#define GOW(HS, CK, AH, OCC)                                                                                        \
+  attention_prefill_wide_kernel<HS, CK, AH, OCC><<<grid, block, 0, stream>>>(                                       \
       (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table, \
       table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks)
+    // chunks of 64 keys (one barrier for twice the work, two score tiles whose sums do not wait for
+    // each other) where the registers hold them and a page holds whole chunks
+    const bool ck64 = page_size % 64 == 0;
     switch (head_dim) {
-      case 32: GOW(32, 2, 3); break;
-      case 64: GOW(64, 2, 3); break;
-      case 96: GOW(96, 2, 2); break;
-      default: GOW(128, 1, 2); break;
+      case 32: if (ck64) GOW(32, 64, 2, 3); else GOW(32, 32, 2, 3); break;
+      case 64: if (ck64) GOW(64, 64, 2, 2); else GOW(64, 32, 2, 3); break;
+      case 96: GOW(96, 32, 2, 2); break;
+      default: GOW(128, 32, 1, 2); break;
     }
 #undef GOW
     GL3_LAUNCH_CHECK();

@@ -586,6 +586,11 @@ def test_attention_prefill(H, Kh, hs, prefill_kernel):
     sk, sv, qs = attention_case(rng, H, Kh, hs, lens_before, new, "bfloat16")
     got, ref = run_attention(prefill_fn(lens_before, new), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng)
     np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+    # pages of 32 and of 96 positions: chunks of 32 keys, several pages or a part of one to a chunk's page
+    for page in (32, 96):
+        got, ref = run_attention(prefill_fn(lens_before, new), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng,
+                                 page=page)
+        np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max(), err_msg=f"pages of {page}")
 
 
 def test_attention_prefill_far_key_and_window_edge(prefill_kernel):
