@@ -185,3 +185,41 @@ def test_chat_loop_keeps_the_dialogue_in_the_cache():
     got = cli.run_interactive(eng, chat, tok, g.select_sampler(cfgd["vocab_size"], 0.0, 1.0, 1), args, lines=lines, out=out)
     assert got == want
     assert out.getvalue().count("> ") == 3 and eng.slots_free() == free
+
+
+def test_command_line_with_a_text_prompt(tmp_path):
+    """--prompt through a tokenizer.json in the model folder: the tokens that the model sees are the
+    chat format's (begin of text, system and user message, the assistant's header), the answer is the
+    plain implementation's greedy continuation, printed as text."""
+    import shutil
+    from tokenizers import Tokenizer, decoders, models, pre_tokenizers
+    from gpullama3_java_amd.chat import SYSTEM, USER, HFTokenizer, LlamaChatFormat, Message
+    folder, cfgd, _ = model("B")
+    mine = str(tmp_path / "model")
+    shutil.copytree(folder, mine)
+    alphabet = sorted(pre_tokenizers.ByteLevel.alphabet())
+    tok = Tokenizer(models.BPE(vocab={ch: i for i, ch in enumerate(alphabet)}, merges=[]))
+    tok.pre_tokenizer = pre_tokenizers.ByteLevel(add_prefix_space=False)
+    tok.decoder = decoders.ByteLevel()
+    tok.add_special_tokens(["<|begin_of_text|>", "<|start_header_id|>", "<|end_header_id|>", "<|eot_id|>",
+                            "<|end_of_text|>"])
+    assert tok.get_vocab_size() <= cfgd["vocab_size"]
+    tok.save(os.path.join(mine, "tokenizer.json"))
+    hf = HFTokenizer(os.path.join(mine, "tokenizer.json"))
+    chat = LlamaChatFormat(hf)
+    assert hf.encode("hi") == [alphabet.index("h"), alphabet.index("i")] and hf.decode(hf.encode("a b")) == "a b"
+    prompt = chat.encode_dialog_prompt(True, [Message(SYSTEM, "s"), Message(USER, "hi there")])
+    limit = len(prompt) + 10
+    want = plain_greedy("B", prompt, 11)
+    if any(t in chat.stop_tokens for t in want):
+        want = want[:[t in chat.stop_tokens for t in want].index(True)]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "llama-hip"), "-m", mine, "-p", " hi there ", "-sp", "s",
+           "--temperature=0", "-n", str(limit), "--stream", "false", "--dtype", "float32"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert r.stdout.rstrip("\n") == hf.decode(want).rstrip("\n")
+    assert f"Tokens: {len(prompt) + len(want)}" in r.stderr
+    chatty = subprocess.run(cmd[:4] + ["--chat", "--temperature=0", "-n", str(limit), "--dtype", "float32"],
+                            input="hi there\nquit\n", capture_output=True, text=True, timeout=300)
+    assert chatty.returncode == 0, chatty.stderr
+    assert chatty.stdout.startswith("> ")
