@@ -541,10 +541,11 @@ def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None):
 
 def mfma_slices(M, N, K):
     """Into how many slices of K the tiled product [M, K] x [N, K] into the residual stream is cut:
-    more than one only where the tiles of 128 x 128 are too few for the chip and K is long enough
-    for a slice to outweigh the extra pass over its sums."""
+    more than one only where the tiles of 128 x 128 are too few for the chip. A block's time is its
+    walk along K (half a microsecond per 64 columns, whatever else runs), so few tiles over a long
+    K are better cut, down to slices of 512 columns; the norm that follows adds the slices up."""
     tiles = -(-M // 128) * -(-N // 128)
-    return max(1, min(4, 512 // tiles, K // 2048))
+    return max(1, min(8, 512 // tiles, K // 512))
 
 
 # ------------------------------------------------------------------ bfloat16 attention of a prefill step
