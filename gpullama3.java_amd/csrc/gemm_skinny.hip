@@ -574,7 +574,7 @@ struct SkCall {
 // Blocks of the resident kernel: every strip its own block while that still leaves CUs idle, else
 // two blocks per CU that walk over the strips.
 static int resident_blocks(int n_strips, int nw) {
-  const int most = nw == 16 ? 256 : 512;
+  const int most = nw == 16 ? 256 : nw == 8 ? 512 : 1024;
   return n_strips < most ? n_strips : most;
 }
 
@@ -602,6 +602,13 @@ static int launch_skinny(int nw, const SkCall& a) {
     }
   }
   if (a.resident) {
+    // very many strips (the head after a prompt): four waves a block, each with four times the share
+    // of K. A block walks over fewer strips, more of them are on their way on a CU at once, and four
+    // partial tiles are merged per strip, not sixteen (the head at one row: 113 -> 100 us). With the
+    // norm folded in (a decode step's head) the sixteen waves are the faster ones: 97 against 103 us.
+    if constexpr (NG * MT == 1 && EPI != SK_QKV && !XNORM) {
+      if (steps <= 64 && n_strips >= 2048) RES(4, 16);
+    }
     // 16 waves a strip where their partial tiles fit, so that a strip's rows are asked for at once
     if constexpr (NG * MT <= 2) {
       if (steps <= 64) RES(16, 4);

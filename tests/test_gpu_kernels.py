@@ -416,7 +416,8 @@ def test_sample_kernel_frequencies_and_rules():
 
 # ------------------------------------------------------------------ bfloat16 product for few rows (matrix cores)
 @pytest.mark.parametrize("M", [1, 8, 17, 64])
-@pytest.mark.parametrize("N, Kd", [(2048, 2048), (130, 64), (48, 40), (3000, 512), (256, 8192)])
+# (the last case has strips enough for the blocks of four waves that very wide products take)
+@pytest.mark.parametrize("N, Kd", [(2048, 2048), (130, 64), (48, 40), (3000, 512), (256, 8192), (33000, 136)])
 def test_gemm_skinny(M, N, Kd):
     rng = np.random.default_rng(M + N)
     a = rounded(rng.standard_normal((M, Kd)), "bfloat16")
