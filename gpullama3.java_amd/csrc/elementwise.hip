@@ -7,7 +7,7 @@
 // ssq (may be null; then n_tokens <= 64): ssq[t] = sum of squares of row t, for a norm that is
 // folded into the product that follows; with it next_weight [d] (float) and xg [n_tokens][d]
 // (may be null): xg = bfloat16(next_weight * row), the rows as that product reads them.
-template <typename TW>
+template <typename TW, bool VEC>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out, int d,
                              float* __restrict__ ssq, const float* __restrict__ next_weight, bf16_t* __restrict__ xg) {
   __shared__ float scratch[16];
@@ -15,11 +15,39 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
   const TW* row = table + (long)ids[t] * d;
   float* o = out + t * d;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    const float v = to_f32<TW>(row[i]);
-    o[i] = v;
-    ss += v * v;
-    if (xg) xg[t * d + i] = static_cast<bf16_t>(next_weight[i] * v);
+  if (VEC) {
+    // eight elements a thread and trip: a row of a decode step is one trip to memory, not eight
+    typedef TW tw8 __attribute__((ext_vector_type(8)));
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+    for (int i = threadIdx.x * 8; i < d; i += blockDim.x * 8) {
+      const tw8 r8 = *(const tw8*)(row + i);
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        v[e] = to_f32<TW>(r8[e]);
+        ss += v[e] * v[e];
+      }
+      *(f32x4*)(o + i) = f32x4{v[0], v[1], v[2], v[3]};
+      *(f32x4*)(o + i + 4) = f32x4{v[4], v[5], v[6], v[7]};
+      if (xg) {
+        const f32x4 w0 = *(const f32x4*)(next_weight + i), w1 = *(const f32x4*)(next_weight + i + 4);
+        bf16x8 g;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          g[e] = static_cast<bf16_t>(w0[e] * v[e]);
+          g[4 + e] = static_cast<bf16_t>(w1[e] * v[4 + e]);
+        }
+        *(bf16x8*)(xg + t * d + i) = g;
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+      const float v = to_f32<TW>(row[i]);
+      o[i] = v;
+      ss += v * v;
+      if (xg) xg[t * d + i] = static_cast<bf16_t>(next_weight[i] * v);
+    }
   }
   if (ssq) {
     ss = block_sum(ss, scratch);
@@ -35,11 +63,15 @@ extern "C" int gl3_embed(const void* table, int table_dtype, const int* ids, flo
   GL3_REQUIRE((next_weight == nullptr) == (xg == nullptr) && (!xg || ssq),
               "gl3_embed: the next norm's weight and its rows come together, with the sums of squares");
   dim3 grid(n_tokens), block(256);
-  if (table_dtype == GL3_F32)
-    embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, ids, out, d, ssq, next_weight, (bf16_t*)xg);
-  else if (table_dtype == GL3_BF16)
-    embed_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)table, ids, out, d, ssq, next_weight, (bf16_t*)xg);
+  // 16-byte units where the rows allow them (a width of a multiple of 8, aligned bases)
+  const bool vec = d % 8 == 0 && (uintptr_t)table % 32 == 0 && (uintptr_t)out % 16 == 0 &&
+                   (!xg || ((uintptr_t)xg % 16 == 0 && (uintptr_t)next_weight % 16 == 0));
+#define GO(TW, VEC)                                                                                              \
+  embed_kernel<TW, VEC><<<grid, block, 0, stream>>>((const TW*)table, ids, out, d, ssq, next_weight, (bf16_t*)xg)
+  if (table_dtype == GL3_F32) { if (vec) GO(float, true); else GO(float, false); }
+  else if (table_dtype == GL3_BF16) { if (vec) GO(bf16_t, true); else GO(bf16_t, false); }
   else GL3_REQUIRE(false, "gl3_embed: unknown dtype %d", table_dtype);
+#undef GO
   GL3_LAUNCH_CHECK();
   return 0;
 }
