@@ -56,6 +56,7 @@ def _declare(lib):
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_sample_work_floats": [I, I],
         "gl3_argmax": [P, L, P, P, I, I, P],
+        "gl3_argmax_static": [P, L, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
         "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P],
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P],

@@ -22,6 +22,8 @@
 // walk that short list, in shared memory, instead of the row. A flat distribution, whose nucleus
 // reaches further down, takes eight passes over the whole row.
 #include "common.h"
+#include "gl3_noalloc.h"
+#include <mutex>
 
 #define SB 1024
 #define SW 16          // waves of a block
@@ -579,6 +581,44 @@ extern "C" int gl3_argmax(const float* logits, long ld, float* work, int* out, i
   GL3_REQUIRE(n_rows <= 65535, "gl3_argmax: too many rows");
   float* pv = work;
   int* pi = (int*)(work + (long)n_rows * ARG_SLICES);
+  argmax_slice_kernel<<<dim3(n_rows, ARG_SLICES), dim3(256), 0, stream>>>(logits, ld, pv, pi, V);
+  GL3_LAUNCH_CHECK();
+  argmax_final_kernel<<<dim3(n_rows), dim3(64), 0, stream>>>(pv, pi, out);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
+// The same without a workspace from the caller (see gl3_noalloc.h): the slices' partial results live
+// in a device array of this library. In host code `scratch` is only a handle for the runtime, not a
+// device address; the address on each GPU is asked for once, with that GPU current, and kept.
+static __device__ __align__(256) float scratch[GL3_ARGMAX_STATIC_ROWS * 2 * ARG_SLICES];
+#define GL3_MAX_DEVICES 64
+static float* g_scratch_ptr[GL3_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+extern "C" int gl3_argmax_static(const float* logits, long ld, int* out, int n_rows, int V, hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  GL3_REQUIRE(logits && out && n_rows > 0 && V > 0 && ld >= V, "gl3_argmax_static: bad arguments");
+  GL3_REQUIRE(n_rows <= GL3_ARGMAX_STATIC_ROWS, "gl3_argmax_static: %d rows exceed the %d that the library's array holds",
+              n_rows, GL3_ARGMAX_STATIC_ROWS);
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  GL3_REQUIRE(e == hipSuccess && dev >= 0 && dev < GL3_MAX_DEVICES, "gl3_argmax_static: no current device (%s)",
+              hipGetErrorString(e));
+  float* work;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      GL3_REQUIRE(e == hipSuccess && p != nullptr, "gl3_argmax_static: the array's address on device %d: %s", dev,
+                  hipGetErrorString(e));
+      g_scratch_ptr[dev] = (float*)p;
+    }
+    work = g_scratch_ptr[dev];
+  }
+  float* pv = work;
+  int* pi = (int*)(work + (long)GL3_ARGMAX_STATIC_ROWS * ARG_SLICES);
   argmax_slice_kernel<<<dim3(n_rows, ARG_SLICES), dim3(256), 0, stream>>>(logits, ld, pv, pi, V);
   GL3_LAUNCH_CHECK();
   argmax_final_kernel<<<dim3(n_rows), dim3(64), 0, stream>>>(pv, pi, out);
