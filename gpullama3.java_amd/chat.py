@@ -1,5 +1,7 @@
-"""The Llama 3 chat format over token ids (J/model/format/LlamaChatFormat.java:21-74,
-J/model/format/ChatFormat.java roles): a message is its header (start-of-header, the role's
+"""The Llama 3 chat format over token ids. The token protocol is fixed by the model family, so the
+functions follow the reference's one for one: ``encode_header`` J/model/format/LlamaChatFormat.java:44-51,
+``encode_message`` :53-59, ``encode_dialog_prompt`` :61-72, the special tokens :21-42, the roles
+J/model/format/ChatFormat.java: a message is its header (start-of-header, the role's
 name, end-of-header, a line feed), its stripped text and end-of-turn; a dialogue starts with
 begin-of-text; generation stops at end-of-text or end-of-turn.
 

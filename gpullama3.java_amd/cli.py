@@ -32,7 +32,7 @@ import os
 import sys
 import time
 
-from .chat import ASSISTANT, SYSTEM, USER, HFTokenizer, LlamaChatFormat, Message
+from .chat import ASSISTANT, SYSTEM, USER, HFTokenizer, Message
 
 DEFAULT_MAX_TOKENS = 1024      # J/Options.java:10
 
@@ -116,8 +116,7 @@ def run_interactive(engine, chat, tokenizer, sampler, args, lines=None, out=None
             if not args.stream:
                 print(tokenizer.decode(response), file=out)
             if not stopped:
-                print("\n Ran out of context length...\n Increase context length with by passing to llama-hip "
-                      "--max-tokens XXX", file=sys.stderr)
+                print("\nThe context is full. A larger --max-tokens gives the conversation more room.", file=sys.stderr)
                 break
             print(file=out)
             _print_metrics(engine)
@@ -127,10 +126,10 @@ def run_interactive(engine, chat, tokenizer, sampler, args, lines=None, out=None
 def main(argv=None):
     args = create_parser().parse_args(argv)
     if not 0 <= args.temperature:
-        print("ERROR Invalid argument: --temperature must be non-negative", file=sys.stderr)
+        print("error: --temperature takes 0 (greedy) or a positive number", file=sys.stderr)
         return 2
     if not 0 <= args.top_p <= 1:
-        print("ERROR Invalid argument: --top-p must be within [0, 1]", file=sys.stderr)
+        print("error: --top-p takes a mass between 0 and 1", file=sys.stderr)
         return 2
     seed = args.seed if args.seed is not None else time.time_ns()
     import gpullama3_java_amd as g
@@ -144,12 +143,14 @@ def main(argv=None):
     tok_path = os.path.join(args.model_path, "tokenizer.json")
     if os.path.isfile(tok_path):
         tokenizer = HFTokenizer(tok_path)
-        chat = LlamaChatFormat(tokenizer)
+        # the dialogue's token protocol belongs to the architecture: its configuration class says which
+        make_format = getattr(g.load_config(args.model_path), "chat_format", None)
+        chat = make_format(tokenizer) if make_format is not None else None
     if args.suffix is not None:
         print("note: --suffix is for fill-in-the-middle models; a Llama model takes none, it is ignored", file=sys.stderr)
     if args.interactive:
         if chat is None:
-            print(f"ERROR --interactive needs {tok_path}", file=sys.stderr)
+            print(f"error: chat mode needs {tok_path} and an architecture with a chat format", file=sys.stderr)
             return 2
         prompt = None
     elif args.prompt_ids:
@@ -157,18 +158,18 @@ def main(argv=None):
         stop_ids = None
     elif args.prompt is not None:
         if chat is None:
-            print(f"ERROR --prompt needs {tok_path}; without a tokenizer give --prompt-ids", file=sys.stderr)
+            print(f"error: a text prompt needs {tok_path} and an architecture with a chat format; "
+                  "--prompt-ids takes token ids as they are", file=sys.stderr)
             return 2
         dialog = [Message(SYSTEM, args.system_prompt)] if args.system_prompt is not None else []
         prompt = chat.encode_dialog_prompt(True, dialog + [Message(USER, args.prompt)])
         stop_ids = chat.stop_tokens
     else:
-        print('ERROR Missing argument: --prompt is required in --instruct mode e.g. --prompt "Why is the sky blue?"',
-              file=sys.stderr)
+        print("error: give --prompt (or --prompt-ids), or --interactive for a dialogue", file=sys.stderr)
         return 2
     engine = g.load_model(args.model_path, context_length=args.max_tokens, dtype=args.dtype,
                           max_tokens=None)
-    sampler = g.select_sampler(engine.config.vocab_size, args.temperature, args.top_p, seed)
+    sampler = g.select_sampler(engine.spec.vocab_size, args.temperature, args.top_p, seed)
     if args.interactive:
         run_interactive(engine, chat, tokenizer, sampler, args)
         return 0

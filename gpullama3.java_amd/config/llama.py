@@ -136,6 +136,12 @@ class LlamaConfiguration:
             d["eos_token_id"] = list(self.stop_ids)
         return d
 
+    def chat_format(self, tokenizer):
+        """The dialogue's token protocol of this architecture over ``tokenizer`` (the command line asks
+        the configuration for it: another architecture brings its own or none)."""
+        from ..chat import LlamaChatFormat
+        return LlamaChatFormat(tokenizer)
+
     def with_stop_ids(self, ids):
         return replace(self, stop_ids=tuple(ids))
 

@@ -115,9 +115,8 @@ def test_first_tokens_of_a_sequence(name, dtype):
     got = np.concatenate([eng.step([(s, [t])]).cpu().numpy() for t in toks])
     eng.give_back_slot(s)
     close(got, ref, dtype, "one by one from position 0")
-    for n in (1, 2, 3):                                          # prompts of 1, 2, 3 tokens in one batch
-        pass
     slots = [eng.take_slot() for _ in range(3)]
+    # prompts of 1, 2, 3 tokens in one batch
     out = eng.step([(slots[i], toks[:i + 1]) for i in range(3)], want="all").cpu().numpy()
     close(out, np.concatenate([ref[:1], ref[:2], ref[:3]]), dtype, "prompts of 1, 2, 3")
 

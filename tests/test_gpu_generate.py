@@ -111,7 +111,7 @@ def test_command_line(tmp_path):
     assert [int(t) for t in r.stdout.split()] == plain_greedy("A", prompt, 8)
     assert "achieved tok/s" in r.stderr and "Tokens: 14" in r.stderr
     bad = subprocess.run(cmd[:4] + ["--top-p", "1.5", "--prompt-ids", "1"], capture_output=True, text=True, timeout=300)
-    assert bad.returncode != 0 and "--top-p must be within [0, 1]" in bad.stderr
+    assert bad.returncode != 0 and "--top-p takes a mass between 0 and 1" in bad.stderr
     noprompt = subprocess.run(cmd[:4] + ["--prompt", "hello"], capture_output=True, text=True, timeout=300)
     assert noprompt.returncode != 0 and "tokenizer.json" in noprompt.stderr
 

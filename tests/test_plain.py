@@ -64,14 +64,88 @@ def test_rope_scaling_factor_one_is_identity_and_branches():
     assert np.all(got[mid] < base[mid]) and np.all(got[mid] > base[mid] / 8.0)
 
 
-def test_rope_scaling_is_continuous_at_both_edges():
-    # freq chosen so that the wavelength sits at a boundary: smooth = 1 at old/hi, 0 at old/lo
-    old, lo, hi, factor = 64.0, 1.0, 4.0, 8.0
-    for wl, expect in ((old / hi, 1.0), (old / lo, 1.0 / factor)):
-        freq = 2 * math.pi / wl
-        smooth = (old / wl - lo) / (hi - lo)
-        val = (1 - smooth) * freq / factor + smooth * freq
-        assert abs(val / freq - expect) < 1e-12
+def _scaled_over_base(fn, wavelen, sc):
+    """``fn``'s scaled frequency over the unscaled one for a head of 4 whose second pair has the
+    wavelength ``wavelen``: theta is chosen so that ``theta ** -0.5 == 2 pi / wavelen``."""
+    theta = (wavelen / (2 * math.pi)) ** 2
+    return float(fn(4, theta, sc)[1]) / float(fn(4, theta, None)[1])
+
+
+# J/inference/operation/RoPE.java:20-27 worked by hand for old=64, lo=1, hi=4 (the band is 16..64):
+# smooth = (old/wavelen - lo)/(hi - lo); scaled/base = (1 - smooth)/factor + smooth.
+#   wavelen 32   -> old/wavelen 2   -> smooth 1/3 -> (2/3)/8 + 1/3 = 5/12
+#   wavelen 25.6 -> old/wavelen 2.5 -> smooth 1/2 -> (1/2)/8 + 1/2 = 9/16
+#   wavelen 64/3 -> old/wavelen 3   -> smooth 2/3 -> (1/3)/8 + 2/3 = 17/24
+# (smooth and 1 - smooth exchanged would give 17/24, 9/16, 5/12: the first and last tell them apart)
+# and for factor 32, old 8192 (the band is 2048..8192): wavelen 4096 -> smooth 1/3 -> (2/3)/32 + 1/3 = 17/48.
+SC_8 = dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=64)
+SC_32 = dict(factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192)
+HAND_VALUES = [(SC_8, 32.0, 5 / 12), (SC_8, 25.6, 9 / 16), (SC_8, 64 / 3, 17 / 24), (SC_32, 4096.0, 17 / 48)]
+
+
+@pytest.mark.parametrize("sc, wavelen, expect", HAND_VALUES)
+def test_rope_interpolation_at_points_worked_by_hand(sc, wavelen, expect):
+    assert abs(_scaled_over_base(P.rope_frequencies, wavelen, sc) - expect) < 2e-6
+
+
+def test_rope_interpolation_falls_from_one_to_one_over_factor_across_the_band():
+    # through the function itself: continuous at both edges of the band, monotone inside it, and
+    # linear in the frequency (smooth is linear in old/wavelen = old * freq / 2 pi)
+    ratio = lambda w: _scaled_over_base(P.rope_frequencies, w, SC_8)
+    assert ratio(15.99) == 1.0 and abs(ratio(16.01) - 1.0) < 1e-3            # old/hi = 16
+    assert abs(ratio(63.99) - 1 / 8) < 1e-4 and abs(ratio(64.01) - 1 / 8) < 1e-6   # old/lo = 64
+    ws = np.linspace(16.5, 63.5, 48)
+    rs = np.array([ratio(w) for w in ws])
+    assert np.all(np.diff(rs) < 0) and rs[0] < 1.0 and rs[-1] > 1 / 8
+    fs = 64.0 / ws                                                           # old/wavelen
+    np.testing.assert_allclose(rs, (1 - (fs - 1) / 3) / 8 + (fs - 1) / 3, atol=2e-6)
+
+
+def _library_forward(cfg, W, toks):
+    """The whole model out of library routines only (torch's rms_norm, scaled_dot_product_attention,
+    silu, complex multiplication for the rotation), float64: an implementation that shares no line
+    with ``plain_llama.forward``. Adjacent pairing rotates the complex numbers (x[2j], x[2j+1]),
+    half pairing (x[j], x[j + hs/2]). The frequencies are ``P.rope_frequencies``, pinned above."""
+    import torch.nn.functional as F
+    d, H, K, hs, Fdim, V, L = dims(cfg)
+    t = lambda n: torch.from_numpy(np.asarray(W[n])).double()
+    T = len(toks)
+    freq = torch.from_numpy(P.rope_frequencies(hs, cfg.get("rope_theta", 10000.0), cfg.get("rope_scaling"))).double()
+    ang = torch.arange(T, dtype=torch.float64)[:, None] * freq[None, :]
+    rot = torch.polar(torch.ones_like(ang), ang)                             # [T, hs/2]
+    adjacent = cfg.get("rope_pairing", "half") == "adjacent"
+
+    def rotate(x):                                                           # [T, heads, hs]
+        pairs = x.reshape(T, -1, hs // 2, 2) if adjacent else torch.stack((x[..., :hs // 2], x[..., hs // 2:]), -1)
+        z = torch.view_as_real(torch.view_as_complex(pairs.contiguous()) * rot[:, None, :])
+        return z.reshape(T, -1, hs) if adjacent else torch.cat((z[..., 0], z[..., 1]), -1)
+
+    eps = cfg.get("rms_norm_eps", 1e-5)
+    x = t("model.embed_tokens.weight")[torch.tensor(toks)]
+    for i in range(L):
+        n = P.layer_names(i)
+        h = F.rms_norm(x, (d,), t(n["attn_norm"]), eps)
+        q = rotate((h @ t(n["q"]).T).reshape(T, H, hs)).transpose(0, 1)     # [H, T, hs]
+        k = rotate((h @ t(n["k"]).T).reshape(T, K, hs)).transpose(0, 1)
+        v = (h @ t(n["v"]).T).reshape(T, K, hs).transpose(0, 1)
+        k, v = k.repeat_interleave(H // K, 0), v.repeat_interleave(H // K, 0)
+        a = F.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]
+        x = x + a.transpose(0, 1).reshape(T, H * hs) @ t(n["o"]).T
+        h = F.rms_norm(x, (d,), t(n["ffn_norm"]), eps)
+        x = x + (F.silu(h @ t(n["gate"]).T) * (h @ t(n["up"]).T)) @ t(n["down"]).T
+    head = t("model.embed_tokens.weight") if cfg.get("tie_word_embeddings", False) else t("lm_head.weight")
+    return (F.rms_norm(x, (d,), t("model.norm.weight"), eps) @ head.T).numpy()
+
+
+@pytest.mark.parametrize("cfg", [TINY_A, {**TINY_A, "rope_pairing": "half"}, TINY_B, TINY_C, TINY_D],
+                         ids=["A", "A-half", "B", "C", "D"])
+def test_whole_model_is_a_composition_of_library_routines(cfg):
+    W = make_weights(cfg, 21, norm_std=0.1)
+    toks = tokens(cfg, 21, 29)
+    got = P.forward(cfg, W, toks)
+    want = _library_forward(cfg, W, toks)
+    scale = float(np.abs(want).max())
+    assert float(np.abs(got - want).max()) < 3e-6 * scale
 
 
 def test_rope_rotation_is_a_complex_multiplication():
