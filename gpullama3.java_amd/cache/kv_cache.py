@@ -9,12 +9,20 @@ last two axes exchanged. A page is
 each entry may own a state area of fixed size per slot, ``[slot, elements]``,
 zeroed when the slot is handed out; the attention of this architecture asks for
 none (the reference has no such state either: J/inference/state/State.java:28-65).
+
+Every group also keeps its block table on the device, one row per slot, ``[n_slots + 1,
+pages of the longest sequence]``: a step names the rows (slot numbers) of its sequences and
+uploads no page numbers. The host changes single entries when a sequence gets or returns a
+page; the changes travel inside a launch (``flush_tables``). Row ``n_slots`` belongs to no
+sequence and names the sink page only: entries that pad a batch to a fixed size use it, and
+the matching row of every state area, so that they touch nothing a sequence owns.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
 from typing import Optional
 
+import numpy as np
 import torch
 
 from .pages import CacheFull, PagePool, SlotTable
@@ -46,6 +54,9 @@ class CacheGroup:
         # values lie transposed inside a page (positions contiguous): the order in which the
         # attention kernels' second product reads them
         self.v = torch.zeros((n, n_pages, need.n_kv_heads, need.head_dim, page_size), dtype=dtype, device=device)
+        self.table = None            # [n_slots + 1, pages of the longest sequence] int32 on the device
+        self.table_host = None       # the same on the host (numpy), the copy that the bookkeeping writes
+        self.dirty = {}              # flat place in the table -> page number, not yet on the device
 
 
 class Cache:
@@ -76,10 +87,15 @@ class Cache:
                 self.group_of[e] = (len(self.groups), i)
             self.groups.append(g)
         self.slots = SlotTable(n_slots, len(self.groups))
+        self._windowed = any(g.need.window for g in self.groups)
+        self.sink_slot = n_slots                             # the row of padded entries: no sequence's
+        for g in self.groups:
+            g.table_host = np.zeros((n_slots + 1, self.max_pages_per_seq), dtype=np.int32)
+            g.table = torch.zeros((n_slots + 1, self.max_pages_per_seq), dtype=torch.int32, device=device)
         self.state = {}
         for e, need in enumerate(state_needs):
             if need is not None and need.elements > 0:
-                self.state[e] = torch.zeros((n_slots, need.elements), dtype=need.dtype, device=device)
+                self.state[e] = torch.zeros((n_slots + 1, need.elements), dtype=need.dtype, device=device)
 
     # ---- slots
     def take_slot(self):
@@ -117,7 +133,28 @@ class Cache:
                                 f"{(group.pool.n_pages - 1) * self.page_size} tokens")
         for s, g, extra in plan:
             if extra > 0:
-                self.slots.pages[s][g].extend(self.groups[g].pool.take(extra))
+                pages = self.slots.pages[s][g]
+                first = len(pages)
+                pages.extend(self.groups[g].pool.take(extra))
+                self._table_set(g, s, first, pages[first:])
+
+    def reserve_one_each(self, slots):
+        """``reserve`` for a step that brings one token per sequence: nothing to do while every
+        sequence's last page has room (the usual case of a decode step)."""
+        page, pages, length = self.page_size, self.slots.pages, self.slots.length
+        for s in slots:
+            n = length[s]
+            if n >= self.max_context or any(n >= len(held) * page for held in pages[s]):
+                return self.reserve({s: 1 for s in slots})
+
+    def advance_one_each(self, slots):
+        if self._windowed:
+            for s in slots:
+                self.advance(s, 1)
+        else:
+            length = self.slots.length
+            for s in slots:
+                length[s] += 1
 
     def advance(self, s, n):
         """The sequence of slot ``s`` has ``n`` more tokens. A group with a window gives back the
@@ -136,6 +173,29 @@ class Cache:
                 group.pool.give_back([pages[i] for i in gone])
                 for i in gone:
                     pages[i] = 0
+                    self._table_set(g, s, i, [0])
+
+    # ---- the block tables on the device
+    def _table_set(self, g, slot, first, pages):
+        group = self.groups[g]
+        base = slot * self.max_pages_per_seq + first
+        for i, p in enumerate(pages):
+            group.table_host[slot, first + i] = p
+            group.dirty[base + i] = p
+
+    def flush_tables(self):
+        """Bring the device tables up to date (on the current stream): only entries that changed since
+        the last call travel, inside the launch of a small kernel."""
+        for group in self.groups:
+            if group.dirty:
+                from ..csrc import lib as K
+                K.scatter_i32(group.table, list(group.dirty.keys()), list(group.dirty.values()))
+                group.dirty = {}
+
+    def device_table(self, group):
+        """``[n_slots + 1, max_pages_per_seq]`` int32: row s holds slot s's pages (call ``flush_tables``
+        before a kernel reads it)."""
+        return self.groups[group].table
 
     # ---- what the kernels read
     def layer_kv(self, entry):

@@ -42,7 +42,7 @@ template <int HS, int GH>
 __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
-    int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
+    const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
     float scale, int q_blocks) {
   constexpr int KK = HS / 32;
   constexpr int DT = HS / 16;
@@ -68,7 +68,8 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   const int before = __builtin_amdgcn_readfirstlane(kv_before[b]);
   const int heads_here = min(GH, g - hg * GH);
   const int h0 = c * g + hg * GH;
-  const int* bt = block_table + (long)b * table_stride;
+  // the sequence's row of the table: its number in the batch, or what `seq_rows` says (a table with a row per cache slot)
+  const int* bt = block_table + (long)(seq_rows ? __builtin_amdgcn_readfirstlane(seq_rows[b]) : b) * table_stride;
   // the block's range of chunks, and the wave's own inside it
   const int blk_first = before + qb * 64, blk_last = before + min(qb * 64 + 63, q_len - 1);
   const int blk_lo = (window > 0 && blk_first + 1 > window) ? blk_first + 1 - window : 0;
@@ -262,7 +263,7 @@ template <int HS, int CK, int AHEAD, int OCC>
 __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ cu_seqlens, const int* __restrict__ kv_before, const int* __restrict__ block_table,
-    int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
+    const int* __restrict__ seq_rows, int table_stride, bf16_t* __restrict__ out, long out_stride, int n_heads, int n_kv, int page_size, int window,
     float scale, int q_blocks) {
   constexpr int KS = HS / 16;             // steps of the score product
   constexpr int DT = HS / 32;             // tiles of 32 dims of the output
@@ -286,7 +287,8 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   const int q_len = __builtin_amdgcn_readfirstlane(cu_seqlens[b + 1]) - tok0;
   if (qb * QB >= q_len) return;            // the whole block: no barrier has been passed yet
   const int before = __builtin_amdgcn_readfirstlane(kv_before[b]);
-  const int* bt = block_table + (long)b * table_stride;
+  // the sequence's row of the table: its number in the batch, or what `seq_rows` says (a table with a row per cache slot)
+  const int* bt = block_table + (long)(seq_rows ? __builtin_amdgcn_readfirstlane(seq_rows[b]) : b) * table_stride;
   const int blk_first = before + qb * QB, blk_last = before + min(qb * QB + QB - 1, q_len - 1);
   const int blk_lo = (window > 0 && blk_first + 1 > window) ? blk_first + 1 - window : 0;
   const int ck0 = blk_lo / CK, ck1 = blk_last / CK;
@@ -458,19 +460,21 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
 }
 
 // From how many tokens of the longest sequence of a step on the kernel with 128 queries a block is
-// taken (settable: tests run both kernels on the same inputs).
-extern "C" int gl3_attention_prefill_wide_from = 256;
+// taken, unless the caller says otherwise.
+#define GL3_PREFILL_WIDE_FROM 256
 
 extern "C" int gl3_attention_prefill_supports(int head_dim, int page_size) {
   return (head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128) && page_size % 32 == 0;
 }
 
 // max_q_len: the most tokens any sequence brings in this step (it sizes the grid).
+// seq_rows (may be null): the row of `block_table` that holds sequence b's pages; null: row b.
+// wide_from: the kernel with 128 queries a block is taken when max_q_len reaches it; <= 0: the default.
 extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k_cache, const void* v_cache,
                                      const int* cu_seqlens, const int* kv_before, const int* block_table,
-                                     int table_stride, void* out, long out_stride, int n_seqs, int max_q_len,
-                                     int n_heads, int n_kv, int head_dim, int page_size, int window, float scale,
-                                     hipStream_t stream) {
+                                     const int* seq_rows, int table_stride, void* out, long out_stride, int n_seqs,
+                                     int max_q_len, int n_heads, int n_kv, int head_dim, int page_size, int window,
+                                     float scale, int wide_from, hipStream_t stream) {
   if (n_seqs == 0 || max_q_len == 0) return 0;
   GL3_REQUIRE(q && k_cache && v_cache && cu_seqlens && kv_before && block_table && out,
               "gl3_attention_prefill: null argument");
@@ -484,7 +488,7 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
               "gl3_attention_prefill: queries must be 16-byte aligned, outputs 8-byte aligned");
   const int g = n_heads / n_kv;
   // query heads per wave: as many as the registers hold with two blocks on a CU
-  const bool wide = max_q_len >= gl3_attention_prefill_wide_from;
+  const bool wide = max_q_len >= (wide_from > 0 ? wide_from : GL3_PREFILL_WIDE_FROM);
   // query heads per wave: as many as the registers hold with two blocks on a CU; one with 32 queries a wave
   const int gh = wide ? 1 : head_dim <= 32 ? 4 : head_dim <= 64 ? 2 : 1;
   const long z = (long)n_kv * ((g + gh - 1) / gh);
@@ -496,7 +500,7 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
 #define GOW(HS, CK, AH, OCC)                                                                                        \
   attention_prefill_wide_kernel<HS, CK, AH, OCC><<<grid, block, 0, stream>>>(                                       \
       (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table, \
-      table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks)
+      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks)
     // chunks of 64 keys (one barrier for twice the work, two score tiles whose sums do not wait for
     // each other) where the registers hold them and a page holds whole chunks
     const bool ck64 = page_size % 64 == 0;
@@ -513,7 +517,7 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
 #define GO(HS, GH)                                                                                                  \
   attention_prefill_kernel<HS, GH><<<grid, block, 0, stream>>>(                                                     \
       (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu_seqlens, kv_before, block_table, \
-      table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks)
+      seq_rows, table_stride, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, q_blocks)
   switch (head_dim) {
     case 32: GO(32, 4); break;
     case 64: GO(64, 2); break;

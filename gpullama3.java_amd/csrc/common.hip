@@ -31,3 +31,88 @@ extern "C" int gl3_fill_u32(void* p, uint32_t v, long n, hipStream_t stream) {
   GL3_LAUNCH_CHECK();
   return 0;
 }
+
+// ---- scatter of a few integers whose places and values travel in the launch itself: how the host
+// changes entries of a table on the device (a page added to a sequence) without staging memory.
+#define GL3_SCATTER_MAX 128
+struct ScatterArgs { int idx[GL3_SCATTER_MAX]; int val[GL3_SCATTER_MAX]; };
+
+__global__ void scatter_i32_kernel(int* dst, int n, ScatterArgs a) {
+  const int i = threadIdx.x;
+  if (i < n) dst[a.idx[i]] = a.val[i];
+}
+
+// dst[idx[i]] = val[i] for i < n (host arrays); `limit`: elements of dst, every idx is checked against it.
+extern "C" int gl3_scatter_i32(int* dst, long limit, const int* idx, const int* val, int n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  GL3_REQUIRE(dst && idx && val, "gl3_scatter_i32: null argument");
+  for (int i = 0; i < n; ++i)
+    GL3_REQUIRE(idx[i] >= 0 && idx[i] < limit, "gl3_scatter_i32: place %d is outside the %ld elements", idx[i], limit);
+  for (int lo = 0; lo < n; lo += GL3_SCATTER_MAX) {
+    ScatterArgs a;
+    const int m = n - lo < GL3_SCATTER_MAX ? n - lo : GL3_SCATTER_MAX;
+    for (int i = 0; i < m; ++i) { a.idx[i] = idx[lo + i]; a.val[i] = val[lo + i]; }
+    for (int i = m; i < GL3_SCATTER_MAX; ++i) { a.idx[i] = 0; a.val[i] = 0; }
+    scatter_i32_kernel<<<dim3(1), dim3(GL3_SCATTER_MAX), 0, stream>>>(dst, m, a);
+    GL3_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+// ---- a copy from pinned host memory to the device on a stream (one call, no tensor objects)
+extern "C" int gl3_upload(void* dst, const void* src, long bytes, hipStream_t stream) {
+  if (bytes <= 0) return 0;
+  GL3_REQUIRE(dst && src, "gl3_upload: null argument");
+  hipError_t e = hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyHostToDevice, stream);
+  GL3_REQUIRE(e == hipSuccess, "gl3_upload: %s", hipGetErrorString(e));
+  return 0;
+}
+
+// ---- the input of a decode step, written into the device buffer that a captured step reads. The
+// numbers travel in the launch itself (no staging memory, nothing to wait for before the host may
+// write the next step's): tokens | positions | tokens held before (the same numbers) | slots, each
+// `n_pad` long; entries from `n` on are padding: token 0 at position 0 of slot `pad_slot`.
+#define GL3_STAGE_MAX 256
+struct StageArgs { int tok[GL3_STAGE_MAX]; int pos[GL3_STAGE_MAX]; int slot[GL3_STAGE_MAX]; };
+
+__global__ void stage_decode_kernel(int* dst, int n_pad, int first, int count, int n, int pad_slot, int* counter,
+                                    StageArgs a) {
+  const int i = threadIdx.x;
+  if (i < count) {
+    const int e = first + i;
+    const bool real = e < n;
+    dst[e] = real ? a.tok[i] : 0;
+    dst[n_pad + e] = real ? a.pos[i] : 0;
+    dst[2 * n_pad + e] = real ? a.pos[i] : 0;
+    dst[3 * n_pad + e] = real ? a.slot[i] : pad_slot;
+  }
+  if (i == 0 && first == 0 && counter) counter[0] = 0;
+}
+
+// tokens, positions, slots: host arrays of n entries. dst: device, at least 4 * n_pad ints. counter (may be
+// null): a device int set to 0 (the step counter of a run of steps).
+extern "C" int gl3_stage_decode(int* dst, int n_pad, int n, const int* tokens, const int* positions, const int* slots,
+                                int pad_slot, int* counter, hipStream_t stream) {
+  GL3_REQUIRE(dst && tokens && positions && slots && n >= 0 && n <= n_pad && n_pad > 0, "gl3_stage_decode: bad arguments");
+  for (int first = 0; first < n_pad; first += GL3_STAGE_MAX) {
+    StageArgs a;
+    const int count = n_pad - first < GL3_STAGE_MAX ? n_pad - first : GL3_STAGE_MAX;
+    for (int i = 0; i < count; ++i) {
+      const int e = first + i;
+      a.tok[i] = e < n ? tokens[e] : 0;
+      a.pos[i] = e < n ? positions[e] : 0;
+      a.slot[i] = e < n ? slots[e] : pad_slot;
+    }
+    stage_decode_kernel<<<dim3(1), dim3(GL3_STAGE_MAX), 0, stream>>>(dst, n_pad, first, count, n, pad_slot, counter, a);
+    GL3_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+// ---- launch of an instantiated graph (a captured decode step) on a stream
+extern "C" int gl3_graph_launch(void* graph_exec, hipStream_t stream) {
+  GL3_REQUIRE(graph_exec, "gl3_graph_launch: null graph");
+  hipError_t e = hipGraphLaunch((hipGraphExec_t)graph_exec, stream);
+  GL3_REQUIRE(e == hipSuccess, "gl3_graph_launch: %s", hipGetErrorString(e));
+  return 0;
+}

@@ -65,7 +65,11 @@ def _declare(lib):
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
-        "gl3_attention_prefill": [P, L, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, P],
+        "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P],
+        "gl3_scatter_i32": [P, L, P, P, I, P],
+        "gl3_upload": [P, P, L, P],
+        "gl3_stage_decode": [P, I, I, P, P, P, I, P, P],
+        "gl3_graph_launch": [P, P],
         "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P],
     }
     for name, args in sigs.items():
@@ -554,19 +558,13 @@ def attention_prefill_fits(head_dim, n_heads, n_kv, page_size):
     return bool(library().gl3_attention_prefill_supports(head_dim, page_size)) and n_heads % n_kv == 0
 
 
-def attention_prefill_wide_from(tokens=None):
-    """From how many tokens of a step's longest sequence on the prefill attention takes its kernel
-    with 128 queries a block; with an argument, sets it (tests run both kernels on the same inputs)."""
-    var = ctypes.c_int.in_dll(library(), "gl3_attention_prefill_wide_from")
-    if tokens is not None:
-        var.value = int(tokens)
-    return var.value
-
-
 def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, out, max_q_len, n_heads, n_kv,
-                      head_dim, page_size, window, scale):
+                      head_dim, page_size, window, scale, seq_rows=None, wide_from=0):
     """Any number of tokens per sequence; ``cu_seqlens`` [B+1] and ``kv_before`` [B] say which tokens
-    of the packed ``q`` belong to which sequence and where they sit in it."""
+    of the packed ``q`` belong to which sequence and where they sit in it. ``seq_rows`` [B] (optional)
+    names each sequence's row of ``block_table``; without it sequence b reads row b. ``wide_from``: from
+    how many tokens of the step's longest sequence on the kernel with 128 queries a block runs
+    (0: the library's choice; tests run both kernels on the same inputs)."""
     _dev(q, "q", torch.bfloat16, contiguous=False); _dev(out, "out", torch.bfloat16, contiguous=False)
     _dev(k_cache, "k_cache", torch.bfloat16); _dev(v_cache, "v_cache", torch.bfloat16)
     _dev(cu_seqlens, "cu_seqlens", torch.int32); _dev(kv_before, "kv_before", torch.int32)
@@ -578,9 +576,56 @@ def attention_prefill(q, k_cache, v_cache, cu_seqlens, kv_before, block_table, o
     if out.shape != (T, n_heads * head_dim) or out.stride(1) != 1:
         raise KernelError(f"attention: out {tuple(out.shape)}")
     _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention")
-    if cu_seqlens.numel() != B + 1 or block_table.dim() != 2 or block_table.shape[0] < B or max_q_len < 1:
+    if cu_seqlens.numel() != B + 1 or block_table.dim() != 2 or max_q_len < 1:
         raise KernelError("attention: cu_seqlens / kv_before / block_table shapes")
+    if seq_rows is not None:
+        _dev(seq_rows, "seq_rows", torch.int32)
+        if seq_rows.numel() != B:
+            raise KernelError("attention: one table row per sequence")
+    elif block_table.shape[0] < B:
+        raise KernelError("attention: the block table has fewer rows than there are sequences")
     _check(library().gl3_attention_prefill(
         _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(cu_seqlens), _ptr(kv_before), _ptr(block_table),
-        block_table.shape[1], _ptr(out), out.stride(0), B, int(max_q_len), n_heads, n_kv, head_dim, page_size,
-        int(window or 0), float(scale), _stream()), "attention_prefill")
+        _ptr(seq_rows), block_table.shape[1], _ptr(out), out.stride(0), B, int(max_q_len), n_heads, n_kv, head_dim,
+        page_size, int(window or 0), float(scale), int(wide_from), _stream()), "attention_prefill")
+
+
+# ------------------------------------------------------------------ host to device without tensor objects
+def scatter_i32(dst, places, values):
+    """dst.view(-1)[places[i]] = values[i]: the places and values travel in the launch itself."""
+    _dev(dst, "dst", torch.int32)
+    n = len(places)
+    if n != len(values):
+        raise KernelError("scatter_i32: as many places as values")
+    if n == 0:
+        return
+    arr = (c_int * n)
+    _check(library().gl3_scatter_i32(_ptr(dst), dst.numel(), arr(*places), arr(*values), n, _stream()), "scatter_i32")
+
+
+def stage_decode(dst, n_pad, tokens, positions, slots, pad_slot, counter=None):
+    """The input of a captured decode step into its device buffer ``dst`` (int32, 4 * n_pad at least):
+    tokens | positions | tokens held before | slots of ``len(tokens)`` sequences, padded to ``n_pad``
+    with one-token sequences in ``pad_slot``. The numbers travel inside the launch."""
+    n = len(tokens)
+    if len(positions) != n or len(slots) != n or n > n_pad or dst.numel() < 4 * n_pad:
+        raise KernelError("stage_decode: sizes")
+    arr = c_int * n
+    _check(library().gl3_stage_decode(_ptr(dst), n_pad, n, arr(*tokens), arr(*positions), arr(*slots), pad_slot,
+                                      _ptr(counter), _stream()), "stage_decode")
+
+
+def graph_launch(graph_exec):
+    """Launch an instantiated graph (its raw handle) on the current stream."""
+    _check(library().gl3_graph_launch(c_void_p(graph_exec), _stream()), "graph_launch")
+
+
+def upload(dst, src_pinned, n_bytes=None):
+    """Copy from pinned host memory to the device on the current stream."""
+    _dev(dst, "dst")
+    if src_pinned.is_cuda or not src_pinned.is_pinned():
+        raise KernelError("upload: the source must be pinned host memory")
+    n = src_pinned.numel() * src_pinned.element_size() if n_bytes is None else int(n_bytes)
+    if n > dst.numel() * dst.element_size() or n > src_pinned.numel() * src_pinned.element_size():
+        raise KernelError("upload: more bytes than the tensors hold")
+    _check(library().gl3_upload(_ptr(dst), c_void_p(src_pinned.data_ptr()), n, _stream()), "upload")

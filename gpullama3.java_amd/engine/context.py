@@ -4,8 +4,11 @@ belongs.
 All index arrays are int32 on the device: ``token_ids[T]``, ``positions[T]`` (a
 token's place in its own sequence), ``seq_of_token[T]`` (which row of the batch),
 ``cu_seqlens[B+1]``, ``kv_before[B]`` (tokens a sequence held before this step),
-and one block table ``[B, width]`` per cache group. Host copies of the lengths are
-kept for launch decisions.
+``slot_ids[B]`` (the cache slot of each sequence), and one block table per cache group
+with ``table_rows[T]`` / ``seq_rows[B]`` naming the table's row of each token / sequence
+(the engine passes the cache's own table, a row per slot, so these are slot numbers; a
+context built by hand may bring a table with a row per sequence and leave both unset).
+Host copies of the lengths are kept for launch decisions.
 """
 from __future__ import annotations
 
@@ -54,9 +57,28 @@ class StepContext:
         self.token_ids = self.positions = self.seq_of_token = self.cu_seqlens = self.kv_before = None
         self.slot_ids = None
         self._tables = []
+        self._table_rows = self._seq_rows = None
 
     def block_table(self, group):
         return self._tables[group]
+
+    @property
+    def table_rows(self):
+        """[T] the row of the block table that holds each token's sequence."""
+        return self._table_rows if self._table_rows is not None else self.seq_of_token
+
+    @table_rows.setter
+    def table_rows(self, v):
+        self._table_rows = v
+
+    @property
+    def seq_rows(self):
+        """[B] the row of the block table of each sequence; None: sequence b has row b."""
+        return self._seq_rows
+
+    @seq_rows.setter
+    def seq_rows(self, v):
+        self._seq_rows = v
 
     def buffer(self, name, shape, dtype):
         return self.engine.workspace.get(name, shape, dtype)
@@ -70,5 +92,6 @@ class StepContext:
         return torch.empty((n_rows, vocab), dtype=torch.float32, device=self.device)
 
     def slot_state(self, entry):
-        """``[n_slots, elements]`` state of one run-order entry; index with ``slot_ids``."""
+        """``[n_slots + 1, elements]`` state of one run-order entry; index with ``slot_ids`` (the last
+        row belongs to the entries that pad a batch: no sequence's)."""
         return self.cache.slot_state(entry)

@@ -10,7 +10,7 @@ final norm and the head run on the wanted rows only.
 """
 from __future__ import annotations
 
-import os
+import contextlib
 import tempfile
 
 import torch
@@ -41,13 +41,21 @@ def _require_gpu(device):
 
 
 RUN_LENGTH = 16     # most decode steps that run on the device before the host looks at the tokens
+_current_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
 class _DecodeGraph:
-    """A captured decode step for one batch bucket: its fixed input buffer and its logits; for runs
-    of steps also the sampling of the next tokens and their feeding back."""
-    graph = logits = host = dev = blank = fhost = fdev = copied = None
-    width = off_before = off_slots = off_tables = off_step = off_sampled = off_hist = 0
+    """A captured decode step for one batch bucket: its input buffer on the device and its logits;
+    for runs of steps also the sampling of the next tokens and their feeding back."""
+    graph = handle = logits = dev = step = fhost = fdev = None
+    B_pad = n_input = off_sampled = off_hist = 0
+
+    def launch(self):
+        from ..csrc import lib as K
+        if self.handle is not None:
+            K.graph_launch(self.handle)
+        else:
+            self.graph.replay()
 
 
 class Engine:
@@ -56,6 +64,8 @@ class Engine:
     def __init__(self, config, weights, dtype="bfloat16", device="cuda:0", max_tokens=None, max_context=None,
                  n_slots=None, page_size=64, use_graphs=True):
         self.device = _require_gpu(device)
+        if self.device.index is None:
+            self.device = torch.device("cuda", torch.cuda.current_device())
         self.dtype = _dtype(dtype)
         limit = config.max_position_embeddings
         max_context = limit if max_context is None or max_context < 0 else min(max_context, limit)
@@ -75,12 +85,12 @@ class Engine:
         self.sampler = DeviceSampler(self.device)
         self.metrics = RunMetrics()
         # Decode steps are replayed from captured graphs when every part's work is made of kernel
-        # launches on the current stream alone and no part keeps per-slot state (a padded entry
-        # of a bucketed batch must not touch a real slot).
+        # launches on the current stream alone. (Per-slot state is no obstacle: an entry that pads a
+        # bucketed batch works on the cache's sink slot, which no sequence owns.)
         parts = [p for b in self.model.blocks for p in b.parts()]
-        self.use_graphs = bool(use_graphs and not self.cache.state
-                               and all(getattr(p, "graph_safe", False) for p in parts))
-        self.fuse = bool(self.dtype == torch.bfloat16 and all(getattr(p, "graph_safe", False) for p in parts))
+        safe = all(getattr(p, "graph_safe", False) for p in parts)
+        self.use_graphs = bool(use_graphs and safe)
+        self.fuse = bool(self.dtype == torch.bfloat16 and safe)
         self._graphs = {}
         self._graphs_generation = 0
 
@@ -138,19 +148,21 @@ class Engine:
         Each sequence's tokens are appended at its own length. ``want``: "last"
         (the last token of every entry), "all", "none", or a list with one list of
         indices into each entry's tokens. Returns ``[rows, vocab]`` float32 on the
-        device, rows in the order of the entries and of their wanted indices. If the
-        cache has no room, ``CacheFull`` is raised and nothing has changed.
+        device, rows in the order of the entries and of their wanted indices: a tensor
+        of its own, which later steps do not touch. If the cache has no room,
+        ``CacheFull`` is raised and nothing has changed.
         """
         B = len(entries)
         if B == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        if want == "last" and self.use_graphs and all(len(e[1]) == 1 for e in entries):
+            return self._step_decode(entries)
         slots = [int(s) for s, _ in entries]
         if len(set(slots)) != B:
             raise ValueError("a slot appears twice in one step")
         V = self.spec.vocab_size
-        token_ids, positions, seq_of, cu, kv_before, want_rows = [], [], [], [0], [], []
+        token_ids, positions, seq_of, cu, kv_before, want_rows, slot_of = [], [], [], [0], [], [], []
         q_lens = []
-        last_only = True
         for b, (slot, toks) in enumerate(entries):
             toks = [int(t) for t in toks]
             if not toks:
@@ -170,11 +182,11 @@ class Engine:
                 idx = [int(i) for i in want[b]]
                 if any(not 0 <= i < n for i in idx):
                     raise ValueError(f"entry {b}: a wanted place is outside its {n} tokens")
-            last_only = last_only and idx == [n - 1]
             want_rows.extend(cu[-1] + i for i in idx)
             token_ids.extend(toks)
             positions.extend(range(start, start + n))
             seq_of.extend([b] * n)
+            slot_of.extend([slots[b]] * n)
             cu.append(cu[-1] + n)
             kv_before.append(start)
             q_lens.append(n)
@@ -182,44 +194,74 @@ class Engine:
         T = cu[-1]
         max_kv = max(k + n for k, n in zip(kv_before, q_lens))
         decode = all(n == 1 for n in q_lens)
-        with torch.cuda.device(self.device):
-            if self.use_graphs and decode and last_only:
-                logits = self._step_graph(B, token_ids, positions, slots, max_kv)
-            else:
-                logits = self._step_eager(B, T, token_ids, positions, seq_of, cu, kv_before, slots, want_rows,
-                                          q_lens, decode, max_kv)
+        with self._on_device():
+            self.cache.flush_tables()
+            ctx = StepContext(self, T, B, q_lens, kv_before, slots, decode=decode, max_q_len=max(q_lens),
+                              max_kv_len=max_kv)
+            dev = torch.tensor(token_ids + positions + seq_of + slot_of + cu + kv_before + slots + want_rows,
+                               dtype=torch.int32).to(self.device)
+            o = 0
+
+            def cut(n):
+                nonlocal o
+                t = dev[o:o + n]
+                o += n
+                return t
+
+            ctx.token_ids, ctx.positions, ctx.seq_of_token, ctx.table_rows = cut(T), cut(T), cut(T), cut(T)
+            ctx.cu_seqlens, ctx.kv_before, ctx.slot_ids = cut(B + 1), cut(B), cut(B)
+            ctx.seq_rows = ctx.slot_ids
+            rows = cut(len(want_rows))
+            ctx._tables = [self.cache.device_table(g) for g in range(len(self.cache.groups))]
+            logits = self.model.forward(ctx, rows)
         for s, n in zip(slots, q_lens):
             self.cache.advance(s, n)
         return logits
-
-    def _step_eager(self, B, T, token_ids, positions, seq_of, cu, kv_before, slots, want_rows, q_lens, decode, max_kv):
-        ctx = StepContext(self, T, B, q_lens, kv_before, slots, decode=decode, max_q_len=max(q_lens),
-                          max_kv_len=max_kv)
-        width = max(1, -(-max_kv // self.cache.page_size))
-        tables = [self.cache.block_rows(g, slots, width) for g in range(len(self.cache.groups))]
-        flat = token_ids + positions + seq_of + cu + kv_before + slots + want_rows
-        for t in tables:
-            for row in t:
-                flat.extend(row)
-        dev = torch.tensor(flat, dtype=torch.int32).to(self.device)
-        o = 0
-
-        def cut(n):
-            nonlocal o
-            t = dev[o:o + n]
-            o += n
-            return t
-
-        ctx.token_ids, ctx.positions, ctx.seq_of_token = cut(T), cut(T), cut(T)
-        ctx.cu_seqlens, ctx.kv_before, ctx.slot_ids = cut(B + 1), cut(B), cut(B)
-        rows = cut(len(want_rows))
-        ctx._tables = [cut(B * width).view(B, width) for _ in tables]
-        return self.model.forward(ctx, rows)
 
     # ------------------------------------------------------------------ decode steps from captured graphs
     @property
     def decode_run_length(self):
         return RUN_LENGTH if self.use_graphs else 1
+
+    def _decode_entries(self, entries):
+        """Checks of a step that brings one token per sequence; returns (slots, tokens, lengths)."""
+        V = self.spec.vocab_size
+        slots, tokens = [], []
+        for slot, tok in entries:
+            t = int(tok[0]) if isinstance(tok, (list, tuple)) else int(tok)
+            if not 0 <= t < V:
+                raise ValueError(f"token id {t} is outside the vocabulary of {V}")
+            slots.append(int(slot))
+            tokens.append(t)
+        if len(set(slots)) != len(slots):
+            raise ValueError("a slot appears twice in one step")
+        return slots, tokens, [self.cache.length(s) for s in slots]
+
+    def _on_device(self):
+        """The engine's device as the current one (entering a device context costs as much as a launch)."""
+        if _current_device is not None and _current_device() == self.device.index:
+            return contextlib.nullcontext()
+        return torch.cuda.device(self.device)
+
+    def _step_decode(self, entries):
+        """One token for each of B sequences: the step's tokens, positions and slot numbers are
+        written into the captured step's input buffer by a small kernel that carries them in its
+        launch, and the captured launches are replayed. The batch is padded to a bucket; a padded
+        entry is a one-token sequence in the cache's sink slot, so it reads and writes nothing
+        that a real sequence owns, and its logits are not returned."""
+        from ..csrc import lib as K
+        slots, tokens, starts = self._decode_entries(entries)
+        B = len(slots)
+        cache = self.cache
+        cache.reserve_one_each(slots)                                  # raises CacheFull, nothing changed
+        with self._on_device():
+            dg = self._graph_for(B, max(starts) + 1, run=False)
+            cache.flush_tables()
+            K.stage_decode(dg.dev, dg.B_pad, tokens, starts, slots, cache.sink_slot)
+            dg.launch()
+            logits = dg.logits[:B].clone()       # the graph's own buffer is overwritten by the next step
+        cache.advance_one_each(slots)
+        return logits
 
     def decode_run(self, entries, n, temperatures, top_ps, uniforms):
         """``n`` decode steps in a row for ``entries = [(slot, token), ...]``: every step samples
@@ -227,34 +269,27 @@ class Engine:
         end. ``uniforms[k][r]`` is step k's uniform number for entry r. Returns the sampled
         tokens ``[n][len(entries)]``. The cache has all n positions reserved before the first
         step, or ``CacheFull`` is raised and nothing has changed."""
-        B = len(entries)
         if not self.use_graphs or not 1 <= n <= RUN_LENGTH:
             raise ValueError(f"a run takes 1..{RUN_LENGTH} steps on an engine that replays graphs")
-        slots = [int(s) for s, _ in entries]
-        tokens = [int(t) for _, t in entries]
-        if len(set(slots)) != B:
-            raise ValueError("a slot appears twice in one step")
-        if any(not 0 <= t < self.spec.vocab_size for t in tokens):
-            raise ValueError("a token id is outside the vocabulary")
-        starts = [self.cache.length(s) for s in slots]
+        from ..csrc import lib as K
+        slots, tokens, starts = self._decode_entries(entries)
+        B = len(slots)
         self.cache.reserve({s: n for s in slots})
-        with torch.cuda.device(self.device):
+        with self._on_device():
             greedy = all(t == 0 for t in temperatures)
             dg = self._graph_for(B, max(starts) + n, run="greedy" if greedy else "sampled")
-            self._fill_graph_input(dg, B, tokens, starts, slots)
+            self.cache.flush_tables()
             B_pad = dg.B_pad
-            f = dg.fhost
+            f = dg.fhost                          # (free again: the last run ended with a wait for its tokens)
             f.zero_()
             f[0:B] = torch.tensor(list(temperatures), dtype=torch.float32)
             f[B_pad:B_pad + B] = torch.tensor(list(top_ps), dtype=torch.float32)
             u = torch.tensor([list(row) for row in uniforms], dtype=torch.float32)        # [n, B]
             f[2 * B_pad:2 * B_pad + RUN_LENGTH * B_pad].view(RUN_LENGTH, B_pad)[:n, :B] = u
             dg.fdev.copy_(f, non_blocking=True)
-            dg.dev.copy_(dg.host, non_blocking=True)
-            dg.copied = torch.cuda.Event()
-            dg.copied.record()
+            K.stage_decode(dg.dev, B_pad, tokens, starts, slots, self.cache.sink_slot, counter=dg.step)
             for _ in range(n):
-                dg.graph.replay()
+                dg.launch()
             hist = dg.dev[dg.off_hist:dg.off_hist + RUN_LENGTH * B_pad].view(RUN_LENGTH, B_pad)[:n, :B].cpu()
         for s in slots:
             self.cache.advance(s, n)
@@ -279,74 +314,44 @@ class Engine:
             self._graphs[key] = dg
         return dg
 
-    def _fill_graph_input(self, dg, B, token_ids, positions, slots):
-        h, W, B_pad = dg.host, dg.width, dg.B_pad
-        if dg.copied is not None:
-            dg.copied.synchronize()              # the last copy out of this pinned buffer has left it
-        h[:] = dg.blank
-        h[0:B] = torch.tensor(token_ids, dtype=torch.int32)
-        h[B_pad:B_pad + B] = torch.tensor(positions, dtype=torch.int32)
-        h[dg.off_before:dg.off_before + B] = h[B_pad:B_pad + B]
-        h[dg.off_slots:dg.off_slots + B] = torch.tensor(slots, dtype=torch.int32)
-        for g in range(len(self.cache.groups)):
-            rows = torch.tensor(self.cache.block_rows(g, slots, W), dtype=torch.int32)
-            o = dg.off_tables + g * B_pad * W
-            h[o:o + B * W] = rows.view(-1)
-
-    def _step_graph(self, B, token_ids, positions, slots, max_kv):
-        """One token for each of B sequences: the step's index arrays go into a fixed buffer and
-        the captured launches are replayed. The batch is padded to a bucket; a padded entry is a
-        one-token sequence whose block table names the sink page only, so it reads and writes
-        nothing that a real sequence owns, and its logits are not returned."""
-        dg = self._graph_for(B, max_kv, run=False)
-        self._fill_graph_input(dg, B, token_ids, positions, slots)
-        dg.dev.copy_(dg.host, non_blocking=True)
-        dg.copied = torch.cuda.Event()
-        dg.copied.record()
-        dg.graph.replay()
-        return dg.logits[:B]
-
     def _capture(self, B_pad, kv_bucket, run=False):
-        W = self.cache.max_pages_per_seq
+        from ..csrc import lib as K
         G = len(self.cache.groups)
         dg = _DecodeGraph()
-        dg.width, dg.B_pad = W, B_pad
-        # layout: tokens | positions | seq_of_token | cu_seqlens | kv_before | slots | rows | tables
-        dg.off_before = 3 * B_pad + B_pad + 1
-        dg.off_slots = dg.off_before + B_pad
-        off_rows = dg.off_slots + B_pad
-        dg.off_tables = off_rows + B_pad
-        dg.off_step = dg.off_tables + G * B_pad * W          # for runs: step counter, sampled tokens, their history
-        dg.off_sampled = dg.off_step + 1
+        dg.B_pad = B_pad
+        # the part that every step brings: tokens | positions | kv_before | slots | step counter;
+        # after it what never changes (sequence of each token, sequence bounds, wanted rows) and, for
+        # runs, the sampled tokens and their history
+        dg.n_input = 4 * B_pad + 1
+        off_seq = dg.n_input
+        off_cu = off_seq + B_pad
+        off_rows = off_cu + B_pad + 1
+        dg.off_sampled = off_rows + B_pad
         dg.off_hist = dg.off_sampled + B_pad
-        n = dg.off_hist + RUN_LENGTH * B_pad if run else dg.off_step
-        blank = torch.zeros(n, dtype=torch.int32)
+        n = dg.off_hist + RUN_LENGTH * B_pad if run else dg.off_sampled
+        fixed = torch.zeros(n, dtype=torch.int32)
+        fixed[3 * B_pad:4 * B_pad] = self.cache.sink_slot          # padded entries live in the sink slot
         ar = torch.arange(B_pad + 1, dtype=torch.int32)
-        blank[2 * B_pad:3 * B_pad] = ar[:B_pad]                   # seq_of_token
-        blank[3 * B_pad:3 * B_pad + B_pad + 1] = ar                # cu_seqlens
-        blank[off_rows:off_rows + B_pad] = ar[:B_pad]             # wanted rows: every entry's only token
-        dg.blank = blank
-        dg.host = torch.zeros(n, dtype=torch.int32).pin_memory()
-        dg.host[:] = blank
-        dg.dev = torch.zeros(n, dtype=torch.int32, device=self.device)
-        dg.dev.copy_(dg.host)
-        ctx = StepContext(self, B_pad, B_pad, [1] * B_pad, [0] * B_pad, [0] * B_pad, decode=True, max_q_len=1,
-                          max_kv_len=kv_bucket)
+        fixed[off_seq:off_seq + B_pad] = ar[:B_pad]                # seq_of_token
+        fixed[off_cu:off_cu + B_pad + 1] = ar                      # cu_seqlens
+        fixed[off_rows:off_rows + B_pad] = ar[:B_pad]              # wanted rows: every entry's only token
+        dg.dev = fixed.to(self.device)
+        ctx = StepContext(self, B_pad, B_pad, [1] * B_pad, [0] * B_pad, [self.cache.sink_slot] * B_pad, decode=True,
+                          max_q_len=1, max_kv_len=kv_bucket)
         ctx.kv_len_hint = kv_bucket
         d = dg.dev
-        ctx.token_ids, ctx.positions, ctx.seq_of_token = d[0:B_pad], d[B_pad:2 * B_pad], d[2 * B_pad:3 * B_pad]
-        ctx.cu_seqlens = d[3 * B_pad:4 * B_pad + 1]
-        ctx.kv_before = d[dg.off_before:dg.off_before + B_pad]
-        ctx.slot_ids = d[dg.off_slots:dg.off_slots + B_pad]
+        ctx.token_ids, ctx.positions, ctx.kv_before = d[0:B_pad], d[B_pad:2 * B_pad], d[2 * B_pad:3 * B_pad]
+        ctx.slot_ids = d[3 * B_pad:4 * B_pad]
+        ctx.table_rows = ctx.seq_rows = ctx.slot_ids               # one token per sequence: its slot is its table row
+        step = dg.step = d[4 * B_pad:4 * B_pad + 1]
+        ctx.seq_of_token = d[off_seq:off_seq + B_pad]
+        ctx.cu_seqlens = d[off_cu:off_cu + B_pad + 1]
         rows = d[off_rows:off_rows + B_pad]
-        ctx._tables = [d[dg.off_tables + g * B_pad * W:dg.off_tables + (g + 1) * B_pad * W].view(B_pad, W)
-                       for g in range(G)]
+        ctx._tables = [self.cache.device_table(g) for g in range(G)]
         if run:
-            from ..csrc import lib as K
             dg.fhost = torch.zeros((2 + RUN_LENGTH) * B_pad, dtype=torch.float32).pin_memory()
             dg.fdev = torch.zeros((2 + RUN_LENGTH) * B_pad, dtype=torch.float32, device=self.device)
             work = torch.empty(K.sample_work_size(B_pad, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-            step = d[dg.off_step:dg.off_step + 1]
             sampled = d[dg.off_sampled:dg.off_sampled + B_pad]
             hist = d[dg.off_hist:dg.off_hist + RUN_LENGTH * B_pad].view(RUN_LENGTH, B_pad)
             temps, tops = dg.fdev[0:B_pad], dg.fdev[B_pad:2 * B_pad]
@@ -376,6 +381,10 @@ class Engine:
                 dg.logits = body()
         finally:
             self.workspace.frozen = False
+        try:
+            dg.handle = int(dg.graph.raw_cuda_graph_exec())    # launched without the wrapper's bookkeeping
+        except Exception:
+            dg.handle = None
         return dg
 
     # ------------------------------------------------------------------ generation

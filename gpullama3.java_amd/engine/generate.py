@@ -142,8 +142,13 @@ def _run_batch(backend, requests, results, ids, on_token, metrics):
             return out.finish_reason is None
 
         def params(rows, k=0):
+            # the draw for the token at a position depends on (seed, request, that position): a sequence
+            # that goes on over several calls in a slot it keeps never meets the same number twice, as
+            # the reference's one generator runs on across the turns of a dialogue
+            # (J/inference/sampler/Sampler.java:63)
             return ([requests[i].sampling.temperature for i in rows], [requests[i].sampling.top_p for i in rows],
-                    [uniform(requests[i].sampling.seed, i, len(results[i].tokens) + k) for i in rows])
+                    [uniform(requests[i].sampling.seed, i,
+                             requests[i].cached + len(requests[i].prompt) + len(results[i].tokens) + k) for i in rows])
 
         # the prompts of the batch in one step, and each sequence's first token
         t0 = time.perf_counter()

@@ -181,6 +181,12 @@ def _linear_wide(a, w, out, epilogue, ctx):
     return True
 
 
+def _table_rows(ctx):
+    """The block table's row of each token: what the context says, else the token's sequence number."""
+    rows = getattr(ctx, "table_rows", None)
+    return rows if rows is not None else ctx.seq_of_token
+
+
 def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_heads, n_kv, head_dim, dtype, writes_kv):
     """Queries, keys and values of the step's tokens: q rotated into a buffer whose rows start
     with the H*hs query columns (returned), k rotated and v into the cache. One kernel when
@@ -193,7 +199,7 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
     if (isinstance(h, Normed) and writes_kv and h.rows is None and "fused" not in disabled
             and K.qkv_rope_cache_fits(h.xg, w_qkv, head_dim, rot)):
         q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
-        K.qkv_rope_cache(h.xg, h.ssq, h.n_partials, h.eps, w_qkv, q, ctx.positions, ctx.seq_of_token,
+        K.qkv_rope_cache(h.xg, h.ssq, h.n_partials, h.eps, w_qkv, q, ctx.positions, _table_rows(ctx),
                          block_table, cos, sin, k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page)
         return q
     if isinstance(h, Normed):
@@ -203,7 +209,7 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
             and K.qkv_rope_cache_fits(h[:64], w_qkv, head_dim, rot) and (T <= 64 or chunks)):
         q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
         for lo, hi in (chunks or [(0, T)]):
-            K.qkv_rope_cache(h[lo:hi], None, 0, 0.0, w_qkv, q[lo:hi], ctx.positions[lo:hi], ctx.seq_of_token[lo:hi],
+            K.qkv_rope_cache(h[lo:hi], None, 0, 0.0, w_qkv, q[lo:hi], ctx.positions[lo:hi], _table_rows(ctx)[lo:hi],
                              block_table, cos, sin, k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page)
         return q
     if writes_kv:
@@ -212,7 +218,7 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
     else:
         qkv = ctx.buffer("qkv", (T, n_heads * head_dim), dtype)
         linear(h, w_q, qkv)
-    K.rope_cache_write(qkv, ctx.positions, ctx.seq_of_token, block_table, cos, sin, k_cache, v_cache,
+    K.rope_cache_write(qkv, ctx.positions, _table_rows(ctx), block_table, cos, sin, k_cache, v_cache,
                        n_heads, n_kv, head_dim, rot, adjacent, page, write_kv=writes_kv)
     return qkv
 
@@ -228,11 +234,12 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
             if splits > 1:
                 part_o = ctx.buffer("attn_part_o", (T, n_heads, splits, head_dim), torch.float32)
                 part_ml = ctx.buffer("attn_part_ml", (T, n_heads, splits, 2), torch.float32)
-            return K.attention_decode(q, k_cache, v_cache, ctx.positions, ctx.seq_of_token, block_table, out, n_heads,
+            return K.attention_decode(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads,
                                       n_kv, head_dim, page, window, scale, splits, part_o, part_ml)
         if (not ctx.decode and "attn_prefill" not in disabled and K.has("gl3_attention_prefill") and scale > 0
                 and K.attention_prefill_fits(head_dim, n_heads, n_kv, page)):
             return K.attention_prefill(q, k_cache, v_cache, ctx.cu_seqlens, ctx.kv_before, block_table, out,
-                                       ctx.max_q_len, n_heads, n_kv, head_dim, page, window, scale)
-    return K.attention_generic(q, k_cache, v_cache, ctx.positions, ctx.seq_of_token, block_table, out, n_heads, n_kv,
+                                       ctx.max_q_len, n_heads, n_kv, head_dim, page, window, scale,
+                                       seq_rows=getattr(ctx, "seq_rows", None))
+    return K.attention_generic(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads, n_kv,
                                head_dim, page, window, scale)

@@ -47,7 +47,7 @@ def test_groups_have_storage_of_their_own():
     assert c.group_of == {0: (0, 0), 1: (0, 1), 2: (1, 0)}
     k, v = c.layer_kv(1)
     assert k.shape == (11, 2, 64, 16) and v.shape == (11, 2, 16, 64) and k.data_ptr() == c.groups[0].k[1].data_ptr()
-    assert c.slot_state(1).shape == (4, 6) and c.slot_state(0) is None
+    assert c.slot_state(1).shape == (5, 6) and c.slot_state(0) is None      # a row per slot and the sink row
 
 
 def test_reserve_is_all_or_nothing():
@@ -144,3 +144,26 @@ def test_a_group_with_a_window_gives_back_the_pages_behind_it():
     assert c.block_rows(1, [s], 7)[0][:4] == [0, 0, 0, 0]       # the places of the pages given back point at the sink
     c.give_back_slot(s)
     assert full.n_free == 8 and windowed.n_free == 8
+
+
+def test_the_table_of_every_group_follows_the_pages():
+    """The host copy of each group's block table (a row per slot, the last row no sequence's) holds what
+    the slots hold, and every change waits in ``dirty`` until it has travelled to the device."""
+    c = Cache([KVNeed(2, 16), KVNeed(1, 32, window=100)], [None, None], 640, 640, 3, torch.float32, "cpu", page_size=64)
+    a, b = c.take_slot(), c.take_slot()
+    c.reserve({a: 200, b: 5}); c.advance(a, 200); c.advance(b, 5)
+    W = c.max_pages_per_seq
+    for g, group in enumerate(c.groups):
+        assert group.table_host.shape == (4, W) and not group.table_host[c.sink_slot].any()
+        for s in (a, b):
+            pages = c.slots.pages[s][g]
+            assert group.table_host[s, :len(pages)].tolist() == pages
+        # after 200 tokens the first page of a lies behind the window of 100: its place names the sink page
+        assert (group.table_host[a, 0] == 0) == (group.need.window is not None)
+        assert {k: v for k, v in group.dirty.items()} == {
+            s * W + i: int(group.table_host[s, i]) for s in (a, b) for i in range(len(c.slots.pages[s][g]))}
+        group.dirty = {}
+    c.reserve({a: 1}); c.advance(a, 1)                       # no new page: nothing to send
+    assert all(not g.dirty for g in c.groups)
+    c.reserve({b: 60}); c.advance(b, 60)                     # b's second page
+    assert all(list(g.dirty) == [b * W + 1] for g in c.groups)

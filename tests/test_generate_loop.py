@@ -83,7 +83,7 @@ def alone(prompt, n, sampling=SamplingParams(), stops=(), index=0, max_context=6
     seq, out = list(prompt), []
     while len(out) < n:
         tok = P.sample(FakeBackend.logits_of(seq), sampling.temperature, sampling.top_p,
-                       uniform(sampling.seed, index, len(out)))
+                       uniform(sampling.seed, index, len(prompt) + len(out)))
         out.append(tok)
         if tok in stops or len(seq) >= max_context:
             break
@@ -230,8 +230,27 @@ def test_a_sequence_that_goes_on_keeps_its_slot_and_runs_single_steps():
     assert first == whole[:4] and be.runs == [] and s in be.seqs
     assert be.cache.length(s) == len(prompt) + 3            # the last sampled token has not been fed
     rest = generate(be, [Request([first[-1]], 5, SamplingParams(), slot=s, cached=be.cache.length(s))])[0].tokens
-    # the draw's index restarts with a request, greedy does not care
     assert first + rest == whole and be.cache.slots.n_free == be.n_slots - 1
+    be.give_back_slot(s)
+    # with temperature too: a draw is keyed by the token's position in its sequence, so a sequence that
+    # goes on over two calls draws what it would have drawn in one, and no turn repeats another's numbers
+    hot = SamplingParams(temperature=1.5, top_p=1.0, seed=4)
+    whole = generate(RunBackend(), [Request(prompt, 9, hot)])[0].tokens
+    s = be.take_slot()
+    first = generate(be, [Request(prompt, 4, hot, slot=s, cached=0)])[0].tokens
+    rest = generate(be, [Request([first[-1]], 5, hot, slot=s, cached=be.cache.length(s))])[0].tokens
+    assert first + rest == whole
+    seen = []
+    import sys
+    G = sys.modules[generate.__module__]
+    real = G.uniform
+    try:
+        G.uniform = lambda seed, r, step: seen.append(step) or real(seed, r, step)
+        generate(be, [Request([rest[-1]], 3, hot, slot=s, cached=be.cache.length(s))])
+        generate(be, [Request([7], 3, hot, slot=s, cached=be.cache.length(s))])
+    finally:
+        G.uniform = real
+    assert len(seen) == len(set(seen))                      # two turns on one state: no uniform is drawn twice
     be.give_back_slot(s)
     with pytest.raises(ValueError, match="no slot"):
         generate(be, [Request([1], 2, SamplingParams(), cached=3)])

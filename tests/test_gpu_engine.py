@@ -277,3 +277,52 @@ def test_replayed_graphs_equal_plain_launches(name, dtype):
         np.testing.assert_array_equal(got, np.stack(outs[0][i]))
         n0 = 8 + 5 * i
         close(got, plain_logits(name, seqs[i])[n0:n0 + 12], dtype, f"request {i}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_logits_of_a_step_outlive_the_steps_after_it(dtype):
+    """A caller may keep what ``step`` returned while it runs further steps of the same batch size
+    and context bucket: decode steps are replayed from a captured graph whose own logits buffer
+    the next replay overwrites, so ``step`` hands out a tensor of its own."""
+    name = "B"
+    eng = engine(name, dtype)
+    assert eng.use_graphs
+    a, b = rand_tokens(name, 40, 30), rand_tokens(name, 41, 21)
+    ref_a, ref_b = plain_logits(name, a), plain_logits(name, b)
+    sa, sb = eng.take_slot(), eng.take_slot()
+    eng.step([(sa, a[:20]), (sb, b[:11])], want="none")
+    kept = [eng.step([(sa, [a[20 + i]]), (sb, [b[11 + i]])]) for i in range(10)]    # ten results held at once
+    torch.cuda.synchronize()
+    assert len({k.data_ptr() for k in kept}) == 10
+    for i, k in enumerate(kept):
+        close(k.cpu().numpy(), np.stack([ref_a[20 + i], ref_b[11 + i]]), dtype, f"step {i} read after step 9")
+
+
+def test_a_decode_step_costs_the_host_little():
+    """The host's share of a decode step at batch 8 with the context of a real Llama 3.2 config.json
+    (131072 positions: 2,048 pages a sequence): no page number is uploaded per step (the block tables
+    live on the device, a row per slot), the step's tokens, positions and slots travel in one launch.
+    A one-layer model, so that the device is not what the loop waits for. The bound is three times
+    what the box measures, not the figure itself (it is printed)."""
+    import time
+    from gpullama3_java_amd.engine import Engine
+    cfg = {"architectures": ["LlamaForCausalLM"], "hidden_size": 256, "intermediate_size": 512, "num_hidden_layers": 1,
+           "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64, "vocab_size": 1024,
+           "max_position_embeddings": 131072, "rms_norm_eps": 1e-5, "rope_theta": 500000.0, "tie_word_embeddings": True}
+    eng = Engine.random(cfg, 0, dtype="bfloat16", max_tokens=8 * 4096, n_slots=8)
+    assert eng.cache.max_pages_per_seq == 2048
+    slots = [eng.take_slot() for _ in range(8)]
+    eng.step([(s, [1, 2, 3]) for s in slots], want="none")
+    entries = [(s, [5]) for s in slots]
+    for _ in range(50):
+        eng.step(entries)
+    torch.cuda.synchronize()
+    best = 1e9
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for _ in range(1000):
+            eng.step(entries)
+        best = min(best, (time.perf_counter() - t0) / 1000)
+        torch.cuda.synchronize()
+    print(f"host time of a decode step at batch 8: {best * 1e6:.1f} us")
+    assert best < 120e-6

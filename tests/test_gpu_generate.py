@@ -89,7 +89,7 @@ def test_sampled_generation_follows_the_logits():
     for i, (p, r) in enumerate(zip(prompts, res)):
         seq = list(p)
         for k, t in enumerate(r.tokens):
-            u = uniform(9, i, k)
+            u = uniform(9, i, len(p) + k)
             l = plain_logits(name, seq)[-1]
             want = P.sample(l, 0.8, 0.95, u)
             if t != want:                                   # allowed only at an edge of the running sum

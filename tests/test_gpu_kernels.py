@@ -560,24 +560,31 @@ def test_gemm_mfma(M, N, Kd):
 
 
 # ------------------------------------------------------------------ bfloat16 attention of a prefill step
-def prefill_fn(lens_before, new):
+WIDE_FROM = {"64 queries a block": 1 << 30, "128 queries a block": 1}
+
+
+def prefill_fn(lens_before, new, kernel, shuffled_rows=False):
     lib = K()
 
     def fn(q, kc, vc, positions, seq_of, table, out, H, Kh, hs, page, window, scale):
         cu = dev(np.concatenate([[0], np.cumsum(new)]), torch.int32)
+        seq_rows = None
+        if shuffled_rows:
+            # the table's rows in another order, with rows of the sink page between them: sequence b reads row seq_rows[b]
+            B = table.shape[0]
+            order = np.random.default_rng(B).permutation(2 * B)[:B]
+            big = torch.zeros((2 * B, table.shape[1]), dtype=torch.int32, device=table.device)
+            big[torch.as_tensor(order, device=table.device)] = table
+            table, seq_rows = big, dev(order, torch.int32)
         lib.attention_prefill(q, kc, vc, cu, dev(lens_before, torch.int32), table, out, max(new), H, Kh, hs, page,
-                              window, scale)
+                              window, scale, seq_rows=seq_rows, wide_from=WIDE_FROM[kernel])
     return fn
 
 
 @pytest.fixture(params=["64 queries a block", "128 queries a block"])
 def prefill_kernel(request):
     """Both kernels of the prefill attention on the same inputs, whatever the step's length."""
-    lib = K()
-    usual = lib.attention_prefill_wide_from()
-    lib.attention_prefill_wide_from(1 if request.param.startswith("128") else 1 << 30)
-    yield request.param
-    lib.attention_prefill_wide_from(usual)
+    return request.param
 
 
 @pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 32), (5, 5, 96), (8, 1, 128), (12, 2, 64), (3, 1, 128)])
@@ -585,12 +592,15 @@ def test_attention_prefill(H, Kh, hs, prefill_kernel):
     rng = np.random.default_rng(H * hs)
     lens_before, new = [0, 70, 0, 130, 5], [33, 1, 200, 17, 64]      # prompts, chunks after a prefix, one token
     sk, sv, qs = attention_case(rng, H, Kh, hs, lens_before, new, "bfloat16")
-    got, ref = run_attention(prefill_fn(lens_before, new), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng)
+    got, ref = run_attention(prefill_fn(lens_before, new, prefill_kernel), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng)
     np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+    got, ref = run_attention(prefill_fn(lens_before, new, prefill_kernel, shuffled_rows=True), sk, sv, qs, lens_before, new, H, Kh, hs,
+                             "bfloat16", rng)
+    np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max(), err_msg="table rows named by seq_rows")
     # pages of 32 and of 96 positions: chunks of 32 keys, several pages or a part of one to a chunk's page
     for page in (32, 96):
-        got, ref = run_attention(prefill_fn(lens_before, new), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng,
-                                 page=page)
+        got, ref = run_attention(prefill_fn(lens_before, new, prefill_kernel), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16",
+                                 rng, page=page)
         np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max(), err_msg=f"pages of {page}")
 
 
@@ -605,14 +615,14 @@ def test_attention_prefill_far_key_and_window_edge(prefill_kernel):
     q[n - 1, 2] = 0; q[n - 1, 2, 5] = 30.0
     k, v, q = (rounded(a, "bfloat16") for a in (k, v, q))
     for before, new in ((0, n), (500, 200)):                       # the whole prompt; a chunk after a prefix
-        got, ref = run_attention(prefill_fn([before], [new]), [k], [v], [q], [before], [new], H, Kh, hs, "bfloat16", rng)
+        got, ref = run_attention(prefill_fn([before], [new], prefill_kernel), [k], [v], [q], [before], [new], H, Kh, hs, "bfloat16", rng)
         np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
         np.testing.assert_allclose(got[-1, 2], v[far, 1], atol=4e-2)
     w = 100
     for hot, inside in ((n - w, True), (n - w - 1, False)):
         k2 = k.copy(); k2[far, 1] = 0.0; k2[hot, 1] = 0; k2[hot, 1, 5] = 30.0
         k2 = rounded(k2, "bfloat16")
-        got, ref = run_attention(prefill_fn([0], [n]), [k2], [v], [q], [0], [n], H, Kh, hs, "bfloat16", rng, window=w)
+        got, ref = run_attention(prefill_fn([0], [n], prefill_kernel), [k2], [v], [q], [0], [n], H, Kh, hs, "bfloat16", rng, window=w)
         np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
         assert (np.abs(got[-1, 2] - v[hot, 1]).max() < 4e-2) == inside
 
