@@ -43,7 +43,8 @@ class NormSpec:
 
 @dataclass(frozen=True)
 class AttentionSpec:
-    """Causal grouped-query attention over a cache of keys and values."""
+    """Causal grouped-query attention over a cache of keys and values. Names ``q_bias``, ``k_bias``,
+    ``v_bias`` (together) and ``o_bias`` among ``names`` add biases to the projections."""
     kind: str = "attention"
     hidden: int = 0
     n_heads: int = 0
@@ -57,7 +58,8 @@ class AttentionSpec:
 
 @dataclass(frozen=True)
 class GatedFeedForwardSpec:
-    """down(act(gate(x)) * up(x))."""
+    """down(act(gate(x)) * up(x)); ``activation``: "silu" or "gelu_tanh". Names ``gate_bias`` and
+    ``up_bias`` (together) and ``down_bias`` among ``names`` add biases to the products."""
     kind: str = "gated"
     hidden: int = 0
     intermediate: int = 0
@@ -101,3 +103,8 @@ class ModelSpec:
     embedding_name: str
     head_name: Optional[str]          # None when tied
     stop_ids: tuple = ()
+    # what other decoders put around the blocks; the reference's model has none of them
+    # (J/inference/InferenceCore.java:69, :175-177):
+    embedding_scale: Optional[float] = None       # the embedding row times this
+    position_table_name: Optional[str] = None     # a stored [max_positions, hidden] table whose row at the token's position is added to it
+    logit_scale: Optional[float] = None           # the logits times this

@@ -90,3 +90,18 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   for (int i = 1; i < nw; ++i) t = fmaxf(t, scratch[i]);
   return t;
 }
+
+// ---- what a product's epilogue may apply besides its own rule: a bias per output column (float;
+// for the gated epilogue the gate's biases, then the up's), and the activation of the gated
+// epilogue. The reference's feed-forward is silu without biases (J/inference/InferenceCore.java:158-166).
+enum { GL3_ACT_SILU = 0, GL3_ACT_GELU_TANH = 1 };
+
+template <bool FAST>
+__device__ __forceinline__ float gl3_activation(float v, int act) {
+  if (act == GL3_ACT_GELU_TANH) {
+    // 0.5 v (1 + tanh(sqrt(2/pi) (v + 0.044715 v^3))) = v / (1 + exp(-2 u))
+    const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+    return v / (1.0f + (FAST ? __expf(-2.0f * u) : expf(-2.0f * u)));
+  }
+  return v / (1.0f + (FAST ? __expf(-v) : expf(-v)));
+}

@@ -32,6 +32,22 @@ extern "C" int gl3_fill_u32(void* p, uint32_t v, long n, hipStream_t stream) {
   return 0;
 }
 
+// ---- p[i] *= s (what a model's logit scale is applied with)
+__global__ void scale_f32_kernel(float* p, float s, long n) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] *= s;
+}
+
+extern "C" int gl3_scale_f32(float* p, float s, long n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  GL3_REQUIRE(p != nullptr, "gl3_scale_f32: null pointer");
+  long blocks = (n + 255) / 256;
+  GL3_REQUIRE(blocks < (1L << 31), "gl3_scale_f32: %ld elements is too many", n);
+  scale_f32_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p, s, n);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---- scatter of a few integers whose places and values travel in the launch itself: how the host
 // changes entries of a table on the device (a page added to a sequence) without staging memory.
 #define GL3_SCATTER_MAX 128

@@ -3,16 +3,21 @@
 #include "common.h"
 
 // ----------------------------------------------------------------- embedding
-// out[t, :] = table[ids[t], :] as float (J/inference/InferenceCore.java:69).
+// out[t, :] = table[ids[t], :] as float (J/inference/InferenceCore.java:69); with `scale` != 1 the row
+// is multiplied by it, with `pos_table` ([positions][d], the table's type) row positions[t] of it is
+// added (the reference's model has neither: an embedding multiplier and learned absolute positions
+// are what other decoders put here).
 // ssq (may be null; then n_tokens <= 64): ssq[t] = sum of squares of row t, for a norm that is
 // folded into the product that follows; with it next_weight [d] (float) and xg [n_tokens][d]
 // (may be null): xg = bfloat16(next_weight * row), the rows as that product reads them.
 template <typename TW, bool VEC>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out, int d,
-                             float* __restrict__ ssq, const float* __restrict__ next_weight, bf16_t* __restrict__ xg) {
+                             float* __restrict__ ssq, const float* __restrict__ next_weight, bf16_t* __restrict__ xg,
+                             float scale, const TW* __restrict__ pos_table, const int* __restrict__ positions) {
   __shared__ float scratch[16];
   const long t = blockIdx.x;
   const TW* row = table + (long)ids[t] * d;
+  const TW* prow = pos_table ? pos_table + (long)positions[t] * d : nullptr;
   float* o = out + t * d;
   float ss = 0.f;
   if (VEC) {
@@ -24,10 +29,18 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
       const tw8 r8 = *(const tw8*)(row + i);
       float v[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        v[e] = to_f32<TW>(r8[e]);
-        ss += v[e] * v[e];
+      for (int e = 0; e < 8; ++e) v[e] = to_f32<TW>(r8[e]);
+      if (scale != 1.0f) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= scale;
       }
+      if (prow) {
+        const tw8 p8 = *(const tw8*)(prow + i);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += to_f32<TW>(p8[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
       *(f32x4*)(o + i) = f32x4{v[0], v[1], v[2], v[3]};
       *(f32x4*)(o + i + 4) = f32x4{v[4], v[5], v[6], v[7]};
       if (xg) {
@@ -43,7 +56,9 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
     }
   } else {
     for (int i = threadIdx.x; i < d; i += blockDim.x) {
-      const float v = to_f32<TW>(row[i]);
+      float v = to_f32<TW>(row[i]);
+      if (scale != 1.0f) v *= scale;
+      if (prow) v += to_f32<TW>(prow[i]);
       o[i] = v;
       ss += v * v;
       if (xg) xg[t * d + i] = static_cast<bf16_t>(next_weight[i] * v);
@@ -56,18 +71,22 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
 }
 
 extern "C" int gl3_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens, int d,
-                         float* ssq, const float* next_weight, void* xg, hipStream_t stream) {
+                         float* ssq, const float* next_weight, void* xg, float scale, const void* pos_table,
+                         const int* positions, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(table && ids && out && n_tokens > 0 && d > 0, "gl3_embed: bad arguments (T=%d d=%d)", n_tokens, d);
   GL3_REQUIRE(!ssq || n_tokens <= 64, "gl3_embed: sums of squares are kept for at most 64 rows");
   GL3_REQUIRE((next_weight == nullptr) == (xg == nullptr) && (!xg || ssq),
               "gl3_embed: the next norm's weight and its rows come together, with the sums of squares");
+  GL3_REQUIRE(!pos_table || positions, "gl3_embed: a table of positions needs the tokens' positions");
   dim3 grid(n_tokens), block(256);
   // 16-byte units where the rows allow them (a width of a multiple of 8, aligned bases)
   const bool vec = d % 8 == 0 && (uintptr_t)table % 32 == 0 && (uintptr_t)out % 16 == 0 &&
+                   (!pos_table || (uintptr_t)pos_table % 32 == 0) &&
                    (!xg || ((uintptr_t)xg % 16 == 0 && (uintptr_t)next_weight % 16 == 0));
 #define GO(TW, VEC)                                                                                              \
-  embed_kernel<TW, VEC><<<grid, block, 0, stream>>>((const TW*)table, ids, out, d, ssq, next_weight, (bf16_t*)xg)
+  embed_kernel<TW, VEC><<<grid, block, 0, stream>>>((const TW*)table, ids, out, d, ssq, next_weight, (bf16_t*)xg, scale, \
+                                                    (const TW*)pos_table, pos_table ? positions : nullptr)
   if (table_dtype == GL3_F32) { if (vec) GO(float, true); else GO(float, false); }
   else if (table_dtype == GL3_BF16) { if (vec) GO(bf16_t, true); else GO(bf16_t, false); }
   else GL3_REQUIRE(false, "gl3_embed: unknown dtype %d", table_dtype);

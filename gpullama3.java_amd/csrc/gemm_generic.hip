@@ -11,7 +11,9 @@
 // Epilogues: store (as float or bfloat16), add into a float matrix in place (the
 // residual stream; the reference fuses the same, TransformerComputeKernelsLayered
 // .java:766-784), and gated: W holds [gate rows | up rows] and the kernel writes
-// silu(gate) * up (J/inference/InferenceCore.java:158-166).
+// act(gate) * up, act = silu as the reference's (J/inference/InferenceCore.java:158-166) or the tanh form
+// of gelu. An optional bias per output column (float; gated: the gate's, then the up's) is added to
+// the sums before anything else.
 #include "common.h"
 
 #define GT 64   // tile edge
@@ -22,7 +24,8 @@ enum { EPI_STORE = 0, EPI_ADD = 1, EPI_GATED = 2 };
 template <typename TA, typename TW, typename TC, int EPI>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
                                                             TC* __restrict__ C, int M, int N, int K, long lda,
-                                                            long ldw, long ldc, long up_offset) {
+                                                            long ldw, long ldc, long up_offset,
+                                                            const float* __restrict__ bias, int act) {
   // N is the number of output columns; for EPI_GATED the up rows of W start at
   // row `up_offset`.
   __shared__ float As[GK][GT + 1];
@@ -81,9 +84,11 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
       const long n = n0 + tx * 4 + j;
       if (n >= N) continue;
       float v = acc[i][j];
+      if (bias) v += bias[n];
       if (EPI == EPI_GATED) {
-        v = v / (1.0f + expf(-v));
-        v = v * accu[i][j];
+        float u = accu[i][j];
+        if (bias) u += bias[up_offset + n];
+        v = gl3_activation<false>(v, act) * u;
       }
       TC* c = C + m * ldc + n;
       if (EPI == EPI_ADD) *c = from_f32<TC>(to_f32<TC>(*c) + v);
@@ -94,35 +99,38 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
 
 template <typename TA, typename TW, typename TC>
 static int launch_generic(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                          int epi, hipStream_t stream) {
+                          int epi, const float* bias, int act, hipStream_t stream) {
   dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT), block(256);
   GL3_REQUIRE(grid.y <= 65535, "gl3_gemm_generic: M=%d is too large for one launch", M);
   const TA* a = (const TA*)A;
   const TW* w = (const TW*)W;
   TC* c = (TC*)C;
-  if (epi == EPI_STORE) gemm_generic_kernel<TA, TW, TC, EPI_STORE><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0);
-  else if (epi == EPI_ADD) gemm_generic_kernel<TA, TW, TC, EPI_ADD><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0);
-  else gemm_generic_kernel<TA, TW, TC, EPI_GATED><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, N);
+  if (epi == EPI_STORE) gemm_generic_kernel<TA, TW, TC, EPI_STORE><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act);
+  else if (epi == EPI_ADD) gemm_generic_kernel<TA, TW, TC, EPI_ADD><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act);
+  else gemm_generic_kernel<TA, TW, TC, EPI_GATED><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, N, bias, act);
   GL3_LAUNCH_CHECK();
   return 0;
 }
 
 // N counts output columns: for the gated epilogue W has 2N rows (gate, then up).
+// bias (may be null): N floats (gated: 2N). act: the gated epilogue's activation (GL3_ACT_*).
 extern "C" int gl3_gemm_generic(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M,
-                                int N, int K, long lda, long ldw, long ldc, int epilogue, hipStream_t stream) {
+                                int N, int K, long lda, long ldw, long ldc, int epilogue, const float* bias, int act,
+                                hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_generic: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gl3_gemm_generic: leading dimensions %ld %ld %ld too small", lda, ldw, ldc);
   GL3_REQUIRE(epilogue >= 0 && epilogue <= 2, "gl3_gemm_generic: unknown epilogue %d", epilogue);
   GL3_REQUIRE(epilogue != EPI_ADD || c_dtype == GL3_F32, "gl3_gemm_generic: the add epilogue needs a float output");
+  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_generic: unknown activation %d", act);
   const int key = a_dtype * 4 + w_dtype * 2 + c_dtype;
   switch (key) {
-    case 0: return launch_generic<float, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
-    case 2: return launch_generic<float, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
-    case 4: return launch_generic<bf16_t, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
-    case 5: return launch_generic<bf16_t, float, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
-    case 6: return launch_generic<bf16_t, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
-    case 7: return launch_generic<bf16_t, bf16_t, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, stream);
+    case 0: return launch_generic<float, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, stream);
+    case 2: return launch_generic<float, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, stream);
+    case 4: return launch_generic<bf16_t, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, stream);
+    case 5: return launch_generic<bf16_t, float, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, stream);
+    case 6: return launch_generic<bf16_t, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, stream);
+    case 7: return launch_generic<bf16_t, bf16_t, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, stream);
     default:
       GL3_REQUIRE(false, "gl3_gemm_generic: unsupported dtypes A=%d W=%d C=%d", a_dtype, w_dtype, c_dtype);
   }

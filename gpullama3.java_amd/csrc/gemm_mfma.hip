@@ -30,7 +30,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
                                                                   const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                   int M, int N, int K, long lda, long ldw, long ldc,
                                                                   int tiles_m, int tiles_n, int k_per_slice,
-                                                                  float* __restrict__ P, long p_stride, long ldp) {
+                                                                  float* __restrict__ P, long p_stride, long ldp,
+                                                                  const float* __restrict__ bias, int act) {
   constexpr int NT = 64 * WM * WN;                       // threads
   constexpr int BM = 32 * TM * WM;                       // rows of a block
   constexpr int BN = 64 * WN;                            // rows of W of a block
@@ -179,8 +180,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
       if (EPI == MF_GATED) {
         const int n = n0 + wn * 32 + lr;
         if (n < N) {
-          const float g = acc[tm][0][v];
-          C[(long)m * ldc + n] = from_f32<TC>(g / (1.0f + __expf(-g)) * acc[tm][1][v]);
+          float g = acc[tm][0][v], u = acc[tm][1][v];
+          if (bias) { g += bias[n]; u += bias[N + n]; }
+          C[(long)m * ldc + n] = from_f32<TC>(gl3_activation<true>(g, act) * u);
         }
       } else {
 #pragma unroll
@@ -188,8 +190,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
           const int n = n0 + wn * 64 + tn * 32 + lr;
           if (n < N) {
             TC* c = C + (long)m * ldc + n;
-            if (EPI == MF_ADD) *c = from_f32<TC>(to_f32<TC>(*c) + acc[tm][tn][v]);
-            else *c = from_f32<TC>(acc[tm][tn][v]);
+            const float s = acc[tm][tn][v] + (bias ? bias[n] : 0.f);
+            if (EPI == MF_ADD) *c = from_f32<TC>(to_f32<TC>(*c) + s);
+            else *c = from_f32<TC>(s);
           }
         }
       }
@@ -199,7 +202,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
 
 template <int EPI, typename TC, int TM, int WM, int WN>
 static int launch_shape(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                        int slices, float* P, long p_stride, long ldp, hipStream_t stream) {
+                        int slices, float* P, long p_stride, long ldp, const float* bias, int act, hipStream_t stream) {
   const int bm = 32 * TM * WM;
   const int ncols = (EPI == MF_GATED) ? 32 * WN : 64 * WN;
   const int tiles_n = (N + ncols - 1) / ncols;
@@ -210,30 +213,31 @@ static int launch_shape(const void* A, const void* W, void* C, int M, int N, int
   const int k_per_slice = ((K + MF_BK - 1) / MF_BK + slices - 1) / slices * MF_BK;
   gemm_mfma_kernel<EPI, TC, TM, WM, WN><<<dim3((unsigned)blocks, slices), dim3(64 * WM * WN), 0, stream>>>(
       (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n, k_per_slice, P, p_stride,
-      ldp);
+      ldp, bias, act);
   GL3_LAUNCH_CHECK();
   return 0;
 }
 
 template <int EPI, typename TC>
 static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                       int slices, float* P, long p_stride, long ldp, hipStream_t stream) {
+                       int slices, float* P, long p_stride, long ldp, const float* bias, int act, hipStream_t stream) {
   // 256 x 256 tiles of sixteen waves where there is at least one for every CU: half the operand
   // traffic per product, and that traffic is what bounds the large products. Otherwise 128 x 128
   // tiles of eight waves, of which several fit a CU and overlap each other's waits.
   const long big_n = (EPI == MF_GATED) ? (N + 127) / 128 : (N + 255) / 256;
   if ((long)((M + 255) / 256) * big_n * slices >= 256)
-    return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, stream);
-  return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, stream);
+    return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
+  return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
 }
 
 // N counts output columns: for the gated epilogue W has 2N rows (gate, then up).
 // slices > 1 (not with the gated epilogue): K is cut into that many slices; the first ends in the
 // epilogue into C, slice s > 0 stores its sums into P[s - 1] ([slices - 1][M][ldp] floats,
 // p_stride elements apart), which the caller adds to C in that order.
+// bias (may be null; not with slices): N floats (gated: 2N). act: the gated epilogue's activation.
 extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
-                             long ldc, int epilogue, int slices, float* P, long p_stride, long ldp,
-                             hipStream_t stream) {
+                             long ldc, int epilogue, int slices, float* P, long p_stride, long ldp, const float* bias,
+                             int act, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_mfma: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gl3_gemm_mfma: K=%d, lda=%ld, ldw=%ld must be multiples of 8",
@@ -249,7 +253,9 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
               slices, K);
   GL3_REQUIRE(slices == 1 || (epilogue != MF_GATED && P && ldp >= N && p_stride >= (long)(M - 1) * ldp + N),
               "gl3_gemm_mfma: slices need a buffer for their sums and another epilogue than the gated one");
-#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, stream
+  GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_mfma: a bias goes with one slice of K");
+  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_mfma: unknown activation %d", act);
+#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream
   if (c_dtype == GL3_F32) {
     if (epilogue == MF_STORE) return launch_mfma<MF_STORE, float>(ARGS);
     if (epilogue == MF_ADD) return launch_mfma<MF_ADD, float>(ARGS);

@@ -52,11 +52,16 @@ struct SkNorm {
   const int* rows;        // may be null: row m of the product reads row rows[m] of A
 };
 
-// For the norm that follows an add epilogue: its weight, and where bfloat16(weight * x) goes.
+// What the end of a product applies or leaves besides its epilogue's own rule. For the norm that
+// follows an add epilogue: its weight, and where bfloat16(weight * x) goes. For any epilogue but
+// the rotation's: a bias per output column, added to the sums first (gated: the gate's biases,
+// then the up's), and the activation of the gated epilogue (GL3_ACT_*).
 struct SkNext {
   const float* weight;    // [N] float; null: nothing is written
   bf16_t* xg;             // [M][ld]
   long ld;
+  const float* bias;      // [N] (gated: [2N]) float; null: none
+  int act;
 };
 
 struct SkRope {
@@ -132,6 +137,7 @@ __device__ __forceinline__ void sk_ssq_partials(float (*sm_ssq)[64], int M, cons
 // token tile `mt`; a lane holds 4 columns of one token.
 struct SkPre {
   f32x4 prev;
+  f32x4 bias, bias_up;   // the biases of this lane's columns (zero without a bias)
   f32x4 next_w;     // the next norm's weight at this lane's columns
   f32x4 co, si;
   int pos;
@@ -142,12 +148,21 @@ template <int MT, int EPI, typename TC, int ROWS = 16>
 __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int N, long ldc, int strip, int hd, int sub,
                                             bool rotated, const SkRope& rp, const SkNext& nx = SkNext{}) {
   SkPre p;
-  p.prev = p.next_w = p.co = p.si = f32x4{0.f, 0.f, 0.f, 0.f};
+  p.prev = p.bias = p.bias_up = p.next_w = p.co = p.si = f32x4{0.f, 0.f, 0.f, 0.f};
   p.pos = 0; p.page = 0;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
   const int m = wave * 16 + r;
   if (wave >= MT || m >= M || 4 * q >= ROWS) return p;
+  if (EPI != SK_QKV && nx.bias) {
+    const int n = strip * ROWS + 4 * q;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      if (n + c < N) {
+        p.bias[c] = nx.bias[n + c];
+        if (EPI == SK_GATED) p.bias_up[c] = nx.bias[N + n + c];
+      }
+  }
   if (EPI == SK_ADD) {
     const int n = strip * ROWS + 4 * q;
     const TC* cp = C + (long)m * ldc + n;
@@ -220,9 +235,13 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
       v *= rms;
       up *= rms;
     }
+    if (EPI != SK_QKV) {
+      v += pre.bias;
+      up += pre.bias_up;
+    }
     if (EPI == SK_GATED) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c) v[c] = v[c] / (1.0f + __expf(-v[c])) * up[c];
+      for (int c = 0; c < 4; ++c) v[c] = gl3_activation<true>(v[c], nx.act) * up[c];
     }
     if (EPI == SK_QKV) {
       const int hs = rp.head_dim;
@@ -486,7 +505,8 @@ template <int MT, int NS, int NW, int EPI, typename TC>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t* __restrict__ A,
                                                                    const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                    int M, int N, int K, long lda, long ldw, long ldc,
-                                                                   long slice_stride, int steps_per_slice, SkRope rp) {
+                                                                   long slice_stride, int steps_per_slice, SkRope rp,
+                                                                   SkNext nx) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   constexpr int UNROLL = 4;
   __shared__ f32x4 red[NW][NG * MT][64];
@@ -511,7 +531,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   SkPre pre[NS];
 #pragma unroll
   for (int g = 0; g < NS; ++g)
-    pre[g] = sk_preload<MT, EPI, TC>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g], rotated[g], rp);
+    pre[g] = sk_preload<MT, EPI, TC>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g], rotated[g], rp, nx);
 
   const int steps = (K + 31) / 32;
   const int s_begin = blockIdx.y * steps_per_slice;
@@ -557,7 +577,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
     if (g) __syncthreads();   // the partial tiles in shared memory are free again
     if (strip0 + g < n_strips)   // the same for all threads of the block
       sk_finish<MT, NW, EPI, TC, false, false>(red, sm_ssq, acc[g], strip0 + g, hd[g], sub[g], rotated[g], out, M, N, K,
-                                                ldc, SkNorm{}, nullptr, rp, SkNext{}, pre[g]);
+                                                ldc, SkNorm{}, nullptr, rp, nx, pre[g]);
   }
 }
 
@@ -681,9 +701,11 @@ static int check_common(const char* who, const void* A, const void* W, const voi
 // row per 8 columns, [ceil(N/8)][64].
 // next_weight, xg (may be null; with ssq_out): the weight [N] (float) of the norm that follows, and
 // where bfloat16(weight * x) of the completed rows goes, [M][ldxg].
+// bias (may be null): N floats (gated: 2N), added to the sums; act: the gated epilogue's activation.
 extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                long ldw, long ldc, int epilogue, int waves, float* ssq_out, int strip_rows,
-                               const float* next_weight, void* xg, long ldxg, hipStream_t stream) {
+                               const float* next_weight, void* xg, long ldxg, const float* bias, int act,
+                               hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny", A, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny: ldc too small");
@@ -696,7 +718,8 @@ extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtyp
   GL3_REQUIRE((next_weight == nullptr) == (xg == nullptr) && (!xg || (ssq_out && ldxg >= N)),
               "gl3_gemm_skinny: the next norm's weight and its rows come together, with the sums of squares");
   SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, ssq_out, SkRope{}, stream, waves == 0, strip_rows};
-  a.nx = SkNext{next_weight, (bf16_t*)xg, ldxg};
+  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny: unknown activation %d", act);
+  a.nx = SkNext{next_weight, (bf16_t*)xg, ldxg, bias, act};
   const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32) {
     if (epilogue == SK_STORE) return pick_mt<SK_STORE, float, false, false>(nw, a);
@@ -720,7 +743,7 @@ static int launch_wide(const SkCall& a, int slices, long slice_stride) {
   gemm_skinny_wide_kernel<MT, NS, NW, EPI, TC>
       <<<dim3((n_strips + NS - 1) / NS, slices), dim3(NW * 64), 0, a.stream>>>(
           (const bf16_t*)a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, slice_stride, per_slice,
-          a.rp);
+          a.rp, a.nx);
   GL3_LAUNCH_CHECK();
   return 0;
 }
@@ -746,9 +769,10 @@ static int wide_strips(int N, int slices, int epilogue) {
 // The product for 33 to 64 rows of A (bfloat16). `slices` > 1 (store epilogue, float output only):
 // K is cut into that many slices and C is [slices][M][ldc] with `slice_stride` elements between
 // slices; the caller adds them up. `strips_per_block`: 0 lets the library choose.
+// bias (may be null; one slice only): N floats (gated: 2N); act: the gated epilogue's activation.
 extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                     long ldw, long ldc, int epilogue, int slices, long slice_stride,
-                                    int strips_per_block, hipStream_t stream) {
+                                    int strips_per_block, const float* bias, int act, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_wide", A, W, C, M, N, K, lda, ldw, 0)) return -1;
   GL3_REQUIRE(M > 32, "gl3_gemm_skinny_wide: M=%d; up to 32 rows are gl3_gemm_skinny's", M);
@@ -762,7 +786,10 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
   if (strips_per_block == 0) strips_per_block = wide_strips(N, slices, epilogue);
   GL3_REQUIRE(strips_per_block == big || strips_per_block == big / 2, "gl3_gemm_skinny_wide: %d strips per block",
               strips_per_block);
-  const SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, nullptr, SkRope{}, stream, false};
+  GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_skinny_wide: a bias goes with one slice of K");
+  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny_wide: unknown activation %d", act);
+  SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, nullptr, SkRope{}, stream, false};
+  a.nx = SkNext{nullptr, nullptr, 0, bias, act};
   if (c_dtype == GL3_F32) {
     if (epilogue == SK_STORE) return pick_wide<SK_STORE, float>(a, strips_per_block, slices, slice_stride);
     if (epilogue == SK_ADD) return pick_wide<SK_ADD, float>(a, strips_per_block, slices, slice_stride);
@@ -778,16 +805,19 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
 // [n_partials][64] partial sums of squares of the rows of x (indexed by the row of x, so x has at
 // most 64 rows); `rows` (may be null) picks the rows of x that the product's rows read.
 // Epilogues: store (float or bfloat16) and gated (bfloat16).
+// bias (may be null): N floats (gated: 2N), added after the 1/rms; act: the gated epilogue's activation.
 extern "C" int gl3_gemm_skinny_norm(const void* xg, const int* rows, const float* ssq, int n_partials, float eps,
                                     const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
-                                    long ldc, int epilogue, int waves, hipStream_t stream) {
+                                    long ldc, int epilogue, int waves, const float* bias, int act, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_norm", xg, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ssq && n_partials > 0, "gl3_gemm_skinny_norm: norm arguments missing");
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny_norm: ldc too small");
   GL3_REQUIRE(epilogue == SK_STORE || epilogue == SK_GATED, "gl3_gemm_skinny_norm: epilogue %d", epilogue);
+  GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny_norm: unknown activation %d", act);
   const SkNorm nrm = {ssq, n_partials, eps, rows};
-  const SkCall a = {xg, W, C, M, N, K, lda, ldw, ldc, nrm, nullptr, SkRope{}, stream, waves == 0};
+  SkCall a = {xg, W, C, M, N, K, lda, ldw, ldc, nrm, nullptr, SkRope{}, stream, waves == 0};
+  a.nx = SkNext{nullptr, nullptr, 0, bias, act};
   const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32 && epilogue == SK_STORE) return pick_mt<SK_STORE, float, true, false>(nw, a);
   if (c_dtype == GL3_BF16 && epilogue == SK_STORE) return pick_mt<SK_STORE, bf16_t, true, false>(nw, a);

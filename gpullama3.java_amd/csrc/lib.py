@@ -17,6 +17,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 EPI_STORE, EPI_ADD, EPI_GATED = 0, 1, 2
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}     # the gated epilogue's activation
 
 _lib = None
 
@@ -47,22 +48,23 @@ def _declare(lib):
     sigs = {
         "gl3_abi_version": [],
         "gl3_fill_u32": [P, c_uint32, L, P],
-        "gl3_embed": [P, I, P, P, I, I, P, P, P, P],
+        "gl3_embed": [P, I, P, P, I, I, P, P, P, F, P, P, P],
+        "gl3_scale_f32": [P, F, L, P],
         "gl3_rmsnorm": [P, P, P, I, P, I, I, I, F, P],
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
-        "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P],
+        "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, P],
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_sample_work_floats": [I, I],
         "gl3_argmax": [P, L, P, P, I, I, P],
         "gl3_argmax_static": [P, L, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
-        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P],
-        "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P],
-        "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P],
+        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P],
+        "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P],
+        "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P],
         "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
-        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P],
+        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
         "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P],
@@ -150,10 +152,33 @@ def _check_next(next_weight, xg, rows, d, who):
             raise KernelError(f"{who}: next weight {tuple(next_weight.shape)}, rows {tuple(xg.shape)} for [{rows}, {d}]")
 
 
-def embed(table, ids, out, ssq=None, next_weight=None, xg=None):
-    """out[t] = table[ids[t]] as float32. The caller has checked ids < rows. ``ssq`` (at least 64
-    floats, at most 64 tokens) receives each row's sum of squares; with it ``xg`` [T, d] bfloat16
-    may receive ``next_weight * out``, the rows as the product after the next norm reads them."""
+def _bias(bias, n, who):
+    """A bias per output column: float32 [n] on the device, or None."""
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.shape != (n,):
+            raise KernelError(f"{who}: bias {tuple(bias.shape)} for {n} columns")
+    return _ptr(bias)
+
+
+def _act(act, who):
+    try:
+        return ACTIVATIONS[act]
+    except KeyError:
+        raise KernelError(f"{who}: activation {act!r} is not built ({sorted(ACTIVATIONS)})") from None
+
+
+def scale_(t, factor):
+    """t *= factor (float32, contiguous)."""
+    _dev(t, "tensor", torch.float32)
+    _check(library().gl3_scale_f32(_ptr(t), float(factor), t.numel(), _stream()), "scale_f32")
+
+
+def embed(table, ids, out, ssq=None, next_weight=None, xg=None, scale=1.0, pos_table=None, positions=None):
+    """out[t] = scale * table[ids[t]] (+ pos_table[positions[t]]) as float32. The caller has checked
+    ids < rows and positions < rows of ``pos_table``. ``ssq`` (at least 64 floats, at most 64 tokens)
+    receives each row's sum of squares; with it ``xg`` [T, d] bfloat16 may receive ``next_weight *
+    out``, the rows as the product after the next norm reads them."""
     _dev(table, "table"); _dev(ids, "ids", torch.int32); _dev(out, "out", torch.float32)
     T, d = out.shape
     if table.dim() != 2 or table.shape[1] != d or ids.numel() != T:
@@ -165,8 +190,13 @@ def embed(table, ids, out, ssq=None, next_weight=None, xg=None):
     _check_next(next_weight, xg, T, d, "embed")
     if xg is not None and (ssq is None or not xg.is_contiguous()):
         raise KernelError("embed: the next norm's rows come with the sums of squares, contiguous")
+    if pos_table is not None:
+        _dev(pos_table, "pos_table", table.dtype); _dev(positions, "positions", torch.int32)
+        if pos_table.dim() != 2 or pos_table.shape[1] != d or positions.numel() != T:
+            raise KernelError(f"embed: table of positions {tuple(pos_table.shape)} for rows of {d}")
     _check(library().gl3_embed(_ptr(table), _code(table, "table"), _ptr(ids), _ptr(out), T, d, _ptr(ssq),
-                               _ptr(next_weight), _ptr(xg), _stream()), "embed")
+                               _ptr(next_weight), _ptr(xg), float(scale), _ptr(pos_table),
+                               _ptr(positions) if pos_table is not None else c_void_p(0), _stream()), "embed")
 
 
 def rmsnorm(x, weight, out, eps, rows=None):
@@ -243,9 +273,10 @@ def rope_cache_write(qkv, positions, seq_of_token, block_table, cos, sin, k_cach
         page_size, int(write_kv), _stream()), "rope_cache_write")
 
 
-def gemm_generic(a, w, out, epilogue=EPI_STORE):
+def gemm_generic(a, w, out, epilogue=EPI_STORE, bias=None, act="silu"):
     """out = a @ w.T with float multiply-adds; see gemm_generic.hip for the epilogues.
-    ``a`` and ``out`` may be row-strided views (last dimension contiguous)."""
+    ``a`` and ``out`` may be row-strided views (last dimension contiguous). ``bias``: float32, one
+    per row of ``w``; ``act``: the gated epilogue's activation."""
     _dev(a, "a", contiguous=False); _dev(w, "w"); _dev(out, "out", contiguous=False)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
         raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
@@ -255,7 +286,8 @@ def gemm_generic(a, w, out, epilogue=EPI_STORE):
     if w.shape != (rows, K) or out.shape[0] != M:
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_generic(_ptr(a), _code(a, "a"), _ptr(w), _code(w, "w"), _ptr(out), _code(out, "out"),
-                                      M, N, K, a.stride(0), w.stride(0), out.stride(0), epilogue, _stream()),
+                                      M, N, K, a.stride(0), w.stride(0), out.stride(0), epilogue,
+                                      _bias(bias, rows, "gemm_generic"), _act(act, "gemm_generic"), _stream()),
            "gemm_generic")
 
 
@@ -339,7 +371,8 @@ def skinny_strip_rows(M, N, K, epilogue):
     return 8 if M <= 16 and epilogue != EPI_GATED and -(-N // 16) <= 160 and K > 4096 else 16
 
 
-def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows=16, next_weight=None, xg=None):
+def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows=16, next_weight=None, xg=None,
+                bias=None, act="silu"):
     """out (=, +=, gated) a @ w.T on the matrix cores for at most 64 rows of ``a``. ``ssq_out``
     [N/strip_rows, 64] float32 (add epilogue): partial sums of squares of the completed rows; with it
     ``xg`` [M, N] bfloat16 may receive ``next_weight * out``, the rows as the product after the next
@@ -361,7 +394,8 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows
         raise KernelError("gemm_skinny: the next norm's rows come with the sums of squares")
     _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                      out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _ptr(next_weight),
-                                     _ptr(xg), xg.stride(0) if xg is not None else 0, _stream()), "gemm_skinny")
+                                     _ptr(xg), xg.stride(0) if xg is not None else 0, _bias(bias, rows, "gemm_skinny"),
+                                     _act(act, "gemm_skinny"), _stream()), "gemm_skinny")
 
 
 def gemm_skinny_wide_fits(a, w, out, epilogue):
@@ -374,7 +408,7 @@ def wide_slices(N, K):
     return max(1, min(8, 256 // -(-N // 64), K // 512))
 
 
-def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0):
+def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="silu"):
     """out (=, +=, gated) a @ w.T for 33 to 64 rows of ``a``. ``out`` with three axes [slices, M, N]
     (float32, store epilogue) takes the sums of one slice of K each: the caller adds them up."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
@@ -389,6 +423,7 @@ def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0):
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_skinny_wide(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0),
                                           w.stride(0), rows.stride(0), epilogue, slices, slice_stride, strips,
+                                          _bias(bias, wrows, "gemm_skinny_wide"), _act(act, "gemm_skinny_wide"),
                                           _stream()), "gemm_skinny_wide")
 
 
@@ -408,7 +443,7 @@ def gemm_skinny_norm_fits(xg, w, out, epilogue):
                  or (epilogue == EPI_GATED and out.dtype == torch.bfloat16)))
 
 
-def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=None, waves=0):
+def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=None, waves=0, bias=None, act="silu"):
     """out (=, gated) RMSNorm(x)[rows] @ w.T, where ``xg`` = bfloat16(norm weight * x) was left by the
     kernel that completed the rows of x, together with their sums of squares as partial sums."""
     _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
@@ -424,7 +459,8 @@ def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=
         raise KernelError(f"gemm: rows {tuple(xg.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_skinny_norm(
         _ptr(xg), _ptr(rows), _ptr(ssq), n_partials, float(eps), _ptr(w), _ptr(out), _code(out, "out"), M, N, K,
-        xg.stride(0), w.stride(0), out.stride(0), epilogue, waves, _stream()), "gemm_skinny_norm")
+        xg.stride(0), w.stride(0), out.stride(0), epilogue, waves, _bias(bias, wrows, "gemm_skinny_norm"),
+        _act(act, "gemm_skinny_norm"), _stream()), "gemm_skinny_norm")
 
 
 def qkv_rope_cache_fits(a, w_qkv, head_dim, rot_dim):
@@ -520,7 +556,7 @@ def gemm_mfma_fits(a, w, out, epilogue):
             and (out.dtype == torch.float32 or (out.dtype == torch.bfloat16 and epilogue != EPI_ADD)))
 
 
-def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None):
+def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None, bias=None, act="silu"):
     """out (=, +=, gated) a @ w.T on the matrix cores, tiled for many rows of ``a``. With
     ``more_slices`` [S, M, N] float32 K is cut into S + 1 slices: the first goes into ``out``, the
     others' sums are stored there, for the caller to add to ``out`` in that order."""
@@ -540,7 +576,8 @@ def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None):
     if w.shape != (rows, K) or out.shape[0] != M:
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_mfma(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
-                                   out.stride(0), epilogue, slices, _ptr(more_slices), p_stride, ldp, _stream()),
+                                   out.stride(0), epilogue, slices, _ptr(more_slices), p_stride, ldp,
+                                   _bias(bias, rows, "gemm_mfma"), _act(act, "gemm_mfma"), _stream()),
            "gemm_mfma")
 
 

@@ -3,7 +3,9 @@
 Order as the reference's layer (J/inference/InferenceCore.java:78-151): q, k, v
 projections (one product over the three matrices stacked by rows), rotation of q
 and k, cache write at the token's position, attention over positions lo..p of the
-token's own sequence, output projection added into the residual stream.
+token's own sequence, output projection added into the residual stream. The reference's
+projections have no biases; a description that names ``q_bias``, ``k_bias``, ``v_bias``
+(together) or ``o_bias`` among its tensors gets them added in the products' epilogues.
 """
 from __future__ import annotations
 
@@ -29,12 +31,21 @@ class GQAAttention:
         self.scale = spec.scale if spec.scale is not None else 1.0 / math.sqrt(self.hs)
         self.position = build_part("position", spec.position, device=device) if spec.position is not None else None
         self.names = spec.names
-        self.w_qkv = self.w_q = self.w_o = None
+        self.biased = "q_bias" in self.names
+        if self.biased and not ("k_bias" in self.names and "v_bias" in self.names):
+            raise ValueError("an attention names the biases of q, k and v together or none of them")
+        self.w_qkv = self.w_q = self.w_o = self.b_qkv = self.b_o = None
 
     def tensors(self):
         n, d, hs = self.names, self.d, self.hs
-        return {n["q"]: TensorSpec((self.H * hs, d)), n["k"]: TensorSpec((self.Kh * hs, d)),
-                n["v"]: TensorSpec((self.Kh * hs, d)), n["o"]: TensorSpec((d, self.H * hs))}
+        out = {n["q"]: TensorSpec((self.H * hs, d)), n["k"]: TensorSpec((self.Kh * hs, d)),
+               n["v"]: TensorSpec((self.Kh * hs, d)), n["o"]: TensorSpec((d, self.H * hs))}
+        if self.biased:
+            out.update({n["q_bias"]: TensorSpec((self.H * hs,), "vector"), n["k_bias"]: TensorSpec((self.Kh * hs,), "vector"),
+                        n["v_bias"]: TensorSpec((self.Kh * hs,), "vector")})
+        if "o_bias" in n:
+            out[n["o_bias"]] = TensorSpec((d,), "vector")
+        return out
 
     def load(self, weights):
         n = self.names
@@ -47,6 +58,10 @@ class GQAAttention:
             self.w_qkv[:qn], self.w_qkv[qn:qn + kn], self.w_qkv[qn + kn:])
         self.w_q = self.w_qkv[:qn]
         self.w_o = weights[n["o"]]
+        if self.biased:     # the epilogues read biases as float
+            self.b_qkv = torch.cat([weights[n[k]].float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()
+        if "o_bias" in n:
+            self.b_o = weights[n["o_bias"]].float().contiguous()
 
     def kv_need(self):
         return KVNeed(self.Kh, self.hs, self.window)
@@ -59,10 +74,10 @@ class GQAAttention:
         k_cache, v_cache = ctx.cache.layer_kv(run.kv_entry)
         table = ctx.block_table(ctx.cache.group_index(run.kv_entry))
         q = ops.qkv_project(ctx, h, self.w_qkv, self.w_q, self.position, k_cache, v_cache, table, H, Kh, hs,
-                            self.dtype, run.writes_kv)
+                            self.dtype, run.writes_kv, bias=self.b_qkv)
         att = ctx.buffer("attn_out", (T, H * hs), self.dtype)
         ops.attention(ctx, q, k_cache, v_cache, table, att, H, Kh, hs, self.window, self.scale)
-        ops.linear(att, self.w_o, x, ops.EPI_ADD, ctx)
+        ops.linear(att, self.w_o, x, ops.EPI_ADD, ctx, bias=self.b_o)
 
 
 register_part("mixer", "attention", GQAAttention)

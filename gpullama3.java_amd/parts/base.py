@@ -13,7 +13,17 @@ Mixer:        ``forward(ctx, h[T,d], x[T,d] float32, run)`` adds its output into
               ``kv_need()`` / ``state_need()`` tell the cache what one run-order entry stores.
 FeedForward:  ``forward(ctx, h[T,d], x[T,d] float32)`` adds its output into ``x``.
 Position:     built by the mixer that uses it from its description (``build_part("position", ...)``).
-Block:        ``forward(ctx, x, run)``; owns the arrangement of norm, mixer and feed-forward.
+Block:        ``parts()`` and ``forward(ctx, x, run)``; owns the arrangement of norm, mixer and
+              feed-forward. Optional: ``cache_needs() -> (KVNeed | None, StateNeed | None)`` (else the
+              one part with ``kv_need`` is asked), and ``first_norm()``, with which the block takes
+              part in the folding of norms into products and is called with ``norm_after=``.
+
+The residual rows ``x`` between parts: parts only ADD to ``x`` (through ``ops.linear`` with the add
+epilogue, or with a kernel of their own followed by ``ops.residual_written``). After a product of 33
+or more rows the sums may still lie in slices that the next norm adds up, so whoever READS ``x``
+other than through a norm calls ``ops.settle_residual(ctx, x)`` first. A block without ``first_norm``
+is handed whole rows, and no product leaves slices or prepared rows while it runs
+(``DecoderModel.forward`` sees to both), so an arrangement of one's own need not know any of this.
 """
 from __future__ import annotations
 

@@ -18,6 +18,9 @@ class PreNormBlock:
     def parts(self):
         return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
 
+    def cache_needs(self):
+        return self.mixer.kv_need(), self.mixer.state_need()
+
     def first_norm(self):
         """The norm that reads the residual rows first: the block before this one may prepare its rows."""
         return self.mixer_norm

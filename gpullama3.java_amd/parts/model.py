@@ -19,12 +19,27 @@ def expected_tensors(spec, dtype=torch.float32, device="cpu"):
     out = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden))}
     if spec.head_name is not None:
         out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden))
+    if spec.position_table_name is not None:
+        out[spec.position_table_name] = TensorSpec((spec.max_positions, spec.hidden))
     out.update(_norm_tensors(spec.final_norm))
     for b in spec.layers:
         block = build_part("block", b, dtype=dtype, device=device)
         for p in block.parts():
             out.update(p.tensors())
     return out
+
+
+def _block_needs(block):
+    """(KVNeed or None, StateNeed or None) of one run of a block: what the block says itself
+    (``cache_needs()``), else what the one of its parts that keeps something per position or per
+    sequence says."""
+    if hasattr(block, "cache_needs"):
+        return block.cache_needs()
+    keepers = [p for p in block.parts() if hasattr(p, "kv_need")]
+    if len(keepers) > 1:
+        raise ValueError("a block with several parts that keep keys, values or state must say what it needs itself "
+                         "(cache_needs)")
+    return (keepers[0].kv_need(), keepers[0].state_need()) if keepers else (None, None)
 
 
 def _norm_tensors(spec):
@@ -45,13 +60,15 @@ class DecoderModel:
                                  "with keys and values of its own")
             self.runs.append(RunInfo(entry=e, kv_entry=e if r.reads is None else r.reads,
                                      writes_kv=r.reads is None))
-        self.embedding = self.head = None
+        self.embedding = self.head = self.position_table = None
         self.weights = {}
 
     def expected(self):
         out = {self.spec.embedding_name: TensorSpec((self.spec.vocab_size, self.spec.hidden))}
         if self.spec.head_name is not None:
             out[self.spec.head_name] = TensorSpec((self.spec.vocab_size, self.spec.hidden))
+        if self.spec.position_table_name is not None:
+            out[self.spec.position_table_name] = TensorSpec((self.spec.max_positions, self.spec.hidden))
         out.update(self.final_norm.tensors())
         for b in self.blocks:
             for p in b.parts():
@@ -62,6 +79,8 @@ class DecoderModel:
         self.weights = weights
         self.embedding = weights[self.spec.embedding_name]
         self.head = self.embedding if self.spec.head_name is None else weights[self.spec.head_name]
+        if self.spec.position_table_name is not None:
+            self.position_table = weights[self.spec.position_table_name].to(self.embedding.dtype)
         self.final_norm.load(weights)
         for b in self.blocks:
             for p in b.parts():
@@ -70,9 +89,9 @@ class DecoderModel:
     def cache_needs(self):
         kv, state = [], []
         for run, r in zip(self.runs, self.spec.run_order):
-            mixer = self.blocks[r.layer].mixer
-            kv.append(mixer.kv_need() if run.writes_kv else None)
-            state.append(mixer.state_need())
+            kv_need, state_need = _block_needs(self.blocks[r.layer])
+            kv.append(kv_need if run.writes_kv else None)
+            state.append(state_need)
         return kv, state
 
     def forward(self, ctx, want_rows):
@@ -82,23 +101,40 @@ class DecoderModel:
         order = [self.blocks[r.layer] for r in self.spec.run_order]
         # the norm that reads the residual rows after entry i of the run order, where the block says which
         firsts = [getattr(b, "first_norm", lambda: None)() for b in order] + [self.final_norm]
+        around = {}
+        if self.spec.embedding_scale is not None:
+            around["scale"] = self.spec.embedding_scale
+        if self.position_table is not None:
+            around.update(pos_table=self.position_table, positions=ctx.positions)
         if getattr(ctx, "fuse", False) and ctx.n_tokens <= ops.FUSE_ROWS and getattr(firsts[0], "folds", False):
             # the first norm's sums of squares, and its rows times its weight, come with the embedding
             ssq = ctx.ssq_buffer(1)
             xg = ctx.buffer("rows_times_norm_weight", (ctx.n_tokens, self.spec.hidden), torch.bfloat16)
-            K.embed(self.embedding, ctx.token_ids, x, ssq, firsts[0].weight_f32, xg)
+            K.embed(self.embedding, ctx.token_ids, x, ssq, firsts[0].weight_f32, xg, **around)
             ops.residual_written(ctx, x, ssq, 1, xg, firsts[0])
         else:
-            K.embed(self.embedding, ctx.token_ids, x)
+            K.embed(self.embedding, ctx.token_ids, x, **around)
             ops.residual_written(ctx, x)
         for i, (run, block) in enumerate(zip(self.runs, order)):
             if hasattr(block, "first_norm"):
                 block.forward(ctx, x, run, norm_after=firsts[i + 1])
             else:
-                block.forward(ctx, x, run)
+                # an arrangement of its own may read the rows as they are: they are made whole first, and
+                # nothing is left in slices or prepared for a folded norm while it runs
+                ops.settle_residual(ctx, x)
+                fuse, ctx.fuse = ctx.fuse, False
+                try:
+                    block.forward(ctx, x, run)
+                finally:
+                    ctx.fuse = fuse
+                if ctx.pending is not None:
+                    raise RuntimeError("a block left sums of a product in slices behind it")
+                ops.residual_written(ctx, x)
         n = want_rows.numel()
         logits = ctx.logits_buffer(n, self.spec.vocab_size)
         if n:
             h = self.final_norm(ctx, x, rows=want_rows, name="final_normed")
             ops.linear(h, self.head, logits, ops.EPI_STORE, ctx)
+            if self.spec.logit_scale is not None:
+                K.scale_(logits, self.spec.logit_scale)
         return logits

@@ -82,17 +82,17 @@ def row_chunks(M, ctx=None):
     return [(lo, min(M, lo + size)) for lo in range(0, M, size)]
 
 
-def _linear_in_chunks(a, w, out, epilogue, ctx, chunks):
+def _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias=None, act="silu"):
     M, Kd = a.shape
     N = out.shape[1]
     if epilogue != EPI_ADD:
         for lo, hi in chunks:
-            linear(a[lo:hi], w, out[lo:hi], epilogue)
+            linear(a[lo:hi], w, out[lo:hi], epilogue, bias=bias, act=act)
         return
-    slices = K.wide_slices(N, Kd)
+    slices = K.wide_slices(N, Kd) if bias is None else 1     # (a bias is added once: no slices of K with one)
     if slices < 2:
         for lo, hi in chunks:
-            K.gemm_skinny(a[lo:hi], w, out[lo:hi], EPI_ADD)
+            K.gemm_skinny(a[lo:hi], w, out[lo:hi], EPI_ADD, bias=bias)
         return residual_written(ctx, out)
     settle_residual(ctx, out)
     part = ctx.buffer(f"slices{slices}", (slices, M, N), torch.float32)
@@ -102,21 +102,23 @@ def _linear_in_chunks(a, w, out, epilogue, ctx, chunks):
     ctx.pending = (out.data_ptr(), part)
 
 
-def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
+def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu"):
     """out (=, +=, gated) a @ w.T. ``a`` may be a ``Normed``. With the add epilogue ``out`` is the
-    residual stream."""
+    residual stream. ``bias`` (float32, one per row of ``w``) is added to the sums before the
+    epilogue's own rule; ``act`` is the gated epilogue's activation (``lib.ACTIVATIONS``)."""
     if isinstance(a, Normed):
         if ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
                 and a.xg.shape[0] <= 64):
-            return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows)
+            return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act)
         a = a.materialize()
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         chunks = row_chunks(a.shape[0], ctx)
         if (chunks and ctx is not None and getattr(ctx, "fuse", False) and not disabled & {"wide", "fused", "skinny"}
                 and K.gemm_skinny_fits(a[:1], w, out[:1], epilogue)
                 and not (epilogue == EPI_STORE and out.shape[1] >= 128 * 512)):     # (the head: the tiled kernel)
-            return _linear_in_chunks(a, w, out, epilogue, ctx, chunks)
-        if "wide" not in disabled and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx):
+            return _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias, act)
+        if ("wide" not in disabled and K.gemm_skinny_wide_fits(a, w, out, epilogue)
+                and _linear_wide(a, w, out, epilogue, ctx, bias, act)):
             return
         if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
             N = out.shape[1]
@@ -127,15 +129,16 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
                 norm, xg = _next_norm(ctx, N)
                 if norm is not None:
                     ssq = ctx.ssq_buffer(N // rows)
-                    K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq, strip_rows=rows, next_weight=norm.weight_f32, xg=xg)
+                    K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq, strip_rows=rows, next_weight=norm.weight_f32, xg=xg,
+                                  bias=bias)
                     return residual_written(ctx, out, ssq, N // rows, xg, norm)
-            K.gemm_skinny(a, w, out, epilogue, strip_rows=rows)
+            K.gemm_skinny(a, w, out, epilogue, strip_rows=rows, bias=bias, act=act)
             if epilogue == EPI_ADD:
                 residual_written(ctx, out)
             return
         if "mfma" not in disabled and K.gemm_mfma_fits(a, w, out, epilogue):
             M, Kd = a.shape
-            slices = K.mfma_slices(M, out.shape[1], Kd) if epilogue == EPI_ADD else 1
+            slices = K.mfma_slices(M, out.shape[1], Kd) if epilogue == EPI_ADD and bias is None else 1
             if slices > 1 and ctx is not None and getattr(ctx, "fuse", False) and "fused" not in disabled:
                 # a long K over few tiles: the first slice adds into the rows, the norm that follows
                 # adds the others
@@ -145,29 +148,31 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None):
                 residual_written(ctx, out)
                 ctx.pending = (out.data_ptr(), part)
                 return
-            K.gemm_mfma(a, w, out, epilogue)
+            K.gemm_mfma(a, w, out, epilogue, bias=bias, act=act)
             if epilogue == EPI_ADD:
                 residual_written(ctx, out)
             return
-    K.gemm_generic(a, w, out, epilogue)
+    K.gemm_generic(a, w, out, epilogue, bias=bias, act=act)
     if epilogue == EPI_ADD:
         residual_written(ctx, out)
 
 
-def _linear_wide(a, w, out, epilogue, ctx):
+def _linear_wide(a, w, out, epilogue, ctx, bias=None, act="silu"):
     """Products of 33 to 64 rows where another kernel than the skinny one is faster. True when done."""
     M, Kd = a.shape
     N = out.shape[1]
     if epilogue == EPI_GATED:
         if N < 32 * 192:          # too few blocks of two strip pairs for the chip
             return False
-        K.gemm_skinny_wide(a, w, out, epilogue)
+        K.gemm_skinny_wide(a, w, out, epilogue, bias=bias, act=act)
         return True
     if epilogue == EPI_STORE:
         # many columns (the head): the tiled kernel, whose blocks share their rows of a
         if N >= 128 * 512 and "mfma" not in disabled and K.gemm_mfma_fits(a, w, out, epilogue):
-            K.gemm_mfma(a, w, out, epilogue)
+            K.gemm_mfma(a, w, out, epilogue, bias=bias)
             return True
+        return False
+    if bias is not None:          # a bias is added once: no slices of K with one
         return False
     # into the residual stream: K in slices, added up by the norm that follows
     slices = K.wide_slices(N, Kd)
@@ -187,16 +192,18 @@ def _table_rows(ctx):
     return rows if rows is not None else ctx.seq_of_token
 
 
-def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_heads, n_kv, head_dim, dtype, writes_kv):
+def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_heads, n_kv, head_dim, dtype, writes_kv,
+                bias=None):
     """Queries, keys and values of the step's tokens: q rotated into a buffer whose rows start
     with the H*hs query columns (returned), k rotated and v into the cache. One kernel when
-    ``h`` is a ``Normed`` and the shapes allow, else product and rotation apart."""
+    ``h`` is a ``Normed`` and the shapes allow, else product and rotation apart (always apart with
+    a ``bias``, float32 over the stacked q, k, v rows, which is added before the rotation)."""
     T = h.shape[0]
     page = k_cache.shape[2]
     cos, sin = (rotary.cos, rotary.sin) if rotary is not None else (None, None)
     rot = rotary.rot_dim if rotary is not None else 0
     adjacent = rotary.adjacent if rotary is not None else False
-    if (isinstance(h, Normed) and writes_kv and h.rows is None and "fused" not in disabled
+    if (isinstance(h, Normed) and writes_kv and h.rows is None and "fused" not in disabled and bias is None
             and K.qkv_rope_cache_fits(h.xg, w_qkv, head_dim, rot)):
         q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
         K.qkv_rope_cache(h.xg, h.ssq, h.n_partials, h.eps, w_qkv, q, ctx.positions, _table_rows(ctx),
@@ -205,7 +212,7 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
     if isinstance(h, Normed):
         h = h.materialize()
     chunks = row_chunks(T, ctx) if getattr(ctx, "fuse", False) and "wide" not in disabled else None
-    if (writes_kv and h.dtype == torch.bfloat16 and "fused" not in disabled and "skinny" not in disabled
+    if (writes_kv and h.dtype == torch.bfloat16 and "fused" not in disabled and "skinny" not in disabled and bias is None
             and K.qkv_rope_cache_fits(h[:64], w_qkv, head_dim, rot) and (T <= 64 or chunks)):
         q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
         for lo, hi in (chunks or [(0, T)]):
@@ -214,10 +221,10 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
         return q
     if writes_kv:
         qkv = ctx.buffer("qkv", (T, (n_heads + 2 * n_kv) * head_dim), dtype)
-        linear(h, w_qkv, qkv)
+        linear(h, w_qkv, qkv, bias=bias)
     else:
         qkv = ctx.buffer("qkv", (T, n_heads * head_dim), dtype)
-        linear(h, w_q, qkv)
+        linear(h, w_q, qkv, bias=None if bias is None else bias[:n_heads * head_dim])
     K.rope_cache_write(qkv, ctx.positions, _table_rows(ctx), block_table, cos, sin, k_cache, v_cache,
                        n_heads, n_kv, head_dim, rot, adjacent, page, write_kv=writes_kv)
     return qkv

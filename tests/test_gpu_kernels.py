@@ -844,3 +844,100 @@ def test_argmax_kernel_takes_the_first_of_the_greatest(V):
     out = torch.empty(R, dtype=torch.int32, device=DEV)
     K().argmax(wide[:, :V], torch.empty(128 * R, device=DEV), out)
     assert out.tolist() == [P.argmax(row) for row in logits]
+
+
+# ------------------------------------------------------------------ biases and the other activation in the products' epilogues
+def gelu_tanh(v):
+    return 0.5 * v * (1 + np.tanh(math.sqrt(2 / math.pi) * (v + 0.044715 * v ** 3)))
+
+
+def epilogue_reference(a, w, epilogue, bias, act, before=None):
+    """What a product's end makes of a @ w.T in float64: bias first, then store / add / act(gate) * up."""
+    s = a.astype(np.float64) @ w.astype(np.float64).T
+    if bias is not None:
+        s = s + bias.astype(np.float64)
+    if epilogue == 2:
+        n = s.shape[1] // 2
+        g = s[:, :n]
+        return (g / (1 + np.exp(-g)) if act == "silu" else gelu_tanh(g)) * s[:, n:]
+    return s + before if epilogue == 1 else s
+
+
+PRODUCTS = ["generic float32", "generic bfloat16", "tiled", "few rows", "few rows, folded norm", "33 to 64 rows"]
+
+
+@pytest.mark.parametrize("which", PRODUCTS)
+@pytest.mark.parametrize("epilogue, act", [(0, "silu"), (1, "silu"), (2, "silu"), (2, "gelu_tanh")])
+def test_products_with_bias_and_activation(which, epilogue, act):
+    """Every product kernel with a bias per output column (the gated epilogue: the gate's, then the
+    up's) and both activations, against the same in float64. The bias is large next to the sums, so
+    that one added twice, to the wrong half or after the activation shows."""
+    lib = K()
+    rng = np.random.default_rng(len(which) * 7 + epilogue)
+    M = {"tiled": 150, "33 to 64 rows": 40}.get(which, 9)
+    N, Kd = 200, 136                                               # output columns: no tile divides them
+    dtype = "float32" if which == "generic float32" else "bfloat16"
+    wrows = 2 * N if epilogue == 2 else N
+    a = rounded(rng.standard_normal((M, Kd)), dtype)
+    w = rounded(rng.standard_normal((wrows, Kd)) * 0.1, dtype)
+    bias = (rng.standard_normal(wrows) * 2).astype(np.float32)
+    before = rng.standard_normal((M, N)).astype(np.float32)
+    out_dtype = torch.float32 if epilogue == 1 or dtype == "float32" else torch.bfloat16
+    out = dev(before, out_dtype) if epilogue == 1 else torch.zeros(M, N, device=DEV, dtype=out_dtype)
+    A, W, B = dev(a, TD[dtype]), dev(w, TD[dtype]), dev(bias)
+    ref_a = a
+    if which.startswith("generic"):
+        lib.gemm_generic(A, W, out, epilogue, bias=B, act=act)
+    elif which == "tiled":
+        lib.gemm_mfma(A, W, out, epilogue, bias=B, act=act)
+    elif which == "few rows":
+        lib.gemm_skinny(A, W, out, epilogue, bias=B, act=act)
+    elif which == "33 to 64 rows":
+        lib.gemm_skinny_wide(A, W, out, epilogue, bias=B, act=act)
+    else:
+        if epilogue == 1:
+            pytest.skip("a folded norm feeds store and gated products only")
+        x = (rng.standard_normal((M, Kd)) * 2).astype(np.float32)
+        nw = (1 + 0.2 * rng.standard_normal(Kd)).astype(np.float32)
+        xg = times_weight(x, nw).to(DEV)
+        ssq = dev(ssq_partials(x, 3))
+        lib.gemm_skinny_norm(xg, ssq, 3, 1e-5, W, out, epilogue, bias=B, act=act)
+        ref_a = xg.float().cpu().numpy() / np.sqrt((x.astype(np.float64) ** 2).mean(1, keepdims=True) + 1e-5)
+    ref = epilogue_reference(ref_a, w, epilogue, bias, act, before)
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref, atol=tol(dtype) * np.abs(ref).max())
+    with pytest.raises(lib.KernelError):
+        lib.gemm_generic(A, W, out, epilogue, bias=B[:-1])
+    with pytest.raises(lib.KernelError, match="activation"):
+        lib.gemm_generic(A, W, out, epilogue, act="relu")
+
+
+def test_embed_with_a_multiplier_and_a_table_of_positions():
+    rng = np.random.default_rng(3)
+    for dtype, d in (("float32", 70), ("bfloat16", 256)):          # scalar and 16-byte paths
+        table = rounded(rng.standard_normal((300, d)), dtype)
+        ptab = rounded(rng.standard_normal((50, d)), dtype)
+        ids, pos = rng.integers(0, 300, 21), rng.integers(0, 50, 21)
+        out = torch.empty(21, d, device=DEV)
+        K().embed(dev(table, TD[dtype]), dev(ids, torch.int32), out, scale=3.5, pos_table=dev(ptab, TD[dtype]),
+                  positions=dev(pos, torch.int32))
+        np.testing.assert_allclose(out.cpu().numpy(), 3.5 * table[ids] + ptab[pos], rtol=1e-6, atol=1e-6)
+        K().embed(dev(table, TD[dtype]), dev(ids, torch.int32), out, scale=0.25)
+        np.testing.assert_array_equal(out.cpu().numpy(), 0.25 * table[ids])
+    t = dev(rng.standard_normal((5, 33)))
+    before = t.clone()
+    K().scale_(t, 1.5)
+    assert torch.equal(t, before * 1.5)
+
+
+def test_scatter_of_table_entries():
+    lib = K()
+    t = torch.zeros(6, 50, dtype=torch.int32, device=DEV)
+    rng = np.random.default_rng(0)
+    places = rng.permutation(300)[:200].tolist()                  # more than one launch holds
+    values = rng.integers(1, 1000, 200).tolist()
+    lib.scatter_i32(t, places, values)
+    want = np.zeros(300, np.int32)
+    want[places] = values
+    assert t.view(-1).cpu().numpy().tolist() == want.tolist()
+    with pytest.raises(lib.KernelError, match="outside"):
+        lib.scatter_i32(t, [300], [1])

@@ -183,8 +183,29 @@ def test_feed_forward_part(dtype):
     part.forward(_ctx_only(dtype), h.to(DEV), x)
     ref = P.feed_forward(h.float().numpy(), *(W[n].float().numpy() for n in ("g", "u", "dn")))
     np.testing.assert_allclose(x.cpu().numpy() - 2, ref, atol=(2e-5 if dtype == "float32" else 2e-2) * np.abs(ref).max())
-    with pytest.raises(ValueError, match="gelu"):
-        build_part("ffn", GatedFeedForwardSpec(hidden=d, intermediate=F, activation="gelu"), dtype=TD[dtype], device=DEV)
+    with pytest.raises(ValueError, match="relu"):
+        build_part("ffn", GatedFeedForwardSpec(hidden=d, intermediate=F, activation="relu"), dtype=TD[dtype], device=DEV)
+    # the other activation, and biases on all three products: a description's matter, no other part
+    names = {"gate": "g", "up": "u", "down": "dn", "gate_bias": "gb", "up_bias": "ub", "down_bias": "db"}
+    part = build_part("ffn", GatedFeedForwardSpec(hidden=d, intermediate=F, activation="gelu_tanh", names=names),
+                      dtype=TD[dtype], device=DEV)
+    assert {k: tuple(v.shape) for k, v in part.tensors().items()} == {"g": (F, d), "u": (F, d), "dn": (d, F), "gb": (F,),
+                                                              "ub": (F,), "db": (d,)}
+    Wb = dict(W, gb=stored(rng.standard_normal(F), "float32"), ub=stored(rng.standard_normal(F), "float32"),
+              db=stored(rng.standard_normal(d), "float32"))
+    part.load({k: v.to(DEV) for k, v in Wb.items()})
+    for rows in (11, 40, 150):                                                # the kernels for few rows, 33 to 64, many
+        h = stored(rng.standard_normal((rows, d)), dtype)
+        x = torch.full((rows, d), 2.0, device=DEV)
+        part.forward(_ctx_only(dtype), h.to(DEV), x)
+        f = lambda n: Wb[n].float().numpy().astype(np.float64)
+        g = h.float().numpy() @ f("g").T + f("gb")
+        act = 0.5 * g * (1 + np.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3))) * (h.float().numpy() @ f("u").T + f("ub"))
+        if dtype == "bfloat16":
+            act = torch.as_tensor(act).to(torch.bfloat16).double().numpy()
+        ref = act @ f("dn").T + f("db")
+        np.testing.assert_allclose(x.cpu().numpy() - 2, ref, atol=(2e-5 if dtype == "float32" else 2e-2) * np.abs(ref).max(),
+                                   err_msg=f"{rows} rows")
 
 
 def test_rotary_part_tables():
@@ -693,3 +714,141 @@ def test_a_mixer_with_state_decodes_from_captured_graphs(tmp_path):
     assert np.array_equal(outs[True], outs[False])
     for i, q in enumerate(seqs):
         np.testing.assert_allclose(outs[True][:, i], toy_plain(cfg, W, q)[3:6], atol=2e-4)
+
+
+# ------------------------------------------------------------------ what other decoders put around and inside the blocks
+class HalvingBlock:
+    """An arrangement of its own that READS the residual rows (it halves them before the usual
+    pre-norm sequence) and offers no ``first_norm``: the decoder makes the rows whole before it
+    runs and lets no product leave its sums in slices meanwhile."""
+
+    def __init__(self, spec, dtype, device):
+        from gpullama3_java_amd.parts.block import PreNormBlock
+        self.inner = PreNormBlock(spec, dtype, device)
+
+    def parts(self):
+        return self.inner.parts()
+
+    def forward(self, ctx, x, run):
+        x.mul_(0.5)
+        self.inner.forward(ctx, x, run)
+
+
+def other_plain(cfg, W, toks):
+    """The toy decoder below in numpy: embedding times a multiplier plus a learned position row, halved
+    rows, attention without rotation and with biases, gelu feed-forward with biases, scaled logits."""
+    d, H, K, hs, L = cfg["hidden"], cfg["heads"], cfg["kv_heads"], cfg["head_dim"], cfg["layers"]
+    T = len(toks)
+    x = W["emb"][toks].astype(np.float32) * np.float32(cfg["embedding_scale"]) + W["wpe"][:T]
+    for l in range(L):
+        p = f"l{l}."
+        if l in cfg["halving_layers"]:
+            x = x * np.float32(0.5)
+        h = P.rmsnorm(x, W[p + "n1"], cfg["eps"])
+        q = (P.linear(h, W[p + "q"]) + W[p + "qb"]).reshape(T, H, hs)
+        k = (P.linear(h, W[p + "k"]) + W[p + "kb"]).reshape(T, K, hs)
+        v = (P.linear(h, W[p + "v"]) + W[p + "vb"]).reshape(T, K, hs)
+        x = x + P.linear(P.attention(q, k, v).reshape(T, H * hs), W[p + "o"]) + W[p + "ob"]
+        h = P.rmsnorm(x, W[p + "n2"], cfg["eps"])
+        g = (P.linear(h, W[p + "g"]) + W[p + "gb"]).astype(np.float64)
+        act = 0.5 * g * (1 + np.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3)))
+        x = x + P.linear((act * (P.linear(h, W[p + "u"]) + W[p + "ub"])).astype(np.float32), W[p + "dn"])
+        if p + "db" in W:
+            x = x + W[p + "db"]
+    return P.linear(P.rmsnorm(x, W["final"], cfg["eps"]), W["emb"]) * np.float32(cfg["logit_scale"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_decoder_of_another_make_from_descriptions_alone(tmp_path, dtype):
+    """Embedding multiplier, learned absolute positions, logit scale, biases on every projection,
+    the other activation and a block kind defined here: all of it is a description and two
+    registrations, no file of the framework changes. 40 tokens in one step take the kernels for 33
+    to 64 rows, whose products into the residual rows leave their sums in slices (K = 1024): the
+    block that reads the rows must find them whole."""
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.config import AttentionSpec, BlockSpec, GatedFeedForwardSpec, ModelSpec, NormSpec, Run
+    from gpullama3_java_amd.engine import Engine
+    from gpullama3_java_amd.parts import register_part
+
+    register_part("block", "toy_halving", HalvingBlock)
+
+    @dataclass(frozen=True)
+    class OtherConfig:
+        d: dict
+        max_position_embeddings: int = 128
+        stop_ids: tuple = ()
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(dict(d))
+
+        def with_context_length(self, n):
+            return self
+
+        def model_spec(self):
+            c = self.d
+            layers = []
+            for l in range(c["layers"]):
+                p = f"l{l}."
+                ffn_names = {"gate": p + "g", "up": p + "u", "down": p + "dn", "gate_bias": p + "gb", "up_bias": p + "ub"}
+                if l in c["down_bias_layers"]:
+                    ffn_names["down_bias"] = p + "db"
+                layers.append(BlockSpec(
+                    kind="toy_halving" if l in c["halving_layers"] else "prenorm",
+                    mixer_norm=NormSpec(dim=c["hidden"], eps=c["eps"], names={"weight": p + "n1"}),
+                    mixer=AttentionSpec(hidden=c["hidden"], n_heads=c["heads"], n_kv_heads=c["kv_heads"],
+                                        head_dim=c["head_dim"], position=None,
+                                        names={"q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o", "q_bias": p + "qb",
+                                               "k_bias": p + "kb", "v_bias": p + "vb", "o_bias": p + "ob"}),
+                    ffn_norm=NormSpec(dim=c["hidden"], eps=c["eps"], names={"weight": p + "n2"}),
+                    ffn=GatedFeedForwardSpec(hidden=c["hidden"], intermediate=c["inter"], activation="gelu_tanh",
+                                             names=ffn_names)))
+            return ModelSpec(architecture="OtherForCausalLM", vocab_size=c["vocab"], hidden=c["hidden"], layers=tuple(layers),
+                             run_order=tuple(Run(i) for i in range(c["layers"])),
+                             final_norm=NormSpec(dim=c["hidden"], eps=c["eps"], names={"weight": "final"}),
+                             max_positions=128, tie_embeddings=True, embedding_name="emb", head_name=None,
+                             embedding_scale=c["embedding_scale"], position_table_name="wpe", logit_scale=c["logit_scale"])
+
+    g.register_architecture("OtherForCausalLM", OtherConfig)
+    # three layers: the usual arrangement whose down projection has no bias (its sums stay in slices
+    # behind it), then the halving one, which reads the rows, then the usual one again
+    cfg = {"architectures": ["OtherForCausalLM"], "hidden": 128, "inter": 1024, "layers": 3, "heads": 4, "kv_heads": 2,
+           "head_dim": 32, "vocab": 300, "eps": 1e-5, "embedding_scale": 3.0, "logit_scale": 0.25,
+           "halving_layers": [1], "down_bias_layers": [1, 2]}
+    rng = np.random.default_rng(4)
+    r = lambda *s, scale=0.05: (rng.standard_normal(s) * scale).astype(np.float32)
+    W = {"emb": r(300, 128, scale=0.3), "wpe": r(128, 128, scale=0.3), "final": 1 + r(128, scale=0.1)}
+    for l in range(3):
+        p = f"l{l}."
+        W.update({p + "n1": 1 + r(128, scale=0.1), p + "n2": 1 + r(128, scale=0.1), p + "q": r(128, 128), p + "k": r(64, 128),
+                  p + "v": r(64, 128), p + "o": r(128, 128), p + "qb": r(128, scale=0.3), p + "kb": r(64, scale=0.3),
+                  p + "vb": r(64, scale=0.3), p + "ob": r(128, scale=0.3), p + "g": r(1024, 128), p + "u": r(1024, 128),
+                  p + "dn": r(128, 1024), p + "gb": r(1024, scale=0.3), p + "ub": r(1024, scale=0.3), p + "db": r(128, scale=0.3)})
+    del W["l0.db"]
+    if dtype == "bfloat16":                                   # what the engine will hold: matrices in bfloat16
+        W = {k: (torch.as_tensor(v).to(torch.bfloat16).float().numpy() if v.ndim == 2 else v) for k, v in W.items()}
+    folder = str(tmp_path / "other")
+    os.makedirs(folder)
+    json.dump(cfg, open(os.path.join(folder, "config.json"), "w"))
+    save_file({k: torch.as_tensor(v).to(TD[dtype] if v.ndim == 2 else torch.float32) for k, v in W.items()},
+              os.path.join(folder, "model.safetensors"))
+    eng = Engine.from_folder(folder, dtype=dtype, max_tokens=512, n_slots=2)
+    toks = rng.integers(0, 300, 45).tolist()
+    ref = other_plain(cfg, W, toks)
+    s = eng.take_slot()
+    got = [eng.step([(s, toks[:40])], want="all").cpu().numpy()]
+    got += [eng.step([(s, [t])]).cpu().numpy() for t in toks[40:]]
+    close(np.concatenate(got), ref, dtype, "a decoder of another make")
+    if dtype == "bfloat16":
+        # the case is the one it claims to be: without the decoder's care the halving block would halve
+        # rows whose last product still lies in slices
+        from gpullama3_java_amd.parts import ops
+        seen = []
+        real = ops.settle_residual
+        ops.settle_residual = lambda ctx, x: seen.append(ctx.pending is not None) or real(ctx, x)
+        try:
+            s2 = eng.take_slot()
+            eng.step([(s2, toks[:40])], want="none")
+        finally:
+            ops.settle_residual = real
+        assert any(seen)
