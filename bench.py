@@ -1,7 +1,7 @@
 """Decode and prefill throughput of the Llama-3.2-1B shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 1b|3b|8b]
-                    [--prompt-len P] [--prefill-len T]
+                    [--prompt-len P] [--prefill-len T] [--workload decode|unequal8]
 
 A step is one decode step of the generation loop: the engine's step for B sequences (one
 token each, from the cache left by 512-token prompts) and the greedy pick of the next
@@ -10,6 +10,13 @@ The same line carries the prefill of one 2,048-token prompt, the decode step's s
 the memory roofline, and decode at batch 1 and 64. Peaks are the published ones of the
 MI355X: 8 TB/s HBM3E, 2.5 PFLOP/s dense bf16 matrix throughput. Other layer sizes (--shape) and
 lengths are for looking further; the default run is the one that is reported.
+
+Two further workloads with lines of the same form:
+  * ``--workload unequal8`` (with the layers of Llama-3.2-3B unless --shape says otherwise): 8 requests
+    whose prompt lengths are drawn uniformly from [64, 2048] with the seed, their prompts in ONE packed
+    step (timed as the prefill), then --steps decode steps (default 128); the bytes of a step are the
+    weights once and the cache at the lengths the sequences really have at that step.
+  * the Llama-3.1-8B pair: ``--shape 8b --batch 64 --prompt-len 1024 --prefill-len 8192 --points ""``.
 """
 import argparse
 import json
@@ -80,7 +87,7 @@ def prefill_flops(c, T, rows=1):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--steps", type=int, default=None, help="timed decode steps (default 64; 128 for unequal8)")
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes; the default is what is reported")
     ap.add_argument("--layers", type=int, default=None,
@@ -91,7 +98,12 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma-separated")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--workload", default="decode", choices=["decode", "unequal8"])
     args = ap.parse_args()
+    if args.workload == "unequal8" and "--shape" not in " ".join(sys.argv):
+        args.shape = "3b"
+    if args.steps is None:
+        args.steps = 128 if args.workload == "unequal8" else 64
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
         return 2
@@ -113,6 +125,10 @@ def main():
     points = [int(b) for b in args.points.split(",") if b]
     biggest = max([args.batch] + points)
     per_seq = -(-(prompt_len + K + W + 1) // 64) * 64
+    if args.workload == "unequal8":
+        args.batch, points, biggest = 8, [], 8
+        per_seq = -(-(2048 + K + W + 1) // 64) * 64
+        prefill_len = 0
     tmp = tempfile.mkdtemp(prefix="gl3-bench-")
     try:
         t0 = time.time()
@@ -127,6 +143,9 @@ def main():
 
     def sync():
         torch.cuda.synchronize()
+
+    if args.workload == "unequal8":
+        return unequal8(args, eng, cfg, rng, shape_name, shape, esize, short, sync)
 
     # ---- prefill: one prompt (2,048 tokens unless told otherwise), logits at its last token
     def prefill_once():
@@ -201,6 +220,74 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
         "points": {f"decode_b{B}": round(B * K / results[B][0], 1) for B in results if B != args.batch},
+    }
+    print(json.dumps(line))
+    return 0
+
+
+def unequal8(args, eng, cfg, rng, shape_name, shape, esize, short, sync):
+    """8 requests with prompts of unequal lengths that start together: the prompts in one packed step,
+    then one token each per step (runs of steps on the device, as the generation loop drives them)."""
+    import torch
+    K, W, V = args.steps, args.warmup, cfg.vocab_size
+    lens = rng.integers(64, 2049, 8).tolist()
+    prompts = [rng.integers(0, V, n).tolist() for n in lens]
+    best = None
+    for _ in range(2):                                   # the first pass sizes the buffers
+        slots = [eng.take_slot() for _ in range(8)]
+        sync(); t = time.perf_counter()
+        eng.step(list(zip(slots, prompts)))
+        sync(); dt = time.perf_counter() - t
+        best = dt if best is None else min(best, dt)
+        if _ == 0:
+            for s in slots:
+                eng.give_back_slot(s)
+    prefill_s = best
+    T = sum(lens)
+    print(f"[bench] packed prefill of {lens} = {T} tokens: {prefill_s * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    temps, tops = [0.0] * 8, [1.0] * 8
+    toks = rng.integers(0, V, 8).tolist()
+    run = eng.decode_run_length
+
+    def steps(toks, n):
+        while n > 0:
+            m = min(run, n)
+            if m > 1:
+                toks = eng.decode_run(list(zip(slots, toks)), m, temps, tops, [[0.0] * 8] * m)[-1]
+            else:
+                toks = eng.sample(eng.step([(s, [t]) for s, t in zip(slots, toks)]), temps, tops, [0.0] * 8)
+            n -= m
+        return toks
+    toks = steps(toks, W)
+    kv = [eng.cache.length(s) for s in slots]
+    sync(); t = time.perf_counter()
+    steps(toks, K)
+    sync(); dt = time.perf_counter() - t
+    nbytes = decode_bytes(cfg, esize, [n + (K + 1) / 2 for n in kv])      # the mean over the K steps
+    ms = dt / K * 1e3
+    achieved = nbytes / (dt / K) / 1e9
+    # the flops of the packed prompts: the products of T tokens, each prompt's own causal attention, 8 head rows
+    flops = prefill_flops(cfg, T, rows=8) - cfg.num_hidden_layers * 4 * cfg.num_attention_heads * cfg.head_dim * (
+        T * (T + 1) // 2 - sum(n * (n + 1) // 2 for n in lens))
+    line = {
+        "metric": f"decode tok/s, 8 requests with prompts of {min(lens)}..{max(lens)} tokens ({shape_name})",
+        "value": round(8 * K / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic: random N(0,0.02) weights, uniform random token ids",
+        "config": {
+            "model": shape_name, "layers": args.layers, "layers_of_shape": shape["num_hidden_layers"],
+            "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
+            "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+            "vocab_size": cfg.vocab_size, "tied_head": cfg.tie_word_embeddings, "global_batch": 8,
+            "seq_len": shape["max_position_embeddings"], "prompt_len_min": min(lens), "prompt_len_max": max(lens),
+            "prompt_tokens": T, "mean_context": round(sum(kv) / 8 + (K + 1) / 2, 1), "new_tokens": K,
+            "parallelism": "single GPU", "sampling": "greedy on device",
+        },
+        "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(flops / prefill_s / (PEAK_TFLOPS[short] * 1e12), 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBS, 4)},
+        "points": {},
     }
     print(json.dumps(line))
     return 0

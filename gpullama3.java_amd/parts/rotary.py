@@ -9,6 +9,7 @@ is part of the kernel that writes the cache.
 from __future__ import annotations
 
 import math
+import weakref
 
 import numpy as np
 import torch
@@ -37,9 +38,18 @@ def frequencies(head_dim, theta, scaling):
     return out
 
 
+class _Tables:
+    """cos and sin of one description on one device."""
+
+    def __init__(self, cos, sin):
+        self.cos, self.sin = cos, sin
+
+
 class Rotary:
-    """cos/sin ``[max_positions, head_dim/2]`` float32 on the device."""
-    _tables = {}
+    """cos/sin ``[max_positions, head_dim/2]`` float32 on the device. The layers of a model (and models
+    with the same description) share one pair of tables; the pair lives as long as a part holds it and
+    is freed with the last engine that used it."""
+    _tables = weakref.WeakValueDictionary()
 
     def __init__(self, spec, device):
         if spec.head_dim % 2:
@@ -48,25 +58,30 @@ class Rotary:
         self.rot_dim = spec.head_dim
         self.adjacent = spec.pairing == "adjacent"
         self.max_positions = spec.max_positions
+        self._held = None
 
     def _table(self):
-        spec = self.spec
-        key = (spec.head_dim, spec.theta, spec.scaling, spec.max_positions, str(self.device))
-        if key not in Rotary._tables:
-            freq = frequencies(spec.head_dim, spec.theta, spec.scaling)
-            pos = np.arange(spec.max_positions, dtype=_F)[:, None]
-            val = (pos * freq[None, :]).astype(_F).astype(np.float64)
-            Rotary._tables[key] = (torch.from_numpy(np.cos(val).astype(_F)).to(self.device),
-                                   torch.from_numpy(np.sin(val).astype(_F)).to(self.device))
-        return Rotary._tables[key]
+        if self._held is None:
+            spec = self.spec
+            key = (spec.head_dim, spec.theta, spec.scaling, spec.max_positions, str(self.device))
+            held = Rotary._tables.get(key)
+            if held is None:
+                freq = frequencies(spec.head_dim, spec.theta, spec.scaling)
+                pos = np.arange(spec.max_positions, dtype=_F)[:, None]
+                val = (pos * freq[None, :]).astype(_F).astype(np.float64)
+                held = _Tables(torch.from_numpy(np.cos(val).astype(_F)).to(self.device),
+                               torch.from_numpy(np.sin(val).astype(_F)).to(self.device))
+                Rotary._tables[key] = held
+            self._held = held
+        return self._held
 
     @property
     def cos(self):
-        return self._table()[0]
+        return self._table().cos
 
     @property
     def sin(self):
-        return self._table()[1]
+        return self._table().sin
 
 
 register_part("position", "rotary", Rotary)

@@ -56,6 +56,9 @@ class SafetensorsFile:
             for s in shape:
                 count *= s
             want = count * torch.empty((), dtype=_DTYPES[dt]).element_size()
+            if b < 0 or end < b:
+                raise SafetensorsError(f"{path}: tensor {name!r} has the byte range {b}..{end}, which is no range "
+                                       "of the data that follows the header")
             if end - b != want:
                 raise SafetensorsError(f"{path}: tensor {name!r} of shape {shape} {dt} needs {want} bytes, "
                                        f"its range holds {end - b}")
@@ -63,6 +66,14 @@ class SafetensorsFile:
                 raise SafetensorsError(f"{path}: file is truncated: tensor {name!r} ends at byte "
                                        f"{self._base + end}, the file has {size}")
             self.entries[name] = (_DTYPES[dt], shape, b, count)
+        # two tensors never share bytes: a header whose ranges overlap would load one tensor's values as another's
+        last_end, last_name = 0, None
+        for name, (dt, shape, b, count) in sorted(self.entries.items(), key=lambda kv: kv[1][2]):
+            if count == 0:
+                continue
+            if b < last_end:
+                raise SafetensorsError(f"{path}: tensors {last_name!r} and {name!r} overlap (byte {b} lies before {last_end})")
+            last_end, last_name = b + count * torch.empty((), dtype=dt).element_size(), name
         self._mm = mmap.mmap(self._f.fileno(), 0, access=mmap.ACCESS_READ) if size else None
 
     def names(self):

@@ -117,3 +117,51 @@ def test_runs_of_decode_steps_at_real_layer_sizes_pick_the_tokens_of_single_step
             eng.give_back_slot(sl)
         for i in range(B):
             assert res[i].tokens == want[i], f"batch {B}, request {i}"
+
+
+@pytest.mark.parametrize("shape", ["1B", "3B", "8B"])
+def test_real_layer_sizes_against_the_plain_implementation(tmp_path, shape):
+    """The kernels that only real widths select (tiles of 256 x 256, strips of 8 rows, the resident
+    kernels of sixteen waves, the head through the tiled kernel, products cut into slices of K) inside
+    a whole model against the plain implementation itself (J/inference/InferenceCore.java:58-180), not
+    against another path of the engine: a prompt of 300 tokens with every row wanted, four single
+    tokens after it, and a batch of 40 short prompts with three decode steps (the kernels for 33 to
+    64 rows, replayed from graphs), in float32 and in bfloat16."""
+    from safetensors.torch import load_file
+
+    import gpullama3_java_amd as g
+    import plain_llama as P
+    from gpullama3_java_amd.engine import Engine
+    cfgd = SHAPES[shape]
+    cfg = g.config_from_dict(cfgd)
+    folder = str(tmp_path / "shape")
+    g.write_random_model(folder, cfg, 13, std=0.02, norm_std=0.1)
+    W = {k: v.float().numpy() for k, v in load_file(folder + "/model.safetensors").items()}
+    rng = np.random.default_rng(2)
+    long_toks = rng.integers(0, cfg.vocab_size, 304).tolist()
+    short = [rng.integers(0, cfg.vocab_size, 7).tolist() for _ in range(40)]
+    ref_long = P.forward(cfgd, W, long_toks)
+    ref_short = [P.forward(cfgd, W, q)[3:] for q in short]                   # rows of the tokens 3, 4, 5, 6
+    del W
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine.from_folder(folder, dtype=dtype, max_context=512, max_tokens=64 * 64, n_slots=64)
+        s = eng.take_slot()
+        got = [eng.step([(s, long_toks[:300])], want="all").cpu().numpy()]
+        got += [eng.step([(s, [t])]).cpu().numpy() for t in long_toks[300:]]
+        eng.give_back_slot(s)
+        got = np.concatenate(got)
+        scale = float(np.abs(ref_long).max())
+        err = np.abs(got - ref_long).max(axis=1)
+        assert err.max() <= TOL[dtype] * scale, f"{dtype}: row {int(err.argmax())} of the long sequence is off by {err.max() / scale:.2e}"
+        slots = [eng.take_slot() for _ in short]
+        rows = [eng.step([(sl, q[:4]) for sl, q in zip(slots, short)]).cpu().numpy()]
+        rows += [eng.step([(sl, [q[k]]) for sl, q in zip(slots, short)]).cpu().numpy() for k in (4, 5, 6)]
+        got = np.stack(rows, axis=1)                                         # [40, 4, vocab]
+        for i, r in enumerate(ref_short):
+            sc = float(np.abs(r).max())
+            e = float(np.abs(got[i] - r).max())
+            assert e <= TOL[dtype] * sc, f"{dtype}: sequence {i} of the batch of 40 is off by {e / sc:.2e}"
+        if dtype == "bfloat16":
+            assert eng._graphs
+        del eng
+        torch.cuda.empty_cache()

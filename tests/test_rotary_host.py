@@ -42,3 +42,17 @@ def test_unscaled_frequencies_are_powers_of_theta():
     f = frequencies(8, 10000.0, None)
     for n in range(4):
         assert abs(float(f[n]) - 10000.0 ** (-2 * n / 8)) < 1e-7 * float(f[n]) + 1e-12
+
+
+def test_tables_are_shared_while_held_and_freed_with_their_last_holder():
+    import gc
+
+    from gpullama3_java_amd.config import RotarySpec
+    from gpullama3_java_amd.parts.rotary import Rotary
+    spec = RotarySpec(head_dim=8, theta=10000.0, scaling=None, pairing="half", max_positions=33)
+    a, b = Rotary(spec, "cpu"), Rotary(spec, "cpu")
+    assert a.cos is b.cos and a.cos.shape == (33, 4)
+    n = len(Rotary._tables)
+    del a, b
+    gc.collect()
+    assert len(Rotary._tables) == n - 1

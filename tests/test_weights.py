@@ -56,6 +56,31 @@ def test_truncated_and_broken_files(tmp_path):
         SafetensorsFile(p)
 
 
+def _with_header(path, header, data_bytes):
+    import json
+    h = json.dumps(header).encode()
+    open(path, "wb").write(struct.pack("<Q", len(h)) + h + bytes(data_bytes))
+
+
+def test_byte_ranges_that_are_no_ranges_or_overlap_are_refused(tmp_path):
+    p = str(tmp_path / "y.safetensors")
+    ok = {"a": {"dtype": "F32", "shape": [4], "data_offsets": [0, 16]}, "b": {"dtype": "F32", "shape": [4], "data_offsets": [16, 32]}}
+    _with_header(p, ok, 32)
+    SafetensorsFile(p).close()
+    # a range that starts before the data (it would read the header's own bytes as weights)
+    _with_header(p, {"a": {"dtype": "F32", "shape": [4], "data_offsets": [-16, 0]}}, 32)
+    with pytest.raises(SafetensorsError, match="no range"):
+        SafetensorsFile(p)
+    _with_header(p, {"a": {"dtype": "F32", "shape": [4], "data_offsets": [16, 0]}}, 32)
+    with pytest.raises(SafetensorsError, match="no range"):
+        SafetensorsFile(p)
+    # two tensors over the same bytes
+    both = {"a": {"dtype": "F32", "shape": [4], "data_offsets": [0, 16]}, "b": {"dtype": "F32", "shape": [4], "data_offsets": [8, 24]}}
+    _with_header(p, both, 32)
+    with pytest.raises(SafetensorsError, match="overlap"):
+        SafetensorsFile(p)
+
+
 def test_random_model_folder(tmp_path):
     cfg = g.config_from_dict(TINY_B)
     d1 = write_random_model(str(tmp_path / "m1"), cfg, seed=5, norm_std=0.1)
