@@ -318,11 +318,17 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
   }
 }
 
-template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ, int ROWS = 16>
+// PACK (strips of 8 rows, at most 8 rows of A, one token tile): the tile's rows 8..15 are the strip's
+// 8 rows again, 32 k further, and its token columns 8..15 the tokens again at those k, so that one
+// instruction covers 64 k of the strip, every lane loads (a row of W and a row of A are read in
+// whole 128-byte lines) and nothing of the tile is idle. Of the 16 x 16 sums the two diagonal
+// 8 x 8 blocks are the product's two halves, added at the end; the other two are dropped.
+template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ, int ROWS = 16, bool PACK = false>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __restrict__ Av, const bf16_t* __restrict__ W,
                                                               TC* __restrict__ C, int M, int N, int K, long lda,
                                                               long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out,
                                                               SkNext nx, SkRope rp) {
+  static_assert(!PACK || (ROWS == 8 && MT == 1 && EPI != SK_GATED && EPI != SK_QKV && !XNORM), "packed strips: 8 rows, one tile");
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   constexpr int UNROLL = 8;
   __shared__ f32x4 red[NW][NG * MT][64];
@@ -333,12 +339,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   int hd, sub;
   bool rotated;
   const int wr = sk_strip_row<EPI, ROWS>(strip, r, N, rp, hd, sub, rotated);
-  const bf16_t* wrow = W + (long)wr * ldw + q * 8;
+  const int koff = PACK ? 32 * (r >> 3) + q * 8 : q * 8;   // the lane's place inside a k-step
+  const bf16_t* wrow = W + (long)wr * ldw + koff;
   const bf16_t* urow = wrow + (long)N * ldw;  // up rows (gated only)
   const void* xrow[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)   // null for rows that do not exist: their lanes ask for nothing
-    xrow[mt] = mt * 16 + r < M ? sk_x_row<XNORM>(Av, lda, mt * 16 + r, nrm) : nullptr;
+  for (int mt = 0; mt < MT; ++mt) {   // null for rows that do not exist: their lanes ask for nothing
+    const int m = PACK ? (r & 7) : mt * 16 + r;
+    xrow[mt] = m < M ? sk_x_row<XNORM>(Av, lda, m, nrm) : nullptr;
+  }
   if (XNORM) sk_ssq_partials<NW>(sm_ssq, M, nrm);
   const SkPre pre = sk_preload<MT, EPI, TC, ROWS>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx);
 
@@ -350,6 +359,27 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
     for (int mt = 0; mt < MT; ++mt) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
+  if (PACK) {
+    // a wave takes steps of 64 k: step wave, wave + NW, ...
+    for (int p0 = wave; p0 * 64 < K; p0 += NW * UNROLL) {
+      bf16x8 wf[UNROLL], xf[UNROLL][MT];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int k = (p0 + NW * u) * 64;
+        const bool ok = k + koff < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
+        wf[u] = ok ? *(const bf16x8*)(wrow + k) : zero;
+        sk_load_x<MT, XNORM>(xf[u], xrow, k + koff, ok, nrm);
+      }
+      __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u)
+        acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u][0], acc[0][0], 0, 0, 0);
+    }
+    // lane (token column j, quarter q) holds tile rows 4q .. 4q+3: the sums over the first 32 k of every
+    // step lie at j < 8, q < 2, those over the second at j >= 8, q >= 2: lane + 40
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[0][0][c] += __shfl_xor(acc[0][0][c], 40, 64);
+  } else {
   // a wave takes pairs of neighbouring k-steps (the two halves of one 128-byte line of a row of W):
   // pair wave, wave + NW, ...
   for (int p0 = wave; 2 * p0 < steps; p0 += NW * (UNROLL / 2)) {
@@ -371,6 +401,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
         if (EPI == SK_GATED) acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u], xf[u][mt], acc[1][mt], 0, 0, 0);
       }
     }
+  }
   }
   sk_finish<MT, NW, EPI, TC, XNORM, SSQ, ROWS>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp,
                                                nx, pre);
@@ -614,9 +645,14 @@ static int launch_skinny(int nw, const SkCall& a) {
   } while (0)
   if constexpr (MT == 1 && !XNORM && (EPI == SK_STORE || EPI == SK_ADD)) {
     if (a.strip_rows == 8) {
-      // strips of 8 rows: twice the blocks, each with half the rows to stream
-      gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
-          a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp);
+      // strips of 8 rows: twice the blocks, each with half the rows to stream; with at most 8 rows of A
+      // the tile's other half takes the next 32 k
+      if (a.M <= 8)
+        gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8, true><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
+            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp);
+      else
+        gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
+            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp);
       GL3_LAUNCH_CHECK();
       return 0;
     }

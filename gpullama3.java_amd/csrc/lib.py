@@ -366,9 +366,13 @@ def gemm_skinny_fits(a, w, out, epilogue):
 
 def skinny_strip_rows(M, N, K, epilogue):
     """Rows of w that a block of the skinny kernel takes: 8 where strips of 16 would leave more than a
-    third of the CUs without a block and K is too long for the kernel that keeps its rows of ``a`` in
-    registers (measured: 17.0 -> 15.8 us at N=2048, K=8192; slower where that kernel applies), else 16."""
-    return 8 if M <= 16 and epilogue != EPI_GATED and -(-N // 16) <= 160 and K > 4096 else 16
+    third of the CUs without a block. With at most 8 rows of ``a`` the half-empty tile of such a strip
+    takes the next 32 k instead (N=2048, 8 rows: K=8192 12.4 -> 9.7 us, K=2048 6.1 -> 4.3 us); with 9
+    to 16 rows half the tile idles, which pays only where K is too long for the kernel that keeps its
+    rows of ``a`` in registers (17.0 -> 15.8 us at N=2048, K=8192). Else 16."""
+    if epilogue == EPI_GATED or -(-N // 16) > 160:
+        return 16
+    return 8 if M <= 8 or (M <= 16 and K > 4096) else 16
 
 
 def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows=16, next_weight=None, xg=None,

@@ -941,3 +941,34 @@ def test_scatter_of_table_entries():
     assert t.view(-1).cpu().numpy().tolist() == want.tolist()
     with pytest.raises(lib.KernelError, match="outside"):
         lib.scatter_i32(t, [300], [1])
+
+
+@pytest.mark.parametrize("M", [1, 5, 8, 9, 16])
+@pytest.mark.parametrize("N, Kd", [(2048, 2048), (2048, 8192), (130, 40), (24, 136), (1000, 72), (8, 64)])
+def test_gemm_skinny_strips_of_eight_rows(M, N, Kd):
+    """Strips of 8 rows of the weights. With at most 8 rows of ``a`` the tile's second half takes the
+    next 32 k (K of no multiple of 64 ends inside such a step); with 9 to 16 rows it idles. One
+    column of the weights is large, so that a half of the sum that is dropped or taken twice shows."""
+    lib = K()
+    rng = np.random.default_rng(M * 1000 + N + Kd)
+    a = rounded(rng.standard_normal((M, Kd)), "bfloat16")
+    w = rounded(rng.standard_normal((N, Kd)) / 10, "bfloat16")
+    w[:, Kd - 1] *= 20; w[:, min(Kd - 1, 37)] *= 20                         # in the last step, and in a second half
+    w = rounded(w, "bfloat16")
+    ref = a.astype(np.float64) @ w.astype(np.float64).T
+    A, W = dev(a, torch.bfloat16), dev(w, torch.bfloat16)
+    out = torch.full((M, N), 7.0, device=DEV)
+    lib.gemm_skinny(A, W, out, lib.EPI_STORE, strip_rows=8)
+    np.testing.assert_allclose(out.cpu().numpy(), ref, atol=2e-5 * np.abs(ref).max() + 1e-5)
+    before = rng.standard_normal((M, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    x = dev(before)
+    ssq = torch.full((-(-N // 8), 64), -1.0, device=DEV)
+    if N % 16 == 0:
+        lib.gemm_skinny(A, W, x, lib.EPI_ADD, ssq_out=ssq, strip_rows=8, bias=dev(bias))
+        new = before + ref + bias
+        np.testing.assert_allclose(ssq[:N // 8, :M].cpu().numpy(), ssq_partials(new.astype(np.float32), N // 8)[:, :M], rtol=1e-4)
+    else:
+        lib.gemm_skinny(A, W, x, lib.EPI_ADD, strip_rows=8, bias=dev(bias))
+        new = before + ref + bias
+    np.testing.assert_allclose(x.cpu().numpy(), new, atol=2e-5 * np.abs(new).max() + 1e-5)
