@@ -54,10 +54,11 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t vs[2][HS][VROW];
   const int g = n_heads / n_kv;
   const int groups = (g + GH - 1) / GH;
-  // the longest query blocks first: blockIdx.x counts down through a sequence
-  const int qb = q_blocks - 1 - blockIdx.x;
+  // the longest query blocks first, of all heads and sequences: blockIdx.z counts down through a
+  // sequence, the heads (x, which varies fastest as blocks are handed out) and sequences inside it
+  const int qb = q_blocks - 1 - blockIdx.z;
   const int b = blockIdx.y;
-  const int c = blockIdx.z / groups, hg = blockIdx.z % groups;
+  const int c = blockIdx.x / groups, hg = blockIdx.x % groups;
   // scalar: what depends on the wave alone (chunk, page) lives in scalar registers
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -277,9 +278,9 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t ks[2][CK][KROW];
   __shared__ __attribute__((aligned(16))) bf16_t vs[2][HS][VROW];
   const int g = n_heads / n_kv;
-  const int qb = q_blocks - 1 - blockIdx.x;
+  const int qb = q_blocks - 1 - blockIdx.z;      // the longest query blocks of all heads and sequences first
   const int b = blockIdx.y;
-  const int head = blockIdx.z, c = head / g;   // one query head to a block
+  const int head = blockIdx.x, c = head / g;   // one query head to a block
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, h = lane >> 5;
@@ -492,10 +493,10 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
   // query heads per wave: as many as the registers hold with two blocks on a CU; one with 32 queries a wave
   const int gh = wide ? 1 : head_dim <= 32 ? 4 : head_dim <= 64 ? 2 : 1;
   const long z = (long)n_kv * ((g + gh - 1) / gh);
-  GL3_REQUIRE(n_seqs <= 65535 && z <= 65535, "gl3_attention_prefill: %d sequences / %ld head groups exceed the grid",
-              n_seqs, z);
   const int q_blocks = wide ? (max_q_len + 127) / 128 : (max_q_len + 63) / 64;
-  dim3 grid(q_blocks, n_seqs, (unsigned)z), block(256);
+  GL3_REQUIRE(n_seqs <= 65535 && q_blocks <= 65535, "gl3_attention_prefill: %d sequences / %d blocks of queries exceed the grid",
+              n_seqs, q_blocks);
+  dim3 grid((unsigned)z, n_seqs, q_blocks), block(256);
   if (wide) {
 #define GOW(HS, CK, AH, OCC)                                                                                        \
   attention_prefill_wide_kernel<HS, CK, AH, OCC><<<grid, block, 0, stream>>>(                                       \

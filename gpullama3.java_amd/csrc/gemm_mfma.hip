@@ -220,7 +220,11 @@ static int launch_shape(const void* A, const void* W, void* C, int M, int N, int
 
 template <int EPI, typename TC>
 static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                       int slices, float* P, long p_stride, long ldp, const float* bias, int act, hipStream_t stream) {
+                       int slices, float* P, long p_stride, long ldp, const float* bias, int act, int shape,
+                       hipStream_t stream) {
+  if (shape == 1) return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
+  if (shape == 2) return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
+  if (shape == 3) return launch_shape<EPI, TC, 4, 2, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
   // 256 x 256 tiles of sixteen waves where there is at least one for every CU: half the operand
   // traffic per product, and that traffic is what bounds the large products. Otherwise 128 x 128
   // tiles of eight waves, of which several fit a CU and overlap each other's waits.
@@ -235,9 +239,11 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
 // epilogue into C, slice s > 0 stores its sums into P[s - 1] ([slices - 1][M][ldp] floats,
 // p_stride elements apart), which the caller adds to C in that order.
 // bias (may be null; not with slices): N floats (gated: 2N). act: the gated epilogue's activation.
+// shape: 0 lets the library choose the tile; 1: 128 x 128, eight waves; 2: 256 x 256, sixteen waves of
+// 64 x 64; 3: 256 x 256, eight waves of 128 x 64.
 extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
                              long ldc, int epilogue, int slices, float* P, long p_stride, long ldp, const float* bias,
-                             int act, hipStream_t stream) {
+                             int act, int shape, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_mfma: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gl3_gemm_mfma: K=%d, lda=%ld, ldw=%ld must be multiples of 8",
@@ -255,7 +261,8 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
               "gl3_gemm_mfma: slices need a buffer for their sums and another epilogue than the gated one");
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_mfma: a bias goes with one slice of K");
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_mfma: unknown activation %d", act);
-#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream
+  GL3_REQUIRE(shape >= 0 && shape <= 3, "gl3_gemm_mfma: unknown tile shape %d", shape);
+#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, shape, stream
   if (c_dtype == GL3_F32) {
     if (epilogue == MF_STORE) return launch_mfma<MF_STORE, float>(ARGS);
     if (epilogue == MF_ADD) return launch_mfma<MF_ADD, float>(ARGS);

@@ -64,7 +64,7 @@ def _declare(lib):
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P],
         "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
-        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, P],
+        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
         "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P],
@@ -560,7 +560,7 @@ def gemm_mfma_fits(a, w, out, epilogue):
             and (out.dtype == torch.float32 or (out.dtype == torch.bfloat16 and epilogue != EPI_ADD)))
 
 
-def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None, bias=None, act="silu"):
+def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None, bias=None, act="silu", shape=0):
     """out (=, +=, gated) a @ w.T on the matrix cores, tiled for many rows of ``a``. With
     ``more_slices`` [S, M, N] float32 K is cut into S + 1 slices: the first goes into ``out``, the
     others' sums are stored there, for the caller to add to ``out`` in that order."""
@@ -581,7 +581,7 @@ def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None, bias=None, act="s
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_mfma(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                    out.stride(0), epilogue, slices, _ptr(more_slices), p_stride, ldp,
-                                   _bias(bias, rows, "gemm_mfma"), _act(act, "gemm_mfma"), _stream()),
+                                   _bias(bias, rows, "gemm_mfma"), _act(act, "gemm_mfma"), int(shape), _stream()),
            "gemm_mfma")
 
 
