@@ -1,6 +1,6 @@
 """The cache on the device: keys and values per run-order entry, per-slot state.
 
-Entries of the run order with the same needs (kv heads, head size, window, dtype)
+Entries of the run order with the same needs (kv heads, head size, window, storage dtype)
 form a group; each group has storage, a page pool and block tables of its own (a group
 with a window holds only the pages its window still reaches):
 ``K: [entry in group, page, kv head, position in page, head_dim]``, ``V`` the same with its
@@ -34,6 +34,7 @@ class KVNeed:
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    dtype: Optional[torch.dtype] = None      # None: the engine's; a mixer whose kernels keep something else says so
 
 
 @dataclass(frozen=True)
@@ -50,6 +51,7 @@ class CacheGroup:
         self.pool = PagePool(n_pages)
         self.page_size = page_size
         n = len(self.entries)
+        dtype = need.dtype or dtype
         self.k = torch.zeros((n, n_pages, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
         # values lie transposed inside a page (positions contiguous): the order in which the
         # attention kernels' second product reads them

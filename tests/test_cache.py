@@ -167,3 +167,9 @@ def test_the_table_of_every_group_follows_the_pages():
     assert all(not g.dirty for g in c.groups)
     c.reserve({b: 60}); c.advance(b, 60)                     # b's second page
     assert all(list(g.dirty) == [b * W + 1] for g in c.groups)
+
+
+def test_a_need_may_name_its_own_storage_type():
+    c = Cache([KVNeed(2, 16), KVNeed(2, 16, dtype=torch.float64), KVNeed(2, 16)], [None] * 3, 256, 256, 2, torch.float32, "cpu")
+    assert len(c.groups) == 2 and c.group_of == {0: (0, 0), 2: (0, 1), 1: (1, 0)}
+    assert c.layer_kv(0)[0].dtype == torch.float32 and c.layer_kv(1)[0].dtype == torch.float64

@@ -165,3 +165,40 @@ def test_real_layer_sizes_against_the_plain_implementation(tmp_path, shape):
             assert eng._graphs
         del eng
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("B", [40, 9])
+def test_sampled_runs_of_decode_steps_in_bfloat16_draw_what_single_steps_draw(tmp_path, B):
+    """Runs of decode steps that sample on the device (temperature and top-p, per-row parameters and
+    uniform numbers read by a step counter on the device) at real layer sizes in bfloat16: 40
+    sequences take the kernels for 33 to 64 rows, 9 a bucket of 16. Every token of a run must be
+    the one that the host's twin of the sampler draws, with the same uniform number, from the logits
+    that a single step of the same engine returns for the same sequence so far."""
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.engine import Engine
+    from gpullama3_java_amd.sampling import sample_host, uniform
+    cfg = g.config_from_dict(SHAPES["1B"])
+    folder = str(tmp_path / "shape")
+    g.write_random_model(folder, cfg, 14, std=0.02, norm_std=0.1)
+    eng = Engine.from_folder(folder, dtype="bfloat16", max_context=256, max_tokens=2 * B * 64, n_slots=2 * B)
+    rng = np.random.default_rng(3)
+    prompts = [rng.integers(0, cfg.vocab_size, 3 + i % 5).tolist() for i in range(B)]
+    temps = [0.0 if i % 7 == 3 else 0.6 + 0.1 * (i % 5) for i in range(B)]          # some rows greedy, the rest at several temperatures
+    tops = [1.0 if i % 4 == 0 else 0.9 for i in range(B)]
+    n = 11
+    us = [[uniform(5, i, k) for i in range(B)] for k in range(n)]
+    slots = [eng.take_slot() for _ in range(B)]
+    first = eng.step(list(zip(slots, prompts))).argmax(-1).tolist()
+    run = eng.decode_run(list(zip(slots, first)), n, temps, tops, us)            # [n][B], sampled on the device
+    assert any(key[2] == "sampled" for key in eng._graphs)
+    again = [eng.take_slot() for _ in range(B)]
+    eng.step(list(zip(again, prompts)), want="none")
+    cur = first
+    for k in range(n):
+        logits = eng.step([(s, [t]) for s, t in zip(again, cur)]).cpu().numpy()
+        for i in range(B):
+            want = sample_host(logits[i], temps[i], tops[i], us[k][i])
+            if run[k][i] != want:        # allowed only at an edge of the running sum (the two paths' logits differ in the last bits)
+                near = {sample_host(logits[i], temps[i], tops[i], min(max(us[k][i] + d, 0.0), 0.9999999)) for d in (-1e-4, 1e-4)}
+                assert run[k][i] in near, f"step {k}, row {i}: {run[k][i]} drawn on the device, {want} by the host"
+        cur = run[k]                     # go on with the device's tokens, so that both follow the same sequences
