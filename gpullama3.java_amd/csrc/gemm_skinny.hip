@@ -525,6 +525,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
   }
 }
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bf16x8 sk_buffer_load(__amdgpu_buffer_rsrc_t buf, unsigned byte_offset) {
+  return __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(buf, byte_offset, 0, 0));
+}
+
 // The wide kernel, for steps of three or four token tiles: there a strip's share of A is as
 // large as the strip of W itself, and reading it again for every strip is what takes the time.
 // A block works on NS strips at once (NS pairs of gate and up strips for the gated epilogue), so
@@ -532,31 +537,72 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
 // chip still has blocks enough. With more than one slice the epilogue is a plain store of the
 // slice's sums into slice `blockIdx.y` of a float buffer [slices][M][ldc]: whoever reads the
 // result next adds the slices up in order, no block waits for another.
+//
+// How the operands arrive. A load in the matrix operand's own layout (lane r, q: row r, 16 bytes
+// at q) touches 16 rows with 64 bytes each; a CU's first-level cache takes one such lane a clock,
+// 37 GB/s a CU, whatever the second-level cache could deliver (measured; the same bytes asked for
+// as 8 rows of whole 128-byte lines come at 110 GB/s). With 64 rows of A a block asks for four
+// bytes of A per byte of W, all from the second-level cache, and that rate is the kernel's time.
+// So a wave loads its share of both operands as whole lines (lane l: row l/8, 16 bytes at l%8;
+// two loads cover a tile of 16 rows over 64 k, two k-steps), writes them into its own piece of
+// shared memory and reads the tile back in the operand's layout. Inside a tile row i lies at line
+// i (i < 8) or 8 + (i+1)%8, and its 16-byte piece c at (c xor i%8): then neither the writes (8 lanes
+// a line) nor the reads (16 rows of one piece) meet in a bank. The piece of shared memory is the
+// wave's own, so only the wave's own order matters: a fence of wavefront scope keeps the compiler
+// from moving the reads over the writes, the hardware works a wave's accesses in order.
 template <int MT, int NS, int NW, int EPI, typename TC>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t* __restrict__ A,
                                                                    const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                    int M, int N, int K, long lda, long ldw, long ldc,
-                                                                   long slice_stride, int steps_per_slice, SkRope rp,
+                                                                   long slice_stride, int pairs_per_slice, SkRope rp,
                                                                    SkNext nx) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
-  constexpr int UNROLL = 4;
-  __shared__ f32x4 red[NW][NG * MT][64];
+  constexpr int NWT = NS * NG;        // tiles of W a pair of k-steps
+  constexpr int NT = NWT + MT;        // tiles a wave stages for a pair of k-steps: 16 rows x 128 bytes each
+  constexpr int STAGE = NW * NT * 2048, RED = NW * NG * MT * 1024;
+  __shared__ __attribute__((aligned(16))) char smem[STAGE > RED ? STAGE : RED];
   __shared__ float sm_ssq[1][64];
+  f32x4 (*red)[NG * MT][64] = (f32x4 (*)[NG * MT][64])smem;   // the partial tiles, once the staging is over
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
+  const int l8 = lane >> 3, c8 = lane & 7;
   const int n_strips = (N + 15) / 16;
   const int strip0 = blockIdx.x * NS;
+  char* stage = smem + wave * (NT * 2048);
+  // where this lane's loads go inside a tile (rows l8 and 8 + l8) and where its operands lie (k-steps 0, 1)
+  const int put0 = l8 * 128 + ((c8 ^ l8) * 16);
+  const int put1 = (8 + ((l8 + 1) & 7)) * 128 + ((c8 ^ l8) * 16);
+  const int line = r < 8 ? r : 8 + ((r + 1) & 7);
+  const int get0 = line * 128 + ((q ^ (r & 7)) * 16);
+  const int get1 = line * 128 + (((4 + q) ^ (r & 7)) * 16);
+
+  // Both operands are read through buffer descriptors: a lane whose row or k does not exist gives
+  // an offset beyond the buffer and gets zeros without a branch around the load, so every wave issues
+  // the same loads in the same order and can wait for exactly the ones it needs.
+  const __amdgpu_buffer_rsrc_t w_buf =
+      __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)((((long)NG * N - 1) * ldw + K) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_buf =
+      __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)((((long)M - 1) * lda + K) * 2), 0x00020000);
+  constexpr unsigned NOWHERE = 0x80000000u;   // beyond any buffer the entry point lets in
   int hd[NS], sub[NS];
   bool rotated[NS];
-  const bf16_t* wrow[NS];
+  unsigned wo[NWT][2];   // byte offsets of this lane's lines at k = 0
 #pragma unroll
-  for (int g = 0; g < NS; ++g) {
-    const int wr = sk_strip_row<EPI>(min(strip0 + g, n_strips - 1), r, N, rp, hd[g], sub[g], rotated[g]);
-    wrow[g] = W + (long)wr * ldw + q * 8;
-  }
-  const bf16_t* xrow[MT];
+  for (int g = 0; g < NS; ++g)
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xrow[mt] = mt * 16 + r < M ? A + (long)(mt * 16 + r) * lda + q * 8 : nullptr;
+    for (int j = 0; j < 2; ++j) {
+      const int wr = sk_strip_row<EPI>(min(strip0 + g, n_strips - 1), 8 * j + l8, N, rp, hd[g], sub[g], rotated[g]);
+#pragma unroll
+      for (int h = 0; h < NG; ++h) wo[g * NG + h][j] = (unsigned)((((long)wr + (long)h * N) * ldw + c8 * 8) * 2);
+    }
+  unsigned xo[MT][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int m = mt * 16 + 8 * j + l8;
+      xo[mt][j] = m < M ? (unsigned)(((long)m * lda + c8 * 8) * 2) : NOWHERE;
+    }
 
   TC* out = C + (long)blockIdx.y * slice_stride;
   SkPre pre[NS];
@@ -564,9 +610,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   for (int g = 0; g < NS; ++g)
     pre[g] = sk_preload<MT, EPI, TC>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g], rotated[g], rp, nx);
 
-  const int steps = (K + 31) / 32;
-  const int s_begin = blockIdx.y * steps_per_slice;
-  const int s_end = min(steps, s_begin + steps_per_slice);
+  const int pairs = (K + 63) / 64;
+  const int p_begin = blockIdx.y * pairs_per_slice;
+  const int p_end = min(pairs, p_begin + pairs_per_slice);
   f32x4 acc[NS][NG][MT];
 #pragma unroll
   for (int g = 0; g < NS; ++g)
@@ -576,36 +622,65 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
       for (int mt = 0; mt < MT; ++mt) acc[g][h][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  for (int s0 = s_begin + wave; s0 < s_end; s0 += NW * UNROLL) {
-    bf16x8 wf[UNROLL][NS], uf[UNROLL][NS], xf[UNROLL][MT];
+  // The lines of one pair of k-steps are on their way while the pair before is worked on. (Asking for
+  // W two pairs ahead, with the waits counted so that the later pair stays on its way, gained 3 % where
+  // the registers allowed it and spilled where they did not.)
+  // A wave's pairs are wave, wave + NW, ...; blocks start at different ones, so that at any time the
+  // chip asks for all parts of the rows of W and not for the same quarter of every row.
+  const int n_it = (p_end - p_begin + NW - 1) / NW;
+  const int rot = n_it > 0 ? (int)(blockIdx.x % (unsigned)n_it) : 0;
+  auto pair_at = [&](int i) {   // (i >= n_it: past the end)
+    const int j = i + rot;
+    return i < n_it ? p_begin + wave + NW * (j < n_it ? j : j - n_it) : p_end;
+  };
+  bf16x8 held[NT][2];
+  auto ask = [&](int p) {
+    const unsigned k2 = (p < p_end && p * 64 + c8 * 8 < K) ? (unsigned)p * 128u : NOWHERE;   // (K is a multiple of 8)
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int st = s0 + NW * u;
-      const int k = st * 32;
-      const bool ok = st < s_end && k + q * 8 < K;
+    for (int t = 0; t < NWT; ++t)
 #pragma unroll
-      for (int g = 0; g < NS; ++g) {
-        wf[u][g] = ok ? *(const bf16x8*)(wrow[g] + k) : zero;
-        if (EPI == SK_GATED) uf[u][g] = ok ? *(const bf16x8*)(wrow[g] + (long)N * ldw + k) : zero;
-      }
+      for (int j = 0; j < 2; ++j) held[t][j] = sk_buffer_load(w_buf, wo[t][j] + k2);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) xf[u][mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)(xrow[mt] + k) : zero;
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        held[NWT + mt][j] = sk_buffer_load(a_buf, ((xo[mt][j] | k2) & NOWHERE) ? NOWHERE : xo[mt][j] + k2);
+  };
+  ask(pair_at(0));
+  for (int i = 0; i < n_it; ++i) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      *(bf16x8*)(stage + t * 2048 + put0) = held[t][0];
+      *(bf16x8*)(stage + t * 2048 + put1) = held[t][1];
     }
-    __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    ask(pair_at(i + 1));
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+    for (int s = 0; s < 2; ++s) {
+      const int get = s ? get1 : get0;
+      bf16x8 xf[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) xf[mt] = *(const bf16x8*)(stage + (NWT + mt) * 2048 + get);
 #pragma unroll
       for (int g = 0; g < NS; ++g)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          acc[g][0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][g], xf[u][mt], acc[g][0][mt], 0, 0, 0);
-          if (EPI == SK_GATED)
-            acc[g][1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u][g], xf[u][mt], acc[g][1][mt], 0, 0, 0);
+        for (int h = 0; h < NG; ++h) {
+          const bf16x8 wf = *(const bf16x8*)(stage + (g * NG + h) * 2048 + get);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[g][h][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[mt], acc[g][h][mt], 0, 0, 0);
         }
+    }
+    // the next pair's lines are written only after this pair's operands have been read
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 #pragma unroll
   for (int g = 0; g < NS; ++g) {
-    if (g) __syncthreads();   // the partial tiles in shared memory are free again
+    __syncthreads();   // the staged lines, then the partial tiles of the strip before, are free
     if (strip0 + g < n_strips)   // the same for all threads of the block
       sk_finish<MT, NW, EPI, TC, false, false>(red, sm_ssq, acc[g], strip0 + g, hd[g], sub[g], rotated[g], out, M, N, K,
                                                 ldc, SkNorm{}, nullptr, rp, nx, pre[g]);
@@ -770,12 +845,17 @@ extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtyp
   return 0;
 }
 
+// The wide kernel addresses its operands with 32-bit byte offsets whose top bit means "nowhere".
+static bool wide_addressable(long M, long w_rows, long K, long lda, long ldw) {
+  return ((M - 1) * lda + K) * 2 < (1L << 31) && ((w_rows - 1) * ldw + K) * 2 < (1L << 31);
+}
+
 template <int MT, int NS, int EPI, typename TC>
 static int launch_wide(const SkCall& a, int slices, long slice_stride) {
   constexpr int NW = 8;
   const int n_strips = (a.N + 15) / 16;
-  const int steps = (a.K + 31) / 32;
-  const int per_slice = (steps + slices - 1) / slices;
+  const int pairs = (a.K + 63) / 64;   // pairs of k-steps
+  const int per_slice = (pairs + slices - 1) / slices;
   gemm_skinny_wide_kernel<MT, NS, NW, EPI, TC>
       <<<dim3((n_strips + NS - 1) / NS, slices), dim3(NW * 64), 0, a.stream>>>(
           (const bf16_t*)a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, slice_stride, per_slice,
@@ -812,9 +892,11 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_wide", A, W, C, M, N, K, lda, ldw, 0)) return -1;
   GL3_REQUIRE(M > 32, "gl3_gemm_skinny_wide: M=%d; up to 32 rows are gl3_gemm_skinny's", M);
+  GL3_REQUIRE(wide_addressable(M, epilogue == SK_GATED ? 2L * N : N, K, lda, ldw),
+              "gl3_gemm_skinny_wide: an operand of 2 GiB or more");
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny_wide: ldc too small");
   GL3_REQUIRE(epilogue >= 0 && epilogue <= 2, "gl3_gemm_skinny_wide: unknown epilogue %d", epilogue);
-  GL3_REQUIRE(slices >= 1 && slices <= (K + 31) / 32, "gl3_gemm_skinny_wide: %d slices of K=%d", slices, K);
+  GL3_REQUIRE(slices >= 1 && slices <= (K + 63) / 64, "gl3_gemm_skinny_wide: %d slices of K=%d", slices, K);
   GL3_REQUIRE(slices == 1 || (epilogue == SK_STORE && c_dtype == GL3_F32 && slice_stride >= (long)(M - 1) * ldc + N),
               "gl3_gemm_skinny_wide: slices need the store epilogue, a float output and room for M rows a slice");
   GL3_REQUIRE(epilogue != SK_ADD || c_dtype == GL3_F32, "gl3_gemm_skinny_wide: the add epilogue needs a float output");
@@ -888,8 +970,8 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
   const SkRope rp = {positions, seq_of_token, block_table, table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
                      (bf16_t*)v_cache, n_heads, n_kv, head_dim, adjacent, page_size};
   const SkCall a = {a_rows, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
-  if (!ssq && waves == 0 && M > 32 && (N + 15) / 16 / 2 >= 160) {
-    // many rows and many strips: two strips a block, so that the rows are read half as often
+  if (!ssq && waves == 0 && M > 32 && wide_addressable(M, N, K, lda, ldw)) {
+    // many rows: two strips a block, so that the rows are read half as often, in whole lines
     return (M + 15) / 16 <= 3 ? launch_wide<3, 2, SK_QKV, bf16_t>(a, 1, 0) : launch_wide<4, 2, SK_QKV, bf16_t>(a, 1, 0);
   }
   if (!ssq) return pick_mt<SK_QKV, bf16_t, false, false>(pick_waves(waves, N, K), a);

@@ -408,8 +408,9 @@ def gemm_skinny_wide_fits(a, w, out, epilogue):
 
 def wide_slices(N, K):
     """Into how many slices of K the wide kernel's product [*, K] x [N, K] is cut: enough blocks for
-    the chip (a block takes 64 columns), at least two k-steps of 32 for each of a block's 8 waves."""
-    return max(1, min(8, 256 // -(-N // 64), K // 512))
+    the chip (a block takes 32 columns where they are few), at least one pair of k-steps (64 k) for
+    each of a block's 8 waves."""
+    return max(1, min(8, 256 // -(-N // 32), K // 512))
 
 
 def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="silu"):

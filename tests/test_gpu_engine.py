@@ -153,7 +153,7 @@ def test_decode_steps_of_33_to_64_sequences(name, dtype, graphs, monkeypatch):
     cut = []
 
     def always(N, Kd):
-        n = 3 if Kd >= 192 else 2 if Kd >= 64 else 1
+        n = 3 if Kd >= 192 else 2 if Kd >= 128 else 1      # (a slice is at least a pair of k-steps, 64 k)
         cut.append(n)
         return n
     monkeypatch.setattr(lib, "wide_slices", always)

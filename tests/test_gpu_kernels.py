@@ -763,11 +763,11 @@ def test_gemm_skinny_wide(M, N, Kd):
         lib.gemm_skinny_wide(A, W[:N], out[:M, :N], lib.EPI_STORE, strips=strips)
         np.testing.assert_allclose(out[:M, :N].cpu().numpy(), ref, atol=tol32, err_msg=f"strips {strips}")
         assert torch.all(out[M] == -1) and torch.all(out[:, N:] == -1)
-        for slices in sorted({s_ for s_ in (2, 3, 8) if s_ <= (Kd + 31) // 32}):
+        for slices in sorted({s_ for s_ in (2, 3, 8) if s_ <= (Kd + 63) // 64}):
             part = torch.full((slices, M, N), 7.0, device=DEV)
             lib.gemm_skinny_wide(A, W[:N], part, lib.EPI_STORE, strips=strips)
             np.testing.assert_allclose(part.sum(0).cpu().numpy(), ref, atol=tol32, err_msg=f"{slices} slices")
-            per = -(-((Kd + 31) // 32) // slices) * 32                        # each slice is its own range of K
+            per = -(-((Kd + 63) // 64) // slices) * 64                        # each slice is its own range of K
             for s_ in range(slices):
                 lo, hi = min(s_ * per, Kd), min((s_ + 1) * per, Kd)
                 np.testing.assert_allclose(part[s_].cpu().numpy(), P.linear(a[:, lo:hi], w[:N, lo:hi]) if hi > lo
@@ -795,8 +795,8 @@ def test_gemm_skinny_wide_refuses_what_it_cannot_do():
     with pytest.raises(lib.KernelError, match="slices"):
         lib.gemm_skinny_wide(a, w, torch.zeros(2, 40, 32, device=DEV), lib.EPI_ADD)            # slices are stored, not added
     with pytest.raises(lib.KernelError, match="slices"):
-        lib.gemm_skinny_wide(a, w, torch.zeros(3, 40, 32, device=DEV))                         # more slices than k-steps
-    assert lib.wide_slices(2048, 8192) == 8 and lib.wide_slices(2048, 2048) == 4 and lib.wide_slices(128256, 2048) == 1
+        lib.gemm_skinny_wide(a, w, torch.zeros(3, 40, 32, device=DEV))                         # more slices than pairs of k-steps
+    assert lib.wide_slices(2048, 8192) == 4 and lib.wide_slices(2048, 2048) == 4 and lib.wide_slices(128256, 2048) == 1
 
 
 @pytest.mark.parametrize("d, wdtype, odtype, S", [(2048, "bfloat16", "bfloat16", 8), (100, "float32", "float32", 5),

@@ -1,13 +1,13 @@
-"""The bfloat16 engine against the float32 engine at the layer sizes of real models.
+"""The engines at the layer sizes of real models.
 
 The tiny configurations of the other tests are too small for several choices that the
 product path makes by size: products of a prompt cut into slices of K, tiles of 256 x 256,
 strips of 8 rows, the kernels for 33 to 64 rows with their slices, the tiled kernel for the
 head. Here the layers have the sizes of Llama-3.2-1B (what bench.py measures), Llama-3.2-3B and Llama-3.1-8B
-(two layers each, to keep the test short),
-and every kind of step is run on both engines with the same weights. The float32 engine is
-the reference: it uses one size-generic kernel per operation, and the other tests compare it
-with the plain implementation."""
+(two layers each, to keep the test short). Every kind of step is run on the bfloat16 and the
+float32 engine with the same weights, both engines are compared with the plain implementation
+at these sizes, and runs of decode steps that sample on the device are compared with the
+host's twin of the sampler on the logits of single steps."""
 import numpy as np
 import pytest
 import torch
@@ -167,6 +167,28 @@ def test_real_layer_sizes_against_the_plain_implementation(tmp_path, shape):
         torch.cuda.empty_cache()
 
 
+def _share_of(logits, temperature, top_p, token, u):
+    """How far the uniform number ``u`` lies from the share of [0, 1) that ``token`` has in the sampler's
+    order of the candidates (by falling probability, the kept ones rescaled to 1): 0 when u draws it.
+    With probabilities this flat the neighbours in that order are tokens from anywhere in the
+    vocabulary, so a draw next to an edge is told by this distance and not by the token's number."""
+    s = np.asarray(logits, np.float32) / np.float32(temperature)
+    e = np.exp(s - s.max()).astype(np.float64)
+    p = e / e.sum()
+    order = np.lexsort((np.arange(len(p)), -p))
+    csum = np.cumsum(p[order])
+    mass = 1.0
+    if 0 < top_p < 1:
+        over = np.flatnonzero(csum > top_p)
+        mass = csum[int(over[0])] if len(over) else csum[-1]
+    else:
+        order = np.arange(len(p))
+        csum = np.cumsum(p)
+    rank = int(np.flatnonzero(order == token)[0])
+    lo, hi = (csum[rank - 1] if rank else 0.0) / mass, csum[rank] / mass
+    return 0.0 if lo <= u < hi else min(abs(u - lo), abs(u - hi))
+
+
 @pytest.mark.parametrize("B", [40, 9])
 def test_sampled_runs_of_decode_steps_in_bfloat16_draw_what_single_steps_draw(tmp_path, B):
     """Runs of decode steps that sample on the device (temperature and top-p, per-row parameters and
@@ -199,6 +221,6 @@ def test_sampled_runs_of_decode_steps_in_bfloat16_draw_what_single_steps_draw(tm
         for i in range(B):
             want = sample_host(logits[i], temps[i], tops[i], us[k][i])
             if run[k][i] != want:        # allowed only at an edge of the running sum (the two paths' logits differ in the last bits)
-                near = {sample_host(logits[i], temps[i], tops[i], min(max(us[k][i] + d, 0.0), 0.9999999)) for d in (-1e-4, 1e-4)}
-                assert run[k][i] in near, f"step {k}, row {i}: {run[k][i]} drawn on the device, {want} by the host"
+                assert _share_of(logits[i], temps[i], tops[i], run[k][i], us[k][i]) < 1e-4, \
+                    f"step {k}, row {i}: {run[k][i]} drawn on the device, {want} by the host"
         cur = run[k]                     # go on with the device's tokens, so that both follow the same sequences
