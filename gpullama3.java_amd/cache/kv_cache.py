@@ -4,7 +4,9 @@ Entries of the run order with the same needs (kv heads, head size, window, stora
 form a group; each group has storage, a page pool and block tables of its own (a group
 with a window holds only the pages its window still reaches):
 ``K: [entry in group, page, kv head, position in page, head_dim]``, ``V`` the same with its
-last two axes exchanged. A page is
+last two axes exchanged; inside a page of one head the elements lie in the tiles that the
+attention kernels read as matrix operands (``layout.py``), so a page is a unit that only
+kernels, and code that goes through ``layout.py``, look into. A page is
 ``page_size`` positions of one sequence for every entry of the group. Beside it
 each entry may own a state area of fixed size per slot, ``[slot, elements]``,
 zeroed when the slot is handed out; the attention of this architecture asks for
@@ -53,8 +55,8 @@ class CacheGroup:
         n = len(self.entries)
         dtype = need.dtype or dtype
         self.k = torch.zeros((n, n_pages, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
-        # values lie transposed inside a page (positions contiguous): the order in which the
-        # attention kernels' second product reads them
+        # values lie transposed inside a page: the order in which the attention kernels' second
+        # product reads them (and both in tiles, see layout.py)
         self.v = torch.zeros((n, n_pages, need.n_kv_heads, need.head_dim, page_size), dtype=dtype, device=device)
         self.table = None            # [n_slots + 1, pages of the longest sequence] int32 on the device
         self.table_host = None       # the same on the host (numpy), the copy that the bookkeeping writes
@@ -201,7 +203,8 @@ class Cache:
 
     # ---- what the kernels read
     def layer_kv(self, entry):
-        """(K, V) of one entry: K [page, kv head, position in page, head_dim], V [page, kv head, head_dim, position]."""
+        """(K, V) of one entry: K [page, kv head, position in page, head_dim], V [page, kv head, head_dim, position];
+        the last two axes in the kernels' order (``layout.py``)."""
         g, i = self.group_of[entry]
         return self.groups[g].k[i], self.groups[g].v[i]
 

@@ -12,7 +12,10 @@
 //   S^T[key, head]  = K[key, :] . Q[head, :]^T      two 16x16 tiles, k = head_dim
 //   O^T[dim, head] += V^T[dim, key] . P^T[key, head]  head_dim/16 tiles, k = 32 keys
 // so a lane's 16 bytes of a key row, and of a row of the transposed value page, are the
-// operands as the instruction wants them, and the probabilities leave the first
+// operands as the instruction wants them (and the cache keeps a page in tiles, gl3_k_offset and
+// gl3_v_offset, in which a wave's operand is 1 KB of consecutive memory: with plain rows every
+// lane of a load touched a line of its own, and a chunk's eight loads kept a CU's first-level
+// cache busy for a quarter of the kernel's time), and the probabilities leave the first
 // product in the register order the second one takes: row i of the first score tile is
 // key 8*(i/4) + i%4 of the chunk and row i of the second is the key 4 further, so that
 // quarter q of the lanes ends up with keys 8q..8q+7, which is one 16-byte load from a
@@ -72,7 +75,6 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   for (int ck0 = c_begin + wave; ck0 < c_end; ck0 += NW * CB) {
     // operands of CB chunks, all asked for before any is used
     bf16x8 ka[CB][KK], kb2[CB][KK], vt[CB][DT];
-    const int krow = 8 * (j >> 2) + (j & 3);   // which key of the chunk is row j of the first score tile
 #pragma unroll
     for (int b = 0; b < CB; ++b) {
       const int ck = ck0 + b * NW;
@@ -80,16 +82,19 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
         const int key0 = ck * 32;
         const long page = __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
         const int po = key0 % page_size;
-        const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
-        const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + po;
+        // the chunk's two key tiles lie one after the other, 16 * HS elements each; a k-step's operand
+        // is 512 consecutive elements of a tile in lane order (gl3_k_offset)
+        const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS + lane * 8;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
-          ka[b][kk] = *(const bf16x8*)(kb + (long)krow * HS + kk * 32 + 8 * qd);
-          kb2[b][kk] = *(const bf16x8*)(kb + (long)(krow + 4) * HS + kk * 32 + 8 * qd);
+          ka[b][kk] = *(const bf16x8*)(kb + kk * 512);
+          kb2[b][kk] = *(const bf16x8*)(kb + 16 * HS + kk * 512);
         }
-        // values: lane (dim j of the tile, quarter qd) takes keys 8qd..8qd+7 of the chunk
+        // values: lane (dim j of the tile, quarter qd) takes keys 8qd..8qd+7 of the chunk: 512
+        // consecutive elements of the tile row of 16 dims (gl3_v_offset)
+        const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + (long)(po / 8) * 128 + lane * 8;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vt[b][dt] = *(const bf16x8*)(vb + (long)(dt * 16 + j) * page_size + 8 * qd);
+        for (int dt = 0; dt < DT; ++dt) vt[b][dt] = *(const bf16x8*)(vb + (long)dt * page_size * 16);
       }
     }
     __builtin_amdgcn_sched_barrier(0);   // every load above is issued before the first is waited for

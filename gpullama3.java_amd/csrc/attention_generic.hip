@@ -37,9 +37,10 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const bool valid = key <= p;
     float s = -INFINITY;
     if (valid) {
-      const T* kp = k_cache + (((long)bt[key / page_size] * n_kv + c) * page_size + key % page_size) * head_dim;
+      const T* kp = k_cache + ((long)bt[key / page_size] * n_kv + c) * page_size * head_dim;
+      const int in_page = key % page_size;
       float dot = 0.f;
-      for (int i = 0; i < head_dim; ++i) dot = fmaf(qs[i], to_f32<T>(kp[i]), dot);
+      for (int i = 0; i < head_dim; ++i) dot = fmaf(qs[i], to_f32<T>(kp[gl3_k_offset(in_page, i, head_dim)]), dot);
       s = dot * scale;
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -54,13 +55,14 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     for (int r = 0; r < ATT_MAX_HS / 64; ++r) acc[r] *= alpha;
     for (int j = 0; j < n_valid; ++j) {
       const int kj = base + j;
-      // values lie transposed in a page: [head_dim][position in page]
-      const T* vp = v_cache + ((long)bt[kj / page_size] * n_kv + c) * page_size * head_dim + kj % page_size;
+      // values lie transposed in a page: [head_dim][position in page], in tiles
+      const T* vp = v_cache + ((long)bt[kj / page_size] * n_kv + c) * page_size * head_dim;
+      const int in_page = kj % page_size;
       const float w = ps[j];
 #pragma unroll
       for (int r = 0; r < ATT_MAX_HS / 64; ++r) {
         const int i = lane + 64 * r;
-        if (i < head_dim) acc[r] = fmaf(w, to_f32<T>(vp[(long)i * page_size]), acc[r]);
+        if (i < head_dim) acc[r] = fmaf(w, to_f32<T>(vp[gl3_v_offset(i, in_page, page_size)]), acc[r]);
       }
     }
     m = m_new;
@@ -86,6 +88,9 @@ extern "C" int gl3_attention_generic(const void* q, long q_stride, const void* k
               ATT_MAX_HS);
   GL3_REQUIRE(n_heads <= 65535, "gl3_attention_generic: %d heads exceed the grid", n_heads);
   GL3_REQUIRE(page_size > 0 && table_stride > 0, "gl3_attention_generic: bad paging");
+  GL3_REQUIRE(page_size % 32 == 0 && head_dim % 16 == 0,
+              "gl3_attention_generic: the cache lies in tiles: page_size %d must be a multiple of 32, head_dim %d of 16", page_size,
+              head_dim);
   dim3 grid(n_tokens, n_heads), block(64);
   if (dtype == GL3_F32)
     attention_generic_kernel<float><<<grid, block, 0, stream>>>(

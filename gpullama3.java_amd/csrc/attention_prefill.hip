@@ -116,14 +116,16 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const int key0 = ck * 32;
     const long page = __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
     const int po = key0 % page_size;
+    // (inside a page both lie in tiles, gl3_k_offset and gl3_v_offset: the chunk's keys are still
+    // 32 * HS consecutive elements, its values 512 consecutive elements for every 16 dims)
     const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
-    const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + po;
+    const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + (long)(po / 8) * 128;
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int u = tid + 256 * i;
       if (UNITS % 256 == 0 || u < UNITS) {
         fk[i] = *(const bf16x8*)(kb + u * 8);
-        fv[i] = *(const bf16x8*)(vb + (long)(u >> 2) * page_size + (u & 3) * 8);
+        fv[i] = *(const bf16x8*)(vb + (long)(u >> 6) * page_size * 16 + (u & 63) * 8);
       }
     }
   };
@@ -132,8 +134,11 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     for (int i = 0; i < NU; ++i) {
       const int u = tid + 256 * i;
       if (UNITS % 256 == 0 || u < UNITS) {
-        *(bf16x8*)&ks[buf][(u * 8) / HS][(u * 8) % HS] = fk[i];
-        *(bf16x8*)&vs[buf][u >> 2][(u & 3) * 8] = fv[i];
+        // unit u of the keys: tile u / (2 HS) of the two, column block (u / 16) % (HS / 8), row u % 16
+        const int row = u & 15, tile = u / (2 * HS);
+        *(bf16x8*)&ks[buf][8 * (row >> 2) + 4 * tile + (row & 3)][((u >> 4) % (HS / 8)) * 8] = fk[i];
+        // unit u of the values: 16 dims u / 64, positions 8 * ((u % 64) / 16) .., dim u % 16 of the 16
+        *(bf16x8*)&vs[buf][(u >> 6) * 16 + (u & 15)][((u >> 4) & 3) * 8] = fv[i];
       }
     }
   };
@@ -322,14 +327,16 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     const int key0 = ck * CK;
     const long page = __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
     const int po = key0 % page_size;
+    // (inside a page both lie in tiles, gl3_k_offset and gl3_v_offset: the chunk's keys are still
+    // CK * HS consecutive elements, its values CK * 16 consecutive elements for every 16 dims)
     const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS;
-    const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + po;
+    const bf16_t* vb = v_cache + (page * n_kv + c) * (long)page_size * HS + (long)(po / 8) * 128;
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int u = tid + 256 * i;
       if (UNITS % 256 == 0 || u < UNITS) {
         fk[i] = *(const bf16x8*)(kb + u * 8);
-        fv[i] = *(const bf16x8*)(vb + (long)(u / VU) * page_size + (u % VU) * 8);
+        fv[i] = *(const bf16x8*)(vb + (long)(u / (2 * CK)) * page_size * 16 + (u % (2 * CK)) * 8);
       }
     }
   };
@@ -338,8 +345,12 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     for (int i = 0; i < NU; ++i) {
       const int u = tid + 256 * i;
       if (UNITS % 256 == 0 || u < UNITS) {
-        *(bf16x8*)&ks[buf][(u * 8) / HS][(u * 8) % HS] = fk[i];
-        *(bf16x8*)&vs[buf][u / VU][(u % VU) * 8] = fv[i];
+        // unit u of the keys: 32 keys u / (4 HS), of their two tiles (u / (2 HS)) % 2, column block
+        // (u / 16) % (HS / 8), row u % 16
+        const int row = u & 15, tile = (u / (2 * HS)) & 1, group = u / (4 * HS);
+        *(bf16x8*)&ks[buf][32 * group + 8 * (row >> 2) + 4 * tile + (row & 3)][((u >> 4) % (HS / 8)) * 8] = fk[i];
+        // unit u of the values: 16 dims u / (2 CK), positions 8 * ((u % (2 CK)) / 16) .., dim u % 16 of the 16
+        *(bf16x8*)&vs[buf][(u / (2 * CK)) * 16 + (u & 15)][((u % (2 * CK)) >> 4) * 8] = fv[i];
       }
     }
   };

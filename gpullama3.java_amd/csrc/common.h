@@ -94,6 +94,29 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 // ---- what a product's epilogue may apply besides its own rule: a bias per output column (float;
 // for the gated epilogue the gate's biases, then the up's), and the activation of the gated
 // epilogue. The reference's feed-forward is silu without biases (J/inference/InferenceCore.java:158-166).
+// How one kv head's keys and values lie inside a page of the cache. A key page holds
+// [position][head_dim] elements, a value page [head_dim][position] (transposed), but not row by
+// row: in tiles of 16 rows x 8 columns (16 bytes of bfloat16 a row), the tiles of the same 16 rows
+// one after another along the columns. A matrix-core operand (lane r, q: row r, the 8 elements at
+// column block q) of 16 rows x 32 columns is then 1 KB of consecutive memory in lane order, where
+// rows lying one after another would make every lane touch a line of its own, which costs a CU's
+// first-level cache four times the time.
+//   values: tile (dim / 16, position / 8), row dim % 16, element position % 8
+//   keys:   32 positions make two tiles: the positions with bit 2 clear, then those with it set, so
+//           row i of the first is position 8 * (i / 4) + i % 4 of the 32 and row i of the second the
+//           position 4 further. (The decode kernel's two score tiles of a chunk of 32 keys: a lane
+//           then holds the probabilities of 8 consecutive keys, one 16-byte load of a value row.)
+// page_size is a multiple of 32, head_dim of 16; 32 positions of a key page are still 32 * head_dim
+// consecutive elements, and 8 elements that are consecutive along a row stay consecutive.
+__device__ __forceinline__ long gl3_k_offset(int position_in_page, int dim, int head_dim) {
+  const int p = position_in_page;
+  const int tile = (p >> 5) * 2 + ((p >> 2) & 1), row = ((p >> 3) & 3) * 4 + (p & 3);
+  return ((long)(tile * (head_dim >> 3) + (dim >> 3)) << 7) + (row << 3) + (dim & 7);
+}
+__device__ __forceinline__ long gl3_v_offset(int dim, int position_in_page, int page_size) {
+  return ((long)((dim >> 4) * (page_size >> 3) + (position_in_page >> 3)) << 7) + ((dim & 15) << 3) + (position_in_page & 7);
+}
+
 enum { GL3_ACT_SILU = 0, GL3_ACT_GELU_TANH = 1 };
 
 template <bool FAST>

@@ -236,9 +236,10 @@ extern "C" int gl3_add_slices_rmsnorm(float* x, const int* rows, const float* P,
 // built on the host (J/inference/operation/RoPE.java:29-31). Elements beyond
 // `rot_dim` pass through. A null table means no rotation at all.
 // One layer's key cache is [page][kv head][position in page][head_dim]; its value cache
-// is [page][kv head][head_dim][position in page]: values lie transposed, positions
-// contiguous, which is the operand order the attention kernels' matrix-core products
-// read. The page of position p of sequence s is block_table[s * table_stride + p / page_size].
+// is [page][kv head][head_dim][position in page]: values lie transposed, and inside a page
+// both lie in tiles of 16 rows x 8 columns (gl3_k_offset, gl3_v_offset), which is the order in
+// which the attention kernels' matrix-core products read them.
+// The page of position p of sequence s is block_table[s * table_stride + p / page_size].
 template <typename T>
 __global__ void rope_cache_kernel(T* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                                   const int* __restrict__ block_table, int table_stride, const float* __restrict__ cos_tab,
@@ -251,22 +252,27 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const int* __restrict__ p
   const long row = (long)t * row_stride;
   T* src = qkv + row + (long)head * head_dim;
   const int half = rot_dim / 2;
-  T* dst = src;
+  T* kpage = nullptr;      // a key head: its page; element i of the row goes to kpage[gl3_k_offset(in_page, i, head_dim)]
+  const int in_page = pos % page_size;
   if (head >= n_heads) {
     if (!write_kv) return;
     const int c = (head - n_heads) % n_kv;
     const int page = block_table[(long)seq_of_token[t] * table_stride + pos / page_size];
     if (head >= n_heads + n_kv) {   // a value head: transposed, no rotation
-      T* vt = v_cache + ((long)page * n_kv + c) * page_size * head_dim + pos % page_size;
-      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) vt[(long)i * page_size] = src[i];
+      T* vpage = v_cache + ((long)page * n_kv + c) * page_size * head_dim;
+      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) vpage[gl3_v_offset(i, in_page, page_size)] = src[i];
       return;
     }
-    dst = k_cache + (((long)page * n_kv + c) * page_size + pos % page_size) * head_dim;
+    kpage = k_cache + ((long)page * n_kv + c) * page_size * head_dim;
   }
+  auto put = [&](int i, T v) {
+    if (kpage) kpage[gl3_k_offset(in_page, i, head_dim)] = v;
+    else src[i] = v;
+  };
   const bool rotate = cos_tab != nullptr && head < n_heads + n_kv;
   if (!rotate) {
-    if (dst != src)
-      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
+    if (kpage)
+      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) put(i, src[i]);
     return;
   }
   for (int j = threadIdx.x; j < half; j += blockDim.x) {
@@ -274,11 +280,11 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const int* __restrict__ p
     const int i1 = adjacent ? 2 * j + 1 : j + half;
     const float c = cos_tab[(long)pos * half + j], s = sin_tab[(long)pos * half + j];
     const float v0 = to_f32<T>(src[i0]), v1 = to_f32<T>(src[i1]);
-    dst[i0] = from_f32<T>(v0 * c - v1 * s);
-    dst[i1] = from_f32<T>(v0 * s + v1 * c);
+    put(i0, from_f32<T>(v0 * c - v1 * s));
+    put(i1, from_f32<T>(v0 * s + v1 * c));
   }
-  if (dst != src)
-    for (int i = rot_dim + threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
+  if (kpage)
+    for (int i = rot_dim + threadIdx.x; i < head_dim; i += blockDim.x) put(i, src[i]);
 }
 
 // The same for bfloat16 rows in units of 8 elements (16 bytes): one block per token, a thread
@@ -312,18 +318,20 @@ __global__ __launch_bounds__(256) void rope_cache_vec_kernel(
       const int u = w - rot_heads * per_head;
       const int ch = u / (head_dim / 8), e0 = (u % (head_dim / 8)) * 8;
       const rc_bf16x8 v = *(const rc_bf16x8*)(row + (long)(n_heads + n_kv + ch) * head_dim + e0);
-      bf16_t* vt = v_cache + ((long)page * n_kv + ch) * page_size * head_dim + in_page;
+      bf16_t* vpage = v_cache + ((long)page * n_kv + ch) * page_size * head_dim;
+      const long at = gl3_v_offset(e0, in_page, page_size);   // dims e0 .. e0+7 lie in one tile, 8 elements apart
 #pragma unroll
-      for (int e = 0; e < 8; ++e) vt[(long)(e0 + e) * page_size] = v[e];
+      for (int e = 0; e < 8; ++e) vpage[at + 8 * e] = v[e];
       continue;
     }
     const int head = w / per_head, u = w % per_head;
     bf16_t* src = row + (long)head * head_dim;
-    bf16_t* dst = src;
-    if (head >= n_heads) dst = k_cache + (((long)page * n_kv + (head - n_heads)) * page_size + in_page) * head_dim;
+    bf16_t* kpage = head >= n_heads ? k_cache + ((long)page * n_kv + (head - n_heads)) * page_size * head_dim : nullptr;
+    // where the 8 elements from e on go: back into the row (a query head) or into the key's page
+    auto dst = [&](int e) { return kpage ? kpage + gl3_k_offset(in_page, e, head_dim) : src + e; };
     if (u >= pair_units) {                      // elements beyond the rotation pass through
       const int e0 = (rotate ? rot_dim : 0) + (u - pair_units) * 8;
-      if (dst != src) *(rc_bf16x8*)(dst + e0) = *(const rc_bf16x8*)(src + e0);
+      if (kpage) *(rc_bf16x8*)dst(e0) = *(const rc_bf16x8*)(src + e0);
       continue;
     }
     const int j0 = u * 8;                        // first of the unit's 8 pairs
@@ -355,8 +363,8 @@ __global__ __launch_bounds__(256) void rope_cache_vec_kernel(
         ob[e] = r1;
       }
     }
-    *(rc_bf16x8*)(dst + ea) = oa;
-    *(rc_bf16x8*)(dst + eb) = ob;
+    *(rc_bf16x8*)dst(ea) = oa;
+    *(rc_bf16x8*)dst(eb) = ob;
   }
 }
 
@@ -371,9 +379,13 @@ extern "C" int gl3_rope_cache_write(void* qkv, int dtype, const int* positions, 
   GL3_REQUIRE(rot_dim >= 0 && rot_dim <= head_dim && rot_dim % 2 == 0, "gl3_rope_cache_write: rot_dim %d of head_dim %d",
               rot_dim, head_dim);
   GL3_REQUIRE((cos_tab == nullptr) == (sin_tab == nullptr), "gl3_rope_cache_write: one table without the other");
-  if (write_kv)
+  if (write_kv) {
     GL3_REQUIRE(k_cache && v_cache && block_table && seq_of_token && page_size > 0 && table_stride > 0,
                 "gl3_rope_cache_write: cache arguments missing");
+    GL3_REQUIRE(page_size % 32 == 0 && head_dim % 16 == 0,
+                "gl3_rope_cache_write: the cache lies in tiles: page_size %d must be a multiple of 32, head_dim %d of 16",
+                page_size, head_dim);
+  }
   const int heads = write_kv ? n_heads + 2 * n_kv : n_heads;   // without the write a row holds queries only
   const long row_stride = (long)heads * head_dim;
   // bfloat16 rows whose sizes allow 16-byte units take the kernel of one block per token

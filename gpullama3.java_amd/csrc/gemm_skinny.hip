@@ -284,12 +284,12 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
             bf16x4 o4;
 #pragma unroll
             for (int c = 0; c < 4; ++c) o4[c] = static_cast<bf16_t>(v[c]);
-            *(bf16x4*)(rp.k_cache + ((page * rp.n_kv + ch) * rp.page_size + in_page) * hs + col) = o4;
+            *(bf16x4*)(rp.k_cache + (page * rp.n_kv + ch) * (long)rp.page_size * hs + gl3_k_offset(in_page, col, hs)) = o4;
           } else {
             const int ch = hd - rp.n_heads - rp.n_kv;
-            bf16_t* vt = rp.v_cache + (page * rp.n_kv + ch) * (long)rp.page_size * hs + in_page;
+            bf16_t* vt = rp.v_cache + (page * rp.n_kv + ch) * (long)rp.page_size * hs + gl3_v_offset(col, in_page, rp.page_size);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) vt[(long)(col + c) * rp.page_size] = static_cast<bf16_t>(v[c]);
+            for (int c = 0; c < 4; ++c) vt[8 * c] = static_cast<bf16_t>(v[c]);   // (col % 4 == 0: the 4 dims lie in one tile)
           }
         }
       }
@@ -945,7 +945,8 @@ extern "C" int gl3_gemm_skinny_norm(const void* xg, const int* rows, const float
 }
 
 // a . Wqkv^T, rotation of q and k, q to `q_out` [M, n_heads*head_dim] (ldq), k and v into the paged
-// cache (keys [page][kv head][position][head_dim], values transposed). One token per row; cos/sin
+// cache (keys [page][kv head][position][head_dim], values transposed, in the tiles of gl3_k_offset
+// and gl3_v_offset inside a page). One token per row; cos/sin
 // null: no rotation. head_dim a multiple of 16; the rotation covers the whole head.
 // ssq null: `a` holds the rows as they are. Else `a` is bfloat16(norm weight * x) and the product
 // is that of RMSNorm(x), with the rows' sums of squares in `ssq` [n_partials][64].
@@ -963,6 +964,7 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
               head_dim);
   GL3_REQUIRE(positions && seq_of_token && block_table && k_cache && v_cache && page_size > 0 && table_stride > 0,
               "gl3_qkv_rope_cache: cache arguments missing");
+  GL3_REQUIRE(page_size % 32 == 0, "gl3_qkv_rope_cache: the cache lies in tiles: page_size %d must be a multiple of 32", page_size);
   GL3_REQUIRE((cos_tab == nullptr) == (sin_tab == nullptr), "gl3_qkv_rope_cache: one table without the other");
   GL3_REQUIRE(ldq >= (long)n_heads * head_dim && ldq % 4 == 0 && (uintptr_t)q_out % 8 == 0,
               "gl3_qkv_rope_cache: q_out stride/alignment");

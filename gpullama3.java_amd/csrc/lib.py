@@ -127,11 +127,16 @@ def _ptr(t):
 
 
 def _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, who):
-    """Keys [pages, kv heads, page, head_dim]; values transposed [pages, kv heads, head_dim, page]."""
+    """Keys [pages, kv heads, page, head_dim]; values transposed [pages, kv heads, head_dim, page]; inside a
+    page both lie in the kernels' tiles (``cache/layout.py``), which needs pages of a multiple of 32 positions
+    and heads of a multiple of 16 elements."""
     if (k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim)
             or tuple(v_cache.shape) != (k_cache.shape[0], n_kv, head_dim, page_size)):
         raise KernelError(f"{who}: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for kv {n_kv} "
                           f"page {page_size} hs {head_dim}")
+    if page_size % 32 or head_dim % 16:
+        raise KernelError(f"{who}: the cache lies in tiles: pages of {page_size} positions must be a multiple of 32, "
+                          f"heads of {head_dim} elements a multiple of 16")
 
 
 # ------------------------------------------------------------------ ops

@@ -1,6 +1,8 @@
 """The cache's bookkeeping: no slot or page lost, held twice or freed twice (no GPU)."""
 import random
 
+import numpy as np
+
 import pytest
 import torch
 
@@ -173,3 +175,23 @@ def test_a_need_may_name_its_own_storage_type():
     c = Cache([KVNeed(2, 16), KVNeed(2, 16, dtype=torch.float64), KVNeed(2, 16)], [None] * 3, 256, 256, 2, torch.float32, "cpu")
     assert len(c.groups) == 2 and c.group_of == {0: (0, 0), 2: (0, 1), 1: (1, 0)}
     assert c.layer_kv(0)[0].dtype == torch.float32 and c.layer_kv(1)[0].dtype == torch.float64
+
+
+def test_order_inside_a_page_host_functions_agree_with_the_formulas():
+    """``cache/layout.py`` (reshapes) against the offset formulas written out as index arrays."""
+    import torch
+    import cache_order as O
+    from gpullama3_java_amd.cache import layout as L
+    for page, hs in ((64, 64), (32, 16), (96, 48), (64, 128)):
+        k = np.arange(3 * page * hs, dtype=np.int64).reshape(3, page, hs)
+        v = np.arange(3 * page * hs, dtype=np.int64).reshape(3, hs, page)
+        assert np.array_equal(L.tile_keys(k), O.tile_keys(k)) and np.array_equal(L.tile_values(v), O.tile_values(v))
+        assert np.array_equal(L.untile_keys(L.tile_keys(k)), k) and np.array_equal(L.untile_values(L.tile_values(v)), v)
+        assert torch.equal(L.tile_keys(torch.as_tensor(k)), torch.as_tensor(O.tile_keys(k)))
+        assert torch.equal(L.untile_values(torch.as_tensor(v)), O.untile_values(torch.as_tensor(v)))
+        # a key row's 8 consecutive elements stay consecutive; 32 positions stay 32 * hs consecutive elements
+        idx = O.key_index(page, hs)
+        assert np.all(np.diff(idx.reshape(page, hs // 8, 8), axis=-1) == 1)
+        assert all(set(idx[g * 32:(g + 1) * 32].ravel()) == set(range(g * 32 * hs, (g + 1) * 32 * hs)) for g in range(page // 32))
+    with pytest.raises(ValueError, match="multiple"):
+        L.tile_keys(np.zeros((48, 16)))

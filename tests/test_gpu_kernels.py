@@ -6,6 +6,7 @@ import pytest
 import torch
 
 import plain_llama as P
+from cache_order import tile_keys, tile_values, untile_keys, untile_values
 from gpullama3_java_amd.sampling import sample_host
 
 pytestmark = pytest.mark.gpu
@@ -129,7 +130,9 @@ def test_gemm_generic_mixed_storage_and_strides():
 
 # ------------------------------------------------------------------ paged cache helpers
 def paged(seqs_k, seqs_v, n_kv, hs, page, dtype, rng, n_pages=None):
-    """Scatter per-sequence ``[len, n_kv, hs]`` keys and values into shuffled pages."""
+    """Scatter per-sequence ``[len, n_kv, hs]`` keys and values into shuffled pages, in the order
+    inside a page that the kernels use. ``untile_keys`` and ``untile_values`` give the plain order
+    ``[page, kv head, position, hs]`` and ``[page, kv head, hs, position]`` back."""
     need = [-(-len(k) // page) for k in seqs_k]
     n_pages = n_pages or sum(need) + 3
     ids = rng.permutation(np.arange(1, n_pages))[:sum(need)].tolist()
@@ -145,7 +148,8 @@ def paged(seqs_k, seqs_v, n_kv, hs, page, dtype, rng, n_pages=None):
             n = chunk.stop - chunk.start
             kc[pid, :, :n] = torch.as_tensor(k[chunk]).to(TD[dtype]).transpose(0, 1)
             vc[pid, :, :, :n] = torch.as_tensor(v[chunk]).to(TD[dtype]).permute(1, 2, 0)
-    return kc.to(DEV), vc.to(DEV), torch.as_tensor(table).to(DEV)
+    # inside a page the kernels keep both in tiles; the tests think in the plain order of the shapes
+    return tile_keys(kc).contiguous().to(DEV), tile_values(vc).contiguous().to(DEV), torch.as_tensor(table).to(DEV)
 
 
 # ------------------------------------------------------------------ rotary + cache write
@@ -178,7 +182,7 @@ def test_rope_cache_write(dtype, pairing, H, Kh, hs):
     t = tol(dtype)
     np.testing.assert_allclose(out[:, :H * hs].reshape(T, H, hs), qr, atol=t * 4)
     np.testing.assert_array_equal(out[:, H * hs:], qkv[:, H * hs:])           # k and v in the buffer are left alone
-    kcpu, vcpu, tab = kc.float().cpu().numpy(), vc.float().cpu().numpy(), table.cpu().numpy()
+    kcpu, vcpu, tab = untile_keys(kc).float().cpu().numpy(), untile_values(vc).float().cpu().numpy(), table.cpu().numpy()
     touched = np.zeros(kc.shape[0], bool)
     for i in range(T):
         pid = tab[seq_of[i], positions[i] // page]
@@ -189,7 +193,7 @@ def test_rope_cache_write(dtype, pairing, H, Kh, hs):
     mask = torch.ones_like(kc, dtype=torch.bool)
     for i in range(T):
         mask[tab[seq_of[i], positions[i] // page], :, positions[i] % page] = False
-    assert torch.equal(kc[mask], before_k[mask])
+    assert torch.equal(untile_keys(kc)[mask], untile_keys(before_k)[mask])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -219,7 +223,7 @@ def test_rope_of_a_part_of_the_head_and_of_queries_only(dtype, pairing):
     np.testing.assert_allclose(buf.float().cpu().numpy()[:, :H * hs].reshape(T, H, hs),
                                rotated(qkv[:, :H * hs].reshape(T, H, hs)), atol=t)
     kr = rotated(qkv[:, H * hs:(H + Kh) * hs].reshape(T, Kh, hs))
-    kcpu, vcpu, tab = kc.float().cpu().numpy(), vc.float().cpu().numpy(), table.cpu().numpy()
+    kcpu, vcpu, tab = untile_keys(kc).float().cpu().numpy(), untile_values(vc).float().cpu().numpy(), table.cpu().numpy()
     for i in range(T):
         pid = tab[seq_of[i], positions[i] // page]
         np.testing.assert_allclose(kcpu[pid, :, positions[i] % page], kr[i], atol=t)
@@ -244,7 +248,7 @@ def test_rope_position_zero_and_no_table():
         K().rope_cache_write(buf, dev([0, 0], torch.int32), dev([0, 1], torch.int32), table, cs[0], cs[1], kc, vc,
                              2, 1, 16, 16 if cs[0] is not None else 0, True, 64)
         np.testing.assert_array_equal(buf.cpu().numpy(), qkv)
-        np.testing.assert_array_equal(kc[1, 0, 0].cpu().numpy(), qkv[0, 32:48])
+        np.testing.assert_array_equal(untile_keys(kc)[1, 0, 0].cpu().numpy(), qkv[0, 32:48])
 
 
 # ------------------------------------------------------------------ attention
@@ -735,7 +739,7 @@ def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs, folded_norm):
         k = P.rope_rotate(k, positions, cos, sin, pairing)
     tol_ = 1.5e-2 * np.abs(qkv).max()
     np.testing.assert_allclose(q_out.float().cpu().numpy().reshape(T, H, hs), q, atol=tol_)
-    kcpu, vcpu, tab = kc.float().cpu().numpy(), vc.float().cpu().numpy(), table.cpu().numpy()
+    kcpu, vcpu, tab = untile_keys(kc).float().cpu().numpy(), untile_values(vc).float().cpu().numpy(), table.cpu().numpy()
     mk, mv = torch.ones_like(kc, dtype=torch.bool), torch.ones_like(vc, dtype=torch.bool)
     for i in range(T):
         pid = tab[i, positions[i] // page]
@@ -743,7 +747,8 @@ def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs, folded_norm):
         np.testing.assert_allclose(vcpu[pid, :, :, positions[i] % page], v[i], atol=tol_)
         mk[pid, :, positions[i] % page] = False
         mv[pid, :, :, positions[i] % page] = False
-    assert torch.equal(kc[mk], before_k[mk]) and torch.equal(vc[mv], before_v[mv])   # nothing else moved
+    assert torch.equal(untile_keys(kc)[mk], untile_keys(before_k)[mk])                # nothing else moved
+    assert torch.equal(untile_values(vc)[mv], untile_values(before_v)[mv])
 
 
 # ------------------------------------------------------------------ the wide kernel for 33 to 64 rows, K in slices
