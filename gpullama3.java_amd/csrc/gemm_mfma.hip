@@ -11,7 +11,8 @@
 // barrier a step. Rows in shared memory are padded by 16 bytes so that the 32 lanes that read one
 // column of 16-byte operands hit different banks.
 // Blocks are numbered so that each XCD (whose second-level cache is its own) works on a
-// contiguous range of tiles, neighbouring tiles sharing their panel of W.
+// contiguous range of tiles, ordered so that the tiles it holds at one time form a rectangle
+// and share their panels of A and of W.
 //
 // Epilogues as in gemm_generic.hip: store, add into a float matrix, gated.
 #include "common.h"
@@ -29,7 +30,7 @@ template <int EPI, typename TC, int TM, int WM, int WN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* __restrict__ A,
                                                                   const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                   int M, int N, int K, long lda, long ldw, long ldc,
-                                                                  int tiles_m, int tiles_n, int k_per_slice,
+                                                                  int tiles_m, int tiles_n, int group_m, int k_per_slice,
                                                                   float* __restrict__ P, long p_stride, long ldp,
                                                                   const float* __restrict__ bias, int act) {
   constexpr int NT = 64 * WM * WN;                       // threads
@@ -50,8 +51,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   const int per_xcd = (n_tiles + 7) / 8;
   const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (tile >= n_tiles) return;
-  const int m0 = (tile % tiles_m) * BM;
-  const int n0 = (tile / tiles_m) * NCOLS;
+  // the tiles in order: bands of group_m row tiles; inside a band column after column, the band's row
+  // tiles of a column one after the other. The tiles that an XCD works on at one time are then a
+  // rectangle of group_m row tiles by a few column tiles, which share their rows of A and of W.
+  const int band = tile / (group_m * tiles_n), in_band = tile % (group_m * tiles_n);
+  const int band_rows = min(group_m, tiles_m - band * group_m);
+  const int m0 = (band * group_m + in_band % band_rows) * BM;
+  const int n0 = (in_band / band_rows) * NCOLS;
 
   // global -> register staging in chunks of 16 bytes. An address is a base that the whole block
   // shares (it lives in scalar registers and takes the k-step) plus a 32-bit offset of the thread
@@ -211,9 +217,13 @@ static int launch_shape(const void* A, const void* W, void* C, int M, int N, int
   const long blocks = ((n_tiles + 7) / 8) * 8;
   GL3_REQUIRE(blocks < (1L << 31), "gl3_gemm_mfma: too many tiles");
   const int k_per_slice = ((K + MF_BK - 1) / MF_BK + slices - 1) / slices * MF_BK;
+  // 32 tiles of 256 x 256 (64 of 128 x 128) run on an XCD at a time: bands of 4 (8) row tiles make
+  // them a rectangle of 4 x 8 (8 x 8), which asks memory for a third of the bytes that one column of
+  // 32 row tiles does (3 to 5% of the time of the large products)
+  const int group_m = tiles_m < (bm == 256 ? 4 : 8) ? tiles_m : (bm == 256 ? 4 : 8);
   gemm_mfma_kernel<EPI, TC, TM, WM, WN><<<dim3((unsigned)blocks, slices), dim3(64 * WM * WN), 0, stream>>>(
-      (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n, k_per_slice, P, p_stride,
-      ldp, bias, act);
+      (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n, group_m, k_per_slice, P,
+      p_stride, ldp, bias, act);
   GL3_LAUNCH_CHECK();
   return 0;
 }

@@ -144,9 +144,12 @@ struct SkPre {
   int page;
 };
 
-template <int MT, int EPI, typename TC, int ROWS = 16>
+// GIVEN (SK_QKV): the caller has asked for the token's position and its row of the block table already
+// (`pos`, `table_row`), so that what depends on them can be asked for without another wait.
+template <int MT, int EPI, typename TC, int ROWS = 16, bool GIVEN = false>
 __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int N, long ldc, int strip, int hd, int sub,
-                                            bool rotated, const SkRope& rp, const SkNext& nx = SkNext{}) {
+                                            bool rotated, const SkRope& rp, const SkNext& nx = SkNext{}, int pos = 0,
+                                            int table_row = 0) {
   SkPre p;
   p.prev = p.bias = p.bias_up = p.next_w = p.co = p.si = f32x4{0.f, 0.f, 0.f, 0.f};
   p.pos = 0; p.page = 0;
@@ -174,8 +177,9 @@ __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int
       }
   }
   if (EPI == SK_QKV) {
-    p.pos = rp.positions[m];
-    if (hd >= rp.n_heads) p.page = rp.block_table[(long)rp.seq_of_token[m] * rp.table_stride + p.pos / rp.page_size];
+    p.pos = GIVEN ? pos : rp.positions[m];
+    if (hd >= rp.n_heads)
+      p.page = rp.block_table[(long)(GIVEN ? table_row : rp.seq_of_token[m]) * rp.table_stride + p.pos / rp.page_size];
     if (rotated) {
       const int half = rp.head_dim / 2;
       if (rp.adjacent) {
@@ -605,10 +609,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
     }
 
   TC* out = C + (long)blockIdx.y * slice_stride;
-  SkPre pre[NS];
-#pragma unroll
-  for (int g = 0; g < NS; ++g)
-    pre[g] = sk_preload<MT, EPI, TC>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g], rotated[g], rp, nx);
+  // The rotation's end needs the token's position, and through it a page number and cos and sin:
+  // two trips to memory one after the other. The position is asked for before the first lines of the
+  // product, what hangs on it right after them, so that both trips run beside the product's first.
+  int tok_pos = 0, tok_row = 0;
+  if (EPI == SK_QKV) {
+    const int m = min(min(wave, MT - 1) * 16 + r, M - 1);
+    tok_pos = rp.positions[m];
+    tok_row = rp.seq_of_token[m];
+  }
 
   const int pairs = (K + 63) / 64;
   const int p_begin = blockIdx.y * pairs_per_slice;
@@ -647,6 +656,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
         held[NWT + mt][j] = sk_buffer_load(a_buf, ((xo[mt][j] | k2) & NOWHERE) ? NOWHERE : xo[mt][j] + k2);
   };
   ask(pair_at(0));
+  SkPre pre[NS];
+#pragma unroll
+  for (int g = 0; g < NS; ++g)
+    pre[g] = sk_preload<MT, EPI, TC, 16, EPI == SK_QKV>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g],
+                                                         rotated[g], rp, nx, tok_pos, tok_row);
   for (int i = 0; i < n_it; ++i) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
