@@ -415,13 +415,27 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
 template <int MT, int NW, int KS, int EPI, typename TC, bool XNORM, bool SSQ>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
     const void* __restrict__ Av, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N, int K, long lda,
-    long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out, SkNext nx, SkRope rp, int n_strips) {
+    long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out, SkNext nx, SkRope rp, int n_strips,
+    const bf16_t* __restrict__ Wt) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   __shared__ f32x4 red[NW][NG * MT][64];
   __shared__ float sm_ssq[XNORM ? NW : 1][64];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // Where a strip's operands lie. In W itself a lane's 16 bytes of k-step s are in its row at 32 s
+  // elements; every lane of a load is then on a line of its own. In the copy in the operands' own
+  // order (Wt, may be null: [strip][k-step][lane][8], k padded with zeros to whole steps, the strips'
+  // rows as sk_strip_row names them) a load is 1 KB of consecutive memory, which the CU's first-level
+  // cache takes in less than half the time.
+  const int steps_all = (K + 31) / 32;
+  const long w_step = Wt ? 512 : 32;                       // elements from one k-step to the next
+  const long w_up = Wt ? (long)(N / 16) * steps_all * 512 : (long)N * ldw;   // from a gate strip to its up strip
+  auto strip_base = [&](int strip_, int& hd_, int& sub_, bool& rot_) {
+    const int wr = sk_strip_row<EPI>(strip_, r, N, rp, hd_, sub_, rot_);
+    return Wt ? Wt + ((long)strip_ * steps_all * 64 + lane) * 8 : W + (long)wr * ldw + q * 8;
+  };
+  auto step_ok = [&](int st) { return Wt ? st < steps_all : st * 32 + q * 8 < K; };
   // Everything the block needs first is asked for before anything is waited for, so that it all
   // arrives in one trip to memory: the first strip's rows of W, the rows' partial sums of squares,
   // and this wave's share of A (k-steps wave, wave + NW, ...).
@@ -430,14 +444,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
   bool rotated;
   bf16x8 wf[KS], uf[KS];
   {
-    const int wr = sk_strip_row<EPI>(strip, r, N, rp, hd, sub, rotated);
-    const bf16_t* wrow = W + (long)wr * ldw + q * 8;
+    const bf16_t* wrow = strip_base(strip, hd, sub, rotated);
 #pragma unroll
     for (int i = 0; i < KS; ++i) {
-      const int k = (wave + NW * i) * 32;
-      const bool ok = k + q * 8 < K;
-      wf[i] = ok ? *(const bf16x8*)(wrow + k) : zero;
-      if (EPI == SK_GATED) uf[i] = ok ? *(const bf16x8*)(wrow + (long)N * ldw + k) : zero;
+      const int st = wave + NW * i;
+      const bool ok = step_ok(st);
+      wf[i] = ok ? *(const bf16x8*)(wrow + st * w_step) : zero;
+      if (EPI == SK_GATED) uf[i] = ok ? *(const bf16x8*)(wrow + w_up + st * w_step) : zero;
     }
   }
   float sq[16];
@@ -473,14 +486,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
     int hd_n = 0, sub_n = 0;
     bool rot_n = false;
     if (next < n_strips) {
-      const int wr = sk_strip_row<EPI>(next, r, N, rp, hd_n, sub_n, rot_n);
-      const bf16_t* wrow = W + (long)wr * ldw + q * 8;
+      const bf16_t* wrow = strip_base(next, hd_n, sub_n, rot_n);
 #pragma unroll
       for (int i = 0; i < KS; ++i) {
-        const int k = (wave + NW * i) * 32;
-        const bool ok = k + q * 8 < K;
-        wn[i] = ok ? *(const bf16x8*)(wrow + k) : zero;
-        if (EPI == SK_GATED) un[i] = ok ? *(const bf16x8*)(wrow + (long)N * ldw + k) : zero;
+        const int st = wave + NW * i;
+        const bool ok = step_ok(st);
+        wn[i] = ok ? *(const bf16x8*)(wrow + st * w_step) : zero;
+        if (EPI == SK_GATED) un[i] = ok ? *(const bf16x8*)(wrow + w_up + st * w_step) : zero;
       }
     }
     const SkPre pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx);
@@ -709,6 +721,7 @@ struct SkCall {
   bool resident = true;
   int strip_rows = 16;
   SkNext nx = SkNext{};
+  const void* Wt = nullptr;   // W in the operands' order (the resident kernel reads it where it is given)
 };
 
 // Blocks of the resident kernel: every strip its own block while that still leaves CUs idle, else
@@ -728,7 +741,8 @@ static int launch_skinny(int nw, const SkCall& a) {
   do {                                                                                                            \
     gemm_skinny_resident_kernel<MT, NW, KS, EPI, TC, XNORM, SSQ>                                                  \
         <<<dim3(resident_blocks(n_strips, NW)), dim3(NW * 64), 0, a.stream>>>(                                    \
-            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp, n_strips); \
+            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp, n_strips, \
+            (const bf16_t*)a.Wt);                                                                                 \
     GL3_LAUNCH_CHECK();                                                                                           \
     return 0;                                                                                                     \
   } while (0)
@@ -827,10 +841,13 @@ static int check_common(const char* who, const void* A, const void* W, const voi
 // next_weight, xg (may be null; with ssq_out): the weight [N] (float) of the norm that follows, and
 // where bfloat16(weight * x) of the completed rows goes, [M][ldxg].
 // bias (may be null): N floats (gated: 2N), added to the sums; act: the gated epilogue's activation.
+// w_tiled (may be null; N % 16 == 0): the same W as [strip of 16 rows][k-step of 32][lane][8 elements], k
+// padded with zeros to whole steps (gated: the strips of the gate rows, then those of the up rows): the
+// kernels that keep their rows of A in registers read W there.
 extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                long ldw, long ldc, int epilogue, int waves, float* ssq_out, int strip_rows,
                                const float* next_weight, void* xg, long ldxg, const float* bias, int act,
-                               hipStream_t stream) {
+                               const void* w_tiled, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny", A, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny: ldc too small");
@@ -845,6 +862,8 @@ extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtyp
   SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, ssq_out, SkRope{}, stream, waves == 0, strip_rows};
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny: unknown activation %d", act);
   a.nx = SkNext{next_weight, (bf16_t*)xg, ldxg, bias, act};
+  GL3_REQUIRE(!w_tiled || (N % 16 == 0 && (uintptr_t)w_tiled % 16 == 0), "gl3_gemm_skinny: a copy of W in the operands' order needs N %% 16 == 0");
+  a.Wt = w_tiled;
   const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32) {
     if (epilogue == SK_STORE) return pick_mt<SK_STORE, float, false, false>(nw, a);
@@ -940,7 +959,8 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
 // bias (may be null): N floats (gated: 2N), added after the 1/rms; act: the gated epilogue's activation.
 extern "C" int gl3_gemm_skinny_norm(const void* xg, const int* rows, const float* ssq, int n_partials, float eps,
                                     const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
-                                    long ldc, int epilogue, int waves, const float* bias, int act, hipStream_t stream) {
+                                    long ldc, int epilogue, int waves, const float* bias, int act, const void* w_tiled,
+                                    hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_norm", xg, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ssq && n_partials > 0, "gl3_gemm_skinny_norm: norm arguments missing");
@@ -950,6 +970,8 @@ extern "C" int gl3_gemm_skinny_norm(const void* xg, const int* rows, const float
   const SkNorm nrm = {ssq, n_partials, eps, rows};
   SkCall a = {xg, W, C, M, N, K, lda, ldw, ldc, nrm, nullptr, SkRope{}, stream, waves == 0};
   a.nx = SkNext{nullptr, nullptr, 0, bias, act};
+  GL3_REQUIRE(!w_tiled || (N % 16 == 0 && (uintptr_t)w_tiled % 16 == 0), "gl3_gemm_skinny_norm: a copy of W in the operands' order needs N %% 16 == 0");
+  a.Wt = w_tiled;
   const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32 && epilogue == SK_STORE) return pick_mt<SK_STORE, float, true, false>(nw, a);
   if (c_dtype == GL3_BF16 && epilogue == SK_STORE) return pick_mt<SK_STORE, bf16_t, true, false>(nw, a);
@@ -969,7 +991,7 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
                                   const int* seq_of_token, const int* block_table, int table_stride,
                                   const float* cos_tab, const float* sin_tab, void* k_cache, void* v_cache,
                                   int n_heads, int n_kv, int head_dim, int adjacent, int page_size, int waves,
-                                  hipStream_t stream) {
+                                  const void* w_tiled, hipStream_t stream) {
   if (M == 0) return 0;
   const int N = (n_heads + 2 * n_kv) * head_dim;
   if (check_common("gl3_qkv_rope_cache", a_rows, Wqkv, q_out, M, N, K, lda, ldw, waves)) return -1;
@@ -985,7 +1007,9 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
   const SkNorm nrm = {ssq, n_partials, eps, nullptr};
   const SkRope rp = {positions, seq_of_token, block_table, table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
                      (bf16_t*)v_cache, n_heads, n_kv, head_dim, adjacent, page_size};
-  const SkCall a = {a_rows, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
+  SkCall a = {a_rows, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
+  GL3_REQUIRE(!w_tiled || (uintptr_t)w_tiled % 16 == 0, "gl3_qkv_rope_cache: the copy of W must be 16-byte aligned");
+  a.Wt = w_tiled;   // (its strips hold the rows that sk_strip_row names: for half-split pairing 8 rows and the 8 half a head further)
   if (!ssq && waves == 0 && M > 32 && wide_addressable(M, N, K, lda, ldw)) {
     // many rows: two strips a block, so that the rows are read half as often, in whole lines
     return (M + 15) / 16 <= 3 ? launch_wide<3, 2, SK_QKV, bf16_t>(a, 1, 0) : launch_wide<4, 2, SK_QKV, bf16_t>(a, 1, 0);

@@ -60,10 +60,10 @@ def _declare(lib):
         "gl3_argmax": [P, L, P, P, I, I, P],
         "gl3_argmax_static": [P, L, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
-        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P],
+        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P],
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P],
-        "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P],
-        "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P],
+        "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P],
+        "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P],
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
@@ -404,7 +404,53 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows
     _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                      out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _ptr(next_weight),
                                      _ptr(xg), xg.stride(0) if xg is not None else 0, _bias(bias, rows, "gemm_skinny"),
-                                     _act(act, "gemm_skinny"), _stream()), "gemm_skinny")
+                                     _act(act, "gemm_skinny"), _tiled(w, rows, K, n_out=N), _stream()), "gemm_skinny")
+
+
+def strip_rows_of(n_rows, qkv=None):
+    """Which row of W is row r of strip t of 16, as the kernels' ``sk_strip_row`` names them: rows
+    16 t + r (the last strip repeats the last row), and for the stacked q, k, v rows with half-split
+    pairing (``qkv`` = (n_heads, n_kv, head_dim, rotated, adjacent)) 8 rows of a rotated head and the
+    8 half a head further, so that both elements of a pair lie in one tile."""
+    n_strips = -(-n_rows // 16)
+    rows = torch.arange(n_strips * 16).clamp(max=n_rows - 1).view(n_strips, 16)
+    if qkv is not None:
+        n_heads, n_kv, hs, rotated, adjacent = qkv
+        if rotated and not adjacent:
+            per_head = hs // 16
+            t = torch.arange(n_strips).view(-1, 1)
+            r = torch.arange(16).view(1, -1)
+            hd, sub = t // per_head, t % per_head
+            paired = hd * hs + 8 * sub + torch.where(r < 8, r, hs // 2 + r - 8)
+            rows = torch.where(hd < n_heads + n_kv, paired, rows)
+    return rows.reshape(-1)
+
+
+def tile_weight(w, qkv=None):
+    """A copy of ``w`` [N, K] (bfloat16, N % 16 == 0) in the order in which the matrix cores take it as an
+    operand: [strip of 16 rows][k-step of 32][lane = 16 * (k block of 8) + row][8 elements], k padded with
+    zeros to whole steps. The products of few rows whose kernels keep their rows of A in registers read
+    it where a weight carries one (``w.tiled``): a load is then 1 KB of consecutive memory."""
+    N, K = w.shape
+    if N % 16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"tile_weight: {tuple(w.shape)} {w.dtype}")
+    steps = -(-K // 32)
+    rows = strip_rows_of(N, qkv).to(w.device)
+    wp = torch.zeros(N, steps * 32, dtype=w.dtype, device=w.device)
+    wp[:, :K] = w[rows]
+    t = wp.view(N // 16, 16, steps, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+    t.tiled_for = qkv
+    return t
+
+
+def _tiled(w, n_rows, K, qkv=None, n_out=None):
+    """The pointer to ``w.tiled`` if the weight carries a copy in the operands' order that fits this call
+    (``n_out``: the output columns, where the gate rows and the up rows must each fill whole strips)."""
+    t = getattr(w, "tiled", None)
+    if (t is None or n_rows % 16 or (n_out is not None and n_out % 16) or t.numel() != n_rows * -(-K // 32) * 32
+            or getattr(t, "tiled_for", None) != qkv):
+        return c_void_p(0)
+    return _ptr(t)
 
 
 def gemm_skinny_wide_fits(a, w, out, epilogue):
@@ -470,7 +516,7 @@ def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=
     _check(library().gl3_gemm_skinny_norm(
         _ptr(xg), _ptr(rows), _ptr(ssq), n_partials, float(eps), _ptr(w), _ptr(out), _code(out, "out"), M, N, K,
         xg.stride(0), w.stride(0), out.stride(0), epilogue, waves, _bias(bias, wrows, "gemm_skinny_norm"),
-        _act(act, "gemm_skinny_norm"), _stream()), "gemm_skinny_norm")
+        _act(act, "gemm_skinny_norm"), _tiled(w, wrows, K, n_out=N), _stream()), "gemm_skinny_norm")
 
 
 def qkv_rope_cache_fits(a, w_qkv, head_dim, rot_dim):
@@ -512,7 +558,8 @@ def qkv_rope_cache(a, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_toke
     _check(library().gl3_qkv_rope_cache(
         _ptr(a), _ptr(ssq), n_partials, float(eps), _ptr(w_qkv), _ptr(q_out), q_out.stride(0), T, K, a.stride(0),
         w_qkv.stride(0), _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], _ptr(cos),
-        _ptr(sin), _ptr(k_cache), _ptr(v_cache), n_heads, n_kv, head_dim, int(adjacent), page_size, waves, _stream()),
+        _ptr(sin), _ptr(k_cache), _ptr(v_cache), n_heads, n_kv, head_dim, int(adjacent), page_size, waves,
+        _tiled(w_qkv, w_qkv.shape[0], K, qkv=(n_heads, n_kv, head_dim, cos is not None, bool(adjacent))), _stream()),
         "qkv_rope_cache")
 
 

@@ -57,6 +57,8 @@ class GQAAttention:
         weights[n["q"]], weights[n["k"]], weights[n["v"]] = (
             self.w_qkv[:qn], self.w_qkv[qn:qn + kn], self.w_qkv[qn + kn:])
         self.w_q = self.w_qkv[:qn]
+        ops.for_few_rows(self.w_qkv, (self.H, self.Kh, self.hs, self.position is not None,
+                                      bool(self.position is not None and self.position.adjacent)))
         self.w_o = weights[n["o"]]
         if self.biased:     # the epilogues read biases as float
             self.b_qkv = torch.cat([weights[n[k]].float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()

@@ -79,6 +79,7 @@ class DecoderModel:
         self.weights = weights
         self.embedding = weights[self.spec.embedding_name]
         self.head = self.embedding if self.spec.head_name is None else weights[self.spec.head_name]
+        ops.for_few_rows(self.head)
         if self.spec.position_table_name is not None:
             self.position_table = weights[self.spec.position_table_name].to(self.embedding.dtype)
         self.final_norm.load(weights)

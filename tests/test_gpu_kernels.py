@@ -977,3 +977,83 @@ def test_gemm_skinny_strips_of_eight_rows(M, N, Kd):
         lib.gemm_skinny(A, W, x, lib.EPI_ADD, strip_rows=8, bias=dev(bias))
         new = before + ref + bias
     np.testing.assert_allclose(x.cpu().numpy(), new, atol=2e-5 * np.abs(new).max() + 1e-5)
+
+
+# ------------------------------------------------------------------ weights in the operands' order
+@pytest.mark.parametrize("N, Kd", [(48, 72), (2048, 2048), (160, 1544), (6144, 256), (1008, 4104)])
+@pytest.mark.parametrize("M", [1, 8, 16, 29])
+def test_products_read_a_weight_copy_in_operand_order(M, N, Kd):
+    """``tile_weight``: [strip][k-step][lane][8] with k padded to whole steps. The kernels that keep the
+    step's rows in registers read it in place of the rows of W; the sums are the same sums, bit for bit."""
+    rng = np.random.default_rng(M + N + Kd)
+    lib = K()
+    w = dev(rounded(rng.standard_normal((2 * N, Kd)) / math.sqrt(Kd), "bfloat16"), torch.bfloat16)
+    t = lib.tile_weight(w)
+    steps = -(-Kd // 32)
+    flat = t.reshape(-1).float().cpu().numpy()
+    wn = w.float().cpu().numpy()
+    for (n, k) in [(0, 0), (17, 9), (2 * N - 1, Kd - 1), (N + 5, Kd // 2), (31, 40 % Kd)]:
+        strip, r, step, q, e = n // 16, n % 16, k // 32, (k % 32) // 8, k % 8
+        assert flat[((strip * steps + step) * 64 + q * 16 + r) * 8 + e] == wn[n, k]
+    x = (rng.standard_normal((M, Kd)) * 2).astype(np.float32)
+    nw = rounded(1 + 0.2 * rng.standard_normal(Kd), "bfloat16")
+    xg, ssq = times_weight(x, nw).to(DEV), dev(ssq_partials(x, 5))
+    a = dev(rounded(x, "bfloat16"), torch.bfloat16)
+    res = {}
+    for tiled in (False, True):
+        if tiled:
+            w.tiled = t
+        g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+        lib.gemm_skinny_norm(xg, ssq, 5, 1e-5, w, g_, lib.EPI_GATED)
+        s_ = torch.zeros(M, 2 * N, device=DEV)
+        lib.gemm_skinny_norm(xg, ssq, 5, 1e-5, w, s_, lib.EPI_STORE)
+        p_ = torch.zeros(M, 2 * N, device=DEV)
+        lib.gemm_skinny(a, w, p_, lib.EPI_STORE)
+        res[tiled] = (g_, s_, p_)
+    for u, v in zip(res[False], res[True]):
+        assert torch.equal(u, v)
+    np.testing.assert_allclose(res[True][2].cpu().numpy(), P.linear(rounded(x, "bfloat16"), wn),
+                               atol=2e-5 * np.abs(wn).max() * np.abs(x).max() * Kd)
+    # a copy that does not belong to the call's rows is not used
+    w.tiled = lib.tile_weight(w[:N].contiguous())
+    p2 = torch.zeros(M, 2 * N, device=DEV)
+    lib.gemm_skinny(a, w, p2, lib.EPI_STORE)
+    assert torch.equal(p2, res[False][2])
+
+
+@pytest.mark.parametrize("pairing", ["adjacent", "half", None])
+@pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 16), (5, 5, 48), (8, 1, 128)])
+def test_qkv_rope_cache_reads_a_weight_copy_in_operand_order(pairing, H, Kh, hs):
+    """The stacked q, k, v rows in the operands' order hold, for half-split pairing, 8 rows of a head and
+    the 8 half a head further in one strip (``strip_rows_of``), as the kernel's strips do."""
+    rng = np.random.default_rng(hs + H)
+    lib = K()
+    d, page, T = 96, 64, 7
+    x = (rng.standard_normal((T, d)) * 2).astype(np.float32)
+    nw = rounded(1 + 0.2 * rng.standard_normal(d), "bfloat16")
+    w = dev(rounded(rng.standard_normal(((H + 2 * Kh) * hs, d)) / math.sqrt(d), "bfloat16"), torch.bfloat16)
+    positions = np.array([70, 0, 129, 63, 64, 5, 31])
+    zk = [np.zeros((b + 1, Kh, hs), np.float32) for b in positions]
+    cos, sin = P.rope_table(256, hs, 50000.0)
+    got = {}
+    for tiled in (False, True):
+        if tiled:
+            w.tiled = lib.tile_weight(w, qkv=(H, Kh, hs, pairing is not None, pairing == "adjacent"))
+        kc, vc, table = paged(zk, zk, Kh, hs, page, "bfloat16", np.random.default_rng(1))
+        q_out = torch.zeros(T, H * hs, device=DEV, dtype=torch.bfloat16)
+        lib.qkv_rope_cache(times_weight(x, nw).to(DEV), dev(ssq_partials(x, 6)), 6, 1e-5, w, q_out,
+                           dev(positions, torch.int32), dev(np.arange(T), torch.int32), table,
+                           dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
+                           pairing == "adjacent", page)
+        got[tiled] = (q_out, kc, vc)
+    for u, v in zip(got[False], got[True]):
+        assert torch.equal(u, v)
+    # a copy made for another pairing is not used
+    w.tiled = lib.tile_weight(w, qkv=(H, Kh, hs, pairing is None, False))
+    kc, vc, table = paged(zk, zk, Kh, hs, page, "bfloat16", np.random.default_rng(1))
+    q2 = torch.zeros(T, H * hs, device=DEV, dtype=torch.bfloat16)
+    lib.qkv_rope_cache(times_weight(x, nw).to(DEV), dev(ssq_partials(x, 6)), 6, 1e-5, w, q2,
+                       dev(positions, torch.int32), dev(np.arange(T), torch.int32), table,
+                       dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
+                       pairing == "adjacent", page)
+    assert torch.equal(q2, got[False][0])
