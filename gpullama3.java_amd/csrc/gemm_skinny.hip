@@ -331,7 +331,7 @@ template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ, int ROWS =
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __restrict__ Av, const bf16_t* __restrict__ W,
                                                               TC* __restrict__ C, int M, int N, int K, long lda,
                                                               long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out,
-                                                              SkNext nx, SkRope rp) {
+                                                              SkNext nx, SkRope rp, const bf16_t* __restrict__ Wt8) {
   static_assert(!PACK || (ROWS == 8 && MT == 1 && EPI != SK_GATED && EPI != SK_QKV && !XNORM), "packed strips: 8 rows, one tile");
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   constexpr int UNROLL = 8;
@@ -365,13 +365,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
 
   if (PACK) {
     // a wave takes steps of 64 k: step wave, wave + NW, ...
+    // (Wt8, may be null: W as [strip of 8 rows][step of 64 k][lane][8], the packed tile's own order, k padded
+    // with zeros to whole steps: a load is then 1 KB of consecutive memory)
+    const int steps64 = (K + 63) / 64;
+    const bf16_t* wbase = Wt8 ? Wt8 + ((long)strip * steps64 * 64 + lane) * 8 : wrow;
+    const long w_step = Wt8 ? 512 : 64;
     for (int p0 = wave; p0 * 64 < K; p0 += NW * UNROLL) {
       bf16x8 wf[UNROLL], xf[UNROLL][MT];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        const int k = (p0 + NW * u) * 64;
+        const int p = p0 + NW * u, k = p * 64;
         const bool ok = k + koff < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
-        wf[u] = ok ? *(const bf16x8*)(wrow + k) : zero;
+        wf[u] = (Wt8 ? p < steps64 : ok) ? *(const bf16x8*)(wbase + p * w_step) : zero;
         sk_load_x<MT, XNORM>(xf[u], xrow, k + koff, ok, nrm);
       }
       __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
@@ -722,6 +727,7 @@ struct SkCall {
   int strip_rows = 16;
   SkNext nx = SkNext{};
   const void* Wt = nullptr;   // W in the operands' order (the resident kernel reads it where it is given)
+  const void* Wt8 = nullptr;  // W in the order of the packed tiles of strips of 8 rows
 };
 
 // Blocks of the resident kernel: every strip its own block while that still leaves CUs idle, else
@@ -752,10 +758,12 @@ static int launch_skinny(int nw, const SkCall& a) {
       // the tile's other half takes the next 32 k
       if (a.M <= 8)
         gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8, true><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
-            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp);
+            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp,
+            (const bf16_t*)a.Wt8);
       else
         gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
-            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp);
+            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp,
+            (const bf16_t*)nullptr);
       GL3_LAUNCH_CHECK();
       return 0;
     }
@@ -787,7 +795,8 @@ static int launch_skinny(int nw, const SkCall& a) {
 #undef RES
 #define GO(NW)                                                                                                    \
   gemm_skinny_kernel<MT, NW, EPI, TC, XNORM, SSQ><<<grid, dim3(NW * 64), 0, a.stream>>>(                          \
-      a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp)
+      a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp,          \
+      (const bf16_t*)nullptr)
   if constexpr (NG * MT <= 2) {
     if (nw >= 16) { GO(16); GL3_LAUNCH_CHECK(); return 0; }
   }
@@ -844,10 +853,12 @@ static int check_common(const char* who, const void* A, const void* W, const voi
 // w_tiled (may be null; N % 16 == 0): the same W as [strip of 16 rows][k-step of 32][lane][8 elements], k
 // padded with zeros to whole steps (gated: the strips of the gate rows, then those of the up rows): the
 // kernels that keep their rows of A in registers read W there.
+// w_tiled8 (may be null; N % 8 == 0): W as [strip of 8 rows][step of 64 k][lane][8 elements], lane (r, q)
+// holding row r % 8 at k = 32 (r / 8) + 8 q: the order of the packed tiles of strips of 8 rows (M <= 8).
 extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                long ldw, long ldc, int epilogue, int waves, float* ssq_out, int strip_rows,
                                const float* next_weight, void* xg, long ldxg, const float* bias, int act,
-                               const void* w_tiled, hipStream_t stream) {
+                               const void* w_tiled, const void* w_tiled8, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny", A, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny: ldc too small");
@@ -864,6 +875,8 @@ extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtyp
   a.nx = SkNext{next_weight, (bf16_t*)xg, ldxg, bias, act};
   GL3_REQUIRE(!w_tiled || (N % 16 == 0 && (uintptr_t)w_tiled % 16 == 0), "gl3_gemm_skinny: a copy of W in the operands' order needs N %% 16 == 0");
   a.Wt = w_tiled;
+  GL3_REQUIRE(!w_tiled8 || (N % 8 == 0 && (uintptr_t)w_tiled8 % 16 == 0), "gl3_gemm_skinny: a copy of W in the packed tiles' order needs N %% 8 == 0");
+  a.Wt8 = w_tiled8;
   const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32) {
     if (epilogue == SK_STORE) return pick_mt<SK_STORE, float, false, false>(nw, a);

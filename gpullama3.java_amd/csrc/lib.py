@@ -60,7 +60,7 @@ def _declare(lib):
         "gl3_argmax": [P, L, P, P, I, I, P],
         "gl3_argmax_static": [P, L, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
-        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P],
+        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P, P],
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P],
         "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P],
@@ -404,7 +404,7 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows
     _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                      out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _ptr(next_weight),
                                      _ptr(xg), xg.stride(0) if xg is not None else 0, _bias(bias, rows, "gemm_skinny"),
-                                     _act(act, "gemm_skinny"), _tiled(w, rows, K, n_out=N), _stream()), "gemm_skinny")
+                                     _act(act, "gemm_skinny"), _tiled(w, rows, K, n_out=N), _tiled8(w, rows, K), _stream()), "gemm_skinny")
 
 
 def strip_rows_of(n_rows, qkv=None):
@@ -441,6 +441,27 @@ def tile_weight(w, qkv=None):
     t = wp.view(N // 16, 16, steps, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
     t.tiled_for = qkv
     return t
+
+
+def tile_weight8(w):
+    """A copy of ``w`` [N, K] (bfloat16, N % 8 == 0) in the order of the packed tiles that the products of
+    at most 8 rows use for strips of 8 weight rows: [strip of 8 rows][step of 64 k][lane][8 elements], lane
+    16 q + r holding row r % 8 at k = 32 (r // 8) + 8 q, k padded with zeros to whole steps."""
+    N, K = w.shape
+    if N % 8 or w.dtype != torch.bfloat16:
+        raise KernelError(f"tile_weight8: {tuple(w.shape)} {w.dtype}")
+    steps = -(-K // 64)
+    wp = torch.zeros(N, steps * 64, dtype=w.dtype, device=w.device)
+    wp[:, :K] = w
+    # [strip, row, step, half, q, element] -> [strip, step, q, half, row, element]
+    return wp.view(N // 8, 8, steps, 2, 4, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
+
+
+def _tiled8(w, n_rows, K):
+    t = getattr(w, "tiled8", None)
+    if t is None or n_rows % 8 or t.numel() != n_rows * -(-K // 64) * 64:
+        return c_void_p(0)
+    return _ptr(t)
 
 
 def _tiled(w, n_rows, K, qkv=None, n_out=None):

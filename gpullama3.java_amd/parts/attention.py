@@ -59,7 +59,7 @@ class GQAAttention:
         self.w_q = self.w_qkv[:qn]
         ops.for_few_rows(self.w_qkv, (self.H, self.Kh, self.hs, self.position is not None,
                                       bool(self.position is not None and self.position.adjacent)))
-        self.w_o = weights[n["o"]]
+        self.w_o = ops.for_eight_rows(weights[n["o"]])
         if self.biased:     # the epilogues read biases as float
             self.b_qkv = torch.cat([weights[n[k]].float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()
         if "o_bias" in n:

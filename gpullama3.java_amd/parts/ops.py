@@ -33,6 +33,15 @@ def for_few_rows(w, qkv=None):
     return w
 
 
+def for_eight_rows(w):
+    """The same for a weight of a product into the residual stream (output and down projection), which
+    steps of at most 8 rows take in strips of 8 weight rows with packed tiles (``lib.tile_weight8``)."""
+    if ("tiled" not in disabled and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 8 == 0
+            and w.is_contiguous()):
+        w.tiled8 = K.tile_weight8(w)
+    return w
+
+
 class Normed:
     """The RMSNorm of (rows of) the float residual stream, not computed yet.
 

@@ -1057,3 +1057,35 @@ def test_qkv_rope_cache_reads_a_weight_copy_in_operand_order(pairing, H, Kh, hs)
                        dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
                        pairing == "adjacent", page)
     assert torch.equal(q2, got[False][0])
+
+
+@pytest.mark.parametrize("N, Kd", [(2048, 2048), (2048, 8192), (40, 72), (136, 1544), (3072, 200)])
+@pytest.mark.parametrize("M", [1, 5, 8])
+def test_strips_of_eight_rows_read_a_weight_copy_in_their_tiles_order(M, N, Kd):
+    """``tile_weight8``: [strip of 8 rows][step of 64 k][lane][8], lane 16 q + r holding row r % 8 at
+    k = 32 (r // 8) + 8 q. The products of at most 8 rows into the residual stream read it; same sums."""
+    rng = np.random.default_rng(M + N + Kd)
+    lib = K()
+    wn = rounded(rng.standard_normal((N, Kd)) / math.sqrt(Kd), "bfloat16")
+    w = dev(wn, torch.bfloat16)
+    t = lib.tile_weight8(w)
+    steps = -(-Kd // 64)
+    flat = t.reshape(-1).float().cpu().numpy()
+    for (n, k) in [(0, 0), (17, 9), (N - 1, Kd - 1), (5, Kd // 2), (31, 40 % Kd), (12, 63 % Kd)]:
+        strip, row, step, half, q, e = n // 8, n % 8, k // 64, (k % 64) // 32, (k % 32) // 8, k % 8
+        assert flat[((strip * steps + step) * 64 + q * 16 + half * 8 + row) * 8 + e] == wn[n, k]
+    a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
+    res0 = rng.standard_normal((M, N)).astype(np.float32)
+    got = {}
+    for tiled in (False, True):
+        if tiled:
+            w.tiled8 = t
+        x = dev(res0)
+        ssq = torch.zeros(N // 8, 64, device=DEV)
+        lib.gemm_skinny(a, w, x, lib.EPI_ADD, strip_rows=8, ssq_out=ssq if N % 16 == 0 else None)
+        s_ = torch.zeros(M, N, device=DEV)
+        lib.gemm_skinny(a, w, s_, lib.EPI_STORE, strip_rows=8)
+        got[tiled] = (x, ssq, s_)
+    for u, v in zip(got[False], got[True]):
+        assert torch.equal(u, v)
+    np.testing.assert_allclose(got[True][2].cpu().numpy(), P.linear(a.float().cpu().numpy(), wn), atol=2e-5 * Kd)
