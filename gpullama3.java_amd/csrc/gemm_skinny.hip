@@ -391,14 +391,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   } else {
   // a wave takes pairs of neighbouring k-steps (the two halves of one 128-byte line of a row of W):
   // pair wave, wave + NW, ...
+  // (strips of 16 rows: Wt8, may be null, is W as [strip][k-step of 32][lane][8], the operands' own order,
+  // k padded with zeros to whole steps; gated: the up strips follow the N / 16 gate strips)
+  const bool tiled = ROWS == 16 && Wt8 != nullptr;
+  const bf16_t* wbase = tiled ? Wt8 + ((long)strip * steps * 64 + lane) * 8 : wrow;
+  const bf16_t* ubase = tiled ? wbase + (long)(N / 16) * steps * 512 : urow;
+  const long w_step = tiled ? 512 : 32;
   for (int p0 = wave; 2 * p0 < steps; p0 += NW * (UNROLL / 2)) {
     bf16x8 wf[UNROLL], uf[UNROLL], xf[UNROLL][MT];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int k = (2 * (p0 + NW * (u / 2)) + (u & 1)) * 32;
+      const int st = 2 * (p0 + NW * (u / 2)) + (u & 1), k = st * 32;
       const bool ok = k + q * 8 < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
-      wf[u] = (ok && r < ROWS) ? *(const bf16x8*)(wrow + k) : zero;   // rows of the tile beyond the strip stay zero
-      if (EPI == SK_GATED) uf[u] = ok ? *(const bf16x8*)(urow + k) : zero;
+      const bool w_ok = tiled ? st < steps : ok;
+      wf[u] = (w_ok && r < ROWS) ? *(const bf16x8*)(wbase + st * w_step) : zero;   // rows of the tile beyond the strip stay zero
+      if (EPI == SK_GATED) uf[u] = w_ok ? *(const bf16x8*)(ubase + st * w_step) : zero;
       sk_load_x<MT, XNORM>(xf[u], xrow, k + q * 8, ok, nrm);
     }
     __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
@@ -796,7 +803,7 @@ static int launch_skinny(int nw, const SkCall& a) {
 #define GO(NW)                                                                                                    \
   gemm_skinny_kernel<MT, NW, EPI, TC, XNORM, SSQ><<<grid, dim3(NW * 64), 0, a.stream>>>(                          \
       a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp,          \
-      (const bf16_t*)nullptr)
+      (const bf16_t*)a.Wt)
   if constexpr (NG * MT <= 2) {
     if (nw >= 16) { GO(16); GL3_LAUNCH_CHECK(); return 0; }
   }

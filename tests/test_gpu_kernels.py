@@ -1003,13 +1003,16 @@ def test_products_read_a_weight_copy_in_operand_order(M, N, Kd):
     for tiled in (False, True):
         if tiled:
             w.tiled = t
-        g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
-        lib.gemm_skinny_norm(xg, ssq, 5, 1e-5, w, g_, lib.EPI_GATED)
-        s_ = torch.zeros(M, 2 * N, device=DEV)
-        lib.gemm_skinny_norm(xg, ssq, 5, 1e-5, w, s_, lib.EPI_STORE)
-        p_ = torch.zeros(M, 2 * N, device=DEV)
-        lib.gemm_skinny(a, w, p_, lib.EPI_STORE)
-        res[tiled] = (g_, s_, p_)
+        outs = []
+        for waves in (0, 8, 16):            # the library's choice; the kernels that stream the rows of A, 8 and 16 waves
+            g_ = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+            lib.gemm_skinny_norm(xg, ssq, 5, 1e-5, w, g_, lib.EPI_GATED, waves=waves)
+            s_ = torch.zeros(M, 2 * N, device=DEV)
+            lib.gemm_skinny_norm(xg, ssq, 5, 1e-5, w, s_, lib.EPI_STORE, waves=waves)
+            p_ = torch.zeros(M, 2 * N, device=DEV)
+            lib.gemm_skinny(a, w, p_, lib.EPI_STORE, waves=waves)
+            outs += [g_, s_, p_]
+        res[tiled] = tuple(outs)
     for u, v in zip(res[False], res[True]):
         assert torch.equal(u, v)
     np.testing.assert_allclose(res[True][2].cpu().numpy(), P.linear(rounded(x, "bfloat16"), wn),
