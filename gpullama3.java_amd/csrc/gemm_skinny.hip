@@ -62,7 +62,17 @@ struct SkNext {
   long ld;
   const float* bias;      // [N] (gated: [2N]) float; null: none
   int act;
+  int pack_out;           // (store and gated epilogues, at most 8 rows) the rows go out in the packed tiles' order, see sk_packed_offset
 };
+
+// Where element k of row m (< 8) of a step lies when the step's rows are kept in the order in which the
+// products of at most 8 rows with packed tiles read them: [step of 64 k][lane 16 q + r][8 elements], lane
+// (r, q) holding row r % 8 at k = 32 (r / 8) + 8 q. Such a product then reads 1 KB of consecutive memory
+// per instruction, where rows one after the other put every lane on a line of its own; with a long K
+// (the down projection) every block reads as many bytes of the step's rows as of its weights.
+__device__ __forceinline__ long sk_packed_offset(int m, int k) {
+  return ((long)(((k >> 6) << 6) + (((k >> 3) & 3) << 4) + (((k >> 5) & 1) << 3) + m) << 3) + (k & 7);
+}
 
 struct SkRope {
   const int* positions;
@@ -300,7 +310,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
       continue;
     }
     const int n = n0 + 4 * q;
-    TC* cp = C + (long)m * ldc + n;
+    TC* cp = (EPI != SK_ADD && nx.pack_out) ? C + sk_packed_offset(m & 7, n) : C + (long)m * ldc + n;
     float sq = 0.f;
     if (m_ok && 4 * q < ROWS) {
 #pragma unroll
@@ -331,7 +341,7 @@ template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ, int ROWS =
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __restrict__ Av, const bf16_t* __restrict__ W,
                                                               TC* __restrict__ C, int M, int N, int K, long lda,
                                                               long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out,
-                                                              SkNext nx, SkRope rp, const bf16_t* __restrict__ Wt8) {
+                                                              SkNext nx, SkRope rp, const bf16_t* __restrict__ Wt8, int a_packed) {
   static_assert(!PACK || (ROWS == 8 && MT == 1 && EPI != SK_GATED && EPI != SK_QKV && !XNORM), "packed strips: 8 rows, one tile");
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   constexpr int UNROLL = 8;
@@ -377,7 +387,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
         const int p = p0 + NW * u, k = p * 64;
         const bool ok = k + koff < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
         wf[u] = (Wt8 ? p < steps64 : ok) ? *(const bf16x8*)(wbase + p * w_step) : zero;
-        sk_load_x<MT, XNORM>(xf[u], xrow, k + koff, ok, nrm);
+        if (a_packed)   // the rows in the packed tiles' order (sk_packed_offset): this lane's 16 bytes of step p
+          xf[u][0] = (ok && xrow[0] != nullptr) ? *(const bf16x8*)((const bf16_t*)Av + ((long)p * 64 + lane) * 8) : zero;
+        else
+          sk_load_x<MT, XNORM>(xf[u], xrow, k + koff, ok, nrm);
       }
       __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
 #pragma unroll
@@ -735,6 +748,7 @@ struct SkCall {
   SkNext nx = SkNext{};
   const void* Wt = nullptr;   // W in the operands' order (the resident kernel reads it where it is given)
   const void* Wt8 = nullptr;  // W in the order of the packed tiles of strips of 8 rows
+  int a_packed = 0;           // the rows of A lie in the packed tiles' order (strips of 8 rows, M <= 8 only)
 };
 
 // Blocks of the resident kernel: every strip its own block while that still leaves CUs idle, else
@@ -766,11 +780,11 @@ static int launch_skinny(int nw, const SkCall& a) {
       if (a.M <= 8)
         gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8, true><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
             a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp,
-            (const bf16_t*)a.Wt8);
+            (const bf16_t*)a.Wt8, a.a_packed);
       else
         gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
             a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp,
-            (const bf16_t*)nullptr);
+            (const bf16_t*)nullptr, 0);
       GL3_LAUNCH_CHECK();
       return 0;
     }
@@ -803,7 +817,7 @@ static int launch_skinny(int nw, const SkCall& a) {
 #define GO(NW)                                                                                                    \
   gemm_skinny_kernel<MT, NW, EPI, TC, XNORM, SSQ><<<grid, dim3(NW * 64), 0, a.stream>>>(                          \
       a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp,          \
-      (const bf16_t*)a.Wt)
+      (const bf16_t*)a.Wt, 0)
   if constexpr (NG * MT <= 2) {
     if (nw >= 16) { GO(16); GL3_LAUNCH_CHECK(); return 0; }
   }
@@ -862,10 +876,12 @@ static int check_common(const char* who, const void* A, const void* W, const voi
 // kernels that keep their rows of A in registers read W there.
 // w_tiled8 (may be null; N % 8 == 0): W as [strip of 8 rows][step of 64 k][lane][8 elements], lane (r, q)
 // holding row r % 8 at k = 32 (r / 8) + 8 q: the order of the packed tiles of strips of 8 rows (M <= 8).
+// a_packed (strip_rows 8, M <= 8): A is not [M][lda] but the step's rows in that same order, [ceil(K / 64)][64][8],
+// as a product with `pack_out` leaves them.
 extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                long ldw, long ldc, int epilogue, int waves, float* ssq_out, int strip_rows,
                                const float* next_weight, void* xg, long ldxg, const float* bias, int act,
-                               const void* w_tiled, const void* w_tiled8, hipStream_t stream) {
+                               const void* w_tiled, const void* w_tiled8, int a_packed, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny", A, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny: ldc too small");
@@ -879,11 +895,14 @@ extern "C" int gl3_gemm_skinny(const void* A, const void* W, void* C, int c_dtyp
               "gl3_gemm_skinny: the next norm's weight and its rows come together, with the sums of squares");
   SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, ssq_out, SkRope{}, stream, waves == 0, strip_rows};
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny: unknown activation %d", act);
-  a.nx = SkNext{next_weight, (bf16_t*)xg, ldxg, bias, act};
+  a.nx = SkNext{next_weight, (bf16_t*)xg, ldxg, bias, act, 0};
   GL3_REQUIRE(!w_tiled || (N % 16 == 0 && (uintptr_t)w_tiled % 16 == 0), "gl3_gemm_skinny: a copy of W in the operands' order needs N %% 16 == 0");
   a.Wt = w_tiled;
   GL3_REQUIRE(!w_tiled8 || (N % 8 == 0 && (uintptr_t)w_tiled8 % 16 == 0), "gl3_gemm_skinny: a copy of W in the packed tiles' order needs N %% 8 == 0");
   a.Wt8 = w_tiled8;
+  GL3_REQUIRE(!a_packed || (strip_rows == 8 && M <= 8 && waves == 0 && epilogue != SK_GATED),
+              "gl3_gemm_skinny: rows in the packed tiles' order are read by the strips of 8 rows with at most 8 rows of A");
+  a.a_packed = a_packed;
   const int nw = pick_waves(waves, N, K);
   if (c_dtype == GL3_F32) {
     if (epilogue == SK_STORE) return pick_mt<SK_STORE, float, false, false>(nw, a);
@@ -960,7 +979,7 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_skinny_wide: a bias goes with one slice of K");
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny_wide: unknown activation %d", act);
   SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, nullptr, SkRope{}, stream, false};
-  a.nx = SkNext{nullptr, nullptr, 0, bias, act};
+  a.nx = SkNext{nullptr, nullptr, 0, bias, act, 0};
   if (c_dtype == GL3_F32) {
     if (epilogue == SK_STORE) return pick_wide<SK_STORE, float>(a, strips_per_block, slices, slice_stride);
     if (epilogue == SK_ADD) return pick_wide<SK_ADD, float>(a, strips_per_block, slices, slice_stride);
@@ -977,19 +996,23 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
 // most 64 rows); `rows` (may be null) picks the rows of x that the product's rows read.
 // Epilogues: store (float or bfloat16) and gated (bfloat16).
 // bias (may be null): N floats (gated: 2N), added after the 1/rms; act: the gated epilogue's activation.
+// pack_out (M <= 8, bfloat16): C is not [M][ldc] but the rows in the packed tiles' order (sk_packed_offset),
+// [ceil(N / 64)][64][8], for a product of strips of 8 rows to read with `a_packed`.
 extern "C" int gl3_gemm_skinny_norm(const void* xg, const int* rows, const float* ssq, int n_partials, float eps,
                                     const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
                                     long ldc, int epilogue, int waves, const float* bias, int act, const void* w_tiled,
-                                    hipStream_t stream) {
+                                    int pack_out, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_norm", xg, W, C, M, N, K, lda, ldw, waves)) return -1;
   GL3_REQUIRE(ssq && n_partials > 0, "gl3_gemm_skinny_norm: norm arguments missing");
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny_norm: ldc too small");
   GL3_REQUIRE(epilogue == SK_STORE || epilogue == SK_GATED, "gl3_gemm_skinny_norm: epilogue %d", epilogue);
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny_norm: unknown activation %d", act);
+  GL3_REQUIRE(!pack_out || (M <= 8 && c_dtype == GL3_BF16),
+              "gl3_gemm_skinny_norm: the packed tiles' order holds at most 8 rows of bfloat16 (C then has 8 * 64 * ceil(N / 64) elements)");
   const SkNorm nrm = {ssq, n_partials, eps, rows};
   SkCall a = {xg, W, C, M, N, K, lda, ldw, ldc, nrm, nullptr, SkRope{}, stream, waves == 0};
-  a.nx = SkNext{nullptr, nullptr, 0, bias, act};
+  a.nx = SkNext{nullptr, nullptr, 0, bias, act, pack_out};
   GL3_REQUIRE(!w_tiled || (N % 16 == 0 && (uintptr_t)w_tiled % 16 == 0), "gl3_gemm_skinny_norm: a copy of W in the operands' order needs N %% 16 == 0");
   a.Wt = w_tiled;
   const int nw = pick_waves(waves, N, K);

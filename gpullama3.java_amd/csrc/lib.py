@@ -60,9 +60,9 @@ def _declare(lib):
         "gl3_argmax": [P, L, P, P, I, I, P],
         "gl3_argmax_static": [P, L, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
-        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P, P],
+        "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P, I, P],
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P],
-        "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P],
+        "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, I, P],
         "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P],
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, P],
         "gl3_attention_decode_supports": [I, I],
@@ -380,13 +380,25 @@ def skinny_strip_rows(M, N, K, epilogue):
     return 8 if M <= 8 or (M <= 16 and K > 4096) else 16
 
 
+def packed_rows(n_columns, dtype, device):
+    """A buffer for at most 8 rows of ``n_columns`` elements in the order in which the products of strips of
+    8 weight rows read them: [step of 64 columns][lane 16 q + r][8 elements], lane (r, q) holding row r % 8 at
+    column 32 (r // 8) + 8 q. A product with ``pack_out`` writes it, one with ``a_packed`` reads it."""
+    return torch.empty((-(-n_columns // 64), 64, 8), dtype=dtype, device=device)
+
+
 def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows=16, next_weight=None, xg=None,
-                bias=None, act="silu"):
+                bias=None, act="silu", a_packed=False):
     """out (=, +=, gated) a @ w.T on the matrix cores for at most 64 rows of ``a``. ``ssq_out``
     [N/strip_rows, 64] float32 (add epilogue): partial sums of squares of the completed rows; with it
     ``xg`` [M, N] bfloat16 may receive ``next_weight * out``, the rows as the product after the next
-    norm reads them."""
+    norm reads them. ``a_packed`` (strips of 8 rows, at most 8 rows): ``a`` is a ``packed_rows`` buffer."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
+    if a_packed:
+        if (w.dim() != 2 or out.dim() != 2 or out.stride(1) != 1 or not a.is_contiguous()
+                or a.numel() < -(-w.shape[1] // 64) * 512 or out.shape[0] > 8 or strip_rows != 8 or waves):
+            raise KernelError("gemm_skinny: rows in the packed order go with strips of 8 weight rows and at most 8 rows")
+        a = a.view(-1)[:8 * w.shape[1]].view(8, w.shape[1])[:out.shape[0]]     # (the shape only: the kernel knows the order)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2 or a.stride(1) != 1 or out.stride(1) != 1:
         raise KernelError("gemm: operands must be 2-d with a contiguous last dimension")
     M, K = a.shape
@@ -404,7 +416,8 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows
     _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                      out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _ptr(next_weight),
                                      _ptr(xg), xg.stride(0) if xg is not None else 0, _bias(bias, rows, "gemm_skinny"),
-                                     _act(act, "gemm_skinny"), _tiled(w, rows, K, n_out=N), _tiled8(w, rows, K), _stream()), "gemm_skinny")
+                                     _act(act, "gemm_skinny"), _tiled(w, rows, K, n_out=N), _tiled8(w, rows, K), int(bool(a_packed)),
+                                     _stream()), "gemm_skinny")
 
 
 def strip_rows_of(n_rows, qkv=None):
@@ -520,9 +533,11 @@ def gemm_skinny_norm_fits(xg, w, out, epilogue):
                  or (epilogue == EPI_GATED and out.dtype == torch.bfloat16)))
 
 
-def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=None, waves=0, bias=None, act="silu"):
+def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=None, waves=0, bias=None, act="silu",
+                     pack_out=False):
     """out (=, gated) RMSNorm(x)[rows] @ w.T, where ``xg`` = bfloat16(norm weight * x) was left by the
-    kernel that completed the rows of x, together with their sums of squares as partial sums."""
+    kernel that completed the rows of x, together with their sums of squares as partial sums.
+    ``pack_out`` (at most 8 rows, bfloat16): ``out`` is a ``packed_rows`` buffer."""
     _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
     K = w.shape[1]
     _check_norm_args(xg, ssq, n_partials, K)
@@ -530,6 +545,11 @@ def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=
     if rows is not None:
         _dev(rows, "rows", torch.int32)
         M = rows.numel()
+    if pack_out:
+        n_out = w.shape[0] // 2 if epilogue == EPI_GATED else w.shape[0]
+        if M > 8 or out.dtype != torch.bfloat16 or not out.is_contiguous() or out.numel() < -(-n_out // 64) * 512:
+            raise KernelError("gemm_skinny_norm: the packed order holds at most 8 rows of bfloat16")
+        out = out.view(-1)[:8 * n_out].view(8, n_out)[:M]                      # (the shape only: the kernel knows the order)
     N = out.shape[1]
     wrows = 2 * N if epilogue == EPI_GATED else N
     if w.shape != (wrows, K) or out.shape[0] != M or out.stride(1) != 1 or M > 64:
@@ -537,7 +557,7 @@ def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=
     _check(library().gl3_gemm_skinny_norm(
         _ptr(xg), _ptr(rows), _ptr(ssq), n_partials, float(eps), _ptr(w), _ptr(out), _code(out, "out"), M, N, K,
         xg.stride(0), w.stride(0), out.stride(0), epilogue, waves, _bias(bias, wrows, "gemm_skinny_norm"),
-        _act(act, "gemm_skinny_norm"), _tiled(w, wrows, K, n_out=N), _stream()), "gemm_skinny_norm")
+        _act(act, "gemm_skinny_norm"), _tiled(w, wrows, K, n_out=N), int(bool(pack_out)), _stream()), "gemm_skinny_norm")
 
 
 def qkv_rope_cache_fits(a, w_qkv, head_dim, rot_dim):

@@ -51,6 +51,11 @@ class GatedFeedForward:
             self.b_down = weights[n["down_bias"]].float().contiguous()
 
     def forward(self, ctx, h, x):
+        if self.b_gate_up is None and self.b_down is None and ops.packs_rows(ctx, h, self.w_gate_up, self.w_down, x):
+            act = ctx.buffer("ffn_act_packed", (-(-self.F // 64), 64, 8), self.dtype)
+            ops.linear(h, self.w_gate_up, act, ops.EPI_GATED, ctx, act=self.act, pack_out=True)
+            ops.linear(act, self.w_down, x, ops.EPI_ADD, ctx, a_packed=True)
+            return
         act = ctx.buffer("ffn_act", (h.shape[0], self.F), self.dtype)
         ops.linear(h, self.w_gate_up, act, ops.EPI_GATED, ctx, bias=self.b_gate_up, act=self.act)
         ops.linear(act, self.w_down, x, ops.EPI_ADD, ctx, bias=self.b_down)

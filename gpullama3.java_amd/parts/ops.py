@@ -124,10 +124,47 @@ def _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias=None, act="silu"):
     ctx.pending = (out.data_ptr(), part)
 
 
-def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu"):
+class _BF16_OUT:      # what the check of a product's output looks at
+    dtype = torch.bfloat16
+
+
+def packs_rows(ctx, h, w_first, w_second, x):
+    """Whether a gated product of ``h`` and the product of its result into the residual rows ``x`` can hand
+    the result over in the packed order (``lib.packed_rows``): a folded norm in front, at most 8 rows, the
+    second product in strips of 8 weight rows. Every block of that product reads all of the step's rows;
+    with a long K they are as many bytes as its weights, and in the packed order a CU's first-level
+    cache takes them in a third of the time."""
+    M = h.shape[0]
+    F = w_second.shape[1]
+    return (isinstance(h, Normed) and M <= 8 and not disabled & {"packed", "fused", "skinny"}
+            and w_first.dtype == torch.bfloat16 and w_second.dtype == torch.bfloat16 and x.dtype == torch.float32
+            and w_first.shape[0] == 2 * F and F % 8 == 0 and w_second.stride(0) % 8 == 0 and w_second.data_ptr() % 16 == 0
+            and K.gemm_skinny_norm_fits(h.xg, w_first, _BF16_OUT, EPI_GATED)
+            and K.skinny_strip_rows(M, x.shape[1], F, EPI_ADD) == 8)
+
+
+def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_out=False, a_packed=False):
     """out (=, +=, gated) a @ w.T. ``a`` may be a ``Normed``. With the add epilogue ``out`` is the
     residual stream. ``bias`` (float32, one per row of ``w``) is added to the sums before the
-    epilogue's own rule; ``act`` is the gated epilogue's activation (``lib.ACTIVATIONS``)."""
+    epilogue's own rule; ``act`` is the gated epilogue's activation (``lib.ACTIVATIONS``).
+    ``pack_out`` / ``a_packed``: ``out`` / ``a`` is a ``lib.packed_rows`` buffer (where ``packs_rows`` said so)."""
+    if pack_out:
+        return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act,
+                                  pack_out=True)
+    if a_packed:
+        M, N = out.shape
+        if (epilogue == EPI_ADD and ctx is not None and getattr(ctx, "fuse", False) and N % 16 == 0
+                and "fused" not in disabled and M == ctx.n_tokens <= FUSE_ROWS):
+            norm, xg = _next_norm(ctx, N)
+            if norm is not None:
+                ssq = ctx.ssq_buffer(N // 8)
+                K.gemm_skinny(a, w, out, epilogue, ssq_out=ssq, strip_rows=8, next_weight=norm.weight_f32, xg=xg, bias=bias,
+                              a_packed=True)
+                return residual_written(ctx, out, ssq, N // 8, xg, norm)
+        K.gemm_skinny(a, w, out, epilogue, strip_rows=8, bias=bias, a_packed=True)
+        if epilogue == EPI_ADD:
+            residual_written(ctx, out)
+        return
     if isinstance(a, Normed):
         if ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
                 and a.xg.shape[0] <= 64):

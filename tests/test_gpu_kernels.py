@@ -1092,3 +1092,37 @@ def test_strips_of_eight_rows_read_a_weight_copy_in_their_tiles_order(M, N, Kd):
     for u, v in zip(got[False], got[True]):
         assert torch.equal(u, v)
     np.testing.assert_allclose(got[True][2].cpu().numpy(), P.linear(a.float().cpu().numpy(), wn), atol=2e-5 * Kd)
+
+
+@pytest.mark.parametrize("d, F", [(2048, 8192), (64, 200), (136, 72), (96, 1544)])
+@pytest.mark.parametrize("M", [1, 5, 8])
+def test_rows_handed_over_in_the_packed_order(M, d, F):
+    """A gated product that leaves its rows in the order of the packed tiles (``pack_out``) and a product of
+    strips of 8 weight rows that reads them there (``a_packed``) give what the two give through plain rows."""
+    rng = np.random.default_rng(M + d + F)
+    lib = K()
+    x = (rng.standard_normal((M, d)) * 2).astype(np.float32)
+    nw = rounded(1 + 0.2 * rng.standard_normal(d), "bfloat16")
+    w1 = dev(rounded(rng.standard_normal((2 * F, d)) / math.sqrt(d), "bfloat16"), torch.bfloat16)
+    w2 = dev(rounded(rng.standard_normal((d, F)) / math.sqrt(F), "bfloat16"), torch.bfloat16)
+    xg, ssq = times_weight(x, nw).to(DEV), dev(ssq_partials(x, 4))
+    res0 = rng.standard_normal((M, d)).astype(np.float32)
+    act = torch.zeros(M, F, device=DEV, dtype=torch.bfloat16)
+    lib.gemm_skinny_norm(xg, ssq, 4, 1e-5, w1, act, lib.EPI_GATED)
+    plain = dev(res0)
+    lib.gemm_skinny(act, w2, plain, lib.EPI_ADD, strip_rows=8)
+    packed = lib.packed_rows(F, torch.bfloat16, DEV)
+    packed.fill_(777.0)                                                      # what is not written is not read
+    lib.gemm_skinny_norm(xg, ssq, 4, 1e-5, w1, packed, lib.EPI_GATED, pack_out=True)
+    flat = packed.reshape(-1).float().cpu().numpy()
+    an = act.float().cpu().numpy()
+    for (m, k) in [(0, 0), (M - 1, F - 1), (M // 2, F // 2), (0, 37 % F), (M - 1, 63 % F)]:
+        assert flat[(((k // 64) * 64 + ((k % 32) // 8) * 16 + ((k % 64) // 32) * 8 + m) * 8) + k % 8] == an[m, k]
+    for tiled in (False, True):
+        if tiled:
+            w2.tiled8 = lib.tile_weight8(w2)
+        got = dev(res0)
+        lib.gemm_skinny(packed, w2, got, lib.EPI_ADD, strip_rows=8, a_packed=True)
+        assert torch.equal(got, plain)
+    with pytest.raises(lib.KernelError):
+        lib.gemm_skinny(packed, w2, dev(res0), lib.EPI_ADD, strip_rows=16, a_packed=True)
