@@ -34,10 +34,12 @@ def for_few_rows(w, qkv=None):
 
 
 def for_eight_rows(w):
-    """The same for a weight of a product into the residual stream (output and down projection), which
-    steps of at most 8 rows take in strips of 8 weight rows with packed tiles (``lib.tile_weight8``)."""
+    """The same for a weight of a product into the residual stream (output and down projection): steps of
+    at most 8 rows take it in strips of 8 weight rows with packed tiles where 16-row strips would leave CUs
+    idle (``lib.skinny_strip_rows``, ``lib.tile_weight8``), everything else of few rows in strips of 16."""
+    for_few_rows(w)
     if ("tiled" not in disabled and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 8 == 0
-            and w.is_contiguous()):
+            and w.is_contiguous() and K.skinny_strip_rows(8, w.shape[0], w.shape[1], EPI_ADD) == 8):
         w.tiled8 = K.tile_weight8(w)
     return w
 
