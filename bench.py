@@ -99,6 +99,8 @@ def main():
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma-separated")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", default="decode", choices=["decode", "unequal8"])
+    ap.add_argument("--without", default="", help="names of fast paths to switch off for a comparison on the same machine, "
+                    "comma-separated (parts/ops.py: tiled, packed, fused, wide, ...); the line then says so in `config`")
     args = ap.parse_args()
     if args.workload == "unequal8" and "--shape" not in " ".join(sys.argv):
         args.shape = "3b"
@@ -112,6 +114,8 @@ def main():
     import torch
     import gpullama3_java_amd as g
     from gpullama3_java_amd.engine import Engine
+    from gpullama3_java_amd.parts import ops
+    ops.disabled.update(n for n in args.without.split(",") if n)
 
     shape_name, shape = SHAPES[args.shape]
     context = shape["max_position_embeddings"]
@@ -213,7 +217,7 @@ def main():
             "vocab_size": cfg.vocab_size, "tied_head": cfg.tie_word_embeddings, "rope_theta": cfg.rope_theta,
             "rope_scaling_factor": cfg.rope_scaling.factor, "rms_norm_eps": cfg.rms_norm_eps,
             "global_batch": args.batch, "seq_len": context, "prompt_len": prompt_len, "prefill_len": prefill_len,
-            "parallelism": "single GPU", "sampling": "greedy on device",
+            "parallelism": "single GPU", "sampling": "greedy on device", **({"without": args.without} if args.without else {}),
         },
         "prefill": {"value": round(prefill_len / prefill_s, 1), "tokens": prefill_len, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / (PEAK_TFLOPS[short] * 1e12), 4)},
@@ -281,7 +285,7 @@ def unequal8(args, eng, cfg, rng, shape_name, shape, esize, short, sync):
             "vocab_size": cfg.vocab_size, "tied_head": cfg.tie_word_embeddings, "global_batch": 8,
             "seq_len": shape["max_position_embeddings"], "prompt_len_min": min(lens), "prompt_len_max": max(lens),
             "prompt_tokens": T, "mean_context": round(sum(kv) / 8 + (K + 1) / 2, 1), "new_tokens": K,
-            "parallelism": "single GPU", "sampling": "greedy on device",
+            "parallelism": "single GPU", "sampling": "greedy on device", **({"without": args.without} if args.without else {}),
         },
         "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(flops / prefill_s / (PEAK_TFLOPS[short] * 1e12), 4)},
