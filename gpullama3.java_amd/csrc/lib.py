@@ -380,6 +380,14 @@ def skinny_strip_rows(M, N, K, epilogue):
     return 8 if M <= 8 or (M <= 16 and K > 4096) else 16
 
 
+def skinny_keeps_operands(M, K):
+    """Whether the skinny product (store epilogue, no folded norm) of ``M`` rows over ``K`` columns runs on
+    the kernel whose waves keep their operands of ``a`` in registers: with 33 to 64 rows that is K up to
+    2,048, with fewer rows up to 4,096. Beyond it the kernel that streams the rows of ``a`` for every strip
+    runs, which a product of very many strips should leave to the tiled kernel."""
+    return K <= (2048 if M > 16 else 4096)
+
+
 def packed_rows(n_columns, dtype, device):
     """A buffer for at most 8 rows of ``n_columns`` elements in the order in which the products of strips of
     8 weight rows read them: [step of 64 columns][lane 16 q + r][8 elements], lane (r, q) holding row r % 8 at

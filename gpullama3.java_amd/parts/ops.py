@@ -169,7 +169,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
         return
     if isinstance(a, Normed):
         if ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
-                and a.xg.shape[0] <= 64):
+                and a.xg.shape[0] <= 64 and not _streams_rows_for_many_strips(out.shape[0], w, epilogue)):
             return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act)
         a = a.materialize()
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
@@ -178,6 +178,9 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
                 and K.gemm_skinny_fits(a[:1], w, out[:1], epilogue)
                 and not (epilogue == EPI_STORE and out.shape[1] >= 128 * 512)):     # (the head: the tiled kernel)
             return _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias, act)
+        if (_streams_rows_for_many_strips(a.shape[0], w, epilogue) and "mfma" not in disabled
+                and K.gemm_mfma_fits(a, w, out, epilogue)):
+            return K.gemm_mfma(a, w, out, epilogue, bias=bias)
         if ("wide" not in disabled and K.gemm_skinny_wide_fits(a, w, out, epilogue)
                 and _linear_wide(a, w, out, epilogue, ctx, bias, act)):
             return
@@ -216,6 +219,15 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
     K.gemm_generic(a, w, out, epilogue, bias=bias, act=act)
     if epilogue == EPI_ADD:
         residual_written(ctx, out)
+
+
+def _streams_rows_for_many_strips(M, w, epilogue):
+    """A head of more than 16 rows over a K beyond what the skinny kernel keeps in registers: that kernel
+    would read the rows of ``a`` again for each of thousands of strips, and the tiled kernel, whose blocks
+    share them, is the faster one (N = 128,256, K = 4,096: 32 rows 354 against 292 us, 64 rows 595 against
+    273 us; K = 3,072: 32 rows 276 against 198 us)."""
+    return (epilogue == EPI_STORE and w.shape[0] >= 128 * 512 and M > 16
+            and not K.skinny_keeps_operands(M, w.shape[1]))
 
 
 def _linear_wide(a, w, out, epilogue, ctx, bias=None, act="silu"):
