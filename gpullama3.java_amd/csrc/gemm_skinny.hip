@@ -36,7 +36,7 @@
 // registers and the block walks over several strips with them, asking for the next strip's
 // rows of W before it finishes the current strip; then the first-level cache carries W and
 // nothing else, which is what limits the streaming kernel when the same A is read for every
-// strip. The wide one, for 33 to 64 rows, takes several strips at once (see there).
+// strip. The wide one, for 17 to 64 rows, takes several strips at once (see there).
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -571,8 +571,8 @@ __device__ __forceinline__ bf16x8 sk_buffer_load(__amdgpu_buffer_rsrc_t buf, uns
   return __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(buf, byte_offset, 0, 0));
 }
 
-// The wide kernel, for steps of three or four token tiles: there a strip's share of A is as
-// large as the strip of W itself, and reading it again for every strip is what takes the time.
+// The wide kernel, for steps of two to four token tiles: there a strip's share of A is as
+// large as the strip of W itself (or larger), and reading it again for every strip is what takes the time.
 // A block works on NS strips at once (NS pairs of gate and up strips for the gated epilogue), so
 // that A is read once for all of them, and on one slice of K only (blockIdx.y), so that the
 // chip still has blocks enough. With more than one slice the epilogue is a plain store of the
@@ -940,6 +940,9 @@ template <int EPI, typename TC>
 static int pick_wide(const SkCall& a, int strips_per_block, int slices, long slice_stride) {
   constexpr int BIG = (EPI == SK_GATED) ? 2 : 4;   // a gated strip is a pair of strips
   const bool big = strips_per_block == BIG;
+  if ((a.M + 15) / 16 <= 2)
+    return big ? launch_wide<2, BIG, EPI, TC>(a, slices, slice_stride)
+               : launch_wide<2, BIG / 2, EPI, TC>(a, slices, slice_stride);
   if ((a.M + 15) / 16 <= 3)
     return big ? launch_wide<3, BIG, EPI, TC>(a, slices, slice_stride)
                : launch_wide<3, BIG / 2, EPI, TC>(a, slices, slice_stride);
@@ -954,7 +957,7 @@ static int wide_strips(int N, int slices, int epilogue) {
   return (n_strips / big) * slices >= 192 ? big : big / 2;
 }
 
-// The product for 33 to 64 rows of A (bfloat16). `slices` > 1 (store epilogue, float output only):
+// The product for 17 to 64 rows of A (bfloat16). `slices` > 1 (store epilogue, float output only):
 // K is cut into that many slices and C is [slices][M][ldc] with `slice_stride` elements between
 // slices; the caller adds them up. `strips_per_block`: 0 lets the library choose.
 // bias (may be null; one slice only): N floats (gated: 2N); act: the gated epilogue's activation.
@@ -963,7 +966,7 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
                                     int strips_per_block, const float* bias, int act, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_wide", A, W, C, M, N, K, lda, ldw, 0)) return -1;
-  GL3_REQUIRE(M > 32, "gl3_gemm_skinny_wide: M=%d; up to 32 rows are gl3_gemm_skinny's", M);
+  GL3_REQUIRE(M > 16, "gl3_gemm_skinny_wide: M=%d; up to 16 rows are gl3_gemm_skinny's", M);
   GL3_REQUIRE(wide_addressable(M, epilogue == SK_GATED ? 2L * N : N, K, lda, ldw),
               "gl3_gemm_skinny_wide: an operand of 2 GiB or more");
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny_wide: ldc too small");
@@ -1053,9 +1056,12 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
   SkCall a = {a_rows, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
   GL3_REQUIRE(!w_tiled || (uintptr_t)w_tiled % 16 == 0, "gl3_qkv_rope_cache: the copy of W must be 16-byte aligned");
   a.Wt = w_tiled;   // (its strips hold the rows that sk_strip_row names: for half-split pairing 8 rows and the 8 half a head further)
-  if (!ssq && waves == 0 && M > 32 && wide_addressable(M, N, K, lda, ldw)) {
+  if (!ssq && waves == 0 && M > 16 && wide_addressable(M, N, K, lda, ldw)) {
     // many rows: two strips a block, so that the rows are read half as often, in whole lines
-    return (M + 15) / 16 <= 3 ? launch_wide<3, 2, SK_QKV, bf16_t>(a, 1, 0) : launch_wide<4, 2, SK_QKV, bf16_t>(a, 1, 0);
+    const int tiles = (M + 15) / 16;
+    return tiles <= 2   ? launch_wide<2, 2, SK_QKV, bf16_t>(a, 1, 0)
+           : tiles == 3 ? launch_wide<3, 2, SK_QKV, bf16_t>(a, 1, 0)
+                        : launch_wide<4, 2, SK_QKV, bf16_t>(a, 1, 0);
   }
   if (!ssq) return pick_mt<SK_QKV, bf16_t, false, false>(pick_waves(waves, N, K), a);
   return pick_mt<SK_QKV, bf16_t, true, false>(pick_waves(waves, N, K), a);

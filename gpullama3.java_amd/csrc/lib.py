@@ -382,7 +382,7 @@ def skinny_strip_rows(M, N, K, epilogue):
 
 def skinny_keeps_operands(M, K):
     """Whether the skinny product (store epilogue, no folded norm) of ``M`` rows over ``K`` columns runs on
-    the kernel whose waves keep their operands of ``a`` in registers: with 33 to 64 rows that is K up to
+    the kernel whose waves keep their operands of ``a`` in registers: with 17 to 64 rows that is K up to
     2,048, with fewer rows up to 4,096. Beyond it the kernel that streams the rows of ``a`` for every strip
     runs, which a product of very many strips should leave to the tiled kernel."""
     return K <= (2048 if M > 16 else 4096)
@@ -496,7 +496,7 @@ def _tiled(w, n_rows, K, qkv=None, n_out=None):
 
 
 def gemm_skinny_wide_fits(a, w, out, epilogue):
-    return 32 < a.shape[0] <= 64 and gemm_skinny_fits(a, w, out, epilogue)
+    return 16 < a.shape[0] <= 64 and gemm_skinny_fits(a, w, out, epilogue)
 
 
 def wide_slices(N, K):
@@ -507,7 +507,7 @@ def wide_slices(N, K):
 
 
 def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="silu"):
-    """out (=, +=, gated) a @ w.T for 33 to 64 rows of ``a``. ``out`` with three axes [slices, M, N]
+    """out (=, +=, gated) a @ w.T for 17 to 64 rows of ``a``. ``out`` with three axes [slices, M, N]
     (float32, store epilogue) takes the sums of one slice of K each: the caller adds them up."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
     M, K = a.shape
@@ -517,7 +517,7 @@ def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="si
         slices, slice_stride, rows = out.shape[0], out.stride(0), out[0]
     N = rows.shape[1]
     wrows = 2 * N if epilogue == EPI_GATED else N
-    if (w.shape != (wrows, K) or rows.shape[0] != M or rows.stride(1) != 1 or a.stride(1) != 1 or not 32 < M <= 64):
+    if (w.shape != (wrows, K) or rows.shape[0] != M or rows.stride(1) != 1 or a.stride(1) != 1 or not 16 < M <= 64):
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_skinny_wide(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0),
                                           w.stride(0), rows.stride(0), epilogue, slices, slice_stride, strips,

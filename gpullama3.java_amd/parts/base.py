@@ -19,7 +19,7 @@ Block:        ``parts()`` and ``forward(ctx, x, run)``; owns the arrangement of 
               part in the folding of norms into products and is called with ``norm_after=``.
 
 The residual rows ``x`` between parts: parts only ADD to ``x`` (through ``ops.linear`` with the add
-epilogue, or with a kernel of their own followed by ``ops.residual_written``). After a product of 33
+epilogue, or with a kernel of their own followed by ``ops.residual_written``). After a product of 17
 or more rows the sums may still lie in slices that the next norm adds up, so whoever READS ``x``
 other than through a norm calls ``ops.settle_residual(ctx, x)`` first. A block without ``first_norm``
 is handed whole rows, and no product leaves slices or prepared rows while it runs

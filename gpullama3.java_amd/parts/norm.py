@@ -6,7 +6,8 @@ import torch
 from ..csrc import lib as K
 from ..weights.loader import TensorSpec
 from .base import register_part
-from .ops import FUSE_ROWS, Normed
+from . import ops
+from .ops import Normed
 
 
 
@@ -32,7 +33,7 @@ class RMSNorm:
         rows, and the kernel that last wrote exactly this tensor prepared the rows for this norm)."""
         rec = getattr(ctx, "ssq", None)
         if (getattr(ctx, "fuse", False) and rec is not None and rec[0] == x.data_ptr() and rec[4] is self
-                and x.shape[0] <= FUSE_ROWS and self.dtype == torch.bfloat16):
+                and x.shape[0] <= ops.FUSE_ROWS and self.dtype == torch.bfloat16):
             return Normed(ctx, x, self.weight, self.eps, self.dtype, rec[3], rec[1], rec[2], rows, name)
         n = x.shape[0] if rows is None else rows.numel()
         out = ctx.buffer(name, (n, self.dim), self.dtype)

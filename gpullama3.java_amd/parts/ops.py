@@ -12,9 +12,16 @@ from ..csrc import lib as K
 
 EPI_STORE, EPI_ADD, EPI_GATED = K.EPI_STORE, K.EPI_ADD, K.EPI_GATED
 
-# a norm is folded into the next product for steps of at most this many tokens (two token tiles);
-# larger steps take the kernels for 33 to 64 rows or the tiled ones, with a norm kernel of its own
-FUSE_ROWS = 32
+# a norm is folded into the next product for steps of at most this many tokens (one token tile); larger
+# steps take the kernels for 17 to 64 rows or the tiled ones, with a norm kernel of its own. (With 17 to 32
+# rows the folded products lose to those kernels: a block of the skinny kernel reads the step's rows again
+# for every strip of 16 weight rows. Decode steps of the 1B / 8B layers at batch 32: 0.474 -> 0.386 ms and
+# 1.008 -> 0.814 ms for four layers and the head.)
+FUSE_ROWS = 16
+# a decode step of up to this many rows is worked on in pieces of at most 64 rows; from 129 rows on the
+# tiled kernel's two row tiles are faster than three pieces (8B layers, 192 rows: 2.03 -> 1.69 ms for
+# four layers and the head)
+CHUNK_ROWS = 128
 
 # switches for tests and measurements: names of fast kernels that must not be used
 disabled = set()
@@ -65,7 +72,7 @@ class Normed:
 
 
 def settle_residual(ctx, x):
-    """A product of 33 to 64 rows into the residual stream may have left its sums as slices that the
+    """A product of 17 to 64 rows into the residual stream may have left its sums as slices that the
     next norm adds up. Whoever else wants to READ the rows (adding to them is always fine) calls
     this first."""
     pending = getattr(ctx, "pending", None)
@@ -93,13 +100,11 @@ def _next_norm(ctx, N):
 
 
 def row_chunks(M, ctx=None):
-    """Steps of 66 to 192 rows are worked on in two or three pieces of 33 to 64 rows: the kernels for
+    """Steps of 66 to 128 rows are worked on in two pieces of 33 to 64 rows: the kernels for
     so few rows stream the weights at several times the rate of the tiled kernel, whose tiles of
     128 rows are too few for the chip at these sizes, and the pieces after the first find the
-    weights in the memory-side cache. A step that is not replayed from a graph pays for every
-    launch on the host: there three pieces cost more than they gain (measured: 128 rows 2.9 ms
-    in pieces, 192 rows 3.6 ms in pieces against 3.2 ms tiled). None: no pieces."""
-    if not 65 < M <= (192 if ctx is None or getattr(ctx, "decode", False) else 128):
+    weights in the memory-side cache. None: no pieces."""
+    if not 65 < M <= CHUNK_ROWS:
         return None
     n = -(-M // 64)
     size = -(-M // n)
@@ -181,7 +186,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
         if (_streams_rows_for_many_strips(a.shape[0], w, epilogue) and "mfma" not in disabled
                 and K.gemm_mfma_fits(a, w, out, epilogue)):
             return K.gemm_mfma(a, w, out, epilogue, bias=bias)
-        if ("wide" not in disabled and K.gemm_skinny_wide_fits(a, w, out, epilogue)
+        if ("wide" not in disabled and a.shape[0] > FUSE_ROWS and K.gemm_skinny_wide_fits(a, w, out, epilogue)
                 and _linear_wide(a, w, out, epilogue, ctx, bias, act)):
             return
         if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
@@ -231,7 +236,7 @@ def _streams_rows_for_many_strips(M, w, epilogue):
 
 
 def _linear_wide(a, w, out, epilogue, ctx, bias=None, act="silu"):
-    """Products of 33 to 64 rows where another kernel than the skinny one is faster. True when done."""
+    """Products of 17 to 64 rows where another kernel than the skinny one is faster. True when done."""
     M, Kd = a.shape
     N = out.shape[1]
     if epilogue == EPI_GATED:

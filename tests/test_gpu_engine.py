@@ -144,8 +144,9 @@ def test_batch_mates_order_and_slot_change_nothing(dtype):
 @pytest.mark.parametrize("name, dtype", [("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16"),
                                          ("D", "bfloat16")])
 @pytest.mark.parametrize("graphs", [False, True])
-def test_decode_steps_of_33_to_64_sequences(name, dtype, graphs, monkeypatch):
-    """Between 33 and 64 tokens a step the products into the residual stream leave their sums in
+@pytest.mark.parametrize("B", [41, 23])
+def test_decode_steps_of_17_to_64_sequences(name, dtype, graphs, B, monkeypatch):
+    """Between 17 and 64 tokens a step the products into the residual stream leave their sums in
     slices of K that the next norm adds up, and rotation and cache write ride on the QKV product.
     The tiny models' K is too short for the rule that cuts it, so the rule is replaced by one that
     always cuts."""
@@ -157,7 +158,6 @@ def test_decode_steps_of_33_to_64_sequences(name, dtype, graphs, monkeypatch):
         cut.append(n)
         return n
     monkeypatch.setattr(lib, "wide_slices", always)
-    B = 41
     eng = engine(name, dtype, n_slots=64, max_tokens=64 * 64, use_graphs=graphs)
     seqs = [rand_tokens(name, 200 + i, 2 + i % 5 + 6) for i in range(B)]
     slots = [eng.take_slot() for _ in range(B)]

@@ -700,13 +700,13 @@ def test_gemm_skinny_leaves_sums_of_squares(M):
                         xg=torch.empty(M, N, device=DEV, dtype=torch.bfloat16))          # not without the sums of squares
 
 
-@pytest.mark.parametrize("folded_norm", [True, False])
+@pytest.mark.parametrize("folded_norm, more_rows", [(True, 0), (False, 45), (False, 21), (False, 0)])
 @pytest.mark.parametrize("pairing", ["adjacent", "half", None])
 @pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 16), (5, 5, 48), (8, 1, 128), (32, 8, 128), (21, 7, 112)])
-def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs, folded_norm):
+def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs, folded_norm, more_rows):
     rng = np.random.default_rng(hs + H)
     d, page = 96, 64
-    lens_before = [70, 0, 129, 63, 64] if folded_norm else [70, 0, 129, 63, 64] + list(range(3, 48))   # 50 rows
+    lens_before = [70, 0, 129, 63, 64] + list(range(3, 3 + more_rows))     # 5, 26 and 50 rows: every kernel
     T = len(lens_before)
     x = (rng.standard_normal((T, d)) * 2).astype(np.float32)
     nw = rounded(1 + 0.2 * rng.standard_normal(d), "bfloat16")
@@ -751,8 +751,8 @@ def test_qkv_rope_cache_in_one_kernel(pairing, H, Kh, hs, folded_norm):
     assert torch.equal(untile_values(vc)[mv], untile_values(before_v)[mv])
 
 
-# ------------------------------------------------------------------ the wide kernel for 33 to 64 rows, K in slices
-@pytest.mark.parametrize("M", [33, 48, 64])
+# ------------------------------------------------------------------ the wide kernel for 17 to 64 rows, K in slices
+@pytest.mark.parametrize("M", [17, 32, 33, 48, 64])
 @pytest.mark.parametrize("N, Kd", [(2048, 2048), (130, 72), (40, 40), (1000, 1544), (6144, 256)])
 def test_gemm_skinny_wide(M, N, Kd):
     rng = np.random.default_rng(M + N)
@@ -796,7 +796,7 @@ def test_gemm_skinny_wide_refuses_what_it_cannot_do():
     a = torch.zeros(40, 64, device=DEV, dtype=torch.bfloat16)
     w = torch.zeros(32, 64, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(lib.KernelError):
-        lib.gemm_skinny_wide(a[:20], w, torch.zeros(20, 32, device=DEV))                       # the skinny kernel's rows
+        lib.gemm_skinny_wide(a[:16], w, torch.zeros(16, 32, device=DEV))                       # the skinny kernel's rows
     with pytest.raises(lib.KernelError, match="slices"):
         lib.gemm_skinny_wide(a, w, torch.zeros(2, 40, 32, device=DEV), lib.EPI_ADD)            # slices are stored, not added
     with pytest.raises(lib.KernelError, match="slices"):
