@@ -591,18 +591,21 @@ __device__ __forceinline__ bf16x8 sk_buffer_load(__amdgpu_buffer_rsrc_t buf, uns
 // a line) nor the reads (16 rows of one piece) meet in a bank. The piece of shared memory is the
 // wave's own, so only the wave's own order matters: a fence of wavefront scope keeps the compiler
 // from moving the reads over the writes, the hardware works a wave's accesses in order.
-template <int MT, int NS, int NW, int EPI, typename TC>
+//
+// XNORM (one slice of K): the product is that of an RMSNorm, as in the other kernels: A holds
+// bfloat16(weight * x) and the rows' 1/rms, from the partial sums of squares, is applied to the sums.
+template <int MT, int NS, int NW, int EPI, typename TC, bool XNORM>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t* __restrict__ A,
                                                                    const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                    int M, int N, int K, long lda, long ldw, long ldc,
                                                                    long slice_stride, int pairs_per_slice, SkRope rp,
-                                                                   SkNext nx) {
+                                                                   SkNext nx, SkNorm nrm) {
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   constexpr int NWT = NS * NG;        // tiles of W a pair of k-steps
   constexpr int NT = NWT + MT;        // tiles a wave stages for a pair of k-steps: 16 rows x 128 bytes each
   constexpr int STAGE = NW * NT * 2048, RED = NW * NG * MT * 1024;
   __shared__ __attribute__((aligned(16))) char smem[STAGE > RED ? STAGE : RED];
-  __shared__ float sm_ssq[1][64];
+  __shared__ float sm_ssq[XNORM ? NW : 1][64];
   f32x4 (*red)[NG * MT][64] = (f32x4 (*)[NG * MT][64])smem;   // the partial tiles, once the staging is over
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
@@ -698,6 +701,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   for (int g = 0; g < NS; ++g)
     pre[g] = sk_preload<MT, EPI, TC, 16, EPI == SK_QKV>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g],
                                                          rotated[g], rp, nx, tok_pos, tok_row);
+  if (XNORM) sk_ssq_partials<NW>(sm_ssq, M, nrm);   // (read after the barrier before the first strip's end)
   for (int i = 0; i < n_it; ++i) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -733,8 +737,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   for (int g = 0; g < NS; ++g) {
     __syncthreads();   // the staged lines, then the partial tiles of the strip before, are free
     if (strip0 + g < n_strips)   // the same for all threads of the block
-      sk_finish<MT, NW, EPI, TC, false, false>(red, sm_ssq, acc[g], strip0 + g, hd[g], sub[g], rotated[g], out, M, N, K,
-                                                ldc, SkNorm{}, nullptr, rp, nx, pre[g]);
+      sk_finish<MT, NW, EPI, TC, XNORM, false>(red, sm_ssq, acc[g], strip0 + g, hd[g], sub[g], rotated[g], out, M, N, K,
+                                                ldc, nrm, nullptr, rp, nx, pre[g]);
   }
 }
 
@@ -922,16 +926,16 @@ static bool wide_addressable(long M, long w_rows, long K, long lda, long ldw) {
   return ((M - 1) * lda + K) * 2 < (1L << 31) && ((w_rows - 1) * ldw + K) * 2 < (1L << 31);
 }
 
-template <int MT, int NS, int EPI, typename TC>
+template <int MT, int NS, int EPI, typename TC, bool XNORM = false>
 static int launch_wide(const SkCall& a, int slices, long slice_stride) {
   constexpr int NW = 8;
   const int n_strips = (a.N + 15) / 16;
   const int pairs = (a.K + 63) / 64;   // pairs of k-steps
   const int per_slice = (pairs + slices - 1) / slices;
-  gemm_skinny_wide_kernel<MT, NS, NW, EPI, TC>
+  gemm_skinny_wide_kernel<MT, NS, NW, EPI, TC, XNORM>
       <<<dim3((n_strips + NS - 1) / NS, slices), dim3(NW * 64), 0, a.stream>>>(
           (const bf16_t*)a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, slice_stride, per_slice,
-          a.rp, a.nx);
+          a.rp, a.nx, a.nrm);
   GL3_LAUNCH_CHECK();
   return 0;
 }
@@ -961,12 +965,19 @@ static int wide_strips(int N, int slices, int epilogue) {
 // K is cut into that many slices and C is [slices][M][ldc] with `slice_stride` elements between
 // slices; the caller adds them up. `strips_per_block`: 0 lets the library choose.
 // bias (may be null; one slice only): N floats (gated: 2N); act: the gated epilogue's activation.
+// ssq (may be null; gated epilogue, at most 16 rows, one slice): the product is that of RMSNorm(x), with A =
+// bfloat16(norm weight * x) and the rows' sums of squares in `ssq` [n_partials][64], as gl3_gemm_skinny_norm takes
+// them; pack_out (with ssq, at most 8 rows): C receives the rows in the packed tiles' order, as there.
 extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                     long ldw, long ldc, int epilogue, int slices, long slice_stride,
-                                    int strips_per_block, const float* bias, int act, hipStream_t stream) {
+                                    int strips_per_block, const float* bias, int act, const float* ssq, int n_partials,
+                                    float eps, int pack_out, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_wide", A, W, C, M, N, K, lda, ldw, 0)) return -1;
-  GL3_REQUIRE(M > 16, "gl3_gemm_skinny_wide: M=%d; up to 16 rows are gl3_gemm_skinny's", M);
+  GL3_REQUIRE(ssq || M > 16, "gl3_gemm_skinny_wide: M=%d; up to 16 rows are gl3_gemm_skinny's", M);
+  GL3_REQUIRE(!ssq || (M <= 16 && epilogue == SK_GATED && c_dtype == GL3_BF16 && slices == 1 && n_partials > 0),
+              "gl3_gemm_skinny_wide: a folded norm goes with the gated epilogue, at most 16 rows and one slice");
+  GL3_REQUIRE(!pack_out || (ssq && M <= 8), "gl3_gemm_skinny_wide: the packed tiles' order holds at most 8 rows of a folded norm's product");
   GL3_REQUIRE(wide_addressable(M, epilogue == SK_GATED ? 2L * N : N, K, lda, ldw),
               "gl3_gemm_skinny_wide: an operand of 2 GiB or more");
   GL3_REQUIRE(ldc >= N, "gl3_gemm_skinny_wide: ldc too small");
@@ -981,8 +992,11 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
               strips_per_block);
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_skinny_wide: a bias goes with one slice of K");
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny_wide: unknown activation %d", act);
-  SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{}, nullptr, SkRope{}, stream, false};
-  a.nx = SkNext{nullptr, nullptr, 0, bias, act, 0};
+  SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{ssq, n_partials, eps, nullptr}, nullptr, SkRope{}, stream, false};
+  a.nx = SkNext{nullptr, nullptr, 0, bias, act, pack_out};
+  if (ssq)
+    return strips_per_block == big ? launch_wide<1, 2, SK_GATED, bf16_t, true>(a, 1, 0)
+                                   : launch_wide<1, 1, SK_GATED, bf16_t, true>(a, 1, 0);
   if (c_dtype == GL3_F32) {
     if (epilogue == SK_STORE) return pick_wide<SK_STORE, float>(a, strips_per_block, slices, slice_stride);
     if (epilogue == SK_ADD) return pick_wide<SK_ADD, float>(a, strips_per_block, slices, slice_stride);

@@ -61,7 +61,7 @@ def _declare(lib):
         "gl3_argmax_static": [P, L, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
         "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P, I, P],
-        "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P],
+        "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P, I, F, I, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, I, P],
         "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P],
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, P],
@@ -522,7 +522,7 @@ def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="si
     _check(library().gl3_gemm_skinny_wide(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0),
                                           w.stride(0), rows.stride(0), epilogue, slices, slice_stride, strips,
                                           _bias(bias, wrows, "gemm_skinny_wide"), _act(act, "gemm_skinny_wide"),
-                                          _stream()), "gemm_skinny_wide")
+                                          None, 0, 0.0, 0, _stream()), "gemm_skinny_wide")
 
 
 def _check_norm_args(xg, ssq, n_partials, K):
@@ -542,10 +542,12 @@ def gemm_skinny_norm_fits(xg, w, out, epilogue):
 
 
 def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=None, waves=0, bias=None, act="silu",
-                     pack_out=False):
+                     pack_out=False, whole_lines=False):
     """out (=, gated) RMSNorm(x)[rows] @ w.T, where ``xg`` = bfloat16(norm weight * x) was left by the
     kernel that completed the rows of x, together with their sums of squares as partial sums.
-    ``pack_out`` (at most 8 rows, bfloat16): ``out`` is a ``packed_rows`` buffer."""
+    ``pack_out`` (at most 8 rows, bfloat16): ``out`` is a ``packed_rows`` buffer. ``whole_lines`` (gated
+    epilogue, at most 16 rows, all rows): the kernel that loads both operands as whole lines and takes
+    several strips a block (``gemm_skinny_wide``'s) does the work."""
     _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
     K = w.shape[1]
     _check_norm_args(xg, ssq, n_partials, K)
@@ -562,6 +564,13 @@ def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=
     wrows = 2 * N if epilogue == EPI_GATED else N
     if w.shape != (wrows, K) or out.shape[0] != M or out.stride(1) != 1 or M > 64:
         raise KernelError(f"gemm: rows {tuple(xg.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
+    if whole_lines:
+        if epilogue != EPI_GATED or rows is not None or M > 16 or waves:
+            raise KernelError("gemm_skinny_norm: whole lines go with the gated epilogue, at most 16 rows, all of them")
+        return _check(library().gl3_gemm_skinny_wide(
+            _ptr(xg), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, xg.stride(0), w.stride(0), out.stride(0), epilogue,
+            1, 0, 0, _bias(bias, wrows, "gemm_skinny_norm"), _act(act, "gemm_skinny_norm"), _ptr(ssq), n_partials,
+            float(eps), int(bool(pack_out)), _stream()), "gemm_skinny_wide")
     _check(library().gl3_gemm_skinny_norm(
         _ptr(xg), _ptr(rows), _ptr(ssq), n_partials, float(eps), _ptr(w), _ptr(out), _code(out, "out"), M, N, K,
         xg.stride(0), w.stride(0), out.stride(0), epilogue, waves, _bias(bias, wrows, "gemm_skinny_norm"),

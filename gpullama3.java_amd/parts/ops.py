@@ -157,7 +157,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
     ``pack_out`` / ``a_packed``: ``out`` / ``a`` is a ``lib.packed_rows`` buffer (where ``packs_rows`` said so)."""
     if pack_out:
         return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act,
-                                  pack_out=True)
+                                  pack_out=True, whole_lines=_whole_lines(a, w, epilogue))
     if a_packed:
         M, N = out.shape
         if (epilogue == EPI_ADD and ctx is not None and getattr(ctx, "fuse", False) and N % 16 == 0
@@ -175,7 +175,8 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
     if isinstance(a, Normed):
         if ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
                 and a.xg.shape[0] <= 64 and not _streams_rows_for_many_strips(out.shape[0], w, epilogue)):
-            return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act)
+            return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act,
+                                      whole_lines=_whole_lines(a, w, epilogue))
         a = a.materialize()
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         chunks = row_chunks(a.shape[0], ctx)
@@ -224,6 +225,13 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
     K.gemm_generic(a, w, out, epilogue, bias=bias, act=act)
     if epilogue == EPI_ADD:
         residual_written(ctx, out)
+
+
+def _whole_lines(a, w, epilogue):
+    """Whether a folded norm's gated product runs on the kernel that loads whole lines: where it has blocks
+    enough for the chip, as for 17 to 64 rows."""
+    return (epilogue == EPI_GATED and a.rows is None and "wide" not in disabled and "widefold" not in disabled
+            and a.xg.shape[0] <= 16 and w.shape[0] // 2 >= 32 * 192 and w.numel() < 2 ** 30)    # (32-bit byte offsets)
 
 
 def _streams_rows_for_many_strips(M, w, epilogue):

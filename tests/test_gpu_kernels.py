@@ -669,6 +669,49 @@ def test_gemm_skinny_with_folded_norm(M, N, Kd, P_):
     np.testing.assert_allclose(g_.float().cpu().numpy(), refg, atol=1.5e-2 * max(np.abs(refg).max(), 1e-3))
 
 
+@pytest.mark.parametrize("M", [1, 7, 8, 16])
+@pytest.mark.parametrize("N, Kd, P_", [(8192, 2048, 256), (6144, 136, 3), (130, 64, 1), (1000, 1544, 7), (24, 8192, 40)])
+def test_gated_product_with_folded_norm_through_whole_lines(M, N, Kd, P_):
+    """The folded norm's gated product on the kernel that loads whole lines, plain rows and rows in the packed
+    tiles' order, against the plain implementation and against the kernel that keeps its rows in registers."""
+    rng = np.random.default_rng(M + N)
+    x = (rng.standard_normal((M + 2, Kd)) * 2).astype(np.float32)
+    nw = rounded(1 + 0.2 * rng.standard_normal(Kd), "float32")
+    w = rounded(rng.standard_normal((2 * N, Kd)) / math.sqrt(Kd), "bfloat16")
+    bias = rng.standard_normal(2 * N).astype(np.float32)
+    lib = K()
+    XG, W = times_weight(x, nw).to(DEV), dev(w, torch.bfloat16)
+    ssq = dev(ssq_partials(x, P_))
+    h = P.rmsnorm(x, nw, 1e-5)[:M]
+    for b in (None, bias):
+        g, u = P.linear(h, w[:N]), P.linear(h, w[N:])
+        if b is not None:
+            g, u = g + b[:N], u + b[N:]
+        ref = P.silu(g) * u
+        out = torch.full((M + 1, N + 8), -1.0, device=DEV, dtype=torch.bfloat16)      # a view with a row stride
+        lib.gemm_skinny_norm(XG[:M], ssq, P_, 1e-5, W, out[:M, :N], lib.EPI_GATED, bias=None if b is None else dev(b),
+                             whole_lines=True)
+        np.testing.assert_allclose(out[:M, :N].float().cpu().numpy(), ref, atol=1.5e-2 * max(np.abs(ref).max(), 1e-3))
+        assert torch.all(out[M] == -1) and torch.all(out[:, N:] == -1)
+        other = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+        lib.gemm_skinny_norm(XG[:M], ssq, P_, 1e-5, W, other, lib.EPI_GATED, bias=None if b is None else dev(b))
+        np.testing.assert_allclose(out[:M, :N].float().cpu().numpy(), other.float().cpu().numpy(),
+                                   atol=1e-2 * max(np.abs(ref).max(), 1e-3))            # (another order of summation)
+    if M <= 8:
+        packed = lib.packed_rows(N, torch.bfloat16, DEV)
+        packed.fill_(777.0)
+        lib.gemm_skinny_norm(XG[:M], ssq, P_, 1e-5, W, packed, lib.EPI_GATED, bias=dev(bias), pack_out=True, whole_lines=True)
+        flat = packed.reshape(-1).cpu()
+        m, k = np.meshgrid(np.arange(M), np.arange(N), indexing="ij")
+        at = (((k // 64) * 64 + ((k % 32) // 8) * 16 + ((k % 64) // 32) * 8 + m) * 8) + k % 8
+        assert torch.equal(flat[torch.as_tensor(at)], out[:M, :N].cpu())
+        untouched = np.ones(flat.numel(), bool)
+        untouched[at.reshape(-1)] = False
+        assert torch.all(flat[torch.as_tensor(untouched)] == 777.0)
+    with pytest.raises(lib.KernelError):
+        lib.gemm_skinny_norm(XG[:M], ssq, P_, 1e-5, W[:N], torch.zeros(M, N, device=DEV), lib.EPI_STORE, whole_lines=True)
+
+
 @pytest.mark.parametrize("M", [1, 8, 40])
 def test_gemm_skinny_leaves_sums_of_squares(M):
     rng = np.random.default_rng(M)
