@@ -38,6 +38,7 @@
 // nothing else, which is what limits the streaming kernel when the same A is read for every
 // strip. The wide one, for 17 to 64 rows, takes several strips at once (see there).
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
@@ -944,6 +945,11 @@ template <int EPI, typename TC>
 static int pick_wide(const SkCall& a, int strips_per_block, int slices, long slice_stride) {
   constexpr int BIG = (EPI == SK_GATED) ? 2 : 4;   // a gated strip is a pair of strips
   const bool big = strips_per_block == BIG;
+  if constexpr (EPI == SK_STORE && std::is_same<TC, float>::value) {   // (9 to 16 rows: slices of a long K only)
+    if (a.M <= 16)
+      return big ? launch_wide<1, BIG, EPI, TC>(a, slices, slice_stride)
+                 : launch_wide<1, BIG / 2, EPI, TC>(a, slices, slice_stride);
+  }
   if ((a.M + 15) / 16 <= 2)
     return big ? launch_wide<2, BIG, EPI, TC>(a, slices, slice_stride)
                : launch_wide<2, BIG / 2, EPI, TC>(a, slices, slice_stride);
@@ -961,7 +967,8 @@ static int wide_strips(int N, int slices, int epilogue) {
   return (n_strips / big) * slices >= 192 ? big : big / 2;
 }
 
-// The product for 17 to 64 rows of A (bfloat16). `slices` > 1 (store epilogue, float output only):
+// The product for 17 to 64 rows of A (bfloat16), and for 9 to 16 with the store epilogue and a float
+// output. `slices` > 1 (store epilogue, float output only):
 // K is cut into that many slices and C is [slices][M][ldc] with `slice_stride` elements between
 // slices; the caller adds them up. `strips_per_block`: 0 lets the library choose.
 // bias (may be null; one slice only): N floats (gated: 2N); act: the gated epilogue's activation.
@@ -974,7 +981,8 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
                                     float eps, int pack_out, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_wide", A, W, C, M, N, K, lda, ldw, 0)) return -1;
-  GL3_REQUIRE(ssq || M > 16, "gl3_gemm_skinny_wide: M=%d; up to 16 rows are gl3_gemm_skinny's", M);
+  GL3_REQUIRE(ssq || M > 16 || (M > 8 && epilogue == SK_STORE && c_dtype == GL3_F32),
+              "gl3_gemm_skinny_wide: M=%d; up to 16 rows are gl3_gemm_skinny's (but 9 to 16 with a float output stored)", M);
   GL3_REQUIRE(!ssq || (M <= 16 && epilogue == SK_GATED && c_dtype == GL3_BF16 && slices == 1 && n_partials > 0),
               "gl3_gemm_skinny_wide: a folded norm goes with the gated epilogue, at most 16 rows and one slice");
   GL3_REQUIRE(!pack_out || (ssq && M <= 8), "gl3_gemm_skinny_wide: the packed tiles' order holds at most 8 rows of a folded norm's product");

@@ -496,7 +496,7 @@ def _tiled(w, n_rows, K, qkv=None, n_out=None):
 
 
 def gemm_skinny_wide_fits(a, w, out, epilogue):
-    return 16 < a.shape[0] <= 64 and gemm_skinny_fits(a, w, out, epilogue)
+    return 8 < a.shape[0] <= 64 and gemm_skinny_fits(a, w, out, epilogue)
 
 
 def wide_slices(N, K):
@@ -508,7 +508,8 @@ def wide_slices(N, K):
 
 def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="silu"):
     """out (=, +=, gated) a @ w.T for 17 to 64 rows of ``a``. ``out`` with three axes [slices, M, N]
-    (float32, store epilogue) takes the sums of one slice of K each: the caller adds them up."""
+    (float32, store epilogue) takes the sums of one slice of K each: the caller adds them up; that form
+    also takes 9 to 16 rows."""
     _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
     M, K = a.shape
     slices, slice_stride = 1, 0
@@ -517,7 +518,8 @@ def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="si
         slices, slice_stride, rows = out.shape[0], out.stride(0), out[0]
     N = rows.shape[1]
     wrows = 2 * N if epilogue == EPI_GATED else N
-    if (w.shape != (wrows, K) or rows.shape[0] != M or rows.stride(1) != 1 or a.stride(1) != 1 or not 16 < M <= 64):
+    if (w.shape != (wrows, K) or rows.shape[0] != M or rows.stride(1) != 1 or a.stride(1) != 1
+            or not (16 < M <= 64 or (8 < M <= 16 and epilogue == EPI_STORE and out.dtype == torch.float32))):
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_skinny_wide(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0),
                                           w.stride(0), rows.stride(0), epilogue, slices, slice_stride, strips,

@@ -187,8 +187,8 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
         if (_streams_rows_for_many_strips(a.shape[0], w, epilogue) and "mfma" not in disabled
                 and K.gemm_mfma_fits(a, w, out, epilogue)):
             return K.gemm_mfma(a, w, out, epilogue, bias=bias)
-        if ("wide" not in disabled and a.shape[0] > FUSE_ROWS and K.gemm_skinny_wide_fits(a, w, out, epilogue)
-                and _linear_wide(a, w, out, epilogue, ctx, bias, act)):
+        if ("wide" not in disabled and (a.shape[0] > FUSE_ROWS or _long_k_of_9_to_16_rows(a, out, epilogue, bias))
+                and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx, bias, act)):
             return
         if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
             N = out.shape[1]
@@ -225,6 +225,14 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
     K.gemm_generic(a, w, out, epilogue, bias=bias, act=act)
     if epilogue == EPI_ADD:
         residual_written(ctx, out)
+
+
+def _long_k_of_9_to_16_rows(a, out, epilogue, bias):
+    """A product of 9 to 16 rows into the residual stream over a K too long for the kernel that keeps its rows
+    in registers: strips of 8 weight rows leave half of every tile idle there, and the kernel of whole lines
+    with K in slices is faster even with the norm kernel that then adds the slices."""
+    return (epilogue == EPI_ADD and bias is None and 8 < a.shape[0] <= 16 and a.shape[1] > 4096
+            and "wide916" not in disabled and out.dtype == torch.float32)
 
 
 def _whole_lines(a, w, epilogue):

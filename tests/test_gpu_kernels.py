@@ -834,12 +834,34 @@ def test_gemm_skinny_wide(M, N, Kd):
         np.testing.assert_allclose(g_.float().cpu().numpy(), refg, atol=1e-2 * max(np.abs(refg).max(), 1e-3))
 
 
+@pytest.mark.parametrize("M", [9, 16])
+@pytest.mark.parametrize("N, Kd", [(2048, 8192), (130, 200), (40, 4104)])
+def test_gemm_skinny_wide_slices_of_9_to_16_rows(M, N, Kd):
+    """9 to 16 rows: only what a long K into the residual stream needs, a float output stored, in slices or whole."""
+    rng = np.random.default_rng(M + N)
+    a = rounded(rng.standard_normal((M, Kd)), "bfloat16")
+    w = rounded(rng.standard_normal((N, Kd)) / math.sqrt(Kd), "bfloat16")
+    A, W = dev(a, torch.bfloat16), dev(w, torch.bfloat16)
+    lib = K()
+    ref = P.linear(a, w)
+    tol32 = 2e-5 * np.abs(ref).max() * math.sqrt(Kd / 64)
+    for slices in (1, 2, 4):
+        part = torch.full((slices, M + 1, N + 3), 7.0, device=DEV)
+        lib.gemm_skinny_wide(A, W, part[:, :M, :N], lib.EPI_STORE)
+        np.testing.assert_allclose(part[:, :M, :N].sum(0).cpu().numpy(), ref, atol=tol32, err_msg=f"{slices} slices")
+        assert torch.all(part[:, M] == 7.0) and torch.all(part[:, :, N:] == 7.0)
+    with pytest.raises(lib.KernelError):
+        lib.gemm_skinny_wide(A, W, torch.zeros(M, N, device=DEV), lib.EPI_ADD)
+    with pytest.raises(lib.KernelError):
+        lib.gemm_skinny_wide(A, W, torch.zeros(M, N, device=DEV, dtype=torch.bfloat16))
+
+
 def test_gemm_skinny_wide_refuses_what_it_cannot_do():
     lib = K()
     a = torch.zeros(40, 64, device=DEV, dtype=torch.bfloat16)
     w = torch.zeros(32, 64, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(lib.KernelError):
-        lib.gemm_skinny_wide(a[:16], w, torch.zeros(16, 32, device=DEV))                       # the skinny kernel's rows
+        lib.gemm_skinny_wide(a[:8], w, torch.zeros(8, 32, device=DEV))                         # the skinny kernel's rows
     with pytest.raises(lib.KernelError, match="slices"):
         lib.gemm_skinny_wide(a, w, torch.zeros(2, 40, 32, device=DEV), lib.EPI_ADD)            # slices are stored, not added
     with pytest.raises(lib.KernelError, match="slices"):
