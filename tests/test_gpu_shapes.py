@@ -38,7 +38,7 @@ SHAPES = {
 
 
 def steps(eng, vocab):
-    """Logits of every kind of step: a long prompt, single tokens after it, batches of 8, 20, 40 and 100
+    """Logits of every kind of step: a long prompt, single tokens after it, batches of 8, 12, 20, 40 and 100
     sequences (short prompts, then decode steps that are replayed from graphs), prompts of 50, a prompt
     of 2,600 tokens and single tokens after it."""
     rng = np.random.default_rng(0)
@@ -49,7 +49,7 @@ def steps(eng, vocab):
     for t in toks[600:]:
         out.append(eng.step([(s, [t])]).cpu().numpy())
     eng.give_back_slot(s)
-    for B in (8, 20, 40, 100):
+    for B in (8, 12, 20, 40, 100):
         slots = [eng.take_slot() for _ in range(B)]
         seqs = [rng.integers(0, vocab, 7).tolist() for _ in range(B)]
         out.append(eng.step([(sl, q[:4]) for sl, q in zip(slots, seqs)]).cpu().numpy())
