@@ -49,6 +49,7 @@ class StepContext:
         self.n_tokens, self.n_seqs = n_tokens, n_seqs
         self.q_lens, self.kv_before_host, self.slots = q_lens, kv_before_host, slots
         self.decode = decode
+        self.replayed = False              # whether the step's launches are being captured into a graph
         self.max_q_len, self.max_kv_len = max_q_len, max_kv_len
         self.fuse = getattr(engine, "fuse", False)   # few-token steps fold norms and rotation into the products
         self.ssq = None                    # (address of the residual stream, its partial sums of squares, how many)

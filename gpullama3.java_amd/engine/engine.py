@@ -339,6 +339,7 @@ class Engine:
         ctx = StepContext(self, B_pad, B_pad, [1] * B_pad, [0] * B_pad, [self.cache.sink_slot] * B_pad, decode=True,
                           max_q_len=1, max_kv_len=kv_bucket)
         ctx.kv_len_hint = kv_bucket
+        ctx.replayed = True
         d = dg.dev
         ctx.token_ids, ctx.positions, ctx.kv_before = d[0:B_pad], d[B_pad:2 * B_pad], d[2 * B_pad:3 * B_pad]
         ctx.slot_ids = d[3 * B_pad:4 * B_pad]
