@@ -1079,8 +1079,14 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
   GL3_REQUIRE(!w_tiled || (uintptr_t)w_tiled % 16 == 0, "gl3_qkv_rope_cache: the copy of W must be 16-byte aligned");
   a.Wt = w_tiled;   // (its strips hold the rows that sk_strip_row names: for half-split pairing 8 rows and the 8 half a head further)
   if (!ssq && waves == 0 && M > 16 && wide_addressable(M, N, K, lda, ldw)) {
-    // many rows: two strips a block, so that the rows are read half as often, in whole lines
+    // many rows, read in whole lines: two strips a block, so that the rows are read half as often, where one
+    // strip a block would be more blocks than CUs (N = 3,072, K = 2,048, 64 rows: 10.0 us with two, 8.9 us with
+    // one; N = 5,120, K = 3,072: 16.3 against 20.7 us)
     const int tiles = (M + 15) / 16;
+    if ((N + 15) / 16 <= 256)
+      return tiles <= 2   ? launch_wide<2, 1, SK_QKV, bf16_t>(a, 1, 0)
+             : tiles == 3 ? launch_wide<3, 1, SK_QKV, bf16_t>(a, 1, 0)
+                          : launch_wide<4, 1, SK_QKV, bf16_t>(a, 1, 0);
     return tiles <= 2   ? launch_wide<2, 2, SK_QKV, bf16_t>(a, 1, 0)
            : tiles == 3 ? launch_wide<3, 2, SK_QKV, bf16_t>(a, 1, 0)
                         : launch_wide<4, 2, SK_QKV, bf16_t>(a, 1, 0);
