@@ -210,17 +210,19 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
             return
         if "mfma" not in disabled and K.gemm_mfma_fits(a, w, out, epilogue):
             M, Kd = a.shape
-            slices = K.mfma_slices(M, out.shape[1], Kd) if epilogue == EPI_ADD and bias is None else 1
-            if slices > 1 and ctx is not None and getattr(ctx, "fuse", False) and "fused" not in disabled:
-                # a long K over few tiles: the first slice adds into the rows, the norm that follows
-                # adds the others
+            shape, slices = 0, 1
+            if (epilogue == EPI_ADD and bias is None and ctx is not None and getattr(ctx, "fuse", False)
+                    and "fused" not in disabled):
+                shape, slices = K.mfma_plan(M, out.shape[1], Kd)
+            if slices > 1:
+                # the first slice adds into the rows, the norm that follows adds the others
                 settle_residual(ctx, out)
                 part = ctx.buffer(f"slices{slices - 1}", (slices - 1, M, out.shape[1]), torch.float32)
-                K.gemm_mfma(a, w, out, epilogue, more_slices=part)
+                K.gemm_mfma(a, w, out, epilogue, more_slices=part, shape=shape)
                 residual_written(ctx, out)
                 ctx.pending = (out.data_ptr(), part)
                 return
-            K.gemm_mfma(a, w, out, epilogue, bias=bias, act=act)
+            K.gemm_mfma(a, w, out, epilogue, bias=bias, act=act, shape=shape)
             if epilogue == EPI_ADD:
                 residual_written(ctx, out)
             return

@@ -1,0 +1,25 @@
+"""The rules that choose a kernel's shape are plain arithmetic on the host: their decisions at the sizes
+they were measured at."""
+from gpullama3_java_amd.csrc import lib
+
+
+def test_few_tiles_are_cut_along_k_down_to_slices_of_512_columns():
+    assert lib.mfma_slices(300, 2048, 8192) == 8          # 48 tiles of 128
+    assert lib.mfma_slices(300, 2048, 2048) == 4          # (a slice is at least 512 columns)
+    assert lib.mfma_slices(2048, 2048, 8192) == 2         # 256 tiles
+    assert lib.mfma_plan(300, 2048, 8192) == (1, 8) and lib.mfma_plan(2048, 2048, 8192) == (1, 2)
+
+
+def test_many_tiles_take_the_plan_with_the_fewest_idle_places():
+    # 8,192 rows of the 8B layers: 512 tiles of 256 are two full rounds; nothing to gain from slices
+    assert lib.mfma_plan(8192, 4096, 14336) == (2, 1) and lib.mfma_plan(8192, 4096, 4096) == (2, 1)
+    # 128 tiles of 256 leave half the chip idle: two slices (measured 308 -> 265 us and 187 -> 170 us)
+    assert lib.mfma_plan(2048, 4096, 14336) == (2, 2) and lib.mfma_plan(4096, 2048, 8192) == (2, 2)
+    # 276 tiles of 256 are 1.08 rounds: slices fill the second (5,886 rows of the 3B layers: 474 -> 417 us)
+    assert lib.mfma_plan(5886, 3072, 8192) in ((2, 2), (2, 3))
+    shape, slices = lib.mfma_plan(1536, 3072, 8192)
+    assert slices > 1                                     # (161 us whole, 119 to 132 us in two or three slices)
+    for M in range(300, 9000, 431):
+        for N, K in ((2048, 8192), (3072, 3072), (4096, 14336), (1000, 520)):
+            shape, slices = lib.mfma_plan(M, N, K)
+            assert shape in (1, 2) and 1 <= slices <= 8 and K // slices >= 512
