@@ -235,11 +235,17 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
   if (shape == 1) return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
   if (shape == 2) return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
   if (shape == 3) return launch_shape<EPI, TC, 4, 2, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
-  // 256 x 256 tiles of sixteen waves where there is at least one for every CU: half the operand
-  // traffic per product, and that traffic is what bounds the large products. Otherwise 128 x 128
-  // tiles of eight waves, of which several fit a CU and overlap each other's waits.
+  // 256 x 256 tiles of sixteen waves, one block a CU, have half the operand traffic per product, and
+  // that traffic is what bounds the large products; of the 128 x 128 tiles of eight waves two fit a CU and
+  // overlap each other's waits. A step of 64 columns takes a chip full of the large tiles 1.7 us and a chip
+  // full of the small ones (twice as many blocks, a quarter of the work each) 1.05 us, and the blocks need
+  // whole rounds on the chip: the tile whose rounds take less time is chosen (240 large tiles are one round
+  // where 960 small ones are two; 276 large ones are two where 1,104 small ones are three).
+  const long small_n = (EPI == MF_GATED) ? (N + 63) / 64 : (N + 127) / 128;
   const long big_n = (EPI == MF_GATED) ? (N + 127) / 128 : (N + 255) / 256;
-  if ((long)((M + 255) / 256) * big_n * slices >= 256)
+  const long small_rounds = ((long)((M + 127) / 128) * small_n * slices + 511) / 512;
+  const long big_rounds = ((long)((M + 255) / 256) * big_n * slices + 255) / 256;
+  if (big_rounds * 170 < small_rounds * 105)
     return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
   return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
 }
