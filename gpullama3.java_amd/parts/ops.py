@@ -336,7 +336,7 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
         if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
                 and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):
             T = q.shape[0]
-            splits = K.decode_splits(T, n_heads, n_kv, ctx.kv_len_hint)
+            splits = K.decode_splits(T, n_heads, n_kv, ctx.kv_len_hint, head_dim)
             part_o = part_ml = None
             if splits > 1:
                 part_o = ctx.buffer("attn_part_o", (T, n_heads, splits, head_dim), torch.float32)

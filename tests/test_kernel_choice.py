@@ -23,3 +23,12 @@ def test_many_tiles_take_the_plan_with_the_fewest_idle_places():
         for N, K in ((2048, 8192), (3072, 3072), (4096, 14336), (1000, 520)):
             shape, slices = lib.mfma_plan(M, N, K)
             assert shape in (1, 2) and 1 <= slices <= 8 and K // slices >= 512
+
+
+def test_decode_attention_splits_the_keys_until_every_cu_has_a_block():
+    s = lib.decode_splits
+    assert s(1, 32, 8, 540) == 1 and s(64, 32, 8, 8200) == 1          # short contexts; blocks enough without
+    assert s(1, 32, 8, 8200) == 8 and s(1, 32, 8, 16400) == 16        # a split walks at least 1,024 keys of 64
+    assert s(1, 32, 8, 2100, 128) == 4 and s(1, 32, 8, 2100, 64) == 2  # (or 512 of 128)
+    assert s(8, 32, 8, 16400) == 4 and s(16, 32, 8, 16400) == 2 and s(32, 32, 8, 16400) == 1   # 256 blocks, not more
+    assert s(2, 64, 2, 100000) == 16                                  # never more than 16
