@@ -16,6 +16,7 @@
 //
 // Epilogues as in gemm_generic.hip: store, add into a float matrix, gated.
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -168,42 +169,48 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
     __syncthreads();
   }
 
-  // lane holds C[row(v)][col]: row(v) = 8*(v/4) + 4*(lane/32) + v%4 inside a 32x32 tile, col = lane%32
+  // lane holds C[row(v)][col]: row(v) = 8*(v/4) + 4*(lane/32) + v%4 inside a 32x32 tile, col = lane%32.
+  // Whole tiles (all but the matrix's last row and column of tiles) store without a test per element.
+  auto finish = [&](auto checked_t) {
+    constexpr bool CHECKED = decltype(checked_t)::value;
 #pragma unroll
-  for (int tm = 0; tm < TM; ++tm) {
+    for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int m = m0 + wm * 32 * TM + tm * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
-      if (m >= M) continue;
-      if (slice > 0) {
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * 32 * TM + tm * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
+        if (CHECKED && m >= M) continue;
+        if (slice > 0) {
 #pragma unroll
-        for (int tn = 0; tn < 2; ++tn) {
-          const int n = n0 + wn * 64 + tn * 32 + lr;
-          if (n < N) P[(long)(slice - 1) * p_stride + (long)m * ldp + n] = acc[tm][tn][v];
+          for (int tn = 0; tn < 2; ++tn) {
+            const int n = n0 + wn * 64 + tn * 32 + lr;
+            if (!CHECKED || n < N) P[(long)(slice - 1) * p_stride + (long)m * ldp + n] = acc[tm][tn][v];
+          }
+          continue;
         }
-        continue;
-      }
-      if (EPI == MF_GATED) {
-        const int n = n0 + wn * 32 + lr;
-        if (n < N) {
-          float g = acc[tm][0][v], u = acc[tm][1][v];
-          if (bias) { g += bias[n]; u += bias[N + n]; }
-          C[(long)m * ldc + n] = from_f32<TC>(gl3_activation<true>(g, act) * u);
-        }
-      } else {
+        if (EPI == MF_GATED) {
+          const int n = n0 + wn * 32 + lr;
+          if (!CHECKED || n < N) {
+            float g = acc[tm][0][v], u = acc[tm][1][v];
+            if (bias) { g += bias[n]; u += bias[N + n]; }
+            C[(long)m * ldc + n] = from_f32<TC>(gl3_activation<true>(g, act) * u);
+          }
+        } else {
 #pragma unroll
-        for (int tn = 0; tn < 2; ++tn) {
-          const int n = n0 + wn * 64 + tn * 32 + lr;
-          if (n < N) {
-            TC* c = C + (long)m * ldc + n;
-            const float s = acc[tm][tn][v] + (bias ? bias[n] : 0.f);
-            if (EPI == MF_ADD) *c = from_f32<TC>(to_f32<TC>(*c) + s);
-            else *c = from_f32<TC>(s);
+          for (int tn = 0; tn < 2; ++tn) {
+            const int n = n0 + wn * 64 + tn * 32 + lr;
+            if (!CHECKED || n < N) {
+              TC* c = C + (long)m * ldc + n;
+              const float s = acc[tm][tn][v] + (bias ? bias[n] : 0.f);
+              if (EPI == MF_ADD) *c = from_f32<TC>(to_f32<TC>(*c) + s);
+              else *c = from_f32<TC>(s);
+            }
           }
         }
       }
     }
-  }
+  };
+  if (m0 + BM <= M && n0 + NCOLS <= N) finish(std::false_type{});
+  else finish(std::true_type{});
 }
 
 template <int EPI, typename TC, int TM, int WM, int WN>
