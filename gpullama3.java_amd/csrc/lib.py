@@ -726,7 +726,7 @@ def mfma_plan(M, N, K):
     best = None
     for shape, tile, places, step_us in ((1, 128, 512, 1.05), (2, 256, 256, 1.7)):
         for slices in (1, 2, 3, 4):
-            if K // slices < 512:
+            if slices > 1 and K // slices < 512:
                 continue
             blocks = -(-M // tile) * -(-N // tile) * slices
             estimate = -(-blocks // places) * -(-K // (64 * slices)) * step_us + 0.35e-6 * (slices + 1.5) * M * N * 4

@@ -20,9 +20,9 @@ def test_many_tiles_take_the_plan_with_the_fewest_idle_places():
     shape, slices = lib.mfma_plan(1536, 3072, 8192)
     assert slices > 1                                     # (161 us whole, 119 to 132 us in two or three slices)
     for M in range(300, 9000, 431):
-        for N, K in ((2048, 8192), (3072, 3072), (4096, 14336), (1000, 520)):
+        for N, K in ((2048, 8192), (3072, 3072), (4096, 14336), (1000, 520), (3072, 272), (6144, 8)):
             shape, slices = lib.mfma_plan(M, N, K)
-            assert shape in (1, 2) and 1 <= slices <= 8 and K // slices >= 512
+            assert shape in (1, 2) and 1 <= slices <= 8 and (slices == 1 or K // slices >= 512)
 
 
 def test_decode_attention_splits_the_keys_until_every_cu_has_a_block():
