@@ -27,8 +27,11 @@ def test_many_tiles_take_the_plan_with_the_fewest_idle_places():
 
 def test_decode_attention_splits_the_keys_until_every_cu_has_a_block():
     s = lib.decode_splits
-    assert s(1, 32, 8, 540) == 1 and s(64, 32, 8, 8200) == 1          # short contexts; blocks enough without
-    assert s(1, 32, 8, 8200) == 8 and s(1, 32, 8, 16400) == 16        # a split walks at least 1,024 keys of 64
-    assert s(1, 32, 8, 2100, 128) == 4 and s(1, 32, 8, 2100, 64) == 2  # (or 512 of 128)
-    assert s(8, 32, 8, 16400) == 4 and s(16, 32, 8, 16400) == 2 and s(32, 32, 8, 16400) == 1   # 256 blocks, not more
+    assert s(1, 32, 8, 1024) == 1 and s(8, 32, 8, 1024, 128) == 1 and s(64, 32, 8, 16384) == 1   # short; blocks enough
+    assert s(8, 32, 8, 1024, 128) == 1 and s(8, 32, 8, 2048, 64) == 1                   # 128 K elements, 64 blocks
+    assert s(8, 32, 8, 2048, 128) == 2 and s(8, 32, 8, 4096, 64) == 2                   # 256 K elements
+    assert s(1, 32, 8, 4096) == 2 and s(1, 32, 8, 16384) == 8 and s(1, 32, 8, 32768) == 16  # a split per 128 K elements
+    assert s(1, 32, 8, 2048, 128) == 2 and s(1, 32, 8, 4096, 128) == 4
+    assert s(8, 32, 8, 8192, 64) == 4 and s(8, 32, 8, 32768) == 4 and s(16, 32, 8, 32768) == 2   # 256 blocks, not more
+    assert s(32, 32, 8, 32768) == 1
     assert s(2, 64, 2, 100000) == 16                                  # never more than 16
