@@ -471,9 +471,16 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
     }
 }
 
-// From how many tokens of the longest sequence of a step on the kernel with 128 queries a block is
-// taken, unless the caller says otherwise.
-#define GL3_PREFILL_WIDE_FROM 256
+// Which of the two kernels a step takes, unless the caller says otherwise. Heads of 32 and 64: the one
+// with 128 queries a block (chunks of 64 keys) from 33 tokens of the longest sequence on; it was the faster
+// one at every length from there (192 tokens, 32 heads of 64: 7.4 against 9.8 us; 1,024: 23 against 33 us).
+// Heads of 96 and 128: only where it has at least two blocks for every CU; below that the kernel of 64
+// queries a block, with twice the blocks, is ahead (32 heads of 128, one sequence: 1,024 tokens 38 against
+// 42 us, 1,536 tokens 59 against 65 us, 2,048 tokens 99 against 84 us).
+static bool prefill_wide(int head_dim, int n_heads, int n_seqs, int max_q_len) {
+  if (head_dim <= 64) return max_q_len > 32;
+  return (long)n_heads * n_seqs * ((max_q_len + 127) / 128) >= 512;
+}
 
 extern "C" int gl3_attention_prefill_supports(int head_dim, int page_size) {
   return (head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128) && page_size % 32 == 0;
@@ -481,7 +488,7 @@ extern "C" int gl3_attention_prefill_supports(int head_dim, int page_size) {
 
 // max_q_len: the most tokens any sequence brings in this step (it sizes the grid).
 // seq_rows (may be null): the row of `block_table` that holds sequence b's pages; null: row b.
-// wide_from: the kernel with 128 queries a block is taken when max_q_len reaches it; <= 0: the default.
+// wide_from: the kernel with 128 queries a block is taken when max_q_len reaches it; <= 0: the library's choice.
 extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k_cache, const void* v_cache,
                                      const int* cu_seqlens, const int* kv_before, const int* block_table,
                                      const int* seq_rows, int table_stride, void* out, long out_stride, int n_seqs,
@@ -500,7 +507,7 @@ extern "C" int gl3_attention_prefill(const void* q, long q_stride, const void* k
               "gl3_attention_prefill: queries must be 16-byte aligned, outputs 8-byte aligned");
   const int g = n_heads / n_kv;
   // query heads per wave: as many as the registers hold with two blocks on a CU
-  const bool wide = max_q_len >= (wide_from > 0 ? wide_from : GL3_PREFILL_WIDE_FROM);
+  const bool wide = wide_from > 0 ? max_q_len >= wide_from : prefill_wide(head_dim, n_heads, n_seqs, max_q_len);
   // query heads per wave: as many as the registers hold with two blocks on a CU; one with 32 queries a wave
   const int gh = wide ? 1 : head_dim <= 32 ? 4 : head_dim <= 64 ? 2 : 1;
   const long z = (long)n_kv * ((g + gh - 1) / gh);
