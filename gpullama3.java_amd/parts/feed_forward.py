@@ -43,7 +43,7 @@ class GatedFeedForward:
         dt = g.dtype if g.dtype == u.dtype else torch.float32
         self.w_gate_up = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
         weights[n["gate"]], weights[n["up"]] = self.w_gate_up[:self.F], self.w_gate_up[self.F:]
-        ops.for_few_rows(self.w_gate_up)
+        ops.for_gated(self.w_gate_up)
         self.w_down = ops.for_eight_rows(weights[n["down"]])
         if self.biased:     # the epilogues read biases as float
             self.b_gate_up = torch.cat([weights[n["gate_bias"]].float(), weights[n["up_bias"]].float()]).contiguous()

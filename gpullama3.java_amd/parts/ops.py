@@ -40,11 +40,28 @@ def for_few_rows(w, qkv=None):
     return w
 
 
+def for_gated(w):
+    """The stacked gate and up rows of a feed-forward: the copy of ``for_few_rows`` only where a product of few
+    rows reads it; the kernel of whole lines, which takes the large ones, reads the rows as they are stored."""
+    return w if gated_on_whole_lines(w) else for_few_rows(w)
+
+
+def gated_on_whole_lines(w):
+    """Whether the gated products of few rows over ``w`` (2N rows) run on the kernel that loads whole lines:
+    where it has blocks enough for the chip, and 32-bit byte offsets reach all of ``w``."""
+    return ("wide" not in disabled and "widefold" not in disabled and w.shape[0] // 2 >= 32 * 192
+            and w.numel() < 2 ** 30)
+
+
 def for_eight_rows(w):
     """The same for a weight of a product into the residual stream (output and down projection): steps of
     at most 8 rows take it in strips of 8 weight rows with packed tiles where 16-row strips would leave CUs
-    idle (``lib.skinny_strip_rows``, ``lib.tile_weight8``), everything else of few rows in strips of 16."""
-    for_few_rows(w)
+    idle (``lib.skinny_strip_rows``, ``lib.tile_weight8``), everything else of few rows in strips of 16;
+    the copy for those is left out where no step reads it (strips of 8 up to 8 rows, and a K so long that 9 to
+    16 rows go to the kernel of whole lines)."""
+    N, Kd = w.shape
+    if K.skinny_strip_rows(8, N, Kd, EPI_ADD) == 16 or Kd <= 4096 or "wide" in disabled or "wide916" in disabled:
+        for_few_rows(w)
     if ("tiled" not in disabled and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 8 == 0
             and w.is_contiguous() and K.skinny_strip_rows(8, w.shape[0], w.shape[1], EPI_ADD) == 8):
         w.tiled8 = K.tile_weight8(w)
@@ -242,8 +259,7 @@ def _long_k_of_9_to_16_rows(a, out, epilogue, bias):
 def _whole_lines(a, w, epilogue):
     """Whether a folded norm's gated product runs on the kernel that loads whole lines: where it has blocks
     enough for the chip, as for 17 to 64 rows."""
-    return (epilogue == EPI_GATED and a.rows is None and "wide" not in disabled and "widefold" not in disabled
-            and a.xg.shape[0] <= 16 and w.shape[0] // 2 >= 32 * 192 and w.numel() < 2 ** 30)    # (32-bit byte offsets)
+    return epilogue == EPI_GATED and a.rows is None and a.xg.shape[0] <= 16 and gated_on_whole_lines(w)
 
 
 def _streams_rows_for_many_strips(M, w, epilogue):
