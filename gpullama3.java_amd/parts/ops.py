@@ -23,7 +23,11 @@ FUSE_ROWS = 16
 # four layers and the head)
 CHUNK_ROWS = 128
 
-# switches for tests and measurements: names of fast kernels that must not be used
+# switches for tests and measurements: names of fast paths that must not be used. "skinny", "wide", "mfma",
+# "attn_decode", "attn_prefill": a family of kernels; "fused": norms, rotation and cache write folded into
+# products; "tiled", "packed": the weights' copies in operand order (read when an engine is built) and the rows
+# handed over in the packed tiles' order; "widefold", "wide916": the kernel of whole lines for the gated product
+# with a folded norm and for products of 9 to 16 rows over a long K.
 disabled = set()
 
 
