@@ -933,7 +933,8 @@ def epilogue_reference(a, w, epilogue, bias, act, before=None):
     return s + before if epilogue == 1 else s
 
 
-PRODUCTS = ["generic float32", "generic bfloat16", "tiled", "few rows", "few rows, folded norm", "33 to 64 rows"]
+PRODUCTS = ["generic float32", "generic bfloat16", "tiled", "few rows", "few rows, folded norm",
+            "few rows, folded norm, whole lines", "17 to 32 rows", "33 to 64 rows"]
 
 
 @pytest.mark.parametrize("which", PRODUCTS)
@@ -944,7 +945,7 @@ def test_products_with_bias_and_activation(which, epilogue, act):
     that one added twice, to the wrong half or after the activation shows."""
     lib = K()
     rng = np.random.default_rng(len(which) * 7 + epilogue)
-    M = {"tiled": 150, "33 to 64 rows": 40}.get(which, 9)
+    M = {"tiled": 150, "33 to 64 rows": 40, "17 to 32 rows": 21}.get(which, 9)
     N, Kd = 200, 136                                               # output columns: no tile divides them
     dtype = "float32" if which == "generic float32" else "bfloat16"
     wrows = 2 * N if epilogue == 2 else N
@@ -962,16 +963,18 @@ def test_products_with_bias_and_activation(which, epilogue, act):
         lib.gemm_mfma(A, W, out, epilogue, bias=B, act=act)
     elif which == "few rows":
         lib.gemm_skinny(A, W, out, epilogue, bias=B, act=act)
-    elif which == "33 to 64 rows":
+    elif which in ("33 to 64 rows", "17 to 32 rows"):
         lib.gemm_skinny_wide(A, W, out, epilogue, bias=B, act=act)
     else:
         if epilogue == 1:
             pytest.skip("a folded norm feeds store and gated products only")
+        if which.endswith("whole lines") and epilogue != 2:
+            pytest.skip("whole lines take the gated product only")
         x = (rng.standard_normal((M, Kd)) * 2).astype(np.float32)
         nw = (1 + 0.2 * rng.standard_normal(Kd)).astype(np.float32)
         xg = times_weight(x, nw).to(DEV)
         ssq = dev(ssq_partials(x, 3))
-        lib.gemm_skinny_norm(xg, ssq, 3, 1e-5, W, out, epilogue, bias=B, act=act)
+        lib.gemm_skinny_norm(xg, ssq, 3, 1e-5, W, out, epilogue, bias=B, act=act, whole_lines=which.endswith("whole lines"))
         ref_a = xg.float().cpu().numpy() / np.sqrt((x.astype(np.float64) ** 2).mean(1, keepdims=True) + 1e-5)
     ref = epilogue_reference(ref_a, w, epilogue, bias, act, before)
     np.testing.assert_allclose(out.float().cpu().numpy(), ref, atol=tol(dtype) * np.abs(ref).max())
