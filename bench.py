@@ -114,8 +114,6 @@ def main():
     import torch
     import gpullama3_java_amd as g
     from gpullama3_java_amd.engine import Engine
-    from gpullama3_java_amd.parts import ops
-    ops.disabled.update(n for n in args.without.split(",") if n)
 
     shape_name, shape = SHAPES[args.shape]
     context = shape["max_position_embeddings"]
@@ -139,7 +137,8 @@ def main():
         g.write_random_model(tmp, cfg, args.seed)
         print(f"[bench] random {args.layers}-layer model written in {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
         eng = Engine.from_folder(tmp, dtype=args.dtype, max_context=context,
-                                 max_tokens=max(biggest * per_seq, prefill_len + 64), n_slots=biggest)
+                                 max_tokens=max(biggest * per_seq, prefill_len + 64), n_slots=biggest,
+                                 without=args.without)
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
     rng = np.random.default_rng(args.seed)

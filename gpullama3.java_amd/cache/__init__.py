@@ -1,4 +1,4 @@
 from .pages import CacheFull, PagePool, SlotTable
-from .kv_cache import Cache, CacheGroup, KVNeed, StateNeed
+from .kv_cache import Cache, CacheGroup, KVNeed, StateNeed, check_layout
 
-__all__ = ["CacheFull", "PagePool", "SlotTable", "Cache", "CacheGroup", "KVNeed", "StateNeed"]
+__all__ = ["CacheFull", "PagePool", "SlotTable", "Cache", "CacheGroup", "KVNeed", "StateNeed", "check_layout"]

@@ -32,11 +32,20 @@ from .pages import CacheFull, PagePool, SlotTable
 
 @dataclass(frozen=True)
 class KVNeed:
-    """What one run-order entry stores per position."""
+    """What one run-order entry stores per position: keys of ``head_dim`` elements and values of
+    ``v_head_dim`` for each of ``n_kv_heads`` heads. A mixer that keeps one vector per position (a
+    latent that both its keys and its values are made from) asks for ``values=False`` and gets the
+    first array alone."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     dtype: Optional[torch.dtype] = None      # None: the engine's; a mixer whose kernels keep something else says so
+    v_head_dim: Optional[int] = None         # None: as the keys'
+    values: bool = True                      # False: no second array (``layer_kv`` then gives (keys, None))
+
+    @property
+    def value_dim(self):
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)
@@ -44,6 +53,24 @@ class StateNeed:
     """What one run-order entry stores per sequence, whatever its length."""
     elements: int
     dtype: torch.dtype = torch.float32
+
+
+def check_layout(kv_needs, page_size):
+    """The cache lies in the tiles of the attention kernels' operands (``layout.py``): pages of a multiple of 32
+    positions, heads of a multiple of 16 elements. Anything else is refused here, by name, before any
+    memory is taken or any weight is read; the kernels would refuse it at their first launch."""
+    if isinstance(page_size, bool) or not isinstance(page_size, int) or page_size < 32 or page_size % 32:
+        raise ValueError(f"page_size {page_size!r}: a page of the cache must be a positive multiple of 32 positions")
+    for e, need in enumerate(kv_needs):
+        if need is None:
+            continue
+        sizes = [("head_dim", need.head_dim)] + ([("v_head_dim", need.value_dim)] if need.values else [])
+        for key, v in sizes:
+            if v < 16 or v % 16:
+                raise ValueError(f"run-order entry {e}: {key} {v} is not a multiple of 16; the cache keeps heads in "
+                                 "tiles of 16 by 8 elements (head sizes in steps of 16)")
+        if need.n_kv_heads < 1:
+            raise ValueError(f"run-order entry {e}: {need.n_kv_heads} kv heads")
 
 
 class CacheGroup:
@@ -57,7 +84,8 @@ class CacheGroup:
         self.k = torch.zeros((n, n_pages, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
         # values lie transposed inside a page: the order in which the attention kernels' second
         # product reads them (and both in tiles, see layout.py)
-        self.v = torch.zeros((n, n_pages, need.n_kv_heads, need.head_dim, page_size), dtype=dtype, device=device)
+        self.v = (torch.zeros((n, n_pages, need.n_kv_heads, need.value_dim, page_size), dtype=dtype, device=device)
+                  if need.values else None)
         self.table = None            # [n_slots + 1, pages of the longest sequence] int32 on the device
         self.table_host = None       # the same on the host (numpy), the copy that the bookkeeping writes
         self.dirty = {}              # flat place in the table -> page number, not yet on the device
@@ -73,6 +101,7 @@ class Cache:
     def __init__(self, kv_needs, state_needs, max_tokens, max_context, n_slots, dtype, device, page_size=64):
         if max_tokens < 1 or max_context < 1 or n_slots < 1:
             raise ValueError("cache sizes must be positive")
+        check_layout(kv_needs, page_size)
         self.page_size = page_size
         self.max_context = max_context
         self.max_pages_per_seq = -(-max_context // page_size)
@@ -203,21 +232,14 @@ class Cache:
 
     # ---- what the kernels read
     def layer_kv(self, entry):
-        """(K, V) of one entry: K [page, kv head, position in page, head_dim], V [page, kv head, head_dim, position];
-        the last two axes in the kernels' order (``layout.py``)."""
+        """(K, V) of one entry: K [page, kv head, position in page, head_dim], V [page, kv head, v_head_dim, position]
+        (None for a need without values); the last two axes in the kernels' order (``layout.py``)."""
         g, i = self.group_of[entry]
-        return self.groups[g].k[i], self.groups[g].v[i]
+        group = self.groups[g]
+        return group.k[i], (group.v[i] if group.v is not None else None)
 
     def group_index(self, entry):
         return self.group_of[entry][0]
-
-    def block_rows(self, group, slots, width):
-        """Rows of page numbers for ``slots``, padded with the sink page."""
-        rows = []
-        for s in slots:
-            p = self.slots.pages[s][group]
-            rows.append(p + [0] * (width - len(p)))
-        return rows
 
     def slot_state(self, entry):
         return self.state.get(entry)

@@ -97,7 +97,7 @@ class ModelSpec:
     hidden: int
     layers: tuple
     run_order: tuple
-    final_norm: object
+    final_norm: object                # the norm in front of the head; None: the head reads the rows as they are
     max_positions: int
     tie_embeddings: bool
     embedding_name: str

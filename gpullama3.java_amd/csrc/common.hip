@@ -125,6 +125,68 @@ extern "C" int gl3_stage_decode(int* dst, int n_pad, int n, const int* tokens, c
   return 0;
 }
 
+// ---- the input of a step that brings any number of tokens per sequence. The host names, per entry, its
+// slot, the tokens its sequence holds already and the tokens it brings; what the kernels read per TOKEN
+// (position, sequence, row of the block table) is expanded on the device. The host's part travels as one
+// copy from pinned memory, laid out as the device buffer's head:
+//   tokens[T] | cu_seqlens[B+1] | kv_before[B] | slots[B] | wanted rows[W] | positions[T] | seq_of_token[T] | table_rows[T]
+// (the last three are written by the kernel). The caller owns `pinned` until the copy has run.
+__global__ void expand_step_kernel(const int* __restrict__ cu, const int* __restrict__ kv_before,
+                                   const int* __restrict__ slots, int B, int T, int* __restrict__ positions,
+                                   int* __restrict__ seq_of, int* __restrict__ table_rows) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  int lo = 0, hi = B - 1;                 // the entry b with cu[b] <= t < cu[b + 1]
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  positions[t] = kv_before[lo] + (t - cu[lo]);
+  seq_of[t] = lo;
+  table_rows[t] = slots[lo];
+}
+
+extern "C" long gl3_stage_step_ints(int T, int B, int W) { return 4L * T + 3L * B + 1 + W; }
+
+// tokens: T host ints (the entries' tokens one after another); slots, starts, counts: B host ints; want: W packed
+// rows. vocab: every token is checked against it. dev: device, gl3_stage_step_ints(T, B, W) ints; pinned: host
+// memory that the device can read, T + 3 B + 1 + W ints.
+extern "C" int gl3_stage_step(int* dev, int* pinned, const int* tokens, int T, const int* slots, const int* starts,
+                              const int* counts, int B, const int* want, int W, int vocab, hipStream_t stream) {
+  GL3_REQUIRE(dev && pinned && tokens && slots && starts && counts && T > 0 && B > 0 && W >= 0 && (want || W == 0),
+              "gl3_stage_step: bad arguments");
+  int* cu = pinned + T;
+  int* before = cu + B + 1;
+  int* sl = before + B;
+  int* wr = sl + B;
+  cu[0] = 0;
+  for (int b = 0; b < B; ++b) {
+    GL3_REQUIRE(counts[b] > 0 && starts[b] >= 0, "gl3_stage_step: entry %d brings %d tokens at %d", b, counts[b], starts[b]);
+    cu[b + 1] = cu[b] + counts[b];
+    before[b] = starts[b];
+    sl[b] = slots[b];
+  }
+  GL3_REQUIRE(cu[B] == T, "gl3_stage_step: the entries bring %d tokens, %d were given", cu[B], T);
+  for (int t = 0; t < T; ++t) {
+    const int v = tokens[t];
+    GL3_REQUIRE(v >= 0 && v < vocab, "gl3_stage_step: token id %d is outside the vocabulary of %d", v, vocab);
+    pinned[t] = v;
+  }
+  for (int i = 0; i < W; ++i) {
+    GL3_REQUIRE(want[i] >= 0 && want[i] < T, "gl3_stage_step: wanted row %d of %d", want[i], T);
+    wr[i] = want[i];
+  }
+  const long head = (long)T + 3L * B + 1 + W;
+  hipError_t e = hipMemcpyAsync(dev, pinned, (size_t)head * sizeof(int), hipMemcpyHostToDevice, stream);
+  GL3_REQUIRE(e == hipSuccess, "gl3_stage_step: %s", hipGetErrorString(e));
+  int* d_cu = dev + T;
+  int* d_pos = dev + head;
+  expand_step_kernel<<<dim3((T + 255) / 256), dim3(256), 0, stream>>>(d_cu, d_cu + B + 1, d_cu + 2 * B + 1, B, T, d_pos,
+                                                                      d_pos + T, d_pos + 2 * T);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---- launch of an instantiated graph (a captured decode step) on a stream
 extern "C" int gl3_graph_launch(void* graph_exec, hipStream_t stream) {
   GL3_REQUIRE(graph_exec, "gl3_graph_launch: null graph");

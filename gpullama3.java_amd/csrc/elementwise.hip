@@ -136,6 +136,27 @@ extern "C" int gl3_rmsnorm(const float* x, const int* rows, const void* w, int w
   return 0;
 }
 
+// ----------------------------------------------------------------- rows of the residual stream as they are
+// out[r, i] = x[rows[r], i] in the activation type: what the head of a decoder without a final norm reads.
+template <typename TO>
+__global__ void gather_rows_kernel(const float* __restrict__ x, const int* __restrict__ rows, TO* __restrict__ out, int d) {
+  const long r = blockIdx.x;
+  const float* xr = x + (long)rows[r] * d;
+  TO* o = out + r * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_f32<TO>(xr[i]);
+}
+
+extern "C" int gl3_gather_rows(const float* x, const int* rows, void* out, int out_dtype, int n_rows, int d,
+                               hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  GL3_REQUIRE(x && rows && out && n_rows > 0 && d > 0, "gl3_gather_rows: bad arguments (rows=%d d=%d)", n_rows, d);
+  if (out_dtype == GL3_F32) gather_rows_kernel<float><<<n_rows, 256, 0, stream>>>(x, rows, (float*)out, d);
+  else if (out_dtype == GL3_BF16) gather_rows_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(x, rows, (bf16_t*)out, d);
+  else GL3_REQUIRE(false, "gl3_gather_rows: unknown dtype %d", out_dtype);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
 // ----------------------------------------------------------------- slices of a product + rmsnorm
 // A product whose K was cut into slices left its sums as P[slice][row][ldp] (float). Here they
 // are added to the residual rows in slice order, x[row] += P[0][row] + P[1][row] + ..., and the

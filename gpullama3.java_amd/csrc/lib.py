@@ -51,6 +51,7 @@ def _declare(lib):
         "gl3_embed": [P, I, P, P, I, I, P, P, P, F, P, P, P],
         "gl3_scale_f32": [P, F, L, P],
         "gl3_rmsnorm": [P, P, P, I, P, I, I, I, F, P],
+        "gl3_gather_rows": [P, P, P, I, I, I, P],
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, P],
@@ -71,6 +72,7 @@ def _declare(lib):
         "gl3_scatter_i32": [P, L, P, P, I, P],
         "gl3_upload": [P, P, L, P],
         "gl3_stage_decode": [P, I, I, P, P, P, I, P, P],
+        "gl3_stage_step": [P, P, P, I, P, P, P, I, P, I, I, P],
         "gl3_graph_launch": [P, P],
         "gl3_attention_decode": [P, L, P, P, P, P, P, I, P, P, L, P, L, I, I, I, I, I, I, F, I, P],
     }
@@ -219,6 +221,15 @@ def rmsnorm(x, weight, out, eps, rows=None):
         raise KernelError(f"rmsnorm: {x.shape[0]} inputs for {n} outputs")
     _check(library().gl3_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _code(weight, "weight"), _ptr(out),
                                  _code(out, "out"), n, d, float(eps), _stream()), "rmsnorm")
+
+
+def gather_rows(x, rows, out):
+    """out[r] = x[rows[r]] in ``out``'s dtype (x float32; the caller has checked rows < rows of x)."""
+    _dev(x, "x", torch.float32); _dev(rows, "rows", torch.int32); _dev(out, "out")
+    if x.dim() != 2 or out.dim() != 2 or out.shape != (rows.numel(), x.shape[1]):
+        raise KernelError(f"gather_rows: x {tuple(x.shape)}, {rows.numel()} rows, out {tuple(out.shape)}")
+    _check(library().gl3_gather_rows(_ptr(x), _ptr(rows), _ptr(out), _code(out, "out"), out.shape[0], x.shape[1],
+                                     _stream()), "gather_rows")
 
 
 def add_slices_rmsnorm(x, slices, weight=None, out=None, eps=0.0, rows=None):
@@ -800,6 +811,35 @@ def stage_decode(dst, n_pad, tokens, positions, slots, pad_slot, counter=None):
     arr = c_int * n
     _check(library().gl3_stage_decode(_ptr(dst), n_pad, n, arr(*tokens), arr(*positions), arr(*slots), pad_slot,
                                       _ptr(counter), _stream()), "stage_decode")
+
+
+def stage_step_ints(T, B, W):
+    """Elements of the device buffer that ``stage_step`` fills."""
+    return 4 * T + 3 * B + 1 + W
+
+
+def stage_step(dev, pinned, tokens, slots, starts, counts, want, vocab):
+    """The input of a step of any shape into its device buffer ``dev`` (int32):
+    tokens[T] | cu_seqlens[B+1] | kv_before[B] | slots[B] | wanted rows[W] | positions[T] | seq_of_token[T] | table_rows[T].
+    ``tokens`` [T], ``want`` [W]: contiguous int32 numpy arrays (the entries' tokens one after another, packed
+    rows); ``slots``, ``starts``, ``counts``: one int per entry. The host's part travels as one copy out of
+    ``pinned`` (pinned int32 host tensor, free again once that copy has run), the per-token arrays are expanded
+    on the device. Token ids are checked against ``vocab``, counts against ``tokens``, rows against T."""
+    _dev(dev, "dev", torch.int32)
+    T, B, W = int(tokens.size), len(slots), int(want.size)
+    if len(starts) != B or len(counts) != B or B == 0 or T == 0:
+        raise KernelError("stage_step: one slot, start and count per entry, and at least one token")
+    if (tokens.dtype != "int32" or want.dtype != "int32" or not tokens.flags.c_contiguous or not want.flags.c_contiguous
+            or tokens.ndim != 1 or want.ndim != 1):
+        raise KernelError("stage_step: tokens and wanted rows are contiguous int32 arrays")
+    if pinned.is_cuda or not pinned.is_pinned() or pinned.dtype != torch.int32 or pinned.numel() < T + 3 * B + 1 + W:
+        raise KernelError("stage_step: the staging buffer must be pinned int32 host memory of T + 3 B + 1 + W elements")
+    if dev.numel() < 4 * T + 3 * B + 1 + W:
+        raise KernelError("stage_step: the device buffer is too small")
+    arr = c_int * B
+    _check(library().gl3_stage_step(_ptr(dev), c_void_p(pinned.data_ptr()), c_void_p(tokens.ctypes.data), T, arr(*slots),
+                                    arr(*starts), arr(*counts), B, c_void_p(want.ctypes.data if W else 0), W, int(vocab),
+                                    _stream()), "stage_step")
 
 
 def graph_launch(graph_exec):

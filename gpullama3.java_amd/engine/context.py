@@ -52,6 +52,7 @@ class StepContext:
         self.replayed = False              # whether the step's launches are being captured into a graph
         self.max_q_len, self.max_kv_len = max_q_len, max_kv_len
         self.fuse = getattr(engine, "fuse", False)   # few-token steps fold norms and rotation into the products
+        self.disabled = getattr(engine, "without", frozenset())   # fast paths that the engine does without
         self.ssq = None                    # (address of the residual stream, its partial sums of squares, how many)
         self.pending = None                # (address of the residual stream, slices of a product still to be added to it)
         self.kv_len_hint = max_kv_len      # what launch shapes are sized for; a replayed graph keeps its own

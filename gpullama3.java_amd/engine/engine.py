@@ -12,10 +12,12 @@ from __future__ import annotations
 
 import contextlib
 import tempfile
+from collections import OrderedDict
 
+import numpy as np
 import torch
 
-from ..cache import Cache, CacheFull
+from ..cache import Cache, CacheFull, check_layout
 from ..config import config_from_dict, load_config
 from ..parts import DecoderModel
 from ..sampling import DeviceSampler, SamplingParams
@@ -58,24 +60,44 @@ class _DecodeGraph:
             self.graph.replay()
 
 
+GRAPHS_KEPT = 24    # captured decode steps that an engine keeps (each owns its logits and the sampler's scratch)
+
+
+def _without(without, weight_copies):
+    from ..parts import ops
+    names = set(ops.switches(without))
+    if not weight_copies:
+        names.add("tiled")
+    return frozenset(names)
+
+
 class Engine:
-    """``config``: a registered architecture's configuration; ``weights``: stored name -> device tensor."""
+    """``config``: a registered architecture's configuration; ``weights``: stored name -> device tensor.
+
+    ``weight_copies``: a bfloat16 engine keeps, beside each matrix that decode steps read (QKV, output and down
+    projection, the head, and the gate/up rows of small models), a copy in the order in which the matrix cores
+    take it: 2.5 -> 4.0 GB for the 1B shape, for about 5% more tokens a second at batch 8. False leaves the
+    copies out. ``without``: names of fast paths (``parts.ops.SWITCHES``) this engine does not use, for
+    measurements and tests. ``max_graphs``: captured decode steps kept at a time; the least recently used
+    one goes first."""
 
     def __init__(self, config, weights, dtype="bfloat16", device="cuda:0", max_tokens=None, max_context=None,
-                 n_slots=None, page_size=64, use_graphs=True):
+                 n_slots=None, page_size=64, use_graphs=True, without=(), weight_copies=True, max_graphs=GRAPHS_KEPT):
         self.device = _require_gpu(device)
         if self.device.index is None:
             self.device = torch.device("cuda", torch.cuda.current_device())
         self.dtype = _dtype(dtype)
+        self.without = _without(without, weight_copies)
         limit = config.max_position_embeddings
         max_context = limit if max_context is None or max_context < 0 else min(max_context, limit)
         self.config = config.with_context_length(max_context)
         self.spec = self.config.model_spec()
         self.max_context = max_context
         max_tokens = max_tokens or max_context
-        self.model = DecoderModel(self.spec, self.dtype, self.device)
-        self.model.load(weights)
+        self.model = DecoderModel(self.spec, self.dtype, self.device, without=self.without)
         kv_needs, state_needs = self.model.cache_needs()
+        check_layout(kv_needs, page_size)                 # before the weights are stacked and copied
+        self.model.load(weights)
         if n_slots is None:
             n_slots = max(1, min(-(-max_tokens // page_size), 256))
         with torch.cuda.device(self.device):
@@ -91,8 +113,13 @@ class Engine:
         safe = all(getattr(p, "graph_safe", False) for p in parts)
         self.use_graphs = bool(use_graphs and safe)
         self.fuse = bool(self.dtype == torch.bfloat16 and safe)
-        self._graphs = {}
+        if max_graphs < 1:
+            raise ValueError("max_graphs must be at least 1")
+        self.max_graphs = int(max_graphs)
+        self._graphs = OrderedDict()                      # (batch bucket, context bucket, kind) -> captured step
         self._graphs_generation = 0
+        self._stage_ring = [(None, None)] * 4             # (pinned buffer, event after the copy out of it)
+        self._stage_next = 0
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -101,6 +128,7 @@ class Engine:
         dev = _require_gpu(device)
         config = load_config(folder)
         probe = DecoderModel(config.model_spec(), _dtype(dtype), "cpu")
+        check_layout(probe.cache_needs()[0], kw.get("page_size", 64))       # before the weights are read
         weights = load_weights(folder, probe.expected(), _dtype(dtype), dev)
         return cls(config, weights, dtype=dtype, device=device, **kw)
 
@@ -145,61 +173,55 @@ class Engine:
     def step(self, entries, want="last"):
         """Run the tokens of ``entries = [(slot, tokens), ...]`` and return logits.
 
-        Each sequence's tokens are appended at its own length. ``want``: "last"
-        (the last token of every entry), "all", "none", or a list with one list of
-        indices into each entry's tokens. Returns ``[rows, vocab]`` float32 on the
+        Each sequence's tokens (a list, a tuple or an array of integers) are appended at its own
+        length. ``want``: "last" (the last token of every entry), "all", "none", or a list with one
+        list of indices into each entry's tokens. Returns ``[rows, vocab]`` float32 on the
         device, rows in the order of the entries and of their wanted indices: a tensor
         of its own, which later steps do not touch. If the cache has no room,
         ``CacheFull`` is raised and nothing has changed.
         """
         B = len(entries)
-        if B == 0:
-            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-        if want == "last" and self.use_graphs and all(len(e[1]) == 1 for e in entries):
-            return self._step_decode(entries)
-        slots = [int(s) for s, _ in entries]
-        if len(set(slots)) != B:
-            raise ValueError("a slot appears twice in one step")
         V = self.spec.vocab_size
-        token_ids, positions, seq_of, cu, kv_before, want_rows, slot_of = [], [], [], [0], [], [], []
-        q_lens = []
-        for b, (slot, toks) in enumerate(entries):
-            toks = [int(t) for t in toks]
-            if not toks:
-                raise ValueError(f"entry {b} brings no token")
-            bad = [t for t in toks if not 0 <= t < V]
-            if bad:
-                raise ValueError(f"entry {b}: token id {bad[0]} is outside the vocabulary of {V}")
-            start = self.cache.length(slot)
-            n = len(toks)
-            if want == "last":
-                idx = [n - 1]
-            elif want == "all":
-                idx = list(range(n))
-            elif want == "none" or want is None:
-                idx = []
-            else:
+        if B == 0:
+            return torch.empty((0, V), dtype=torch.float32, device=self.device)
+        slots, arrays = self._entries(entries)
+        counts = [a.size for a in arrays]
+        single = max(counts) == 1
+        if single and want != "last" and isinstance(want, (list, tuple)) and len(want) == B \
+                and all(len(w) == 1 and w[0] == 0 for w in want):
+            want = "last"                         # the only token of every entry: the same step
+        if single and want == "last" and self.use_graphs:
+            return self._step_decode(slots, [int(a[0]) for a in arrays])
+        starts = [self.cache.length(s) for s in slots]
+        T = sum(counts)
+        tokens = arrays[0] if B == 1 else np.concatenate(arrays)
+        if want == "last":
+            rows = np.cumsum(counts, dtype=np.int32) - 1
+        elif want == "all":
+            rows = np.arange(T, dtype=np.int32)
+        elif want == "none" or want is None:
+            rows = np.empty(0, dtype=np.int32)
+        else:
+            if len(want) != B:
+                raise ValueError(f"{len(want)} lists of wanted places for {B} entries")
+            rows, first = [], 0
+            for b, n in enumerate(counts):
                 idx = [int(i) for i in want[b]]
                 if any(not 0 <= i < n for i in idx):
                     raise ValueError(f"entry {b}: a wanted place is outside its {n} tokens")
-            want_rows.extend(cu[-1] + i for i in idx)
-            token_ids.extend(toks)
-            positions.extend(range(start, start + n))
-            seq_of.extend([b] * n)
-            slot_of.extend([slots[b]] * n)
-            cu.append(cu[-1] + n)
-            kv_before.append(start)
-            q_lens.append(n)
-        self.cache.reserve({s: n for s, n in zip(slots, q_lens)})      # raises CacheFull, nothing changed
-        T = cu[-1]
-        max_kv = max(k + n for k, n in zip(kv_before, q_lens))
-        decode = all(n == 1 for n in q_lens)
+                rows.extend(first + i for i in idx)
+                first += n
+            rows = np.asarray(rows, dtype=np.int32)
+        self.cache.reserve(dict(zip(slots, counts)))                   # raises CacheFull, nothing changed
+        W = int(rows.size)
+        max_kv = max(k + n for k, n in zip(starts, counts))
+        from ..csrc import lib as K
         with self._on_device():
             self.cache.flush_tables()
-            ctx = StepContext(self, T, B, q_lens, kv_before, slots, decode=decode, max_q_len=max(q_lens),
-                              max_kv_len=max_kv)
-            dev = torch.tensor(token_ids + positions + seq_of + slot_of + cu + kv_before + slots + want_rows,
-                               dtype=torch.int32).to(self.device)
+            ctx = StepContext(self, T, B, counts, starts, slots, decode=single, max_q_len=max(counts), max_kv_len=max_kv)
+            dev = torch.empty(K.stage_step_ints(T, B, W), dtype=torch.int32, device=self.device)
+            K.stage_step(dev, self._staging(T + 3 * B + 1 + W), tokens, slots, starts, counts, rows, V)
+            self._staged()
             o = 0
 
             def cut(n):
@@ -208,34 +230,66 @@ class Engine:
                 o += n
                 return t
 
-            ctx.token_ids, ctx.positions, ctx.seq_of_token, ctx.table_rows = cut(T), cut(T), cut(T), cut(T)
-            ctx.cu_seqlens, ctx.kv_before, ctx.slot_ids = cut(B + 1), cut(B), cut(B)
+            ctx.token_ids, ctx.cu_seqlens, ctx.kv_before, ctx.slot_ids = cut(T), cut(B + 1), cut(B), cut(B)
+            want_rows = cut(W)
+            ctx.positions, ctx.seq_of_token, ctx.table_rows = cut(T), cut(T), cut(T)
             ctx.seq_rows = ctx.slot_ids
-            rows = cut(len(want_rows))
             ctx._tables = [self.cache.device_table(g) for g in range(len(self.cache.groups))]
-            logits = self.model.forward(ctx, rows)
-        for s, n in zip(slots, q_lens):
+            logits = self.model.forward(ctx, want_rows)
+        for s, n in zip(slots, counts):
             self.cache.advance(s, n)
         return logits
+
+    def _entries(self, entries):
+        """What every step checks before anything changes: ``(slots, one int32 array of tokens per entry)``.
+        Slots are integers that appear once; tokens are integers inside the vocabulary, at least one an entry."""
+        V = self.spec.vocab_size
+        slots, arrays = [], []
+        for b, (slot, toks) in enumerate(entries):
+            if type(toks) is list and len(toks) == 1 and type(toks[0]) is int:       # (the usual decode step)
+                a = np.array(toks, dtype=np.int64)
+            else:
+                a = np.asarray(toks.cpu() if isinstance(toks, torch.Tensor) else toks)
+                if a.ndim == 0:
+                    a = a.reshape(1)
+                if a.ndim != 1 or (a.size and a.dtype.kind not in "iu"):
+                    raise ValueError(f"entry {b}: tokens must be a flat sequence of integers")
+            if a.size == 0:
+                raise ValueError(f"entry {b} brings no token")
+            lo, hi = int(a.min()), int(a.max())
+            if lo < 0 or hi >= V:
+                raise ValueError(f"entry {b}: token id {lo if lo < 0 else hi} is outside the vocabulary of {V}")
+            slots.append(int(slot))
+            arrays.append(a.astype(np.int32, copy=False))
+        if len(set(slots)) != len(slots):
+            raise ValueError("a slot appears twice in one step")
+        return slots, arrays
+
+    def _staging(self, n):
+        """Pinned host memory for the next step's input: one of a ring of buffers, free once the copy out of it
+        (of the step that used it last) has run."""
+        ring = self._stage_ring
+        self._stage_next = (self._stage_next + 1) % len(ring)
+        buf, event = ring[self._stage_next]
+        if event is not None:
+            event.synchronize()
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(4096, 2 * n), dtype=torch.int32).pin_memory()
+        ring[self._stage_next] = (buf, event)
+        return buf
+
+    def _staged(self):
+        buf, event = self._stage_ring[self._stage_next]
+        if event is None:
+            event = torch.cuda.Event()
+        event.record()
+        self._stage_ring[self._stage_next] = (buf, event)
 
     # ------------------------------------------------------------------ decode steps from captured graphs
     @property
     def decode_run_length(self):
         return RUN_LENGTH if self.use_graphs else 1
 
-    def _decode_entries(self, entries):
-        """Checks of a step that brings one token per sequence; returns (slots, tokens, lengths)."""
-        V = self.spec.vocab_size
-        slots, tokens = [], []
-        for slot, tok in entries:
-            t = int(tok[0]) if isinstance(tok, (list, tuple)) else int(tok)
-            if not 0 <= t < V:
-                raise ValueError(f"token id {t} is outside the vocabulary of {V}")
-            slots.append(int(slot))
-            tokens.append(t)
-        if len(set(slots)) != len(slots):
-            raise ValueError("a slot appears twice in one step")
-        return slots, tokens, [self.cache.length(s) for s in slots]
 
     def _on_device(self):
         """The engine's device as the current one (entering a device context costs as much as a launch)."""
@@ -243,14 +297,14 @@ class Engine:
             return contextlib.nullcontext()
         return torch.cuda.device(self.device)
 
-    def _step_decode(self, entries):
-        """One token for each of B sequences: the step's tokens, positions and slot numbers are
+    def _step_decode(self, slots, tokens):
+        """One token for each of B sequences (checked by ``_entries``): the step's tokens, positions and slot numbers are
         written into the captured step's input buffer by a small kernel that carries them in its
         launch, and the captured launches are replayed. The batch is padded to a bucket; a padded
         entry is a one-token sequence in the cache's sink slot, so it reads and writes nothing
         that a real sequence owns, and its logits are not returned."""
         from ..csrc import lib as K
-        slots, tokens, starts = self._decode_entries(entries)
+        starts = [self.cache.length(s) for s in slots]
         B = len(slots)
         cache = self.cache
         cache.reserve_one_each(slots)                                  # raises CacheFull, nothing changed
@@ -272,7 +326,11 @@ class Engine:
         if not self.use_graphs or not 1 <= n <= RUN_LENGTH:
             raise ValueError(f"a run takes 1..{RUN_LENGTH} steps on an engine that replays graphs")
         from ..csrc import lib as K
-        slots, tokens, starts = self._decode_entries(entries)
+        slots, arrays = self._entries([(s, [t] if isinstance(t, int) else t) for s, t in entries])
+        if any(a.size != 1 for a in arrays):
+            raise ValueError("a run of decode steps starts from one token per sequence")
+        tokens = [int(a[0]) for a in arrays]
+        starts = [self.cache.length(s) for s in slots]
         B = len(slots)
         self.cache.reserve({s: n for s in slots})
         with self._on_device():
@@ -306,12 +364,18 @@ class Engine:
         key = (B_pad, kv_bucket, run)
         dg = self._graphs.get(key)
         if dg is None:
+            if len(self._graphs) >= self.max_graphs:
+                torch.cuda.synchronize(self.device)                      # no replay of it is still running
+            while len(self._graphs) >= self.max_graphs:                  # the least recently used one goes
+                self._graphs.popitem(last=False)
             dg = self._capture(B_pad, kv_bucket, run)
             if self._graphs_generation != self.workspace.generation:    # the warm-up grew a buffer
                 self._graphs.clear()
                 self._graphs_generation = self.workspace.generation
                 dg = self._capture(B_pad, kv_bucket, run)
             self._graphs[key] = dg
+        else:
+            self._graphs.move_to_end(key)
         return dg
 
     def _capture(self, B_pad, kv_bucket, run=False):

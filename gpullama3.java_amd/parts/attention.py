@@ -21,6 +21,7 @@ from .base import build_part, register_part
 
 class GQAAttention:
     graph_safe = True      # kernel launches on the current stream only, sizes fixed by (T, B)
+    adds_only = True       # never reads the residual rows: sums of the product before it may still lie in slices
 
     def __init__(self, spec, dtype, device):
         self.spec, self.dtype = spec, dtype
@@ -57,9 +58,10 @@ class GQAAttention:
         weights[n["q"]], weights[n["k"]], weights[n["v"]] = (
             self.w_qkv[:qn], self.w_qkv[qn:qn + kn], self.w_qkv[qn + kn:])
         self.w_q = self.w_qkv[:qn]
+        without = getattr(self, "without", frozenset())      # the fast paths that the engine does without
         ops.for_few_rows(self.w_qkv, (self.H, self.Kh, self.hs, self.position is not None,
-                                      bool(self.position is not None and self.position.adjacent)))
-        self.w_o = ops.for_eight_rows(weights[n["o"]])
+                                      bool(self.position is not None and self.position.adjacent)), without=without)
+        self.w_o = ops.for_eight_rows(weights[n["o"]], without=without)
         if self.biased:     # the epilogues read biases as float
             self.b_qkv = torch.cat([weights[n[k]].float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()
         if "o_bias" in n:

@@ -5,6 +5,7 @@ stream keeps the sum (J/inference/InferenceCore.java:74, :151, :154, :172).
 """
 from __future__ import annotations
 
+from . import ops
 from .base import build_part, register_part
 
 
@@ -27,14 +28,24 @@ class PreNormBlock:
 
     def forward(self, ctx, x, run, norm_after=None):
         """``norm_after``: the norm that reads the residual rows after this block, if known."""
-        h = self.mixer_norm(ctx, x)
+        h = self._whole_rows_for(self.mixer_norm, "takes_slices", ctx, x)(ctx, x)
         ctx.next_norm = self.ffn_norm if self.ffn is not None else norm_after
-        self.mixer.forward(ctx, h, x, run)
+        self._whole_rows_for(self.mixer, "adds_only", ctx, x).forward(ctx, h, x, run)
         if self.ffn is not None:
-            h = self.ffn_norm(ctx, x)
+            h = self._whole_rows_for(self.ffn_norm, "takes_slices", ctx, x)(ctx, x)
             ctx.next_norm = norm_after
-            self.ffn.forward(ctx, h, x)
+            self._whole_rows_for(self.ffn, "adds_only", ctx, x).forward(ctx, h, x)
         ctx.next_norm = None
+
+    @staticmethod
+    def _whole_rows_for(part, declares, ctx, x):
+        """A product of 17 or more rows may have left its sums in slices beside the residual rows. A norm
+        that adds them up itself says so (``takes_slices``), a mixer or feed-forward that only adds to the rows
+        says that (``adds_only``); for any other part the rows are made whole before it runs, so a part that
+        knows nothing of slices reads what it expects."""
+        if not getattr(part, declares, False):
+            ops.settle_residual(ctx, x)
+        return part
 
 
 register_part("block", "prenorm", PreNormBlock)

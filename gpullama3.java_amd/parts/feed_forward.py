@@ -15,6 +15,7 @@ from .base import register_part
 
 class GatedFeedForward:
     graph_safe = True      # kernel launches on the current stream only, sizes fixed by (T, B)
+    adds_only = True       # never reads the residual rows: sums of the product before it may still lie in slices
 
     def __init__(self, spec, dtype, device):
         if spec.activation not in ACTIVATIONS:
@@ -43,8 +44,9 @@ class GatedFeedForward:
         dt = g.dtype if g.dtype == u.dtype else torch.float32
         self.w_gate_up = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
         weights[n["gate"]], weights[n["up"]] = self.w_gate_up[:self.F], self.w_gate_up[self.F:]
-        ops.for_gated(self.w_gate_up)
-        self.w_down = ops.for_eight_rows(weights[n["down"]])
+        without = getattr(self, "without", frozenset())      # the fast paths that the engine does without
+        ops.for_gated(self.w_gate_up, without=without)
+        self.w_down = ops.for_eight_rows(weights[n["down"]], without=without)
         if self.biased:     # the epilogues read biases as float
             self.b_gate_up = torch.cat([weights[n["gate_bias"]].float(), weights[n["up_bias"]].float()]).contiguous()
         if "down_bias" in n:

@@ -21,7 +21,8 @@ def expected_tensors(spec, dtype=torch.float32, device="cpu"):
         out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden))
     if spec.position_table_name is not None:
         out[spec.position_table_name] = TensorSpec((spec.max_positions, spec.hidden))
-    out.update(_norm_tensors(spec.final_norm))
+    if spec.final_norm is not None:
+        out.update(_norm_tensors(spec.final_norm))
     for b in spec.layers:
         block = build_part("block", b, dtype=dtype, device=device)
         for p in block.parts():
@@ -47,10 +48,17 @@ def _norm_tensors(spec):
 
 
 class DecoderModel:
-    def __init__(self, spec, dtype, device):
+    """``without``: names of fast paths (``ops.SWITCHES``) that this model's engine does without; every part
+    finds them as its attribute ``without`` when it loads its weights."""
+
+    def __init__(self, spec, dtype, device, without=frozenset()):
         self.spec, self.dtype, self.device = spec, dtype, device
+        self.without = ops.switches(without)
         self.blocks = [build_part("block", b, dtype=dtype, device=device) for b in spec.layers]
-        self.final_norm = build_part("norm", spec.final_norm, dtype=dtype)
+        self.final_norm = build_part("norm", spec.final_norm, dtype=dtype) if spec.final_norm is not None else None
+        for part in [p for b in self.blocks for p in b.parts()] + [self.final_norm]:
+            if part is not None:
+                part.without = self.without
         self.runs = []
         for e, r in enumerate(spec.run_order):
             if not 0 <= r.layer < len(self.blocks):
@@ -69,7 +77,8 @@ class DecoderModel:
             out[self.spec.head_name] = TensorSpec((self.spec.vocab_size, self.spec.hidden))
         if self.spec.position_table_name is not None:
             out[self.spec.position_table_name] = TensorSpec((self.spec.max_positions, self.spec.hidden))
-        out.update(self.final_norm.tensors())
+        if self.final_norm is not None:
+            out.update(self.final_norm.tensors())
         for b in self.blocks:
             for p in b.parts():
                 out.update(p.tensors())
@@ -79,10 +88,11 @@ class DecoderModel:
         self.weights = weights
         self.embedding = weights[self.spec.embedding_name]
         self.head = self.embedding if self.spec.head_name is None else weights[self.spec.head_name]
-        ops.for_few_rows(self.head)
+        ops.for_few_rows(self.head, without=self.without)
         if self.spec.position_table_name is not None:
             self.position_table = weights[self.spec.position_table_name].to(self.embedding.dtype)
-        self.final_norm.load(weights)
+        if self.final_norm is not None:
+            self.final_norm.load(weights)
         for b in self.blocks:
             for p in b.parts():
                 p.load(weights)
@@ -134,7 +144,13 @@ class DecoderModel:
         n = want_rows.numel()
         logits = ctx.logits_buffer(n, self.spec.vocab_size)
         if n:
-            h = self.final_norm(ctx, x, rows=want_rows, name="final_normed")
+            if self.final_norm is not None:
+                h = self.final_norm(ctx, x, rows=want_rows, name="final_normed")
+            else:
+                # a decoder without a final norm: the head reads the wanted rows as they are
+                ops.settle_residual(ctx, x)
+                h = ctx.buffer("head_rows", (n, self.spec.hidden), self.dtype)
+                K.gather_rows(x, want_rows, h)
             ops.linear(h, self.head, logits, ops.EPI_STORE, ctx)
             if self.spec.logit_scale is not None:
                 K.scale_(logits, self.spec.logit_scale)

@@ -14,6 +14,7 @@ from .ops import Normed
 class RMSNorm:
     graph_safe = True      # kernel launches on the current stream only, sizes fixed by (T, B)
     folds = True           # a product can take over this norm's work (see ``ops.Normed``)
+    takes_slices = True    # adds up the slices that the product before it left, while it reads the rows anyway
 
     def __init__(self, spec, dtype):
         self.dim, self.eps, self.dtype = spec.dim, spec.eps, dtype

@@ -23,50 +23,68 @@ FUSE_ROWS = 16
 # four layers and the head)
 CHUNK_ROWS = 128
 
-# switches for tests and measurements: names of fast paths that must not be used. "skinny", "wide", "mfma",
-# "attn_decode", "attn_prefill": a family of kernels; "fused": norms, rotation and cache write folded into
-# products; "tiled", "packed": the weights' copies in operand order (read when an engine is built) and the rows
-# handed over in the packed tiles' order; "widefold", "wide916": the kernel of whole lines for the gated product
-# with a folded norm and for products of 9 to 16 rows over a long K.
-disabled = set()
+# Switches for tests and measurements: names of fast paths that an engine must not use (``Engine(without=...)``;
+# a step reads them as ``ctx.disabled``, a part that makes copies of its weights as its attribute ``without``, which
+# the decoder sets before ``load``). "skinny", "wide", "mfma", "attn_decode", "attn_prefill": a family of kernels;
+# "fused": norms, rotation and cache write folded into products; "tiled", "packed": the weights' copies in operand
+# order and the rows handed over in the packed tiles' order; "widefold", "wide916": the kernel of whole lines for
+# the gated product with a folded norm and for products of 9 to 16 rows over a long K.
+SWITCHES = frozenset({"skinny", "wide", "mfma", "attn_decode", "attn_prefill", "fused", "tiled", "packed", "widefold",
+                      "wide916"})
+_NONE = frozenset()
 
 
-def for_few_rows(w, qkv=None):
+def switches(names):
+    """``names`` (a string with commas, or any collection) as a frozen set; an unknown name is an error."""
+    if isinstance(names, str):
+        names = [n for n in names.split(",") if n]
+    names = frozenset(names or ())
+    if names - SWITCHES:
+        raise ValueError(f"unknown fast path {sorted(names - SWITCHES)}; known: {sorted(SWITCHES)}")
+    return names
+
+
+def _off(ctx):
+    """The fast paths that the step's engine has switched off."""
+    return getattr(ctx, "disabled", _NONE) if ctx is not None else _NONE
+
+
+def for_few_rows(w, qkv=None, without=_NONE):
     """Gives a bfloat16 weight on the GPU whose products are often ones of few rows (a decode step's
     QKV, gate/up and head) a second copy in the order in which the matrix cores take it as an operand
     (``lib.tile_weight``): the kernels that keep the step's rows in registers then read 1 KB of
     consecutive memory per instruction, where rows of ``w`` itself put every lane on a line of its own
     (gate/up 20.7 -> 19.2 us, the head 118 -> 103 us alone at 8 rows). Costs the weight's size again.
     ``qkv``: the stacked q, k, v rows of an attention, ``(n_heads, n_kv, head_dim, rotated, adjacent)``."""
-    if ("tiled" not in disabled and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 16 == 0
+    if ("tiled" not in without and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 16 == 0
             and w.is_contiguous()):
         w.tiled = K.tile_weight(w, qkv)
     return w
 
 
-def for_gated(w):
+def for_gated(w, without=_NONE):
     """The stacked gate and up rows of a feed-forward: the copy of ``for_few_rows`` only where a product of few
     rows reads it; the kernel of whole lines, which takes the large ones, reads the rows as they are stored."""
-    return w if gated_on_whole_lines(w) else for_few_rows(w)
+    return w if gated_on_whole_lines(w, without) else for_few_rows(w, without=without)
 
 
-def gated_on_whole_lines(w):
+def gated_on_whole_lines(w, without=_NONE):
     """Whether the gated products of few rows over ``w`` (2N rows) run on the kernel that loads whole lines:
     where it has blocks enough for the chip, and 32-bit byte offsets reach all of ``w``."""
-    return ("wide" not in disabled and "widefold" not in disabled and w.shape[0] // 2 >= 32 * 192
+    return ("wide" not in without and "widefold" not in without and w.shape[0] // 2 >= 32 * 192
             and w.numel() < 2 ** 30)
 
 
-def for_eight_rows(w):
+def for_eight_rows(w, without=_NONE):
     """The same for a weight of a product into the residual stream (output and down projection): steps of
     at most 8 rows take it in strips of 8 weight rows with packed tiles where 16-row strips would leave CUs
     idle (``lib.skinny_strip_rows``, ``lib.tile_weight8``), everything else of few rows in strips of 16;
     the copy for those is left out where no step reads it (strips of 8 up to 8 rows, and a K so long that 9 to
     16 rows go to the kernel of whole lines)."""
     N, Kd = w.shape
-    if K.skinny_strip_rows(8, N, Kd, EPI_ADD) == 16 or Kd <= 4096 or "wide" in disabled or "wide916" in disabled:
-        for_few_rows(w)
-    if ("tiled" not in disabled and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 8 == 0
+    if K.skinny_strip_rows(8, N, Kd, EPI_ADD) == 16 or Kd <= 4096 or "wide" in without or "wide916" in without:
+        for_few_rows(w, without=without)
+    if ("tiled" not in without and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 8 == 0
             and w.is_contiguous() and K.skinny_strip_rows(8, w.shape[0], w.shape[1], EPI_ADD) == 8):
         w.tiled8 = K.tile_weight8(w)
     return w
@@ -139,7 +157,7 @@ def _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias=None, act="silu"):
     N = out.shape[1]
     if epilogue != EPI_ADD:
         for lo, hi in chunks:
-            linear(a[lo:hi], w, out[lo:hi], epilogue, bias=bias, act=act)
+            linear(a[lo:hi], w, out[lo:hi], epilogue, ctx, bias=bias, act=act)
         return
     slices = K.wide_slices(N, Kd) if bias is None else 1     # (a bias is added once: no slices of K with one)
     if slices < 2:
@@ -166,7 +184,7 @@ def packs_rows(ctx, h, w_first, w_second, x):
     cache takes them in a third of the time."""
     M = h.shape[0]
     F = w_second.shape[1]
-    return (isinstance(h, Normed) and M <= 8 and not disabled & {"packed", "fused", "skinny"}
+    return (isinstance(h, Normed) and M <= 8 and not _off(ctx) & {"packed", "fused", "skinny"}
             and w_first.dtype == torch.bfloat16 and w_second.dtype == torch.bfloat16 and x.dtype == torch.float32
             and w_first.shape[0] == 2 * F and F % 8 == 0 and w_second.stride(0) % 8 == 0 and w_second.data_ptr() % 16 == 0
             and K.gemm_skinny_norm_fits(h.xg, w_first, _BF16_OUT, EPI_GATED)
@@ -178,6 +196,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
     residual stream. ``bias`` (float32, one per row of ``w``) is added to the sums before the
     epilogue's own rule; ``act`` is the gated epilogue's activation (``lib.ACTIVATIONS``).
     ``pack_out`` / ``a_packed``: ``out`` / ``a`` is a ``lib.packed_rows`` buffer (where ``packs_rows`` said so)."""
+    disabled = _off(ctx if ctx is not None else getattr(a, "ctx", None))
     if pack_out:
         return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act,
                                   pack_out=True, whole_lines=_whole_lines(a, w, epilogue))
@@ -210,7 +229,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
         if (_streams_rows_for_many_strips(a.shape[0], w, epilogue) and "mfma" not in disabled
                 and K.gemm_mfma_fits(a, w, out, epilogue)):
             return K.gemm_mfma(a, w, out, epilogue, bias=bias)
-        if ("wide" not in disabled and (a.shape[0] > FUSE_ROWS or _long_k_of_9_to_16_rows(a, out, epilogue, bias))
+        if ("wide" not in disabled and (a.shape[0] > FUSE_ROWS or _long_k_of_9_to_16_rows(a, out, epilogue, bias, disabled))
                 and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx, bias, act)):
             return
         if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
@@ -252,7 +271,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
         residual_written(ctx, out)
 
 
-def _long_k_of_9_to_16_rows(a, out, epilogue, bias):
+def _long_k_of_9_to_16_rows(a, out, epilogue, bias, disabled=_NONE):
     """A product of 9 to 16 rows into the residual stream over a K too long for the kernel that keeps its rows
     in registers: strips of 8 weight rows leave half of every tile idle there, and the kernel of whole lines
     with K in slices is faster even with the norm kernel that then adds the slices."""
@@ -263,7 +282,7 @@ def _long_k_of_9_to_16_rows(a, out, epilogue, bias):
 def _whole_lines(a, w, epilogue):
     """Whether a folded norm's gated product runs on the kernel that loads whole lines: where it has blocks
     enough for the chip, as for 17 to 64 rows."""
-    return epilogue == EPI_GATED and a.rows is None and a.xg.shape[0] <= 16 and gated_on_whole_lines(w)
+    return epilogue == EPI_GATED and a.rows is None and a.xg.shape[0] <= 16 and gated_on_whole_lines(w, _off(a.ctx))
 
 
 def _streams_rows_for_many_strips(M, w, epilogue):
@@ -277,6 +296,7 @@ def _streams_rows_for_many_strips(M, w, epilogue):
 
 def _linear_wide(a, w, out, epilogue, ctx, bias=None, act="silu"):
     """Products of 17 to 64 rows where another kernel than the skinny one is faster. True when done."""
+    disabled = _off(ctx)
     M, Kd = a.shape
     N = out.shape[1]
     if epilogue == EPI_GATED:
@@ -318,6 +338,7 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
     with the H*hs query columns (returned), k rotated and v into the cache. One kernel when
     ``h`` is a ``Normed`` and the shapes allow, else product and rotation apart (always apart with
     a ``bias``, float32 over the stacked q, k, v rows, which is added before the rotation)."""
+    disabled = _off(ctx)
     T = h.shape[0]
     page = k_cache.shape[2]
     cos, sin = (rotary.cos, rotary.sin) if rotary is not None else (None, None)
@@ -352,6 +373,7 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
 
 def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_dim, window, scale):
     page = k_cache.shape[2]          # keys are [page, kv head, position in page, head_dim]
+    disabled = _off(ctx)
     if q.dtype == torch.bfloat16:
         if (ctx.decode and "attn_decode" not in disabled and K.has("gl3_attention_decode")
                 and K.attention_decode_fits(head_dim, n_heads, n_kv, page)):

@@ -124,12 +124,12 @@ def test_random_traffic_keeps_the_books():
     assert all(g.pool.n_free == t for g, t in zip(c.groups, total_pages))
 
 
-def test_block_rows_pad_with_the_sink():
+def test_a_slots_table_row_names_its_pages_then_the_sink():
     c = make()
     a = c.take_slot()
     c.reserve({a: 70})
-    rows = c.block_rows(0, [a], 4)
-    assert rows[0][:2] == c.slots.pages[a][0] and rows[0][2:] == [0, 0]
+    row = c.groups[0].table_host[a].tolist()
+    assert row[:2] == c.slots.pages[a][0] and not any(row[2:])
 
 
 def test_a_group_with_a_window_gives_back_the_pages_behind_it():
@@ -143,7 +143,7 @@ def test_a_group_with_a_window_gives_back_the_pages_behind_it():
     assert all(c.slots.pages[s][0]) and full.n_free == 8 - 3    # the group without a window keeps everything
     c.reserve({s: 200}); c.advance(s, 200)                      # 334 tokens: from 265 on, pages 4 and 5 of 6
     assert [bool(p) for p in c.slots.pages[s][1]] == [False] * 4 + [True] * 2 and windowed.n_free == 8 - 2
-    assert c.block_rows(1, [s], 7)[0][:4] == [0, 0, 0, 0]       # the places of the pages given back point at the sink
+    assert c.groups[1].table_host[s, :4].tolist() == [0, 0, 0, 0]    # the places of the pages given back point at the sink
     c.give_back_slot(s)
     assert full.n_free == 8 and windowed.n_free == 8
 
@@ -169,6 +169,65 @@ def test_the_table_of_every_group_follows_the_pages():
     assert all(not g.dirty for g in c.groups)
     c.reserve({b: 60}); c.advance(b, 60)                     # b's second page
     assert all(list(g.dirty) == [b * W + 1] for g in c.groups)
+
+
+def test_sizes_that_the_tiles_do_not_fit_are_refused_when_the_cache_is_built():
+    """Pages of a multiple of 32 positions and heads of a multiple of 16 elements: refused by name before
+    any memory is taken, not by the first kernel launch."""
+    def build(needs, **kw):
+        return Cache(needs, [None] * len(needs), 256, 256, 2, torch.float32, "cpu", **kw)
+    with pytest.raises(ValueError, match="head_dim 24"):
+        build([KVNeed(2, 16), KVNeed(2, 24)])
+    with pytest.raises(ValueError, match="v_head_dim 40"):
+        build([KVNeed(2, 16, v_head_dim=40)])
+    for page in (48, 16, 0, 70):
+        with pytest.raises(ValueError, match="page_size"):
+            build([KVNeed(2, 16)], page_size=page)
+    assert build([KVNeed(2, 16)], page_size=96).page_size == 96
+    build([KVNeed(2, 16, v_head_dim=40, values=False)])        # a size that is not stored is not checked
+
+
+def test_values_of_another_size_or_none_at_all():
+    """A need may ask for values of another head size than its keys, or for the first array alone (one
+    vector per position); needs that differ in either form groups of their own."""
+    c = Cache([KVNeed(2, 32), KVNeed(2, 32, v_head_dim=16), KVNeed(1, 48, values=False), KVNeed(2, 32)], [None] * 4,
+              256, 256, 2, torch.float32, "cpu")
+    assert len(c.groups) == 3 and c.group_of[0][0] == c.group_of[3][0]
+    n_pages = 256 // 64 + 1
+    k, v = c.layer_kv(0)
+    assert k.shape == (n_pages, 2, 64, 32) and v.shape == (n_pages, 2, 32, 64)
+    k, v = c.layer_kv(1)
+    assert k.shape == (n_pages, 2, 64, 32) and v.shape == (n_pages, 2, 16, 64)
+    k, v = c.layer_kv(2)
+    assert k.shape == (n_pages, 1, 64, 48) and v is None
+    s = c.take_slot()
+    c.reserve({s: 100}); c.advance(s, 100)                     # every group hands out its own pages
+    assert all(len(c.slots.pages[s][g]) == 2 for g in range(3))
+    c.give_back_slot(s)
+    assert all(g.pool.n_free == n_pages - 1 for g in c.groups)
+
+
+def test_a_slot_that_is_taken_again_overwrites_its_rows_old_entries():
+    """A slot's row of the block table keeps the page numbers of the sequence that held it before; the
+    next sequence's pages overwrite them from the first place on, and every change is queued for the
+    device."""
+    c = Cache([KVNeed(2, 16)], [None], 640, 640, 2, torch.float32, "cpu")
+    a = c.take_slot()
+    c.reserve({a: 300}); c.advance(a, 300)
+    old = list(c.slots.pages[a][0])
+    other = c.take_slot()
+    c.reserve({other: 64}); c.advance(other, 64)
+    c.groups[0].dirty = {}
+    c.give_back_slot(a)
+    b = c.take_slot()
+    assert b == a and c.length(b) == 0
+    c.reserve({b: 70}); c.advance(b, 70)
+    new = c.slots.pages[b][0]
+    W = c.max_pages_per_seq
+    assert len(new) == 2 and c.groups[0].table_host[b, :2].tolist() == new
+    assert c.groups[0].dirty == {b * W + i: p for i, p in enumerate(new)}
+    assert c.groups[0].table_host[b, 2:5].tolist() == old[2:5]         # stale, beyond the sequence's length: never read
+    assert not c.groups[0].table_host[c.sink_slot].any()
 
 
 def test_a_need_may_name_its_own_storage_type():

@@ -16,8 +16,8 @@ class FakeBackend:
 
     def __init__(self, max_tokens=1024, max_context=64, n_slots=4):
         import torch
-        self.cache = Cache([KVNeed(1, 2)], [None], max_tokens, max_context, n_slots, torch.float32, "cpu", 16)
-        self.max_context, self.n_slots, self.page_size = max_context, n_slots, 16
+        self.cache = Cache([KVNeed(1, 16)], [None], max_tokens, max_context, n_slots, torch.float32, "cpu", 32)
+        self.max_context, self.n_slots, self.page_size = max_context, n_slots, 32
         self.seqs = {}
         self.steps = []          # per step: list of (slot, n tokens)
         self.taken = []
@@ -195,7 +195,7 @@ def test_a_failing_step_gives_the_slots_back():
     be.tokens_capacity = lambda: 10**6          # let the plan through so that the step itself fails
     with pytest.raises(CacheFull):
         generate(be, [Request([1] * 30, 2), Request([1] * 30, 2)])
-    assert be.cache.slots.live == set() and be.cache.groups[0].pool.n_free == 2
+    assert be.cache.slots.live == set() and be.cache.groups[0].pool.n_free == 1      # one page of 32 positions
 
 
 def test_runs_of_steps_give_the_same_tokens_and_respect_every_budget():

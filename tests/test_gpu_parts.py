@@ -44,8 +44,11 @@ class Harness:
         ctx.seq_of_token = i32(np.concatenate([[i] * n for i, n in enumerate(q_lens)]))
         ctx.cu_seqlens = i32(np.concatenate([[0], np.cumsum(q_lens)]))
         ctx.kv_before, ctx.slot_ids = i32(before), i32(slots)
-        width = max(1, -(-ctx.max_kv_len // self.cache.page_size))
-        ctx._tables = [i32(self.cache.block_rows(g, slots, width)) for g in range(len(self.cache.groups))]
+        # the block tables as the engine passes them: the cache's own, a row per slot, named by slot numbers
+        self.cache.flush_tables()
+        ctx._tables = [self.cache.device_table(g) for g in range(len(self.cache.groups))]
+        ctx.table_rows = i32(np.concatenate([[s] * n for s, n in entries])) if entries else None
+        ctx.seq_rows = ctx.slot_ids
         for s, n in entries:
             self.cache.advance(s, n)
         return ctx
@@ -852,3 +855,136 @@ def test_a_decoder_of_another_make_from_descriptions_alone(tmp_path, dtype):
         finally:
             ops.settle_residual = real
         assert any(seen)
+
+
+# ------------------------------------------------------------------ no final norm; a norm that knows nothing of slices
+class PlainRMS:
+    """A norm kind of the test's own that reads the residual rows with no thought for sums that a
+    product may have left in slices beside them, as any part written from the interface alone would."""
+    graph_safe = True          # one kernel launch on the current stream
+
+    def __init__(self, spec, dtype):
+        self.dim, self.eps, self.dtype, self.name = spec.dim, spec.eps, dtype, spec.names["weight"]
+
+    def tensors(self):
+        from gpullama3_java_amd.weights.loader import TensorSpec
+        return {self.name: TensorSpec((self.dim,), "vector")}
+
+    def load(self, weights):
+        self.weight = weights[self.name]
+
+    def __call__(self, ctx, x, rows=None, name="normed"):
+        from gpullama3_java_amd.csrc import lib as K
+        out = ctx.buffer("toy_" + name, (x.shape[0] if rows is None else rows.numel(), self.dim), self.dtype)
+        K.rmsnorm(x, self.weight, out, self.eps, rows)
+        return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_decoder_without_a_final_norm_and_with_a_norm_that_knows_nothing_of_slices(tmp_path, dtype):
+    """``ModelSpec.final_norm = None``: the head reads the wanted rows as they are. The feed-forward's norm is
+    a kind defined here that just reads the rows; in a step of 40 tokens the output projection before it
+    (K = 1,024) leaves its sums in slices, so the stock block must make the rows whole for it."""
+    import gpullama3_java_amd as g
+    from gpullama3_java_amd.config import AttentionSpec, BlockSpec, GatedFeedForwardSpec, ModelSpec, NormSpec, Run
+    from gpullama3_java_amd.engine import Engine
+    from gpullama3_java_amd.parts import ops, register_part
+
+    register_part("norm", "toy_plain_rms", PlainRMS)
+    d, H, Kh, hs, F, V, L, eps = 128, 8, 2, 128, 1024, 300, 2, 1e-5
+
+    @dataclass(frozen=True)
+    class BareConfig:
+        d: dict
+        max_position_embeddings: int = 128
+        stop_ids: tuple = ()
+
+        @classmethod
+        def from_dict(cls, dd):
+            return cls(dict(dd))
+
+        def with_context_length(self, n):
+            return self
+
+        def model_spec(self):
+            layers = []
+            for l in range(L):
+                p = f"l{l}."
+                layers.append(BlockSpec(
+                    mixer_norm=NormSpec(dim=d, eps=eps, names={"weight": p + "n1"}),
+                    mixer=AttentionSpec(hidden=d, n_heads=H, n_kv_heads=Kh, head_dim=hs, position=None,
+                                        names={"q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"}),
+                    ffn_norm=NormSpec(kind="toy_plain_rms", dim=d, eps=eps, names={"weight": p + "n2"}),
+                    ffn=GatedFeedForwardSpec(hidden=d, intermediate=F, names={"gate": p + "g", "up": p + "u", "down": p + "dn"})))
+            return ModelSpec(architecture="BareForCausalLM", vocab_size=V, hidden=d, layers=tuple(layers),
+                             run_order=tuple(Run(i) for i in range(L)), final_norm=None, max_positions=128,
+                             tie_embeddings=False, embedding_name="emb", head_name="head")
+
+    g.register_architecture("BareForCausalLM", BareConfig)
+    rng = np.random.default_rng(9)
+    r = lambda *s, scale=0.05: (rng.standard_normal(s) * scale).astype(np.float32)
+    W = {"emb": r(V, d, scale=0.3), "head": r(V, d, scale=0.1)}
+    for l in range(L):
+        p = f"l{l}."
+        W.update({p + "n1": 1 + r(d, scale=0.1), p + "n2": 1 + r(d, scale=0.1), p + "q": r(H * hs, d), p + "k": r(Kh * hs, d),
+                  p + "v": r(Kh * hs, d), p + "o": r(d, H * hs), p + "g": r(F, d), p + "u": r(F, d), p + "dn": r(d, F)})
+    if dtype == "bfloat16":
+        W = {k: (torch.as_tensor(v).to(torch.bfloat16).float().numpy() if v.ndim == 2 else v) for k, v in W.items()}
+
+    def plain(toks):
+        T = len(toks)
+        x = W["emb"][toks].astype(np.float32)
+        for l in range(L):
+            p = f"l{l}."
+            h = P.rmsnorm(x, W[p + "n1"], eps)
+            q, k, v = (P.linear(h, W[p + n]).reshape(T, heads, hs) for n, heads in (("q", H), ("k", Kh), ("v", Kh)))
+            x = x + P.linear(P.attention(q, k, v).reshape(T, H * hs), W[p + "o"])
+            h = P.rmsnorm(x, W[p + "n2"], eps)
+            x = x + P.linear(P.silu(P.linear(h, W[p + "g"])) * P.linear(h, W[p + "u"]), W[p + "dn"])
+        return P.linear(x, W["head"])                       # no final norm
+
+    folder = str(tmp_path / "bare")
+    os.makedirs(folder)
+    json.dump({"architectures": ["BareForCausalLM"]}, open(os.path.join(folder, "config.json"), "w"))
+    save_file({k: torch.as_tensor(v).to(TD[dtype] if v.ndim == 2 else torch.float32) for k, v in W.items()},
+              os.path.join(folder, "model.safetensors"))
+    eng = Engine.from_folder(folder, dtype=dtype, max_tokens=512, n_slots=2)
+    assert eng.model.final_norm is None
+    toks = rng.integers(0, V, 46).tolist()
+    ref = plain(toks)
+    seen = []
+    real = ops.settle_residual
+    ops.settle_residual = lambda ctx, x: seen.append(ctx.pending is not None) or real(ctx, x)
+    try:
+        s = eng.take_slot()
+        got = [eng.step([(s, toks[:40])], want=[[0, 17, 39]]).cpu().numpy()]
+    finally:
+        ops.settle_residual = real
+    got += [eng.step([(s, [t])]).cpu().numpy() for t in toks[40:]]
+    close(np.concatenate(got), ref[[0, 17, 39] + list(range(40, 46))], dtype, "no final norm, a norm that only reads")
+    if dtype == "bfloat16":
+        assert any(seen)           # the case is the one it claims to be: slices lay beside the rows when the toy norm came
+
+
+def test_two_engines_in_one_process_keep_their_own_switches():
+    """The fast paths that an engine does without belong to that engine: another engine of the same process,
+    built before or after it, keeps all of them; both give the plain implementation's logits."""
+    from gpu_helpers import plain_logits
+    from gpullama3_java_amd.engine import Engine
+    folder, _, _ = model("D")
+    bare = Engine.from_folder(folder, dtype="bfloat16", max_tokens=1024, without="tiled,fused,wide")
+    full = Engine.from_folder(folder, dtype="bfloat16", max_tokens=1024)
+    lean = Engine.from_folder(folder, dtype="bfloat16", max_tokens=1024, weight_copies=False)
+    assert bare.without == {"tiled", "fused", "wide"} and full.without == frozenset() and lean.without == {"tiled"}
+    copies = lambda e: [getattr(b.mixer.w_qkv, "tiled", None) is not None for b in e.model.blocks]
+    assert copies(full) == [True, True] and copies(bare) == [False, False] and copies(lean) == [False, False]
+    toks = rand_tokens("D", 3, 30)
+    ref = plain_logits("D", toks)
+    for eng in (bare, full, lean, bare):
+        s = eng.take_slot()
+        got = [eng.step([(s, toks[:20])], want="all").cpu().numpy()]
+        got += [eng.step([(s, [t])]).cpu().numpy() for t in toks[20:]]
+        eng.give_back_slot(s)
+        close(np.concatenate(got), ref, "bfloat16")
+    with pytest.raises(ValueError, match="unknown fast path"):
+        Engine.from_folder(folder, dtype="bfloat16", max_tokens=1024, without="tiled,quick")
