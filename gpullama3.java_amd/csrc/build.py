@@ -18,8 +18,11 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ARCH = "gfx950"
+# (kernarg preload: a kernel's first arguments arrive in scalar registers with the dispatch, where a kernel would
+# otherwise begin with a trip to memory for them)
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 _NOISE = "is not a recognized feature for this target"
 
 

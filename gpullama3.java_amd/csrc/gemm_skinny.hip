@@ -46,6 +46,23 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 enum { SK_STORE = 0, SK_ADD = 1, SK_GATED = 2, SK_QKV = 3 };
 
+// Time stamps inside a kernel, for measurements (compiled in with -DSK_STAMPS only, never in the library's own
+// build): stage i of wave w (0 or the last) of block b (0 or the middle one) goes to sk_stamps[b][w][i].
+#ifdef SK_STAMPS
+__device__ long long sk_stamps[2][2][16];
+extern "C" int gl3_sk_stamps(long long* out) {
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(sk_stamps), sizeof(sk_stamps)) == hipSuccess ? 0 : -1;
+}
+#define SK_STAMP(i)                                                                                              \
+  do {                                                                                                           \
+    const int w_ = threadIdx.x >> 6, nw_ = blockDim.x >> 6;                                                      \
+    if ((blockIdx.x == 0 || blockIdx.x == gridDim.x / 2) && (threadIdx.x & 63) == 0 && (w_ == 0 || w_ == nw_ - 1)) \
+      sk_stamps[blockIdx.x == 0 ? 0 : 1][w_ == 0 ? 0 : 1][i] = (i) == 0 || (i) == 15 ? wall_clock64() : clock64(); \
+  } while (0)
+#else
+#define SK_STAMP(i) do {} while (0)
+#endif
+
 struct SkNorm {
   const float* ssq;       // [n_partials][64] partial sums of squares of the rows of x
   int n_partials;
@@ -85,55 +102,150 @@ struct SkRope {
   bf16_t* k_cache;
   bf16_t* v_cache;
   int n_heads, n_kv, head_dim, adjacent, page_size;
+  // what hangs on a token's position, looked up once per step for all layers (gl3_token_facts; may be null):
+  // the page its keys and values go to, and its row of cos and sin, [tokens][head_dim]: cos, then sin
+  const int* token_pages;
+  const float* token_rot;
 };
 
 // Which row of W is row r of a strip's tile, and for SK_QKV which head the strip belongs to.
 // A strip is ROWS rows of W: 16, or 8 (then rows 8..15 of the tile repeat rows 0..7 and are not
 // written: half a tile is wasted for twice as many blocks where 16-row strips leave CUs idle).
-template <int EPI, int ROWS = 16>
-__device__ __forceinline__ int sk_strip_row(int strip, int r, int N, const SkRope& rp, int& hd, int& sub, bool& rotated) {
-  int wr = min(strip * ROWS + (r % ROWS), N - 1);
+// sk_strip_head is what costs (a division), once per strip; sk_strip_row_of is the row of one lane.
+template <int EPI>
+__device__ __forceinline__ void sk_strip_head(int strip, const SkRope& rp, int& hd, int& sub, bool& rotated) {
   hd = 0; sub = 0; rotated = false;
   if (EPI == SK_QKV) {
     const int per_head = rp.head_dim / 16;
     hd = strip / per_head;
-    sub = strip % per_head;
+    sub = strip - hd * per_head;
     rotated = rp.cos_tab != nullptr && hd < rp.n_heads + rp.n_kv;
-    if (rotated && !rp.adjacent)
-      wr = hd * rp.head_dim + 8 * sub + (r < 8 ? r : rp.head_dim / 2 + r - 8);
   }
-  return wr;
+}
+template <int EPI, int ROWS = 16>
+__device__ __forceinline__ int sk_strip_row_of(int strip, int r, int N, const SkRope& rp, int hd, int sub, bool rotated) {
+  if (EPI == SK_QKV && rotated && !rp.adjacent) return hd * rp.head_dim + 8 * sub + (r < 8 ? r : rp.head_dim / 2 + r - 8);
+  return min(strip * ROWS + (r % ROWS), N - 1);
+}
+template <int EPI, int ROWS = 16>
+__device__ __forceinline__ int sk_strip_row(int strip, int r, int N, const SkRope& rp, int& hd, int& sub, bool& rotated) {
+  sk_strip_head<EPI>(strip, rp, hd, sub, rotated);
+  return sk_strip_row_of<EPI, ROWS>(strip, r, N, rp, hd, sub, rotated);
 }
 
-template <bool XNORM>
-__device__ __forceinline__ const void* sk_x_row(const void* Av, long lda, int m, const SkNorm& nrm) {
-  if (XNORM && nrm.rows) m = nrm.rows[m];
-  return (const bf16_t*)Av + (long)m * lda;
-}
+// ---- loads without branches. Everything a block reads before its first product is asked for in one go, so
+// that it arrives in one trip to memory. A branch around a load defeats that: at the point where the
+// branches meet again the compiler waits for all loads on their way, and a prologue of conditional loads
+// becomes a chain of trips (nine of them before the first matrix instruction of the QKV product, as
+// compiled). So every load here goes through a buffer descriptor and is always issued: a lane that has
+// nothing to read gives an offset beyond the buffer (SK_NOWHERE always is), gets zeros and touches no
+// memory, and a null pointer makes an empty buffer.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned SK_NOWHERE = 0x80000000u;   // beyond any buffer: descriptors span less than 2 GiB
 
-// A operands of one k-step for MT token tiles: elements k .. k+7 of each tile's row.
-template <int MT, bool XNORM>
-__device__ __forceinline__ void sk_load_x(bf16x8 (&xf)[MT], const void* const (&xrow)[MT], int k, bool ok,
-                                          const SkNorm& nrm) {
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t sk_rsrc(const void* p, long bytes) {
+  const long n = p ? (bytes < 0x7fffffffL ? bytes : 0x7fffffffL) : 0;
+  return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, (int)n, 0x00020000);
+}
+__device__ __forceinline__ bf16x8 sk_ld_b128(__amdgpu_buffer_rsrc_t buf, unsigned byte_offset) {
+  return __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(buf, byte_offset, 0, 0));
+}
+__device__ __forceinline__ f32x4 sk_ld_f32x4(__amdgpu_buffer_rsrc_t buf, unsigned byte_offset) {
+  return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(buf, byte_offset, 0, 0));
+}
+__device__ __forceinline__ float sk_ld_f32(__amdgpu_buffer_rsrc_t buf, unsigned byte_offset) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(buf, byte_offset, 0, 0));
+}
+__device__ __forceinline__ int sk_ld_i32(__amdgpu_buffer_rsrc_t buf, unsigned byte_offset) {
+  return (int)__builtin_amdgcn_raw_buffer_load_b32(buf, byte_offset, 0, 0);
+}
+// 4 floats at element `first` of a float array of `count` elements; elements from `count` on read as zero.
+// (Single loads: the array may start anywhere.)
+__device__ __forceinline__ f32x4 sk_ld_4f(__amdgpu_buffer_rsrc_t buf, bool wanted, int first, int count) {
+  f32x4 v;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-    xf[mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
+  for (int c = 0; c < 4; ++c) v[c] = sk_ld_f32(buf, (wanted && first + c < count) ? (unsigned)(first + c) * 4u : SK_NOWHERE);
+  return v;
 }
 
-// Partial sums of squares of the rows: wave w adds the partials w, w+NW, ... of row `lane`.
-template <int NW>
-__device__ __forceinline__ void sk_ssq_partials(float (*sm_ssq)[64], int M, const SkNorm& nrm) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+// The row of A that row m of the product reads (XNORM with `rows`: the product is one of chosen rows). Called
+// before anything else is on its way: the value is used at once, and the wait for it waits for nothing else.
+template <bool XNORM>
+__device__ __forceinline__ int sk_a_row(int m, int M, const SkNorm& nrm) {
+  int row = min(m, M - 1);
+  if (XNORM && nrm.rows) {   // (the same for the whole grid)
+    row = nrm.rows[row];
+    asm volatile("" : "+v"(row));
+  }
+  return row;
+}
+
+// Rows of A as [rows][lda] bfloat16 behind a descriptor; a row's offset is SK_NOWHERE when the row does not
+// exist, so that its lanes ask for nothing: a CU draws a bounded number of bytes a second through its
+// first-level cache, whatever they are.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t sk_a_rsrc(const void* Av, int M, int K, long lda, const SkNorm* nrm) {
+  const long rows = (nrm && nrm->rows) ? 64 : M;   // (chosen rows: A has at most 64; offsets of rows that exist are all that is asked for)
+  return sk_rsrc(Av, ((rows - 1) * lda + K) * 2);
+}
+__device__ __forceinline__ unsigned sk_x_off(int row, bool exists, long lda) {
+  return exists ? (unsigned)((long)row * lda * 2) : SK_NOWHERE;
+}
+// A operands of one k-step for MT token tiles: elements k .. k+7 of each tile's row (`kb`: 2 k, or SK_NOWHERE).
+template <int MT>
+__device__ __forceinline__ void sk_load_x(bf16x8 (&xf)[MT], __amdgpu_buffer_rsrc_t a_buf, const unsigned (&xo)[MT], unsigned kb) {
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) xf[mt] = sk_ld_b128(a_buf, ((xo[mt] | kb) & SK_NOWHERE) ? SK_NOWHERE : xo[mt] + kb);
+}
+
+// Partial sums of squares of the rows, added up in a fixed order: sm_ssq[w][row] receives wave w's share, the
+// strip's end adds the waves' shares. `sq_row`: the lane's row's row of A (the partial sums are stored by it).
+// One token tile (at most 16 rows, every decode step that folds a norm): the lanes are 4 groups of 16 rows, group j
+// of wave w takes the partials w + NW (4 i + j), and the first four of each lane (64 NW partials in all) are
+// asked for with the block's first loads (sk_ssq_ask); sk_ssq_sum, at the first strip's end, adds them, fetches
+// any further ones, and adds the groups. More token tiles: lane = row, sixteen partials at a time, all in sk_ssq_sum.
+template <int NW, int MT>
+__device__ __forceinline__ void sk_ssq_ask(float (&sq)[4], int M, const SkNorm& nrm, int sq_row) {
+  if (MT != 1) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const __amdgpu_buffer_rsrc_t buf = sk_rsrc(nrm.ssq, (long)nrm.n_partials * 256);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int p = wave + NW * (4 * i + (lane >> 4));
+    sq[i] = sk_ld_f32(buf, ((lane & 15) < M && p < nrm.n_partials) ? (unsigned)((p * 64 + sq_row) * 4) : SK_NOWHERE);
+  }
+}
+// `after`: a result of the product's matrix instructions. The sums are wanted at the strip's end; tied to that
+// value they cannot be added up, and waited for, at the point where they were asked for, in front of loads
+// that should be on their way first.
+template <int NW, int MT>
+__device__ __forceinline__ void sk_ssq_sum(float (*sm_ssq)[64], float (&sq)[4], int M, const SkNorm& nrm, int sq_row,
+                                           float after) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const __amdgpu_buffer_rsrc_t buf = sk_rsrc(nrm.ssq, (long)nrm.n_partials * 256);
   float sp = 0.f;
-  if (lane < M) {
-    const int row = nrm.rows ? nrm.rows[lane] : lane;   // the partial sums are stored by row of A
+  if (MT == 1) {
+    asm volatile("" : "+v"(sq[0]) : "v"(after));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sp += sq[i];
+    for (int p0 = wave + NW * 16; p0 < nrm.n_partials; p0 += NW * 16) {   // further partial sums, four a lane at a time
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int p = p0 + NW * (4 * i + (lane >> 4));
+        v[i] = sk_ld_f32(buf, ((lane & 15) < M && p < nrm.n_partials) ? (unsigned)((p * 64 + sq_row) * 4) : SK_NOWHERE);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sp += v[i];
+    }
+    sp += __shfl_xor(sp, 16, 64);
+    sp += __shfl_xor(sp, 32, 64);
+  } else {
     for (int p0 = wave; p0 < nrm.n_partials; p0 += NW * 16) {
       float v[16];   // sixteen loads in flight, then added in order
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int p = p0 + NW * i;
-        v[i] = p < nrm.n_partials ? nrm.ssq[(long)p * 64 + row] : 0.f;
+        v[i] = sk_ld_f32(buf, (lane < M && p < nrm.n_partials) ? (unsigned)((p * 64 + sq_row) * 4) : SK_NOWHERE);
       }
 #pragma unroll
       for (int i = 0; i < 16; ++i) sp += v[i];
@@ -155,55 +267,85 @@ struct SkPre {
   int page;
 };
 
-// GIVEN (SK_QKV): the caller has asked for the token's position and its row of the block table already
-// (`pos`, `table_row`), so that what depends on them can be asked for without another wait.
-template <int MT, int EPI, typename TC, int ROWS = 16, bool GIVEN = false>
+// A block's prologue is what its time goes to before the loads are on their way: sixteen waves that each work
+// through several hundred instructions, most of them scalar, share one scalar unit. So what only the END of a
+// strip needs (sk_token, sk_preload) is computed by the waves that finish a token tile alone (wave < MT: the
+// caller's branch, the same for a whole wave), and offsets are 32-bit (the entry points bound the sizes).
+//
+// A token's position and its row of the block table (SK_QKV), asked for before the product's own loads so
+// that what hangs on them (page number, cos and sin) can be asked for while those are still on their way.
+struct SkToken { int pos, row; };
+__device__ __forceinline__ SkToken sk_token(int M, const SkRope& rp) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r = threadIdx.x & 15;
+  const int m = wave * 16 + r;
+  const unsigned at = m < M ? (unsigned)m * 4u : SK_NOWHERE;
+  SkToken t;
+  t.pos = sk_ld_i32(sk_rsrc(rp.positions, (long)M * 4), at);
+  t.row = sk_ld_i32(sk_rsrc(rp.seq_of_token, (long)M * 4), at);
+  return t;
+}
+
+// For a wave that finishes token tile `wave` (the caller sees to wave < MT). SK_QKV: `tok` is what sk_token
+// returned. No branch surrounds a load: see sk_rsrc.
+template <int MT, int EPI, typename TC, int ROWS = 16>
 __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int N, long ldc, int strip, int hd, int sub,
-                                            bool rotated, const SkRope& rp, const SkNext& nx = SkNext{}, int pos = 0,
-                                            int table_row = 0) {
+                                            bool rotated, const SkRope& rp, const SkNext& nx = SkNext{},
+                                            SkToken tok = SkToken{0, 0}) {
   SkPre p;
   p.prev = p.bias = p.bias_up = p.next_w = p.co = p.si = f32x4{0.f, 0.f, 0.f, 0.f};
   p.pos = 0; p.page = 0;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // (What is computed here is for the calling waves alone. Much of it does not change from strip to strip, and
+  // the compiler would move that in front of the caller's loop over the strips, where every wave pays for it:
+  // the values it all hangs on pass through an empty volatile statement, which stays where it is.)
+  asm volatile("" : "+v"(tok.pos), "+v"(tok.row), "+s"(strip));
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
   const int m = wave * 16 + r;
-  if (wave >= MT || m >= M || 4 * q >= ROWS) return p;
-  if (EPI != SK_QKV && nx.bias) {
-    const int n = strip * ROWS + 4 * q;
+  const bool live = m < M && 4 * q < ROWS;
+  const int n = strip * ROWS + 4 * q;
+  if (EPI != SK_QKV && nx.bias) {   // (the same for the whole grid; nothing hangs on these loads before the strip's end)
+    const __amdgpu_buffer_rsrc_t b_buf = sk_rsrc(nx.bias, (long)(EPI == SK_GATED ? 2 * N : N) * 4);
+    p.bias = sk_ld_4f(b_buf, live, n, N);
+    if (EPI == SK_GATED) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
-      if (n + c < N) {
-        p.bias[c] = nx.bias[n + c];
-        if (EPI == SK_GATED) p.bias_up[c] = nx.bias[N + n + c];
-      }
+      for (int c = 0; c < 4; ++c) p.bias_up[c] = sk_ld_f32(b_buf, (live && n + c < N) ? (unsigned)(N + n + c) * 4u : SK_NOWHERE);
+    }
   }
   if (EPI == SK_ADD) {
-    const int n = strip * ROWS + 4 * q;
-    const TC* cp = C + (long)m * ldc + n;
+    static_assert(EPI != SK_ADD || sizeof(TC) == 4, "the add epilogue adds into a float matrix");
+    const __amdgpu_buffer_rsrc_t c_buf = sk_rsrc(C, ((long)(M - 1) * ldc + N) * 4);
+    const unsigned at = ((unsigned)m * (unsigned)ldc + (unsigned)n) * 4u;
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
-      if (n + c < N) {
-        p.prev[c] = to_f32<TC>(cp[c]);
-        if (nx.weight) p.next_w[c] = nx.weight[n + c];
-      }
+    for (int c = 0; c < 4; ++c) p.prev[c] = sk_ld_f32(c_buf, (live && n + c < N) ? at + 4u * c : SK_NOWHERE);
+    p.next_w = sk_ld_4f(sk_rsrc(nx.weight, (long)N * 4), live, n, N);
   }
   if (EPI == SK_QKV) {
-    p.pos = GIVEN ? pos : rp.positions[m];
-    if (hd >= rp.n_heads)
-      p.page = rp.block_table[(long)(GIVEN ? table_row : rp.seq_of_token[m]) * rp.table_stride + p.pos / rp.page_size];
-    if (rotated) {
-      const int half = rp.head_dim / 2;
-      if (rp.adjacent) {
-        const int jj = (16 * sub + 4 * q) / 2;
-        p.co[0] = rp.cos_tab[(long)p.pos * half + jj];     p.si[0] = rp.sin_tab[(long)p.pos * half + jj];
-        p.co[1] = rp.cos_tab[(long)p.pos * half + jj + 1]; p.si[1] = rp.sin_tab[(long)p.pos * half + jj + 1];
-      } else {
-        const int jj = 8 * sub + 4 * (q & 1);
+    p.pos = tok.pos;
+    // (the tables' sizes are not known here: the descriptors span what a descriptor can, and only lanes of
+    // tokens that exist, whose entries the caller vouches for, give an offset inside)
+    const bool kv = live && hd >= rp.n_heads;
+    const unsigned half = (unsigned)rp.head_dim / 2u;
+    const bool turn = live && rotated;
+    const int pairs = rp.adjacent ? 2 : 4;                                                    // (the same for the whole grid)
+    const unsigned pair0 = rp.adjacent ? (16u * sub + 4u * q) / 2u : 8u * sub + 4u * (q & 1);
+    if (rp.token_pages) {   // (the same for the whole grid) looked up once per step: nothing here waits for the position
+      p.page = sk_ld_i32(sk_rsrc(rp.token_pages, (long)M * 4), kv ? (unsigned)m * 4u : SK_NOWHERE);
+      const __amdgpu_buffer_rsrc_t rot_buf = sk_rsrc(rp.token_rot, (long)M * rp.head_dim * 4);
+      const unsigned at = ((unsigned)m * (unsigned)rp.head_dim + pair0) * 4u;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          p.co[c] = rp.cos_tab[(long)p.pos * half + jj + c];
-          p.si[c] = rp.sin_tab[(long)p.pos * half + jj + c];
-        }
+      for (int c = 0; c < 4; ++c) {
+        p.co[c] = sk_ld_f32(rot_buf, (turn && c < pairs) ? at + 4u * c : SK_NOWHERE);
+        p.si[c] = sk_ld_f32(rot_buf, (turn && c < pairs) ? at + (half + c) * 4u : SK_NOWHERE);
+      }
+    } else {
+      const unsigned page_at = (unsigned)tok.row * (unsigned)rp.table_stride + (unsigned)tok.pos / (unsigned)rp.page_size;
+      p.page = sk_ld_i32(sk_rsrc(rp.block_table, 0x7fffffffL), kv ? page_at * 4u : SK_NOWHERE);
+      const __amdgpu_buffer_rsrc_t co_buf = sk_rsrc(rp.cos_tab, 0x7fffffffL), si_buf = sk_rsrc(rp.sin_tab, 0x7fffffffL);
+      const unsigned at = ((unsigned)tok.pos * half + pair0) * 4u;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        p.co[c] = sk_ld_f32(co_buf, (turn && c < pairs) ? at + 4u * c : SK_NOWHERE);
+        p.si[c] = sk_ld_f32(si_buf, (turn && c < pairs) ? at + 4u * c : SK_NOWHERE);
       }
     }
   }
@@ -228,6 +370,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) red[wave][g * MT + mt][lane] = acc[g][mt];
   __syncthreads();
+  SK_STAMP(6);
   for (int t = wave; t < NG * MT; t += NW) {
     f32x4 v = red[0][t][lane];
 #pragma unroll
@@ -235,6 +378,7 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
     red[0][t][lane] = v;   // only this thread touches red[*][t][lane] before the barrier
   }
   __syncthreads();
+  SK_STAMP(7);
 
   // epilogue: lane holds tile rows 4q .. 4q+3 (columns of C) of token mt*16 + r
   for (int mt = wave; mt < MT; mt += NW) {
@@ -348,50 +492,67 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   constexpr int UNROLL = 8;
   __shared__ f32x4 red[NW][NG * MT][64];
   __shared__ float sm_ssq[XNORM ? NW : 1][64];
+  SK_STAMP(0); SK_STAMP(1);
   const int strip = blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
+  // which rows of A the tiles' rows are (a look-up for chosen rows), before anything else is on its way
+  unsigned xo[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {   // nowhere for rows that do not exist: their lanes ask for nothing
+    const int m = PACK ? (r & 7) : mt * 16 + r;
+    xo[mt] = sk_x_off(sk_a_row<XNORM>(m, M, nrm), m < M, lda);
+  }
+  const int sq_row = XNORM ? sk_a_row<XNORM>(MT == 1 ? (lane & 15) : lane, M, nrm) : 0;
+  const bool ender = wave < MT;   // this wave finishes token tile `wave`
+  SkToken tok = {0, 0};
+  if (EPI == SK_QKV && ender) tok = sk_token(M, rp);
   int hd, sub;
   bool rotated;
   const int wr = sk_strip_row<EPI, ROWS>(strip, r, N, rp, hd, sub, rotated);
+  const int w0 = sk_strip_row_of<EPI, ROWS>(strip, 0, N, rp, hd, sub, rotated);   // the strip's first row: the same for the block
   const int koff = PACK ? 32 * (r >> 3) + q * 8 : q * 8;   // the lane's place inside a k-step
-  const bf16_t* wrow = W + (long)wr * ldw + koff;
-  const bf16_t* urow = wrow + (long)N * ldw;  // up rows (gated only)
-  const void* xrow[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {   // null for rows that do not exist: their lanes ask for nothing
-    const int m = PACK ? (r & 7) : mt * 16 + r;
-    xrow[mt] = m < M ? sk_x_row<XNORM>(Av, lda, m, nrm) : nullptr;
-  }
-  if (XNORM) sk_ssq_partials<NW>(sm_ssq, M, nrm);
-  const SkPre pre = sk_preload<MT, EPI, TC, ROWS>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx);
-
   const int steps = (K + 31) / 32;   // k-steps of 32
+  const int steps64 = (K + 63) / 64;
+  // W behind descriptors that start at the strip: as it is stored (the lane's row, 16 bytes at its place in
+  // a k-step), or the copy in the order of the operands (Wt8: strips of 16 rows [strip][k-step of 32][lane][8],
+  // gated: the up strips follow the N / 16 gate strips; PACK: [strip of 8 rows][step of 64 k][lane][8]; k
+  // padded with zeros to whole steps), where a load is 1 KB of consecutive memory.
+  const bool tiled = Wt8 != nullptr && (PACK || ROWS == 16);
+  const long tile_bytes = PACK ? (long)steps64 * 1024 : (long)steps * 1024;
+  const __amdgpu_buffer_rsrc_t w_buf =
+      tiled ? sk_rsrc(Wt8 + (long)strip * (tile_bytes / 2), tile_bytes)
+            : sk_rsrc(W + (long)w0 * ldw, (((long)(EPI == SK_QKV ? N : min(N, (strip + 1) * ROWS)) - 1 - w0) * ldw + K) * 2);
+  const __amdgpu_buffer_rsrc_t u_buf =   // up rows (gated only)
+      tiled ? sk_rsrc(Wt8 + ((long)(N / 16) + strip) * (tile_bytes / 2), tile_bytes)
+            : sk_rsrc(W + ((long)N + w0) * ldw, (((long)min(N, (strip + 1) * ROWS) - 1 - w0) * ldw + K) * 2);
+  const unsigned w_lane = tiled ? (unsigned)lane * 16u : (unsigned)(((long)(wr - w0) * ldw + koff) * 2);
+  const unsigned w_step = tiled ? 1024u : (PACK ? 128u : 64u);   // bytes from one step to the next
+  const __amdgpu_buffer_rsrc_t a_buf = a_packed ? sk_rsrc(Av, (long)steps64 * 1024) : sk_a_rsrc(Av, M, K, lda, XNORM ? &nrm : nullptr);
+  float sq[4];
+  if (XNORM) sk_ssq_ask<NW, MT>(sq, M, nrm, sq_row);
+  SkPre pre;
+  if (ender) pre = sk_preload<MT, EPI, TC, ROWS>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx, tok);
+  SK_STAMP(2);
+
   f32x4 acc[NG][MT];
 #pragma unroll
   for (int g = 0; g < NG; ++g)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
   if (PACK) {
     // a wave takes steps of 64 k: step wave, wave + NW, ...
-    // (Wt8, may be null: W as [strip of 8 rows][step of 64 k][lane][8], the packed tile's own order, k padded
-    // with zeros to whole steps: a load is then 1 KB of consecutive memory)
-    const int steps64 = (K + 63) / 64;
-    const bf16_t* wbase = Wt8 ? Wt8 + ((long)strip * steps64 * 64 + lane) * 8 : wrow;
-    const long w_step = Wt8 ? 512 : 64;
     for (int p0 = wave; p0 * 64 < K; p0 += NW * UNROLL) {
       bf16x8 wf[UNROLL], xf[UNROLL][MT];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const int p = p0 + NW * u, k = p * 64;
         const bool ok = k + koff < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
-        wf[u] = (Wt8 ? p < steps64 : ok) ? *(const bf16x8*)(wbase + p * w_step) : zero;
-        if (a_packed)   // the rows in the packed tiles' order (sk_packed_offset): this lane's 16 bytes of step p
-          xf[u][0] = (ok && xrow[0] != nullptr) ? *(const bf16x8*)((const bf16_t*)Av + ((long)p * 64 + lane) * 8) : zero;
-        else
-          sk_load_x<MT, XNORM>(xf[u], xrow, k + koff, ok, nrm);
+        wf[u] = sk_ld_b128(w_buf, (tiled ? p < steps64 : ok) ? w_lane + (unsigned)p * w_step : SK_NOWHERE);
+        // (a_packed: the rows in the packed tiles' order, sk_packed_offset: this lane's 16 bytes of step p)
+        const unsigned at = a_packed ? (unsigned)(p * 64 + lane) * 16u : xo[0] + (unsigned)(k + koff) * 2u;
+        xf[u][0] = sk_ld_b128(a_buf, (ok && (r & 7) < M) ? at : SK_NOWHERE);
       }
       __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
 #pragma unroll
@@ -405,12 +566,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   } else {
   // a wave takes pairs of neighbouring k-steps (the two halves of one 128-byte line of a row of W):
   // pair wave, wave + NW, ...
-  // (strips of 16 rows: Wt8, may be null, is W as [strip][k-step of 32][lane][8], the operands' own order,
-  // k padded with zeros to whole steps; gated: the up strips follow the N / 16 gate strips)
-  const bool tiled = ROWS == 16 && Wt8 != nullptr;
-  const bf16_t* wbase = tiled ? Wt8 + ((long)strip * steps * 64 + lane) * 8 : wrow;
-  const bf16_t* ubase = tiled ? wbase + (long)(N / 16) * steps * 512 : urow;
-  const long w_step = tiled ? 512 : 32;
   for (int p0 = wave; 2 * p0 < steps; p0 += NW * (UNROLL / 2)) {
     bf16x8 wf[UNROLL], uf[UNROLL], xf[UNROLL][MT];
 #pragma unroll
@@ -418,9 +573,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
       const int st = 2 * (p0 + NW * (u / 2)) + (u & 1), k = st * 32;
       const bool ok = k + q * 8 < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
       const bool w_ok = tiled ? st < steps : ok;
-      wf[u] = (w_ok && r < ROWS) ? *(const bf16x8*)(wbase + st * w_step) : zero;   // rows of the tile beyond the strip stay zero
-      if (EPI == SK_GATED) uf[u] = w_ok ? *(const bf16x8*)(ubase + st * w_step) : zero;
-      sk_load_x<MT, XNORM>(xf[u], xrow, k + q * 8, ok, nrm);
+      wf[u] = sk_ld_b128(w_buf, (w_ok && r < ROWS) ? w_lane + (unsigned)st * w_step : SK_NOWHERE);   // rows of the tile beyond the strip stay zero
+      if (EPI == SK_GATED) uf[u] = sk_ld_b128(u_buf, w_ok ? w_lane + (unsigned)st * w_step : SK_NOWHERE);
+      sk_load_x<MT>(xf[u], a_buf, xo, ok ? (unsigned)(k + q * 8) * 2u : SK_NOWHERE);
     }
     __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
 #pragma unroll
@@ -433,8 +588,79 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
     }
   }
   }
+#ifdef SK_STAMPS
+  asm volatile("s_nop 0" :: "v"(acc[0][0][0]));
+  SK_STAMP(4);
+#endif
+  if (XNORM) sk_ssq_sum<NW, MT>(sm_ssq, sq, M, nrm, sq_row, acc[0][0][0]);
+  SK_STAMP(5);
   sk_finish<MT, NW, EPI, TC, XNORM, SSQ, ROWS>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp,
                                                nx, pre);
+  SK_STAMP(9); SK_STAMP(15);
+}
+
+// The packed strips of 8 rows (PACK above) over the copy of W in their own order, with the prologue cut down to
+// what the loads' addresses take (see gemm_skinny_decode_kernel): the output and down projections of a decode
+// step of at most 8 rows. A: the step's rows as they are, [M][lda], or in the packed tiles' order (`a_packed`).
+// No test whether a step of W or a row of A exists: the descriptors end where the data ends, so a load beyond it
+// reads zeros; a step that does not exist for the whole wave is not asked for at all. Elements of A from K on are
+// not read (what lies there need not be a number, and the zeros of W that it would meet do not make it one).
+template <int NW, int EPI, typename TC, bool SSQ>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_pack_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wt8,
+                                                                   TC* __restrict__ C, int M, int N, int K, int lda, long ldc,
+                                                                   float* __restrict__ ssq_out, SkNext nx, int a_packed) {
+  constexpr int UNROLL = 8, MT = 1;
+  __shared__ f32x4 red[NW][1][64];
+  __shared__ float sm_ssq[1][64];
+  SK_STAMP(0); SK_STAMP(1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const int strip = blockIdx.x;
+  const int steps64 = (K + 63) >> 6;
+  const unsigned tile_bytes = (unsigned)steps64 << 10;   // a strip of the copy: 1 KB a step of 64 k
+  const __amdgpu_buffer_rsrc_t w_buf = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Wt8 + (long)strip * tile_bytes), 0, (int)tile_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_buf = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)A, 0, a_packed ? (int)tile_bytes : (int)((((unsigned)M - 1u) * (unsigned)lda + (unsigned)K) * 2u), 0x00020000);
+  const unsigned w_at = (unsigned)lane * 16u + (unsigned)wave * 1024u;
+  // lane (r, q) holds row r % 8 at k = 64 p + 32 (r / 8) + 8 q; in the packed order that is the lane's own 16 bytes of step p
+  const unsigned x_at = a_packed ? ((r & 7) < M ? w_at : SK_NOWHERE)
+                                 : ((unsigned)(r & 7) * (unsigned)lda + 32u * (r >> 3) + 8u * q + (unsigned)wave * 64u) * 2u;
+  const unsigned x_step = a_packed ? 1024u : 128u;
+  const int k_lane = 32 * (r >> 3) + 8 * q;   // the lane's k inside a step (K is a multiple of 8: its 8 elements are all in or all out)
+  SkPre pre;
+  if (wave == 0) pre = sk_preload<MT, EPI, TC, 8>(C, M, N, ldc, strip, 0, 0, false, SkRope{}, nx);
+  f32x4 acc[1][MT];
+  acc[0][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // a wave takes steps of 64 k: step wave, wave + NW, ...
+  for (int p0 = wave; p0 < steps64; p0 += NW * UNROLL) {
+    bf16x8 wf[UNROLL], xf[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      wf[u] = zero; xf[u] = zero;
+      if (p0 + NW * u < steps64) {   // (the same for the wave)
+        const unsigned p = (unsigned)(p0 - wave + NW * u);
+        wf[u] = sk_ld_b128(w_buf, w_at + p * 1024u);
+        xf[u] = sk_ld_b128(a_buf, ((x_at & SK_NOWHERE) || 64 * (p0 + NW * u) + k_lane >= K) ? SK_NOWHERE : x_at + p * x_step);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);   // all of the batch's loads are issued before the first is waited for
+    SK_STAMP(2);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+      acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[u], acc[0][0], 0, 0, 0);
+  }
+  // lane (token column j, quarter q) holds tile rows 4q .. 4q+3: the sums over the first 32 k of every
+  // step lie at j < 8, q < 2, those over the second at j >= 8, q >= 2: lane + 40
+#pragma unroll
+  for (int c = 0; c < 4; ++c) acc[0][0][c] += __shfl_xor(acc[0][0][c], 40, 64);
+#ifdef SK_STAMPS
+  asm volatile("s_nop 0" :: "v"(acc[0][0][0]));
+  SK_STAMP(4); SK_STAMP(5);
+#endif
+  sk_finish<MT, NW, EPI, TC, false, SSQ, 8>(red, sm_ssq, acc, strip, 0, 0, false, C, M, N, K, ldc, SkNorm{}, ssq_out, SkRope{}, nx,
+                                            pre);
+  SK_STAMP(9); SK_STAMP(15);
 }
 
 // The resident kernel: K <= 32 * NW * KS. `n_strips` strips are shared out over the blocks.
@@ -448,81 +674,95 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
   __shared__ float sm_ssq[XNORM ? NW : 1][64];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  SK_STAMP(0); SK_STAMP(1);
+  const bool ender = wave < MT;   // this wave finishes token tile `wave` of every strip
+  // The order below is the order of need: the token's position first (the longest chain hangs on it), then the
+  // loads that every wave's matrix instructions wait for, with as few instructions in front of them as can be;
+  // everything else (which head a strip belongs to, what the strip's end reads) while those are on their way.
+  SkToken tok = {0, 0};
+  if (EPI == SK_QKV && ender) tok = sk_token(M, rp);
+  // which rows of A the tiles' rows are (a look-up for chosen rows)
+  unsigned xo[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)   // nowhere for rows that do not exist: their lanes ask for nothing
+    xo[mt] = sk_x_off(sk_a_row<XNORM>(mt * 16 + r, M, nrm), mt * 16 + r < M, lda);
+  const int sq_row = XNORM ? sk_a_row<XNORM>(MT == 1 ? (lane & 15) : lane, M, nrm) : 0;
   // Where a strip's operands lie. In W itself a lane's 16 bytes of k-step s are in its row at 32 s
   // elements; every lane of a load is then on a line of its own. In the copy in the operands' own
   // order (Wt, may be null: [strip][k-step][lane][8], k padded with zeros to whole steps, the strips'
-  // rows as sk_strip_row names them) a load is 1 KB of consecutive memory, which the CU's first-level
-  // cache takes in less than half the time.
+  // rows as sk_strip_row names them; gated: the up strips follow the N / 16 gate strips) a load is 1 KB of
+  // consecutive memory, which the CU's first-level cache takes in less than half the time. Either way the
+  // strip lies behind a descriptor that starts at its first row (see sk_rsrc).
   const int steps_all = (K + 31) / 32;
-  const long w_step = Wt ? 512 : 32;                       // elements from one k-step to the next
-  const long w_up = Wt ? (long)(N / 16) * steps_all * 512 : (long)N * ldw;   // from a gate strip to its up strip
-  auto strip_base = [&](int strip_, int& hd_, int& sub_, bool& rot_) {
-    const int wr = sk_strip_row<EPI>(strip_, r, N, rp, hd_, sub_, rot_);
-    return Wt ? Wt + ((long)strip_ * steps_all * 64 + lane) * 8 : W + (long)wr * ldw + q * 8;
+  const unsigned w_step = Wt ? 1024u : 64u;                // bytes from one k-step to the next
+  const long tile = (long)steps_all * 512;                 // elements of a strip of the copy
+  struct Strip { __amdgpu_buffer_rsrc_t w, u; unsigned lane_at; };
+  auto strip_at = [&](int strip_) {
+    Strip t;
+    if (Wt) {   // (the same for the whole grid)
+      t.w = sk_rsrc(Wt + strip_ * tile, tile * 2);
+      t.u = sk_rsrc(Wt + ((long)(N / 16) + strip_) * tile, tile * 2);
+      t.lane_at = (unsigned)lane * 16u;
+    } else {
+      int hd, sub;
+      bool rotated;
+      const int wr = sk_strip_row<EPI>(strip_, r, N, rp, hd, sub, rotated);
+      const int w0 = sk_strip_row_of<EPI>(strip_, 0, N, rp, hd, sub, rotated);   // the strip's first row: the same for the block
+      const long bytes = (((EPI == SK_QKV ? N : min(N, (strip_ + 1) * 16)) - w0 - 1) * ldw + K) * 2;
+      t.w = sk_rsrc(W + (long)w0 * ldw, bytes);
+      t.u = sk_rsrc(W + ((long)N + w0) * ldw, bytes);
+      t.lane_at = ((unsigned)(wr - w0) * (unsigned)ldw + (unsigned)q * 8u) * 2u;
+    }
+    return t;
   };
-  auto step_ok = [&](int st) { return Wt ? st < steps_all : st * 32 + q * 8 < K; };
-  // Everything the block needs first is asked for before anything is waited for, so that it all
-  // arrives in one trip to memory: the first strip's rows of W, the rows' partial sums of squares,
-  // and this wave's share of A (k-steps wave, wave + NW, ...).
+  auto step_at = [&](const Strip& t, int st) {   // the offset of this lane's 16 bytes of k-step st
+    return (Wt ? st < steps_all : st * 32 + q * 8 < K) ? t.lane_at + (unsigned)st * w_step : SK_NOWHERE;
+  };
   int strip = blockIdx.x;
-  int hd, sub;
-  bool rotated;
+  Strip cur = strip_at(strip);
   bf16x8 wf[KS], uf[KS];
-  {
-    const bf16_t* wrow = strip_base(strip, hd, sub, rotated);
 #pragma unroll
-    for (int i = 0; i < KS; ++i) {
-      const int st = wave + NW * i;
-      const bool ok = step_ok(st);
-      wf[i] = ok ? *(const bf16x8*)(wrow + st * w_step) : zero;
-      if (EPI == SK_GATED) uf[i] = ok ? *(const bf16x8*)(wrow + w_up + st * w_step) : zero;
-    }
-  }
-  float sq[16];
-  int sq_row = 0;
-  if (XNORM) {
-    sq_row = (lane < M && nrm.rows) ? nrm.rows[lane] : lane;   // the partial sums are stored by row of A
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int p = wave + NW * i;
-      sq[i] = (lane < M && p < nrm.n_partials) ? nrm.ssq[(long)p * 64 + sq_row] : 0.f;
-    }
+  for (int i = 0; i < KS; ++i) {
+    wf[i] = sk_ld_b128(cur.w, step_at(cur, wave + NW * i));
+    if (EPI == SK_GATED) uf[i] = sk_ld_b128(cur.u, step_at(cur, wave + NW * i));
   }
   bf16x8 xf[KS][MT];
   {
-    const void* xrow[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)   // null for rows that do not exist: their lanes ask for nothing
-      xrow[mt] = mt * 16 + r < M ? sk_x_row<XNORM>(Av, lda, mt * 16 + r, nrm) : nullptr;
+    const __amdgpu_buffer_rsrc_t a_buf = sk_a_rsrc(Av, M, K, lda, XNORM ? &nrm : nullptr);
 #pragma unroll
     for (int i = 0; i < KS; ++i) {
       const int k = (wave + NW * i) * 32 + q * 8;
-      const bool ok = k < K;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        xf[i][mt] = (ok && xrow[mt] != nullptr) ? *(const bf16x8*)((const bf16_t*)xrow[mt] + k) : zero;
+      sk_load_x<MT>(xf[i], a_buf, xo, k < K ? (unsigned)k * 2u : SK_NOWHERE);
     }
   }
+  float sq[4];
+  if (XNORM) sk_ssq_ask<NW, MT>(sq, M, nrm, sq_row);
+  __builtin_amdgcn_sched_barrier(0);   // all of that is on its way before anything else is computed
+  SK_STAMP(2);
   bool first_strip = true;
   while (strip < n_strips) {
-    // ask for the next strip's rows before this strip's are used
+    // what the strip's end reads, then the next strip's rows, both before this strip's rows are used: the
+    // end then waits for its own loads only, and the next rows travel while this strip is finished
+    int hd = 0, sub = 0;
+    bool rotated = false;
+    SkPre pre;
+    if (ender) {
+      sk_strip_head<EPI>(strip, rp, hd, sub, rotated);
+      pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx, tok);
+    }
     const int next = strip + gridDim.x;
+    Strip nxt = cur;
     bf16x8 wn[KS], un[KS];
-    int hd_n = 0, sub_n = 0;
-    bool rot_n = false;
-    if (next < n_strips) {
-      const bf16_t* wrow = strip_base(next, hd_n, sub_n, rot_n);
+    if (next < n_strips) {   // (the same for the block; what is loaded here is used after the strip's end)
+      nxt = strip_at(next);
 #pragma unroll
       for (int i = 0; i < KS; ++i) {
-        const int st = wave + NW * i;
-        const bool ok = step_ok(st);
-        wn[i] = ok ? *(const bf16x8*)(wrow + st * w_step) : zero;
-        if (EPI == SK_GATED) un[i] = ok ? *(const bf16x8*)(wrow + w_up + st * w_step) : zero;
+        wn[i] = sk_ld_b128(nxt.w, step_at(nxt, wave + NW * i));
+        if (EPI == SK_GATED) un[i] = sk_ld_b128(nxt.u, step_at(nxt, wave + NW * i));
       }
     }
-    const SkPre pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx);
     __builtin_amdgcn_sched_barrier(0);   // the next strip's loads are on their way before this strip's are used
+    SK_STAMP(3);
     f32x4 acc[NG][MT];
 #pragma unroll
     for (int g = 0; g < NG; ++g)
@@ -536,26 +776,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
         if (EPI == SK_GATED) acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[i], xf[i][mt], acc[1][mt], 0, 0, 0);
       }
     }
+#ifdef SK_STAMPS
+    asm volatile("s_nop 0" :: "v"(acc[0][0][0]));
+    SK_STAMP(4);
+#endif
     if (XNORM && first_strip) {
-      // (waited for only now: the second strip's rows of W were asked for in the same trip)
-      float sp = 0.f;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sp += sq[i];
-      for (int p0 = wave + NW * 16; p0 < nrm.n_partials; p0 += NW * 16) {   // further partial sums, sixteen at a time
-        float more[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int p = p0 + NW * i;
-          more[i] = (lane < M && p < nrm.n_partials) ? nrm.ssq[(long)p * 64 + sq_row] : 0.f;
-        }
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sp += more[i];
-      }
-      sm_ssq[wave][lane] = sp;
+      sk_ssq_sum<NW, MT>(sm_ssq, sq, M, nrm, sq_row, acc[0][0][0]);   // (read after the barrier before the first strip's end)
       first_strip = false;
     }
-    sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp,
-                                           nx, pre);
+    SK_STAMP(5);
+    sk_finish<MT, NW, EPI, TC, XNORM, SSQ>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp, nx,
+                                           pre);
+    SK_STAMP(9); SK_STAMP(15);
     if (next >= n_strips) break;
     __syncthreads();   // the partial tiles in shared memory are free again
 #pragma unroll
@@ -563,13 +795,132 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
       wf[i] = wn[i];
       if (EPI == SK_GATED) uf[i] = un[i];
     }
-    strip = next; hd = hd_n; sub = sub_n; rotated = rot_n;
+    strip = next;
+    cur = nxt;
   }
 }
 
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ bf16x8 sk_buffer_load(__amdgpu_buffer_rsrc_t buf, unsigned byte_offset) {
-  return __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(buf, byte_offset, 0, 0));
+// The resident kernel for the products of a decode step proper: a folded norm in front (XNORM), at most 16 rows
+// (one token tile), all of them in order, W as the copy in the operands' order. What it leaves out is the
+// general kernel's choices at run time (which W, which rows), not work: a block's sixteen waves share the CU's
+// one scalar unit, and before the loads are on their way every wave works through the same prologue; measured
+// inside the QKV product of the 1B layers, the last of sixteen waves had its loads out 2.2 us after it started
+// with the general prologue. Here the prologue is what the loads' addresses take and no more:
+//  * no test whether a k-step, a row or a partial sum exists. The descriptors end where the data ends (a strip
+//    of the copy, the rows of A, the partial sums), so a load beyond it reads zeros: k-steps beyond K (the copy
+//    is padded with zeros to whole steps, and rows of A are tested against K for the case lda > K), rows of A
+//    from M on (they start beyond the last row's end), partial sums from n_partials on;
+//  * what only the end of a strip needs is computed by wave 0 alone, after the loads are out.
+template <int NW, int KS, int EPI, typename TC>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
+    const bf16_t* __restrict__ xg, const bf16_t* __restrict__ Wt, TC* __restrict__ C, int M, int N, int K, int lda,
+    long ldc, SkNorm nrm, SkNext nx, SkRope rp, int n_strips) {
+  constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
+  constexpr int MT = 1;
+  __shared__ f32x4 red[NW][NG][64];
+  __shared__ float sm_ssq[NW][64];
+  SK_STAMP(0); SK_STAMP(1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const bool ender = wave == 0;
+  SkToken tok = {0, 0};
+  if (EPI == SK_QKV && ender) tok = sk_token(M, rp);
+  const unsigned tile_bytes = (unsigned)((K + 31) >> 5) << 10;   // a strip of the copy: 1 KB a k-step
+  const unsigned up_strips = (unsigned)N >> 4;                   // (gated) the up strips follow the gate strips
+  int strip = blockIdx.x;
+  const unsigned w_at = (unsigned)lane * 16u + (unsigned)wave * 1024u;
+  bf16x8 wf[KS], uf[KS];
+  {
+    const __amdgpu_buffer_rsrc_t w_buf = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Wt + (long)strip * tile_bytes), 0, (int)tile_bytes, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < KS; ++i) wf[i] = sk_ld_b128(w_buf, w_at + (unsigned)i * (NW * 1024u));
+    if (EPI == SK_GATED) {
+      const __amdgpu_buffer_rsrc_t u_buf = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Wt + (long)(up_strips + strip) * tile_bytes), 0, (int)tile_bytes, 0x00020000);
+#pragma unroll
+      for (int i = 0; i < KS; ++i) uf[i] = sk_ld_b128(u_buf, w_at + (unsigned)i * (NW * 1024u));
+    }
+  }
+  bf16x8 xf[KS][MT];
+  {
+    const __amdgpu_buffer_rsrc_t a_buf = __builtin_amdgcn_make_buffer_rsrc((void*)xg, 0, (int)((((unsigned)M - 1u) * (unsigned)lda + (unsigned)K) * 2u), 0x00020000);
+    const unsigned k0 = (unsigned)wave * 32u + (unsigned)q * 8u;
+    const unsigned x_at = ((unsigned)r * (unsigned)lda + k0) * 2u;
+#pragma unroll
+    for (int i = 0; i < KS; ++i) xf[i][0] = sk_ld_b128(a_buf, k0 + (unsigned)i * (NW * 32u) < (unsigned)K ? x_at + (unsigned)i * (NW * 64u) : SK_NOWHERE);
+  }
+  float sq[4];
+  const __amdgpu_buffer_rsrc_t s_buf = __builtin_amdgcn_make_buffer_rsrc((void*)nrm.ssq, 0, nrm.n_partials * 256, 0x00020000);
+  const unsigned s_at = ((unsigned)wave + (unsigned)q * NW) * 256u + (unsigned)r * 4u;   // partial wave + NW (4 i + q) of row r
+#pragma unroll
+  for (int i = 0; i < 4; ++i) sq[i] = sk_ld_f32(s_buf, s_at + (unsigned)i * (NW * 1024u));
+  __builtin_amdgcn_sched_barrier(0);   // all of that is on its way before anything else is computed
+  SK_STAMP(2);
+  bool first_strip = true;
+  while (true) {
+    int hd = 0, sub = 0;
+    bool rotated = false;
+    SkPre pre;
+    if (ender) {
+      sk_strip_head<EPI>(strip, rp, hd, sub, rotated);
+      pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx, tok);
+    }
+    const int next = strip + gridDim.x;
+    bf16x8 wn[KS], un[KS];
+    if (next < n_strips) {   // (the same for the block; what is loaded here is used after the strip's end)
+      const __amdgpu_buffer_rsrc_t w_buf = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Wt + (long)next * tile_bytes), 0, (int)tile_bytes, 0x00020000);
+#pragma unroll
+      for (int i = 0; i < KS; ++i) wn[i] = sk_ld_b128(w_buf, w_at + (unsigned)i * (NW * 1024u));
+      if (EPI == SK_GATED) {
+        const __amdgpu_buffer_rsrc_t u_buf = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Wt + (long)(up_strips + next) * tile_bytes), 0, (int)tile_bytes, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < KS; ++i) un[i] = sk_ld_b128(u_buf, w_at + (unsigned)i * (NW * 1024u));
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);   // the next strip's loads are on their way before this strip's are used
+    SK_STAMP(3);
+    f32x4 acc[NG][MT];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) acc[g][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], xf[i][0], acc[0][0], 0, 0, 0);
+      if (EPI == SK_GATED) acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[i], xf[i][0], acc[1][0], 0, 0, 0);
+    }
+#ifdef SK_STAMPS
+    asm volatile("s_nop 0" :: "v"(acc[0][0][0]));
+    SK_STAMP(4);
+#endif
+    if (first_strip) {
+      // the waves' shares of the rows' sums of squares (tied to a result of the matrix instructions: see sk_ssq_sum)
+      // (the order of sk_ssq_sum, so that both kernels give the same sums)
+      asm volatile("" : "+v"(sq[0]) : "v"(acc[0][0][0]));
+      float sp = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sp += sq[i];
+      for (int p0 = wave + NW * 16; p0 < nrm.n_partials; p0 += NW * 16) {   // further partial sums, four a lane at a time
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = sk_ld_f32(s_buf, s_at + (unsigned)(p0 - wave) * 256u + (unsigned)i * (NW * 1024u));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sp += v[i];
+      }
+      sp += __shfl_xor(sp, 16, 64);
+      sp += __shfl_xor(sp, 32, 64);
+      sm_ssq[wave][lane] = sp;
+      first_strip = false;
+    }
+    SK_STAMP(5);
+    sk_finish<MT, NW, EPI, TC, true, false>(red, sm_ssq, acc, strip, hd, sub, rotated, C, M, N, K, ldc, nrm, nullptr, rp, nx, pre);
+    SK_STAMP(9); SK_STAMP(15);
+    if (next >= n_strips) break;
+    __syncthreads();   // the partial tiles in shared memory are free again
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      wf[i] = wn[i];
+      if (EPI == SK_GATED) uf[i] = un[i];
+    }
+    strip = next;
+  }
 }
 
 // The wide kernel, for steps of two to four token tiles: there a strip's share of A is as
@@ -604,6 +955,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   constexpr int NWT = NS * NG;        // tiles of W a pair of k-steps
   constexpr int NT = NWT + MT;        // tiles a wave stages for a pair of k-steps: 16 rows x 128 bytes each
+  SK_STAMP(0); SK_STAMP(1);
   constexpr int STAGE = NW * NT * 2048, RED = NW * NG * MT * 1024;
   __shared__ __attribute__((aligned(16))) char smem[STAGE > RED ? STAGE : RED];
   __shared__ float sm_ssq[XNORM ? NW : 1][64];
@@ -628,7 +980,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
       __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)((((long)NG * N - 1) * ldw + K) * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t a_buf =
       __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)((((long)M - 1) * lda + K) * 2), 0x00020000);
-  constexpr unsigned NOWHERE = 0x80000000u;   // beyond any buffer the entry point lets in
+  constexpr unsigned NOWHERE = SK_NOWHERE;   // beyond any buffer the entry point lets in
   int hd[NS], sub[NS];
   bool rotated[NS];
   unsigned wo[NWT][2];   // byte offsets of this lane's lines at k = 0
@@ -653,12 +1005,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   // The rotation's end needs the token's position, and through it a page number and cos and sin:
   // two trips to memory one after the other. The position is asked for before the first lines of the
   // product, what hangs on it right after them, so that both trips run beside the product's first.
-  int tok_pos = 0, tok_row = 0;
-  if (EPI == SK_QKV) {
-    const int m = min(min(wave, MT - 1) * 16 + r, M - 1);
-    tok_pos = rp.positions[m];
-    tok_row = rp.seq_of_token[m];
-  }
+  const bool ender = wave < MT;   // this wave finishes token tile `wave` of every strip
+  SkToken tok = {0, 0};
+  if (EPI == SK_QKV && ender) tok = sk_token(M, rp);
+  const int sq_row = MT == 1 ? (lane & 15) : lane;   // (a folded norm's product of all rows, in order)
+  float sq[4];
 
   const int pairs = (K + 63) / 64;
   const int p_begin = blockIdx.y * pairs_per_slice;
@@ -689,20 +1040,22 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
 #pragma unroll
     for (int t = 0; t < NWT; ++t)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) held[t][j] = sk_buffer_load(w_buf, wo[t][j] + k2);
+      for (int j = 0; j < 2; ++j) held[t][j] = sk_ld_b128(w_buf, wo[t][j] + k2);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int j = 0; j < 2; ++j)
-        held[NWT + mt][j] = sk_buffer_load(a_buf, ((xo[mt][j] | k2) & NOWHERE) ? NOWHERE : xo[mt][j] + k2);
+        held[NWT + mt][j] = sk_ld_b128(a_buf, ((xo[mt][j] | k2) & NOWHERE) ? NOWHERE : xo[mt][j] + k2);
   };
   ask(pair_at(0));
+  SK_STAMP(2);
   SkPre pre[NS];
+  if (ender) {
 #pragma unroll
-  for (int g = 0; g < NS; ++g)
-    pre[g] = sk_preload<MT, EPI, TC, 16, EPI == SK_QKV>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g],
-                                                         rotated[g], rp, nx, tok_pos, tok_row);
-  if (XNORM) sk_ssq_partials<NW>(sm_ssq, M, nrm);   // (read after the barrier before the first strip's end)
+    for (int g = 0; g < NS; ++g)
+      pre[g] = sk_preload<MT, EPI, TC>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g], rotated[g], rp, nx, tok);
+  }
+  if (XNORM) sk_ssq_ask<NW, MT>(sq, M, nrm, sq_row);
   for (int i = 0; i < n_it; ++i) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -734,6 +1087,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
+#ifdef SK_STAMPS
+  asm volatile("s_nop 0" :: "v"(acc[0][0][0][0]));
+  SK_STAMP(4);
+#endif
+  if (XNORM) sk_ssq_sum<NW, MT>(sm_ssq, sq, M, nrm, sq_row, acc[0][0][0][0]);   // (read after the barrier before the first strip's end)
+  SK_STAMP(5);
 #pragma unroll
   for (int g = 0; g < NS; ++g) {
     __syncthreads();   // the staged lines, then the partial tiles of the strip before, are free
@@ -741,6 +1100,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
       sk_finish<MT, NW, EPI, TC, XNORM, false>(red, sm_ssq, acc[g], strip0 + g, hd[g], sub[g], rotated[g], out, M, N, K,
                                                 ldc, nrm, nullptr, rp, nx, pre[g]);
   }
+  SK_STAMP(9); SK_STAMP(15);
 }
 
 struct SkCall {
@@ -782,7 +1142,10 @@ static int launch_skinny(int nw, const SkCall& a) {
     if (a.strip_rows == 8) {
       // strips of 8 rows: twice the blocks, each with half the rows to stream; with at most 8 rows of A
       // the tile's other half takes the next 32 k
-      if (a.M <= 8)
+      if (a.M <= 8 && a.Wt8 && a.lda < (1L << 24) && a.K < (1 << 24))   // (32-bit byte offsets inside a strip and inside A)
+        gemm_skinny_pack_kernel<16, EPI, TC, SSQ><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
+            (const bf16_t*)a.A, (const bf16_t*)a.Wt8, (TC*)a.C, a.M, a.N, a.K, (int)a.lda, a.ldc, a.ssq_out, a.nx, a.a_packed);
+      else if (a.M <= 8)
         gemm_skinny_kernel<MT, 16, EPI, TC, XNORM, SSQ, 8, true><<<dim3((a.N + 7) / 8), dim3(16 * 64), 0, a.stream>>>(
             a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp,
             (const bf16_t*)a.Wt8, a.a_packed);
@@ -792,6 +1155,23 @@ static int launch_skinny(int nw, const SkCall& a) {
             (const bf16_t*)nullptr, 0);
       GL3_LAUNCH_CHECK();
       return 0;
+    }
+  }
+  if constexpr (MT == 1 && XNORM && !SSQ) {
+    // a decode step's products with a folded norm over the copy of W: the kernel with the short prologue
+    if (a.resident && a.Wt && !a.nrm.rows && a.lda < (1L << 24) && a.K < (1 << 24) && (long)steps * 1024 < (1L << 31)) {
+#define DEC(KS)                                                                                                  \
+  do {                                                                                                           \
+    gemm_skinny_decode_kernel<16, KS, EPI, TC><<<dim3(resident_blocks(n_strips, 16)), dim3(16 * 64), 0, a.stream>>>( \
+        (const bf16_t*)a.A, (const bf16_t*)a.Wt, (TC*)a.C, a.M, a.N, a.K, (int)a.lda, a.ldc, a.nrm, a.nx, a.rp, n_strips); \
+    GL3_LAUNCH_CHECK();                                                                                          \
+    return 0;                                                                                                    \
+  } while (0)
+      if (steps <= 64) DEC(4);
+      if constexpr (EPI == SK_STORE) {
+        if (steps <= 128) DEC(8);
+      }
+#undef DEC
     }
   }
   if (a.resident) {
@@ -1065,7 +1445,7 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
                                   const int* seq_of_token, const int* block_table, int table_stride,
                                   const float* cos_tab, const float* sin_tab, void* k_cache, void* v_cache,
                                   int n_heads, int n_kv, int head_dim, int adjacent, int page_size, int waves,
-                                  const void* w_tiled, hipStream_t stream) {
+                                  const void* w_tiled, const int* token_pages, const float* token_rot, hipStream_t stream) {
   if (M == 0) return 0;
   const int N = (n_heads + 2 * n_kv) * head_dim;
   if (check_common("gl3_qkv_rope_cache", a_rows, Wqkv, q_out, M, N, K, lda, ldw, waves)) return -1;
@@ -1079,8 +1459,9 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
   GL3_REQUIRE(ldq >= (long)n_heads * head_dim && ldq % 4 == 0 && (uintptr_t)q_out % 8 == 0,
               "gl3_qkv_rope_cache: q_out stride/alignment");
   const SkNorm nrm = {ssq, n_partials, eps, nullptr};
+  GL3_REQUIRE(!token_pages || !cos_tab || token_rot, "gl3_qkv_rope_cache: the tokens' pages come with their rows of cos and sin");
   const SkRope rp = {positions, seq_of_token, block_table, table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
-                     (bf16_t*)v_cache, n_heads, n_kv, head_dim, adjacent, page_size};
+                     (bf16_t*)v_cache, n_heads, n_kv, head_dim, adjacent, page_size, token_pages, token_rot};
   SkCall a = {a_rows, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
   GL3_REQUIRE(!w_tiled || (uintptr_t)w_tiled % 16 == 0, "gl3_qkv_rope_cache: the copy of W must be 16-byte aligned");
   a.Wt = w_tiled;   // (its strips hold the rows that sk_strip_row names: for half-split pairing 8 rows and the 8 half a head further)

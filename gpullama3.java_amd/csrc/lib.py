@@ -64,7 +64,8 @@ def _declare(lib):
         "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P, I, P],
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P, I, F, I, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, I, P],
-        "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P],
+        "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
+        "gl3_token_facts": [P, P, P, I, I, P, P, I, P, P, I, P],
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
@@ -599,11 +600,34 @@ def qkv_rope_cache_fits(a, w_qkv, head_dim, rot_dim):
             and head_dim % 16 == 0 and rot_dim in (0, head_dim))
 
 
+def token_facts(positions, table_rows, block_table, page_size, cos, sin, pages, rot):
+    """What hangs on each token's position, looked up once for all layers of a step: ``pages`` [T] int32
+    receives the page of the token's position (``block_table[table_rows[t]][positions[t] // page_size]``) and
+    ``rot`` [T, 2 * half] float32 its rows of ``cos`` and ``sin`` one after the other (``cos``, ``sin``, ``rot``
+    all None: no rotation, the pages alone). ``qkv_rope_cache`` takes both in place of its own look-ups."""
+    _dev(positions, "positions", torch.int32); _dev(table_rows, "table_rows", torch.int32)
+    _dev(block_table, "block_table", torch.int32); _dev(pages, "pages", torch.int32)
+    T = positions.numel()
+    if table_rows.numel() != T or pages.numel() != T or block_table.dim() != 2:
+        raise KernelError("token_facts: one row of the table and one page per token")
+    half = 0
+    if cos is not None:
+        _dev(cos, "cos", torch.float32); _dev(sin, "sin", torch.float32); _dev(rot, "rot", torch.float32)
+        half = cos.shape[1]
+        if cos.shape != sin.shape or cos.dim() != 2 or rot.shape != (T, 2 * half):
+            raise KernelError(f"token_facts: tables {tuple(cos.shape)}, rows {tuple(rot.shape)} for {T} tokens")
+    elif sin is not None or rot is not None:
+        raise KernelError("token_facts: the tables and the rows for them come together")
+    _check(library().gl3_token_facts(_ptr(positions), _ptr(table_rows), _ptr(block_table), block_table.shape[1], int(page_size),
+                                     _ptr(cos), _ptr(sin), half, _ptr(pages), _ptr(rot), T, _stream()), "token_facts")
+
+
 def qkv_rope_cache(a, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_token, block_table, cos, sin,
-                   k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page_size, waves=0):
+                   k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page_size, waves=0, token_pages=None, token_rot=None):
     """a @ w_qkv.T, rotation, q into ``q_out`` [T, H*hs] bfloat16, k and v into the cache. ``ssq`` None:
     ``a`` holds the rows as they are; else ``a`` = bfloat16(norm weight * x) and the product is that
-    of RMSNorm(x), the rows' sums of squares coming as partial sums."""
+    of RMSNorm(x), the rows' sums of squares coming as partial sums. ``token_pages``, ``token_rot``: what
+    ``token_facts`` made of the same positions, table and rotation (then the kernel does not look them up)."""
     _dev(w_qkv, "w_qkv", torch.bfloat16); _dev(q_out, "q_out", torch.bfloat16, contiguous=False)
     K = w_qkv.shape[1]
     if ssq is None:
@@ -626,11 +650,21 @@ def qkv_rope_cache(a, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_toke
         _dev(cos, "cos", torch.float32); _dev(sin, "sin", torch.float32)
         if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != head_dim // 2:
             raise KernelError(f"qkv_rope_cache: table {tuple(cos.shape)} for head_dim {head_dim}")
+    # (the kernel reads the tables through 32-bit byte offsets)
+    if block_table.numel() >= 2 ** 29 or (cos is not None and cos.numel() >= 2 ** 29):
+        raise KernelError("qkv_rope_cache: a block table or rotation table of 2 GiB or more")
+    if token_pages is not None:
+        _dev(token_pages, "token_pages", torch.int32)
+        if token_pages.numel() != T or (cos is not None and (token_rot is None or token_rot.dtype != torch.float32
+                                                             or token_rot.shape != (T, head_dim) or not token_rot.is_cuda
+                                                             or not token_rot.is_contiguous())):
+            raise KernelError("qkv_rope_cache: a page per token, and with a rotation a row [head_dim] of cos and sin per token")
     _check(library().gl3_qkv_rope_cache(
         _ptr(a), _ptr(ssq), n_partials, float(eps), _ptr(w_qkv), _ptr(q_out), q_out.stride(0), T, K, a.stride(0),
         w_qkv.stride(0), _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], _ptr(cos),
         _ptr(sin), _ptr(k_cache), _ptr(v_cache), n_heads, n_kv, head_dim, int(adjacent), page_size, waves,
-        _tiled(w_qkv, w_qkv.shape[0], K, qkv=(n_heads, n_kv, head_dim, cos is not None, bool(adjacent))), _stream()),
+        _tiled(w_qkv, w_qkv.shape[0], K, qkv=(n_heads, n_kv, head_dim, cos is not None, bool(adjacent))),
+        _ptr(token_pages), _ptr(token_rot if token_pages is not None and cos is not None else None), _stream()),
         "qkv_rope_cache")
 
 

@@ -184,14 +184,16 @@ class Engine:
         V = self.spec.vocab_size
         if B == 0:
             return torch.empty((0, V), dtype=torch.float32, device=self.device)
-        slots, arrays = self._entries(entries)
-        counts = [a.size for a in arrays]
-        single = max(counts) == 1
+        slots, arrays, ints = self._entries(entries)          # (ints: every entry is a list of one int, kept as ints)
+        counts = [1] * B if ints else [a.size for a in arrays]
+        single = ints or max(counts) == 1
         if single and want != "last" and isinstance(want, (list, tuple)) and len(want) == B \
                 and all(len(w) == 1 and w[0] == 0 for w in want):
             want = "last"                         # the only token of every entry: the same step
         if single and want == "last" and self.use_graphs:
-            return self._step_decode(slots, [int(a[0]) for a in arrays])
+            return self._step_decode(slots, arrays if ints else [int(a[0]) for a in arrays])
+        if ints:
+            arrays = [np.array([t], dtype=np.int32) for t in arrays]
         starts = [self.cache.length(s) for s in slots]
         T = sum(counts)
         tokens = arrays[0] if B == 1 else np.concatenate(arrays)
@@ -241,29 +243,36 @@ class Engine:
         return logits
 
     def _entries(self, entries):
-        """What every step checks before anything changes: ``(slots, one int32 array of tokens per entry)``.
-        Slots are integers that appear once; tokens are integers inside the vocabulary, at least one an entry."""
+        """What every step checks before anything changes: ``(slots, tokens per entry, all_single)``. Slots are
+        integers that appear once; tokens are integers inside the vocabulary, at least one an entry. When every
+        entry brings a list of one int (the usual decode step) the tokens come back as those ints and
+        ``all_single`` is true; else as one int32 array per entry."""
         V = self.spec.vocab_size
-        slots, arrays = [], []
+        slots, arrays, all_single = [], [], True
         for b, (slot, toks) in enumerate(entries):
-            if type(toks) is list and len(toks) == 1 and type(toks[0]) is int:       # (the usual decode step)
-                a = np.array(toks, dtype=np.int64)
+            if type(toks) is list and len(toks) == 1 and type(toks[0]) is int:
+                a = toks[0]
+                lo = hi = a
             else:
+                all_single = False
                 a = np.asarray(toks.cpu() if isinstance(toks, torch.Tensor) else toks)
                 if a.ndim == 0:
                     a = a.reshape(1)
                 if a.ndim != 1 or (a.size and a.dtype.kind not in "iu"):
                     raise ValueError(f"entry {b}: tokens must be a flat sequence of integers")
-            if a.size == 0:
-                raise ValueError(f"entry {b} brings no token")
-            lo, hi = int(a.min()), int(a.max())
+                if a.size == 0:
+                    raise ValueError(f"entry {b} brings no token")
+                lo, hi = int(a.min()), int(a.max())
+                a = a.astype(np.int32, copy=False)
             if lo < 0 or hi >= V:
                 raise ValueError(f"entry {b}: token id {lo if lo < 0 else hi} is outside the vocabulary of {V}")
             slots.append(int(slot))
-            arrays.append(a.astype(np.int32, copy=False))
+            arrays.append(a)
         if len(set(slots)) != len(slots):
             raise ValueError("a slot appears twice in one step")
-        return slots, arrays
+        if not all_single:
+            arrays = [np.array([a], dtype=np.int32) if type(a) is int else a for a in arrays]
+        return slots, arrays, all_single
 
     def _staging(self, n):
         """Pinned host memory for the next step's input: one of a ring of buffers, free once the copy out of it
@@ -326,10 +335,10 @@ class Engine:
         if not self.use_graphs or not 1 <= n <= RUN_LENGTH:
             raise ValueError(f"a run takes 1..{RUN_LENGTH} steps on an engine that replays graphs")
         from ..csrc import lib as K
-        slots, arrays = self._entries([(s, [t] if isinstance(t, int) else t) for s, t in entries])
-        if any(a.size != 1 for a in arrays):
+        slots, arrays, ints = self._entries([(s, [t] if isinstance(t, int) else t) for s, t in entries])
+        if not ints and any(a.size != 1 for a in arrays):
             raise ValueError("a run of decode steps starts from one token per sequence")
-        tokens = [int(a[0]) for a in arrays]
+        tokens = arrays if ints else [int(a[0]) for a in arrays]
         starts = [self.cache.length(s) for s in slots]
         B = len(slots)
         self.cache.reserve({s: n for s in slots})

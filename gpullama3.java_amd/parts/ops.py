@@ -332,6 +332,23 @@ def _table_rows(ctx):
     return rows if rows is not None else ctx.seq_of_token
 
 
+def _token_facts(ctx, block_table, cos, sin, page_size):
+    """The page of each token's position and its rows of cos and sin, looked up once per step for all layers
+    that share the block table and the rotation (``lib.token_facts``): in the QKV product of every layer they
+    would be a second trip to memory behind the token's position. A step's context keeps them by the tables
+    they were made from."""
+    made = ctx.__dict__.setdefault("token_facts", {})
+    key = (block_table.data_ptr(), cos.data_ptr() if cos is not None else 0, page_size)
+    if key not in made:
+        n = len(made)
+        T = ctx.positions.numel()
+        pages = ctx.buffer(f"token_pages{n}", (T,), torch.int32)
+        rot = ctx.buffer(f"token_rot{n}", (T, 2 * cos.shape[1]), torch.float32) if cos is not None else None
+        K.token_facts(ctx.positions, _table_rows(ctx), block_table, page_size, cos, sin, pages, rot)
+        made[key] = (pages, rot)
+    return made[key]
+
+
 def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_heads, n_kv, head_dim, dtype, writes_kv,
                 bias=None):
     """Queries, keys and values of the step's tokens: q rotated into a buffer whose rows start
@@ -347,8 +364,10 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
     if (isinstance(h, Normed) and writes_kv and h.rows is None and "fused" not in disabled and bias is None
             and K.qkv_rope_cache_fits(h.xg, w_qkv, head_dim, rot)):
         q = ctx.buffer("q", (T, n_heads * head_dim), dtype)
+        pages, rows_of_rotation = _token_facts(ctx, block_table, cos, sin, page)
         K.qkv_rope_cache(h.xg, h.ssq, h.n_partials, h.eps, w_qkv, q, ctx.positions, _table_rows(ctx),
-                         block_table, cos, sin, k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page)
+                         block_table, cos, sin, k_cache, v_cache, n_heads, n_kv, head_dim, adjacent, page,
+                         token_pages=pages, token_rot=rows_of_rotation)
         return q
     if isinstance(h, Normed):
         h = h.materialize()

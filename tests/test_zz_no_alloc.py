@@ -45,6 +45,33 @@ def test_static_argmax_matches_the_workspace_one_on_two_calls_in_a_row():
             torch.cuda.synchronize()
             assert got.tolist() == want.tolist()
             assert got[0].item() == 11 and got[1].item() == vocab - 1 and got[2].item() == 0
+            # an answer that no kernel of the library had a hand in (no ties beyond row 0's)
+            assert got[1:].tolist() == torch.argmax(logits[1:], dim=1).tolist()
+
+
+def test_static_argmax_at_the_edges_of_its_array_and_of_a_row():
+    """On one stream, after a large call that fills the library's array: as many rows as the array holds
+    (the last row's partial results lie at its very end), a strided view of wider rows, and a row shorter
+    than the 64 slices it is cut into (most slices are empty). Checked against ``torch.argmax``."""
+    K, lib, static = _calls()
+    dev = "cuda:0"
+    g = torch.Generator(device="cpu").manual_seed(6)
+    with torch.cuda.device(dev):
+        cases = []
+        full = torch.randn(256, 3001, generator=g).to(dev)
+        cases.append(full)
+        wide = torch.randn(9, 700, generator=g).to(dev)
+        cases.append(wide[:, :333])                              # rows 700 floats apart, 333 of them read
+        wide[:, 333:] = 100.0                                    # what lies beyond a row's end must not win
+        cases.append(torch.randn(5, 41, generator=g).to(dev))    # fewer columns than slices
+        cases.append(torch.randn(2, 1, generator=g).to(dev))
+        for logits in cases:
+            rows, vocab = logits.shape
+            got = torch.full((rows,), -1, dtype=torch.int32, device=dev)
+            rc = static(logits.data_ptr(), logits.stride(0), got.data_ptr(), rows, vocab, _stream())
+            assert rc == 0, lib.gl3_last_error().decode()
+            torch.cuda.synchronize()
+            assert got.tolist() == torch.argmax(logits, dim=1).tolist(), (rows, vocab)
 
 
 def test_static_argmax_refuses_more_rows_than_its_array_holds():
