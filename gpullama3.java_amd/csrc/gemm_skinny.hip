@@ -203,13 +203,15 @@ __device__ __forceinline__ void sk_load_x(bf16x8 (&xf)[MT], __amdgpu_buffer_rsrc
 // of wave w takes the partials w + NW (4 i + j), and the first four of each lane (64 NW partials in all) are
 // asked for with the block's first loads (sk_ssq_ask); sk_ssq_sum, at the first strip's end, adds them, fetches
 // any further ones, and adds the groups. More token tiles: lane = row, sixteen partials at a time, all in sk_ssq_sum.
+// (SK_SQN: how many a lane asks for at the start: 512 partial sums a block, what strips of 8 columns of rows of 4,096 leave)
+#define SK_SQN(NW) (128 / (NW))
 template <int NW, int MT>
-__device__ __forceinline__ void sk_ssq_ask(float (&sq)[4], int M, const SkNorm& nrm, int sq_row) {
+__device__ __forceinline__ void sk_ssq_ask(float (&sq)[SK_SQN(NW)], int M, const SkNorm& nrm, int sq_row) {
   if (MT != 1) return;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const __amdgpu_buffer_rsrc_t buf = sk_rsrc(nrm.ssq, (long)nrm.n_partials * 256);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < SK_SQN(NW); ++i) {
     const int p = wave + NW * (4 * i + (lane >> 4));
     sq[i] = sk_ld_f32(buf, ((lane & 15) < M && p < nrm.n_partials) ? (unsigned)((p * 64 + sq_row) * 4) : SK_NOWHERE);
   }
@@ -218,7 +220,7 @@ __device__ __forceinline__ void sk_ssq_ask(float (&sq)[4], int M, const SkNorm& 
 // value they cannot be added up, and waited for, at the point where they were asked for, in front of loads
 // that should be on their way first.
 template <int NW, int MT>
-__device__ __forceinline__ void sk_ssq_sum(float (*sm_ssq)[64], float (&sq)[4], int M, const SkNorm& nrm, int sq_row,
+__device__ __forceinline__ void sk_ssq_sum(float (*sm_ssq)[64], float (&sq)[SK_SQN(NW)], int M, const SkNorm& nrm, int sq_row,
                                            float after) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const __amdgpu_buffer_rsrc_t buf = sk_rsrc(nrm.ssq, (long)nrm.n_partials * 256);
@@ -226,8 +228,8 @@ __device__ __forceinline__ void sk_ssq_sum(float (*sm_ssq)[64], float (&sq)[4], 
   if (MT == 1) {
     asm volatile("" : "+v"(sq[0]) : "v"(after));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) sp += sq[i];
-    for (int p0 = wave + NW * 16; p0 < nrm.n_partials; p0 += NW * 16) {   // further partial sums, four a lane at a time
+    for (int i = 0; i < SK_SQN(NW); ++i) sp += sq[i];
+    for (int p0 = wave + NW * 4 * SK_SQN(NW); p0 < nrm.n_partials; p0 += NW * 16) {   // further partial sums, four a lane at a time
       float v[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -275,9 +277,9 @@ struct SkPre {
 // A token's position and its row of the block table (SK_QKV), asked for before the product's own loads so
 // that what hangs on them (page number, cos and sin) can be asked for while those are still on their way.
 struct SkToken { int pos, row; };
-__device__ __forceinline__ SkToken sk_token(int M, const SkRope& rp) {
+__device__ __forceinline__ SkToken sk_token(int M, const SkRope& rp, int tile = -1) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r = threadIdx.x & 15;
-  const int m = wave * 16 + r;
+  const int m = (tile < 0 ? wave : tile) * 16 + r;
   const unsigned at = m < M ? (unsigned)m * 4u : SK_NOWHERE;
   SkToken t;
   t.pos = sk_ld_i32(sk_rsrc(rp.positions, (long)M * 4), at);
@@ -290,7 +292,7 @@ __device__ __forceinline__ SkToken sk_token(int M, const SkRope& rp) {
 template <int MT, int EPI, typename TC, int ROWS = 16>
 __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int N, long ldc, int strip, int hd, int sub,
                                             bool rotated, const SkRope& rp, const SkNext& nx = SkNext{},
-                                            SkToken tok = SkToken{0, 0}) {
+                                            SkToken tok = SkToken{0, 0}, int tile = -1) {
   SkPre p;
   p.prev = p.bias = p.bias_up = p.next_w = p.co = p.si = f32x4{0.f, 0.f, 0.f, 0.f};
   p.pos = 0; p.page = 0;
@@ -300,7 +302,7 @@ __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int
   asm volatile("" : "+v"(tok.pos), "+v"(tok.row), "+s"(strip));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
-  const int m = wave * 16 + r;
+  const int m = (tile < 0 ? wave : tile) * 16 + r;   // (`tile`: the token tile that the wave finishes, its own number unless said)
   const bool live = m < M && 4 * q < ROWS;
   const int n = strip * ROWS + 4 * q;
   if (EPI != SK_QKV && nx.bias) {   // (the same for the whole grid; nothing hangs on these loads before the strip's end)
@@ -352,6 +354,109 @@ __device__ __forceinline__ SkPre sk_preload(const TC* __restrict__ C, int M, int
   return p;
 }
 
+// The end of one token tile of a strip, by one wave: `v` (gated: and `up`) are the strip's sums for token tile `mt`,
+// a lane holding tile rows 4q .. 4q+3 (columns of C) of token mt*16 + r. `sub`, `hd`, `rotated` describe the strip
+// for SK_QKV; `pre` is what sk_preload asked for.
+template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ, int ROWS = 16>
+__device__ __forceinline__ void sk_end_tile(f32x4 v, f32x4 up, int mt, float (*sm_ssq)[64], int strip, int hd, int sub,
+                                            bool rotated, TC* __restrict__ C, int M, int N, int K, long ldc,
+                                            const SkNorm& nrm, float* __restrict__ ssq_out, const SkRope& rp,
+                                            const SkNext& nx, const SkPre& pre) {
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const int n0 = strip * ROWS;
+  const int m = mt * 16 + r;
+  const bool m_ok = m < M;
+  if (XNORM) {
+    float ss = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) ss += sm_ssq[w][min(m, 63)];
+    const float rms = 1.0f / sqrtf(ss / (float)K + nrm.eps);
+    v *= rms;
+    up *= rms;
+  }
+  if (EPI != SK_QKV) {
+    v += pre.bias;
+    up += pre.bias_up;
+  }
+  if (EPI == SK_GATED) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v[c] = gl3_activation<true>(v[c], nx.act) * up[c];
+  }
+  if (EPI == SK_QKV) {
+    const int hs = rp.head_dim;
+    const int pos = pre.pos;
+    int col = 16 * sub + 4 * q;          // first of this lane's 4 columns inside the head
+    if (rotated) {
+      const int half = hs / 2;
+      if (rp.adjacent) {
+        const float c0 = pre.co[0], s0 = pre.si[0];
+        const float c1 = pre.co[1], s1 = pre.si[1];
+        const f32x4 o = v;
+        v[0] = o[0] * c0 - o[1] * s0;
+        v[1] = o[0] * s0 + o[1] * c0;
+        v[2] = o[2] * c1 - o[3] * s1;
+        v[3] = o[2] * s1 + o[3] * c1;
+      } else {
+        // quarters 0,1 hold the first elements of 8 pairs, quarters 2,3 their partners
+        const bool first = q < 2;
+        const int jj = 8 * sub + 4 * (q & 1);
+        col = (first ? 0 : half) + jj;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const float other = __shfl_xor(v[c], 32, 64);
+          const float co = pre.co[c], si = pre.si[c];
+          v[c] = first ? v[c] * co - other * si : other * si + v[c] * co;
+        }
+      }
+    }
+    if (m_ok) {
+      if (hd < rp.n_heads) {
+        bf16x4 o4;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) o4[c] = static_cast<bf16_t>(v[c]);
+        *(bf16x4*)((bf16_t*)C + (long)m * ldc + (long)hd * hs + col) = o4;
+      } else {
+        const long page = pre.page;
+        const int in_page = pos % rp.page_size;
+        if (hd < rp.n_heads + rp.n_kv) {
+          const int ch = hd - rp.n_heads;
+          bf16x4 o4;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) o4[c] = static_cast<bf16_t>(v[c]);
+          *(bf16x4*)(rp.k_cache + (page * rp.n_kv + ch) * (long)rp.page_size * hs + gl3_k_offset(in_page, col, hs)) = o4;
+        } else {
+          const int ch = hd - rp.n_heads - rp.n_kv;
+          bf16_t* vt = rp.v_cache + (page * rp.n_kv + ch) * (long)rp.page_size * hs + gl3_v_offset(col, in_page, rp.page_size);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) vt[8 * c] = static_cast<bf16_t>(v[c]);   // (col % 4 == 0: the 4 dims lie in one tile)
+        }
+      }
+    }
+    return;
+  }
+  const int n = n0 + 4 * q;
+  TC* cp = (EPI != SK_ADD && nx.pack_out) ? C + sk_packed_offset(m & 7, n) : C + (long)m * ldc + n;
+  float sq = 0.f;
+  if (m_ok && 4 * q < ROWS) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (n + c < N) {
+        float o = v[c];
+        if (EPI == SK_ADD) o += pre.prev[c];
+        cp[c] = from_f32<TC>(o);
+        sq += o * o;
+        if (SSQ && nx.weight) nx.xg[(long)m * nx.ld + n + c] = static_cast<bf16_t>(pre.next_w[c] * o);
+      }
+    }
+  }
+  if (SSQ) {
+    sq += __shfl_xor(sq, 16, 64);
+    sq += __shfl_xor(sq, 32, 64);
+    if (q == 0 && m_ok) ssq_out[(long)strip * 64 + m] = sq;
+  }
+}
+
 // The end of a strip: the waves' partial tiles are summed in wave order by the wave that owns
 // the tile, then the epilogue runs. `sub`, `hd`, `rotated` describe the strip for SK_QKV.
 template <int MT, int NW, int EPI, typename TC, bool XNORM, bool SSQ, int ROWS = 16>
@@ -381,100 +486,9 @@ __device__ __forceinline__ void sk_finish(f32x4 (*red)[((EPI == SK_GATED) ? 2 : 
   SK_STAMP(7);
 
   // epilogue: lane holds tile rows 4q .. 4q+3 (columns of C) of token mt*16 + r
-  for (int mt = wave; mt < MT; mt += NW) {
-    const int m = mt * 16 + r;
-    const bool m_ok = m < M;
-    f32x4 v = red[0][mt][lane];
-    f32x4 up = (EPI == SK_GATED) ? red[0][MT + mt][lane] : zero4;
-    if (XNORM) {
-      float ss = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) ss += sm_ssq[w][min(m, 63)];
-      const float rms = 1.0f / sqrtf(ss / (float)K + nrm.eps);
-      v *= rms;
-      up *= rms;
-    }
-    if (EPI != SK_QKV) {
-      v += pre.bias;
-      up += pre.bias_up;
-    }
-    if (EPI == SK_GATED) {
-#pragma unroll
-      for (int c = 0; c < 4; ++c) v[c] = gl3_activation<true>(v[c], nx.act) * up[c];
-    }
-    if (EPI == SK_QKV) {
-      const int hs = rp.head_dim;
-      const int pos = pre.pos;
-      int col = 16 * sub + 4 * q;          // first of this lane's 4 columns inside the head
-      if (rotated) {
-        const int half = hs / 2;
-        if (rp.adjacent) {
-          const float c0 = pre.co[0], s0 = pre.si[0];
-          const float c1 = pre.co[1], s1 = pre.si[1];
-          const f32x4 o = v;
-          v[0] = o[0] * c0 - o[1] * s0;
-          v[1] = o[0] * s0 + o[1] * c0;
-          v[2] = o[2] * c1 - o[3] * s1;
-          v[3] = o[2] * s1 + o[3] * c1;
-        } else {
-          // quarters 0,1 hold the first elements of 8 pairs, quarters 2,3 their partners
-          const bool first = q < 2;
-          const int jj = 8 * sub + 4 * (q & 1);
-          col = (first ? 0 : half) + jj;
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const float other = __shfl_xor(v[c], 32, 64);
-            const float co = pre.co[c], si = pre.si[c];
-            v[c] = first ? v[c] * co - other * si : other * si + v[c] * co;
-          }
-        }
-      }
-      if (m_ok) {
-        if (hd < rp.n_heads) {
-          bf16x4 o4;
-#pragma unroll
-          for (int c = 0; c < 4; ++c) o4[c] = static_cast<bf16_t>(v[c]);
-          *(bf16x4*)((bf16_t*)C + (long)m * ldc + (long)hd * hs + col) = o4;
-        } else {
-          const long page = pre.page;
-          const int in_page = pos % rp.page_size;
-          if (hd < rp.n_heads + rp.n_kv) {
-            const int ch = hd - rp.n_heads;
-            bf16x4 o4;
-#pragma unroll
-            for (int c = 0; c < 4; ++c) o4[c] = static_cast<bf16_t>(v[c]);
-            *(bf16x4*)(rp.k_cache + (page * rp.n_kv + ch) * (long)rp.page_size * hs + gl3_k_offset(in_page, col, hs)) = o4;
-          } else {
-            const int ch = hd - rp.n_heads - rp.n_kv;
-            bf16_t* vt = rp.v_cache + (page * rp.n_kv + ch) * (long)rp.page_size * hs + gl3_v_offset(col, in_page, rp.page_size);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) vt[8 * c] = static_cast<bf16_t>(v[c]);   // (col % 4 == 0: the 4 dims lie in one tile)
-          }
-        }
-      }
-      continue;
-    }
-    const int n = n0 + 4 * q;
-    TC* cp = (EPI != SK_ADD && nx.pack_out) ? C + sk_packed_offset(m & 7, n) : C + (long)m * ldc + n;
-    float sq = 0.f;
-    if (m_ok && 4 * q < ROWS) {
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        if (n + c < N) {
-          float o = v[c];
-          if (EPI == SK_ADD) o += pre.prev[c];
-          cp[c] = from_f32<TC>(o);
-          sq += o * o;
-          if (SSQ && nx.weight) nx.xg[(long)m * nx.ld + n + c] = static_cast<bf16_t>(pre.next_w[c] * o);
-        }
-      }
-    }
-    if (SSQ) {
-      sq += __shfl_xor(sq, 16, 64);
-      sq += __shfl_xor(sq, 32, 64);
-      if (q == 0 && m_ok) ssq_out[(long)strip * 64 + m] = sq;
-    }
-  }
+  for (int mt = wave; mt < MT; mt += NW)
+    sk_end_tile<MT, NW, EPI, TC, XNORM, SSQ, ROWS>(red[0][mt][lane], (EPI == SK_GATED) ? red[0][MT + mt][lane] : zero4, mt, sm_ssq,
+                                                   strip, hd, sub, rotated, C, M, N, K, ldc, nrm, ssq_out, rp, nx, pre);
 }
 
 // PACK (strips of 8 rows, at most 8 rows of A, one token tile): the tile's rows 8..15 are the strip's
@@ -529,7 +543,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   const unsigned w_lane = tiled ? (unsigned)lane * 16u : (unsigned)(((long)(wr - w0) * ldw + koff) * 2);
   const unsigned w_step = tiled ? 1024u : (PACK ? 128u : 64u);   // bytes from one step to the next
   const __amdgpu_buffer_rsrc_t a_buf = a_packed ? sk_rsrc(Av, (long)steps64 * 1024) : sk_a_rsrc(Av, M, K, lda, XNORM ? &nrm : nullptr);
-  float sq[4];
+  float sq[SK_SQN(NW)];
   if (XNORM) sk_ssq_ask<NW, MT>(sq, M, nrm, sq_row);
   SkPre pre;
   if (ender) pre = sk_preload<MT, EPI, TC, ROWS>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx, tok);
@@ -735,7 +749,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
       sk_load_x<MT>(xf[i], a_buf, xo, k < K ? (unsigned)k * 2u : SK_NOWHERE);
     }
   }
-  float sq[4];
+  float sq[SK_SQN(NW)];
   if (XNORM) sk_ssq_ask<NW, MT>(sq, M, nrm, sq_row);
   __builtin_amdgcn_sched_barrier(0);   // all of that is on its way before anything else is computed
   SK_STAMP(2);
@@ -848,11 +862,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
 #pragma unroll
     for (int i = 0; i < KS; ++i) xf[i][0] = sk_ld_b128(a_buf, k0 + (unsigned)i * (NW * 32u) < (unsigned)K ? x_at + (unsigned)i * (NW * 64u) : SK_NOWHERE);
   }
-  float sq[4];
+  float sq[SK_SQN(NW)];
   const __amdgpu_buffer_rsrc_t s_buf = __builtin_amdgcn_make_buffer_rsrc((void*)nrm.ssq, 0, nrm.n_partials * 256, 0x00020000);
   const unsigned s_at = ((unsigned)wave + (unsigned)q * NW) * 256u + (unsigned)r * 4u;   // partial wave + NW (4 i + q) of row r
 #pragma unroll
-  for (int i = 0; i < 4; ++i) sq[i] = sk_ld_f32(s_buf, s_at + (unsigned)i * (NW * 1024u));
+  for (int i = 0; i < SK_SQN(NW); ++i) sq[i] = sk_ld_f32(s_buf, s_at + (unsigned)i * (NW * 1024u));
   __builtin_amdgcn_sched_barrier(0);   // all of that is on its way before anything else is computed
   SK_STAMP(2);
   bool first_strip = true;
@@ -896,8 +910,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
       asm volatile("" : "+v"(sq[0]) : "v"(acc[0][0][0]));
       float sp = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sp += sq[i];
-      for (int p0 = wave + NW * 16; p0 < nrm.n_partials; p0 += NW * 16) {   // further partial sums, four a lane at a time
+      for (int i = 0; i < SK_SQN(NW); ++i) sp += sq[i];
+      for (int p0 = wave + NW * 4 * SK_SQN(NW); p0 < nrm.n_partials; p0 += NW * 16) {   // further partial sums, four a lane at a time
         float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = sk_ld_f32(s_buf, s_at + (unsigned)(p0 - wave) * 256u + (unsigned)i * (NW * 1024u));
@@ -956,15 +970,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   constexpr int NWT = NS * NG;        // tiles of W a pair of k-steps
   constexpr int NT = NWT + MT;        // tiles a wave stages for a pair of k-steps: 16 rows x 128 bytes each
   SK_STAMP(0); SK_STAMP(1);
-  constexpr int STAGE = NW * NT * 2048, RED = NW * NG * MT * 1024;
+  constexpr int NTILES = NS * NG * MT;   // the partial tiles of a wave: all of the block's strips end together
+  constexpr int STAGE = NW * NT * 2048, RED = NW * NTILES * 1024;
   __shared__ __attribute__((aligned(16))) char smem[STAGE > RED ? STAGE : RED];
   __shared__ float sm_ssq[XNORM ? NW : 1][64];
-  f32x4 (*red)[NG * MT][64] = (f32x4 (*)[NG * MT][64])smem;   // the partial tiles, once the staging is over
+  f32x4 (*red)[NTILES][64] = (f32x4 (*)[NTILES][64])smem;   // the partial tiles, once the staging is over
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int r = lane & 15, q = lane >> 4;
   const int l8 = lane >> 3, c8 = lane & 7;
   const int n_strips = (N + 15) / 16;
   const int strip0 = blockIdx.x * NS;
+  SK_STAMP(10);
   char* stage = smem + wave * (NT * 2048);
   // where this lane's loads go inside a tile (rows l8 and 8 + l8) and where its operands lie (k-steps 0, 1)
   const int put0 = l8 * 128 + ((c8 ^ l8) * 16);
@@ -990,7 +1006,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
     for (int j = 0; j < 2; ++j) {
       const int wr = sk_strip_row<EPI>(min(strip0 + g, n_strips - 1), 8 * j + l8, N, rp, hd[g], sub[g], rotated[g]);
 #pragma unroll
-      for (int h = 0; h < NG; ++h) wo[g * NG + h][j] = (unsigned)((((long)wr + (long)h * N) * ldw + c8 * 8) * 2);
+      for (int h = 0; h < NG; ++h)   // (32-bit: the entry point lets in operands below 2 GiB only)
+        wo[g * NG + h][j] = ((unsigned)(wr + h * N) * (unsigned)ldw + (unsigned)c8 * 8u) * 2u;
     }
   unsigned xo[MT][2];
 #pragma unroll
@@ -998,18 +1015,25 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int m = mt * 16 + 8 * j + l8;
-      xo[mt][j] = m < M ? (unsigned)(((long)m * lda + c8 * 8) * 2) : NOWHERE;
+      xo[mt][j] = m < M ? ((unsigned)m * (unsigned)lda + (unsigned)c8 * 8u) * 2u : NOWHERE;
     }
 
+  SK_STAMP(11);
   TC* out = C + (long)blockIdx.y * slice_stride;
   // The rotation's end needs the token's position, and through it a page number and cos and sin:
   // two trips to memory one after the other. The position is asked for before the first lines of the
   // product, what hangs on it right after them, so that both trips run beside the product's first.
-  const bool ender = wave < MT;   // this wave finishes token tile `wave` of every strip
-  SkToken tok = {0, 0};
-  if (EPI == SK_QKV && ender) tok = sk_token(M, rp);
+  // wave w finishes the token tiles w, w + NW, ... of the block's NS * MT (tile i: token tile i % MT of strip i / MT)
+  constexpr int ENDS = (NS * MT + NW - 1) / NW;
+  const bool ender = wave < NS * MT;
+  SkToken tok[ENDS];
+#pragma unroll
+  for (int e = 0; e < ENDS; ++e) {
+    tok[e] = SkToken{0, 0};
+    if (EPI == SK_QKV && wave + e * NW < NS * MT) tok[e] = sk_token(M, rp, (wave + e * NW) % MT);
+  }
   const int sq_row = MT == 1 ? (lane & 15) : lane;   // (a folded norm's product of all rows, in order)
-  float sq[4];
+  float sq[SK_SQN(NW)];
 
   const int pairs = (K + 63) / 64;
   const int p_begin = blockIdx.y * pairs_per_slice;
@@ -1029,7 +1053,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   // A wave's pairs are wave, wave + NW, ...; blocks start at different ones, so that at any time the
   // chip asks for all parts of the rows of W and not for the same quarter of every row.
   const int n_it = (p_end - p_begin + NW - 1) / NW;
-  const int rot = n_it > 0 ? (int)(blockIdx.x % (unsigned)n_it) : 0;
+  // (any spread will do; a remainder by a number not known before costs some forty instructions in every wave)
+  const int rot = (n_it & (n_it - 1)) == 0 ? (int)(blockIdx.x & (unsigned)(n_it - 1)) : (int)(((blockIdx.x & 255u) * (unsigned)n_it) >> 8);
   auto pair_at = [&](int i) {   // (i >= n_it: past the end)
     const int j = i + rot;
     return i < n_it ? p_begin + wave + NW * (j < n_it ? j : j - n_it) : p_end;
@@ -1047,13 +1072,24 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
       for (int j = 0; j < 2; ++j)
         held[NWT + mt][j] = sk_ld_b128(a_buf, ((xo[mt][j] | k2) & NOWHERE) ? NOWHERE : xo[mt][j] + k2);
   };
+  SK_STAMP(12);
   ask(pair_at(0));
   SK_STAMP(2);
-  SkPre pre[NS];
-  if (ender) {
+  SkPre pre[ENDS];
+  int end_hd[ENDS], end_sub[ENDS];
+  bool end_rot[ENDS];
 #pragma unroll
-    for (int g = 0; g < NS; ++g)
-      pre[g] = sk_preload<MT, EPI, TC>(out, M, N, ldc, min(strip0 + g, n_strips - 1), hd[g], sub[g], rotated[g], rp, nx, tok);
+  for (int e = 0; e < ENDS; ++e) {
+    end_hd[e] = end_sub[e] = 0;
+    end_rot[e] = false;
+    if (wave + e * NW < NS * MT) {   // (the same for the wave)
+      const int end_g = (wave + e * NW) / MT;
+#pragma unroll
+      for (int g = 0; g < NS; ++g)
+        if (g == end_g) { end_hd[e] = hd[g]; end_sub[e] = sub[g]; end_rot[e] = rotated[g]; }
+      pre[e] = sk_preload<MT, EPI, TC>(out, M, N, ldc, min(strip0 + end_g, n_strips - 1), end_hd[e], end_sub[e], end_rot[e], rp,
+                                       nx, tok[e], (wave + e * NW) % MT);
+    }
   }
   if (XNORM) sk_ssq_ask<NW, MT>(sq, M, nrm, sq_row);
   for (int i = 0; i < n_it; ++i) {
@@ -1093,12 +1129,35 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
 #endif
   if (XNORM) sk_ssq_sum<NW, MT>(sm_ssq, sq, M, nrm, sq_row, acc[0][0][0][0]);   // (read after the barrier before the first strip's end)
   SK_STAMP(5);
+  // All strips of the block end together: every wave's partial tiles go to shared memory, tile t is summed in wave
+  // order by wave t % NW, and wave g * MT + mt finishes token tile mt of strip g (three barriers a block, not three a strip).
+  __syncthreads();   // the staged lines are free
 #pragma unroll
-  for (int g = 0; g < NS; ++g) {
-    __syncthreads();   // the staged lines, then the partial tiles of the strip before, are free
-    if (strip0 + g < n_strips)   // the same for all threads of the block
-      sk_finish<MT, NW, EPI, TC, XNORM, false>(red, sm_ssq, acc[g], strip0 + g, hd[g], sub[g], rotated[g], out, M, N, K,
-                                                ldc, nrm, nullptr, rp, nx, pre[g]);
+  for (int g = 0; g < NS; ++g)
+#pragma unroll
+    for (int h = 0; h < NG; ++h)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) red[wave][(g * NG + h) * MT + mt][lane] = acc[g][h][mt];
+  __syncthreads();
+  SK_STAMP(6);
+  for (int t = wave; t < NTILES; t += NW) {
+    f32x4 v = red[0][t][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) v += red[w][t][lane];
+    red[0][t][lane] = v;   // only this thread touches red[*][t][lane] before the barrier
+  }
+  __syncthreads();
+  SK_STAMP(7);
+#pragma unroll
+  for (int e = 0; e < ENDS; ++e) {
+    const int end_g = (wave + e * NW) / MT, end_mt = (wave + e * NW) % MT;
+    if (wave + e * NW < NS * MT && strip0 + end_g < n_strips) {
+      const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+      sk_end_tile<MT, NW, EPI, TC, XNORM, false>(red[0][end_g * NG * MT + end_mt][lane],
+                                                 (EPI == SK_GATED) ? red[0][(end_g * NG + 1) * MT + end_mt][lane] : zero4, end_mt,
+                                                 sm_ssq, strip0 + end_g, end_hd[e], end_sub[e], end_rot[e], out, M, N, K, ldc, nrm,
+                                                 nullptr, rp, nx, pre[e]);
+    }
   }
   SK_STAMP(9); SK_STAMP(15);
 }
@@ -1160,9 +1219,12 @@ static int launch_skinny(int nw, const SkCall& a) {
   if constexpr (MT == 1 && XNORM && !SSQ) {
     // a decode step's products with a folded norm over the copy of W: the kernel with the short prologue
     if (a.resident && a.Wt && !a.nrm.rows && a.lda < (1L << 24) && a.K < (1 << 24) && (long)steps * 1024 < (1L << 31)) {
+#ifndef SK_DEC_NW
+#define SK_DEC_NW 16
+#endif
 #define DEC(KS)                                                                                                  \
   do {                                                                                                           \
-    gemm_skinny_decode_kernel<16, KS, EPI, TC><<<dim3(resident_blocks(n_strips, 16)), dim3(16 * 64), 0, a.stream>>>( \
+    gemm_skinny_decode_kernel<SK_DEC_NW, KS * 16 / SK_DEC_NW, EPI, TC><<<dim3(resident_blocks(n_strips, SK_DEC_NW)), dim3(SK_DEC_NW * 64), 0, a.stream>>>( \
         (const bf16_t*)a.A, (const bf16_t*)a.Wt, (TC*)a.C, a.M, a.N, a.K, (int)a.lda, a.ldc, a.nrm, a.nx, a.rp, n_strips); \
     GL3_LAUNCH_CHECK();                                                                                          \
     return 0;                                                                                                    \
