@@ -29,6 +29,22 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// Time stamps inside the kernel, for measurements (compiled in with -DAD_STAMPS only, never in the library's own build).
+#ifdef AD_STAMPS
+__device__ long long ad_stamps[2][2][16];
+extern "C" int gl3_ad_stamps(long long* out) {
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(ad_stamps), sizeof(ad_stamps)) == hipSuccess ? 0 : -1;
+}
+#define AD_STAMP(i)                                                                                              \
+  do {                                                                                                           \
+    const int w_ = threadIdx.x >> 6, nw_ = blockDim.x >> 6;                                                      \
+    if ((blockIdx.x == 0 || blockIdx.x == gridDim.x / 2) && (threadIdx.x & 63) == 0 && (w_ == 0 || w_ == nw_ - 1)) \
+      ad_stamps[blockIdx.x == 0 ? 0 : 1][w_ == 0 ? 0 : 1][i] = (i) == 0 || (i) == 15 ? wall_clock64() : clock64(); \
+  } while (0)
+#else
+#define AD_STAMP(i) do {} while (0)
+#endif
+
 template <int HS, int NW, int CB>
 __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -39,6 +55,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   constexpr int DT = HS / 16;   // row tiles of the second product
   __shared__ float sm_m[NW][16], sm_l[NW][16];
   __shared__ f32x4 sm_o[NW][DT][64];
+  AD_STAMP(0); AD_STAMP(1);
   const int g = n_heads / n_kv;
   const int groups = (g + 15) / 16;
   const int t = blockIdx.x / (n_kv * groups);
@@ -52,13 +69,22 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   const int heads_here = min(16, g - hg * 16);
   const int h0 = c * g + hg * 16;
 
+  // The token's row of the block table: row seq_of_token[t], or (seq_of_token null) row t of a table that the step
+  // made of its own tokens' rows. Then nothing stands between the kernel's start and the page numbers: those of the
+  // chunks that this wave would take first in a sequence read from its start (no window, one split: every decode
+  // step of a short context) are asked for together with the token's position, one trip to memory instead of two.
+  const int* bt = block_table + (long)(seq_of_token ? __builtin_amdgcn_readfirstlane(seq_of_token[t]) : t) * table_stride;
+  int first_pages[CB];
+#pragma unroll
+  for (int b = 0; b < CB; ++b)
+    first_pages[b] = __builtin_amdgcn_readfirstlane(bt[min(((wave + b * NW) * 32) / page_size, table_stride - 1)]);
   const int kv_len = __builtin_amdgcn_readfirstlane(positions[t]) + 1;
   const int lo = (window > 0 && kv_len > window) ? kv_len - window : 0;
   const int chunk_lo = lo / 32, chunk_hi = (kv_len + 31) / 32;
   const int per_split = (chunk_hi - chunk_lo + n_splits - 1) / n_splits;
   const int c_begin = chunk_lo + split * per_split;
   const int c_end = min(chunk_hi, c_begin + per_split);
-  const int* bt = block_table + (long)__builtin_amdgcn_readfirstlane(seq_of_token[t]) * table_stride;
+  AD_STAMP(2);
 
   // Q^T operand: lane (head j, quarter qd) holds Q[h0 + j][kk*32 + 8*qd .. +7]
   bf16x8 qt[KK];
@@ -80,7 +106,8 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
       const int ck = ck0 + b * NW;
       if (ck < c_end) {
         const int key0 = ck * 32;
-        const long page = __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
+        // (the first chunks from the sequence's start: their pages are here already)
+        const long page = (c_begin == 0 && ck0 == wave) ? first_pages[b] : __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
         const int po = key0 % page_size;
         // the chunk's two key tiles lie one after the other, 16 * HS elements each; a k-step's operand
         // is 512 consecutive elements of a tile in lane order (gl3_k_offset)
@@ -98,6 +125,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
       }
     }
     __builtin_amdgcn_sched_barrier(0);   // every load above is issued before the first is waited for
+    AD_STAMP(3);
 #pragma unroll
     for (int b = 0; b < CB; ++b) {
       const int ck = ck0 + b * NW;
@@ -142,6 +170,10 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     }
   }
 
+#ifdef AD_STAMPS
+  asm volatile("s_nop 0" :: "v"(o[0][0]));
+  AD_STAMP(4);
+#endif
   // merge the waves, in wave order
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
@@ -149,6 +181,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) sm_o[wave][dt][lane] = o[dt];
   __syncthreads();
+  AD_STAMP(5);
   float M = sm_m[0][j];
 #pragma unroll
   for (int w = 1; w < NW; ++w) M = fmaxf(M, sm_m[w][j]);
@@ -179,6 +212,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     ml[0] = M;
     ml[1] = L;
   }
+  AD_STAMP(9); AD_STAMP(15);
 }
 
 // Merge the splits of one (token, head): in split order, so the result has one order of summation.
@@ -214,7 +248,7 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
                                     long out_stride, int n_tokens, int n_heads, int n_kv, int head_dim, int page_size,
                                     int window, float scale, int n_splits, hipStream_t stream) {
   if (n_tokens == 0) return 0;
-  GL3_REQUIRE(q && k_cache && v_cache && positions && seq_of_token && block_table && out,
+  GL3_REQUIRE(q && k_cache && v_cache && positions && block_table && out && table_stride > 0,
               "gl3_attention_decode: null argument");
   GL3_REQUIRE(gl3_attention_decode_supports(head_dim, page_size),
               "gl3_attention_decode: head_dim %d / page_size %d is not built (32, 64, 96, 128; pages of a multiple of 32)",

@@ -440,14 +440,19 @@ extern "C" int gl3_rope_cache_write(void* qkv, int dtype, const int* positions, 
 // A decode step's QKV products need, per token, the page its keys and values go to and its row of cos and sin:
 // look-ups that wait for the token's position, a second trip to memory in each of them. They are the same for
 // every layer that shares the block table and the rotation, so one small kernel makes them once per step:
-// pages[t] = table[rows[t]][positions[t] / page_size]; rot[t] = cos[positions[t]] | sin[positions[t]] (half each).
+// pages[t] = table[rows[t]][positions[t] / page_size]; rot[t] = cos[positions[t]] | sin[positions[t]] (half each);
+// tables[t] (may be null) = the token's row of the block table up to its position's page, so that the attention of
+// a decode step finds the pages of token t in row t, without the look-up of which row is the token's.
 __global__ void token_facts_kernel(const int* __restrict__ positions, const int* __restrict__ rows,
                                    const int* __restrict__ block_table, int table_stride, int page_size,
                                    const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int half,
-                                   int* __restrict__ pages, float* __restrict__ rot) {
+                                   int* __restrict__ pages, float* __restrict__ rot, int* __restrict__ tables) {
   const int t = blockIdx.x;
   const int pos = positions[t];
-  if (threadIdx.x == 0) pages[t] = block_table[(long)rows[t] * table_stride + pos / page_size];
+  const int* row = block_table + (long)rows[t] * table_stride;
+  if (threadIdx.x == 0) pages[t] = row[pos / page_size];
+  if (tables)
+    for (int j = threadIdx.x; j <= pos / page_size; j += blockDim.x) tables[(long)t * table_stride + j] = row[j];
   if (rot)
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
       rot[(long)t * 2 * half + j] = cos_tab[(long)pos * half + j];
@@ -458,14 +463,14 @@ __global__ void token_facts_kernel(const int* __restrict__ positions, const int*
 // cos_tab, sin_tab, rot: all three or none (no rotation: the pages alone).
 extern "C" int gl3_token_facts(const int* positions, const int* rows, const int* block_table, int table_stride,
                                int page_size, const float* cos_tab, const float* sin_tab, int half, int* pages, float* rot,
-                               int n_tokens, hipStream_t stream) {
+                               int* tables, int n_tokens, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(positions && rows && block_table && pages && table_stride > 0 && page_size > 0 && n_tokens > 0,
               "gl3_token_facts: bad arguments");
   GL3_REQUIRE((cos_tab != nullptr) == (sin_tab != nullptr) && (cos_tab != nullptr) == (rot != nullptr) && (!rot || half > 0),
               "gl3_token_facts: the tables and the rows for them come together");
   token_facts_kernel<<<dim3(n_tokens), dim3(64), 0, stream>>>(positions, rows, block_table, table_stride, page_size,
-                                                              cos_tab, sin_tab, half, pages, rot);
+                                                              cos_tab, sin_tab, half, pages, rot, tables);
   GL3_LAUNCH_CHECK();
   return 0;
 }

@@ -820,10 +820,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
 // one scalar unit, and before the loads are on their way every wave works through the same prologue; measured
 // inside the QKV product of the 1B layers, the last of sixteen waves had its loads out 2.2 us after it started
 // with the general prologue. Here the prologue is what the loads' addresses take and no more:
-//  * no test whether a k-step, a row or a partial sum exists. The descriptors end where the data ends (a strip
-//    of the copy, the rows of A, the partial sums), so a load beyond it reads zeros: k-steps beyond K (the copy
-//    is padded with zeros to whole steps, and rows of A are tested against K for the case lda > K), rows of A
-//    from M on (they start beyond the last row's end), partial sums from n_partials on;
+//  * no test whether a k-step or a partial sum exists. The descriptors end where the data ends (a strip of the
+//    copy, the partial sums), so a load beyond it reads zeros: k-steps beyond K (the copy is padded with zeros to
+//    whole steps; elements of A from K on are not read), partial sums from n_partials on;
 //  * what only the end of a strip needs is computed by wave 0 alone, after the loads are out.
 template <int NW, int KS, int EPI, typename TC>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
@@ -839,6 +838,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
   const bool ender = wave == 0;
   SkToken tok = {0, 0};
   if (EPI == SK_QKV && ender) tok = sk_token(M, rp);
+  // the row of A that the product's row r reads: r itself, or a chosen one (the head on the wanted rows)
+  int a_row = r;
+  if (nrm.rows) {   // (the same for the whole grid; nothing else is on its way yet)
+    a_row = nrm.rows[min(r, M - 1)];
+    asm volatile("" : "+v"(a_row));
+  }
   const unsigned tile_bytes = (unsigned)((K + 31) >> 5) << 10;   // a strip of the copy: 1 KB a k-step
   const unsigned up_strips = (unsigned)N >> 4;                   // (gated) the up strips follow the gate strips
   int strip = blockIdx.x;
@@ -856,15 +861,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
   }
   bf16x8 xf[KS][MT];
   {
-    const __amdgpu_buffer_rsrc_t a_buf = __builtin_amdgcn_make_buffer_rsrc((void*)xg, 0, (int)((((unsigned)M - 1u) * (unsigned)lda + (unsigned)K) * 2u), 0x00020000);
+    // (A has at most 64 rows; only rows that exist give an offset)
+    const __amdgpu_buffer_rsrc_t a_buf = __builtin_amdgcn_make_buffer_rsrc((void*)xg, 0, (int)((63u * (unsigned)lda + (unsigned)K) * 2u), 0x00020000);
     const unsigned k0 = (unsigned)wave * 32u + (unsigned)q * 8u;
-    const unsigned x_at = ((unsigned)r * (unsigned)lda + k0) * 2u;
+    const unsigned x_at = r < M ? ((unsigned)a_row * (unsigned)lda + k0) * 2u : SK_NOWHERE;
 #pragma unroll
-    for (int i = 0; i < KS; ++i) xf[i][0] = sk_ld_b128(a_buf, k0 + (unsigned)i * (NW * 32u) < (unsigned)K ? x_at + (unsigned)i * (NW * 64u) : SK_NOWHERE);
+    for (int i = 0; i < KS; ++i)
+      xf[i][0] = sk_ld_b128(a_buf, (r < M && k0 + (unsigned)i * (NW * 32u) < (unsigned)K) ? x_at + (unsigned)i * (NW * 64u) : SK_NOWHERE);
   }
   float sq[SK_SQN(NW)];
   const __amdgpu_buffer_rsrc_t s_buf = __builtin_amdgcn_make_buffer_rsrc((void*)nrm.ssq, 0, nrm.n_partials * 256, 0x00020000);
-  const unsigned s_at = ((unsigned)wave + (unsigned)q * NW) * 256u + (unsigned)r * 4u;   // partial wave + NW (4 i + q) of row r
+  const unsigned s_at = ((unsigned)wave + (unsigned)q * NW) * 256u + (unsigned)a_row * 4u;   // partial wave + NW (4 i + q) of the row (they are stored by row of A)
 #pragma unroll
   for (int i = 0; i < SK_SQN(NW); ++i) sq[i] = sk_ld_f32(s_buf, s_at + (unsigned)i * (NW * 1024u));
   __builtin_amdgcn_sched_barrier(0);   // all of that is on its way before anything else is computed
@@ -1218,7 +1225,7 @@ static int launch_skinny(int nw, const SkCall& a) {
   }
   if constexpr (MT == 1 && XNORM && !SSQ) {
     // a decode step's products with a folded norm over the copy of W: the kernel with the short prologue
-    if (a.resident && a.Wt && !a.nrm.rows && a.lda < (1L << 24) && a.K < (1 << 24) && (long)steps * 1024 < (1L << 31)) {
+    if (a.resident && a.Wt && a.lda < (1L << 24) && a.K < (1 << 24) && (long)steps * 1024 < (1L << 31)) {
 #ifndef SK_DEC_NW
 #define SK_DEC_NW 16
 #endif

@@ -65,7 +65,7 @@ def _declare(lib):
         "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P, I, F, I, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, I, P],
         "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
-        "gl3_token_facts": [P, P, P, I, I, P, P, I, P, P, I, P],
+        "gl3_token_facts": [P, P, P, I, I, P, P, I, P, P, P, I, P],
         "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
@@ -600,11 +600,13 @@ def qkv_rope_cache_fits(a, w_qkv, head_dim, rot_dim):
             and head_dim % 16 == 0 and rot_dim in (0, head_dim))
 
 
-def token_facts(positions, table_rows, block_table, page_size, cos, sin, pages, rot):
+def token_facts(positions, table_rows, block_table, page_size, cos, sin, pages, rot, tables=None):
     """What hangs on each token's position, looked up once for all layers of a step: ``pages`` [T] int32
     receives the page of the token's position (``block_table[table_rows[t]][positions[t] // page_size]``) and
     ``rot`` [T, 2 * half] float32 its rows of ``cos`` and ``sin`` one after the other (``cos``, ``sin``, ``rot``
-    all None: no rotation, the pages alone). ``qkv_rope_cache`` takes both in place of its own look-ups."""
+    all None: no rotation, the pages alone). ``qkv_rope_cache`` takes both in place of its own look-ups.
+    ``tables`` [T, width of ``block_table``] int32 (optional) receives each token's row of the block table up to
+    its position's page: ``attention_decode`` reads it with ``seq_of_token=None``."""
     _dev(positions, "positions", torch.int32); _dev(table_rows, "table_rows", torch.int32)
     _dev(block_table, "block_table", torch.int32); _dev(pages, "pages", torch.int32)
     T = positions.numel()
@@ -618,8 +620,13 @@ def token_facts(positions, table_rows, block_table, page_size, cos, sin, pages, 
             raise KernelError(f"token_facts: tables {tuple(cos.shape)}, rows {tuple(rot.shape)} for {T} tokens")
     elif sin is not None or rot is not None:
         raise KernelError("token_facts: the tables and the rows for them come together")
+    if tables is not None:
+        _dev(tables, "tables", torch.int32)
+        if tables.shape != (T, block_table.shape[1]):
+            raise KernelError(f"token_facts: the tokens' rows {tuple(tables.shape)} of a table {tuple(block_table.shape)}")
     _check(library().gl3_token_facts(_ptr(positions), _ptr(table_rows), _ptr(block_table), block_table.shape[1], int(page_size),
-                                     _ptr(cos), _ptr(sin), half, _ptr(pages), _ptr(rot), T, _stream()), "token_facts")
+                                     _ptr(cos), _ptr(sin), half, _ptr(pages), _ptr(rot), _ptr(tables), T, _stream()),
+           "token_facts")
 
 
 def qkv_rope_cache(a, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_token, block_table, cos, sin,
@@ -691,18 +698,21 @@ def decode_splits(n_tokens, n_heads, n_kv, kv_len, head_dim=64):
 def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,
                      page_size, window, scale, n_splits, part_o=None, part_ml=None):
     """One token per sequence. ``part_o`` [T, H, splits, hs] and ``part_ml`` [T, H, splits, 2] float32
-    are needed when ``n_splits`` > 1 (contiguous, adjacent is not required)."""
+    are needed when ``n_splits`` > 1 (contiguous, adjacent is not required). ``seq_of_token`` None: token t's
+    pages are row t of ``block_table`` (a table of the step's own, as ``token_facts`` makes it)."""
     _dev(q, "q", torch.bfloat16, contiguous=False); _dev(out, "out", torch.bfloat16, contiguous=False)
     _dev(k_cache, "k_cache", torch.bfloat16); _dev(v_cache, "v_cache", torch.bfloat16)
-    _dev(positions, "positions", torch.int32); _dev(seq_of_token, "seq_of_token", torch.int32)
-    _dev(block_table, "block_table", torch.int32)
+    _dev(positions, "positions", torch.int32); _dev(block_table, "block_table", torch.int32)
+    if seq_of_token is not None:
+        _dev(seq_of_token, "seq_of_token", torch.int32)
     T = q.shape[0]
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < n_heads * head_dim:
         raise KernelError(f"attention: q {tuple(q.shape)} for {n_heads} heads of {head_dim}")
     if out.shape != (T, n_heads * head_dim) or out.stride(1) != 1:
         raise KernelError(f"attention: out {tuple(out.shape)}")
     _check_cache(k_cache, v_cache, n_kv, page_size, head_dim, "attention")
-    if positions.numel() != T or seq_of_token.numel() != T or block_table.dim() != 2:
+    if (positions.numel() != T or block_table.dim() != 2
+            or (seq_of_token.numel() != T if seq_of_token is not None else block_table.shape[0] < T)):
         raise KernelError("attention: positions / seq_of_token / block_table shapes")
     floats = 0
     if n_splits > 1:

@@ -109,7 +109,7 @@ class DecoderModel:
         """Logits ``[len(want_rows), vocab]`` float32 at the wanted packed rows."""
         x = ctx.buffer("residual", (ctx.n_tokens, self.spec.hidden), torch.float32)
         ctx.ssq = ctx.pending = ctx.next_norm = None   # a context may run more than one forward pass: nothing is left over
-        ctx.token_facts = {}
+        ctx.token_facts, ctx.token_tables = {}, {}
         order = [self.blocks[r.layer] for r in self.spec.run_order]
         # the norm that reads the residual rows after entry i of the run order, where the block says which
         firsts = [getattr(b, "first_norm", lambda: None)() for b in order] + [self.final_norm]

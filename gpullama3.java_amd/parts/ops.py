@@ -344,8 +344,12 @@ def _token_facts(ctx, block_table, cos, sin, page_size):
         T = ctx.positions.numel()
         pages = ctx.buffer(f"token_pages{n}", (T,), torch.int32)
         rot = ctx.buffer(f"token_rot{n}", (T, 2 * cos.shape[1]), torch.float32) if cos is not None else None
-        K.token_facts(ctx.positions, _table_rows(ctx), block_table, page_size, cos, sin, pages, rot)
+        # a decode step's attention reads the tokens' own rows of the block table (row t: token t)
+        tables = ctx.buffer(f"token_tables{n}", (T, block_table.shape[1]), torch.int32) if ctx.decode else None
+        K.token_facts(ctx.positions, _table_rows(ctx), block_table, page_size, cos, sin, pages, rot, tables)
         made[key] = (pages, rot)
+        if tables is not None:
+            ctx.__dict__.setdefault("token_tables", {})[block_table.data_ptr()] = tables
     return made[key]
 
 
@@ -402,6 +406,10 @@ def attention(ctx, q, k_cache, v_cache, block_table, out, n_heads, n_kv, head_di
             if splits > 1:
                 part_o = ctx.buffer("attn_part_o", (T, n_heads, splits, head_dim), torch.float32)
                 part_ml = ctx.buffer("attn_part_ml", (T, n_heads, splits, 2), torch.float32)
+            own = getattr(ctx, "token_tables", {}).get(block_table.data_ptr())    # (made with the step's token facts)
+            if own is not None:
+                return K.attention_decode(q, k_cache, v_cache, ctx.positions, None, own, out, n_heads, n_kv, head_dim, page,
+                                          window, scale, splits, part_o, part_ml)
             return K.attention_decode(q, k_cache, v_cache, ctx.positions, _table_rows(ctx), block_table, out, n_heads,
                                       n_kv, head_dim, page, window, scale, splits, part_o, part_ml)
         if (not ctx.decode and "attn_prefill" not in disabled and K.has("gl3_attention_prefill") and scale > 0
