@@ -242,17 +242,30 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
   if (shape == 1) return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
   if (shape == 2) return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
   if (shape == 3) return launch_shape<EPI, TC, 4, 2, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
+  if (shape == 4) return launch_shape<EPI, TC, 2, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
+  if (shape == 5) return launch_shape<EPI, TC, 1, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
   // 256 x 256 tiles of sixteen waves, one block a CU, have half the operand traffic per product, and
   // that traffic is what bounds the large products; of the 128 x 128 tiles of eight waves two fit a CU and
   // overlap each other's waits. A step of 64 columns takes a chip full of the large tiles 1.7 us and a chip
   // full of the small ones (twice as many blocks, a quarter of the work each) 1.05 us, and the blocks need
-  // whole rounds on the chip: the tile whose rounds take less time is chosen (240 large tiles are one round
+  // rounds on the chip: the tile whose rounds take less time is chosen (240 large tiles are one round
   // where 960 small ones are two; 276 large ones are two where 1,104 small ones are three).
+  // A third tile, 128 rows x 256 of sixteen waves of 32 x 64, is for the products in between: more tiles of 128 x 128
+  // than one for every CU, but not enough work to fill the chip with the large tiles (2,048 rows of the 1B layers'
+  // QKV product, 384 tiles of 128 x 128 or 192 of 128 x 256: 45 -> 40 us); a step of it takes a full chip about 0.95 us.
+  // Tiles of 128 x 128 that are at most one a CU run faster than two that share one (0.8 of the time a step).
   const long small_n = (EPI == MF_GATED) ? (N + 63) / 64 : (N + 127) / 128;
   const long big_n = (EPI == MF_GATED) ? (N + 127) / 128 : (N + 255) / 256;
-  const long small_rounds = ((long)((M + 127) / 128) * small_n * slices + 511) / 512;
-  const long big_rounds = ((long)((M + 255) / 256) * big_n * slices + 255) / 256;
-  if (big_rounds * 170 < small_rounds * 105)
+  const long small_tiles = (long)((M + 127) / 128) * small_n * slices, wide_tiles = (long)((M + 127) / 128) * big_n * slices;
+  const long big_tiles = (long)((M + 255) / 256) * big_n * slices;
+  // rounds on the chip, in thousandths: whole rounds, and a last, partly empty one that costs half a round and
+  // half of the share of the places it fills (a chip half full works through its blocks faster, not twice as fast)
+  auto rounds = [](long tiles, long places) { return tiles / places * 1000 + (tiles % places ? 500 + tiles % places * 500 / places : 0); };
+  const long small_cost = rounds(small_tiles, 512) * (small_tiles <= 256 ? 84 : 105), big_cost = rounds(big_tiles, 256) * 170;
+  const long wide_cost = rounds(wide_tiles, 256) * (wide_tiles <= 128 ? 119 : 95);
+  if (wide_cost < small_cost && wide_cost < big_cost && slices == 1)
+    return launch_shape<EPI, TC, 1, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
+  if (big_cost < small_cost)
     return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
   return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
 }
@@ -263,7 +276,8 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
 // p_stride elements apart), which the caller adds to C in that order.
 // bias (may be null; not with slices): N floats (gated: 2N). act: the gated epilogue's activation.
 // shape: 0 lets the library choose the tile; 1: 128 x 128, eight waves; 2: 256 x 256, sixteen waves of
-// 64 x 64; 3: 256 x 256, eight waves of 128 x 64.
+// 64 x 64; 3: 256 x 256, eight waves of 128 x 64; 4: 256 rows x 128, eight waves of 64 x 64; 5: 128 rows x 256,
+// sixteen waves of 32 x 64.
 extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
                              long ldc, int epilogue, int slices, float* P, long p_stride, long ldp, const float* bias,
                              int act, int shape, hipStream_t stream) {
@@ -284,7 +298,7 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
               "gl3_gemm_mfma: slices need a buffer for their sums and another epilogue than the gated one");
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_mfma: a bias goes with one slice of K");
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_mfma: unknown activation %d", act);
-  GL3_REQUIRE(shape >= 0 && shape <= 3, "gl3_gemm_mfma: unknown tile shape %d", shape);
+  GL3_REQUIRE(shape >= 0 && shape <= 5, "gl3_gemm_mfma: unknown tile shape %d", shape);
 #define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, shape, stream
   if (c_dtype == GL3_F32) {
     if (epilogue == MF_STORE) return launch_mfma<MF_STORE, float>(ARGS);
