@@ -319,8 +319,13 @@ __global__ __launch_bounds__(256) void rope_cache_vec_kernel(
     bf16_t* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
     const int* __restrict__ block_table, int table_stride, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int n_heads, int n_kv,
-    int head_dim, int rot_dim, int adjacent, int page_size, int write_kv, long row_stride) {
-  const int t = blockIdx.x;
+    int head_dim, int rot_dim, int adjacent, int page_size, int write_kv, long row_stride, int n_tokens) {
+  // Blocks with consecutive numbers go to different XCDs, each with a second-level cache of its own. The values
+  // of 8 consecutive positions of a sequence share 16 bytes of a transposed page, one 2-byte store per token;
+  // with neighbouring tokens on one XCD those stores meet in one cache and leave it as whole lines.
+  const int per_xcd = (n_tokens + 7) / 8;
+  const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (t >= n_tokens) return;
   const int pos = positions[t];
   bf16_t* row = qkv + (long)t * row_stride;
   const int half = rot_dim / 2;
@@ -414,9 +419,9 @@ extern "C" int gl3_rope_cache_write(void* qkv, int dtype, const int* positions, 
                      (!cos_tab || ((uintptr_t)cos_tab % 16 == 0 && (uintptr_t)sin_tab % 16 == 0)) &&
                      (!write_kv || ((uintptr_t)k_cache % 16 == 0));
   if (units) {
-    rope_cache_vec_kernel<<<dim3(n_tokens), dim3(256), 0, stream>>>(
+    rope_cache_vec_kernel<<<dim3((n_tokens + 7) / 8 * 8), dim3(256), 0, stream>>>(
         (bf16_t*)qkv, positions, seq_of_token, block_table, table_stride, cos_tab, sin_tab, (bf16_t*)k_cache,
-        (bf16_t*)v_cache, n_heads, n_kv, head_dim, cos_tab ? rot_dim : 0, adjacent, page_size, write_kv, row_stride);
+        (bf16_t*)v_cache, n_heads, n_kv, head_dim, cos_tab ? rot_dim : 0, adjacent, page_size, write_kv, row_stride, n_tokens);
     GL3_LAUNCH_CHECK();
     return 0;
   }

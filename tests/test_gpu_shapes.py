@@ -126,7 +126,9 @@ def test_real_layer_sizes_against_the_plain_implementation(tmp_path, shape):
     a whole model against the plain implementation itself (J/inference/InferenceCore.java:58-180), not
     against another path of the engine: a prompt of 300 tokens with every row wanted, four single
     tokens after it, and a batch of 40 short prompts with three decode steps (the kernels for 33 to
-    64 rows, replayed from graphs), in float32 and in bfloat16."""
+    64 rows, replayed from graphs), in float32 and in bfloat16. Then batches of 12, 24 and 100 sequences
+    (products of 9 to 16 rows over a long K, the variant for two token tiles, steps worked on in pieces
+    of 64 rows), of which the sequences at the edges of the token tiles are compared."""
     from safetensors.torch import load_file
 
     import gpullama3_java_amd as g
@@ -142,9 +144,12 @@ def test_real_layer_sizes_against_the_plain_implementation(tmp_path, shape):
     short = [rng.integers(0, cfg.vocab_size, 7).tolist() for _ in range(40)]
     ref_long = P.forward(cfgd, W, long_toks)
     ref_short = [P.forward(cfgd, W, q)[3:] for q in short]                   # rows of the tokens 3, 4, 5, 6
+    more = {B: [rng.integers(0, cfg.vocab_size, 7).tolist() for _ in range(B)] for B in (12, 24, 100)}
+    watched = {12: [0, 7, 8, 11], 24: [0, 15, 16, 23], 100: [0, 31, 32, 49, 50, 63, 64, 99]}
+    ref_more = {B: {i: P.forward(cfgd, W, more[B][i])[3:] for i in watched[B]} for B in more}
     del W
     for dtype in ("float32", "bfloat16"):
-        eng = Engine.from_folder(folder, dtype=dtype, max_context=512, max_tokens=64 * 64, n_slots=64)
+        eng = Engine.from_folder(folder, dtype=dtype, max_context=512, max_tokens=128 * 64, n_slots=128)
         s = eng.take_slot()
         got = [eng.step([(s, long_toks[:300])], want="all").cpu().numpy()]
         got += [eng.step([(s, [t])]).cpu().numpy() for t in long_toks[300:]]
@@ -156,13 +161,61 @@ def test_real_layer_sizes_against_the_plain_implementation(tmp_path, shape):
         slots = [eng.take_slot() for _ in short]
         rows = [eng.step([(sl, q[:4]) for sl, q in zip(slots, short)]).cpu().numpy()]
         rows += [eng.step([(sl, [q[k]]) for sl, q in zip(slots, short)]).cpu().numpy() for k in (4, 5, 6)]
+        for sl in slots:
+            eng.give_back_slot(sl)
         got = np.stack(rows, axis=1)                                         # [40, 4, vocab]
         for i, r in enumerate(ref_short):
             sc = float(np.abs(r).max())
             e = float(np.abs(got[i] - r).max())
             assert e <= TOL[dtype] * sc, f"{dtype}: sequence {i} of the batch of 40 is off by {e / sc:.2e}"
+        for B, seqs in more.items():
+            slots = [eng.take_slot() for _ in seqs]
+            rows = [eng.step([(sl, q[:4]) for sl, q in zip(slots, seqs)]).cpu().numpy()]
+            rows += [eng.step([(sl, [q[k]]) for sl, q in zip(slots, seqs)]).cpu().numpy() for k in (4, 5, 6)]
+            for sl in slots:
+                eng.give_back_slot(sl)
+            got = np.stack(rows, axis=1)                                     # [B, 4, vocab]
+            for i, r in ref_more[B].items():
+                sc = float(np.abs(r).max())
+                e = float(np.abs(got[i] - r).max())
+                assert e <= TOL[dtype] * sc, f"{dtype}: sequence {i} of the batch of {B} is off by {e / sc:.2e}"
         if dtype == "bfloat16":
             assert eng._graphs
+        del eng
+        torch.cuda.empty_cache()
+
+
+def test_a_long_context_at_real_layer_sizes_against_the_plain_implementation(tmp_path):
+    """A prompt of 2,600 tokens (the largest tiles of the products, the longest blocks of the prompt's attention)
+    and three single tokens after it, whose attention is split over the keys and merged (heads of 64 at a
+    context beyond 2,048), with the layers of Llama-3.2-1B against the plain implementation itself, in float32
+    and in bfloat16: the prompt's first, middle and last row and the three tokens' rows."""
+    from safetensors.torch import load_file
+
+    import gpullama3_java_amd as g
+    import plain_llama as P
+    from gpullama3_java_amd.csrc import lib
+    from gpullama3_java_amd.engine import Engine
+    cfgd = SHAPES["1B"]
+    cfg = g.config_from_dict(cfgd)
+    folder = str(tmp_path / "shape")
+    g.write_random_model(folder, cfg, 14, std=0.02, norm_std=0.1)
+    W = {k: v.float().numpy() for k, v in load_file(folder + "/model.safetensors").items()}
+    toks = np.random.default_rng(3).integers(0, cfg.vocab_size, 2603).tolist()
+    watched = [0, 1299, 2599, 2600, 2601, 2602]
+    _, hidden = P.forward(cfgd, W, toks, return_hidden=True)
+    ref = P.linear(P.rmsnorm(hidden[watched], W["model.norm.weight"], cfgd["rms_norm_eps"]), W["model.embed_tokens.weight"])
+    del W, hidden
+    assert lib.decode_splits(1, 32, 8, 4096, 64) > 1           # the case is the one it claims to be
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine.from_folder(folder, dtype=dtype, max_context=4096, max_tokens=2688, n_slots=1)
+        s = eng.take_slot()
+        got = [eng.step([(s, toks[:2600])], want=[[0, 1299, 2599]]).cpu().numpy()]
+        got += [eng.step([(s, [t])]).cpu().numpy() for t in toks[2600:]]
+        got = np.concatenate(got)
+        scale = float(np.abs(ref).max())
+        err = np.abs(got - ref).max(axis=1)
+        assert err.max() <= TOL[dtype] * scale, f"{dtype}: row {watched[int(err.argmax())]} is off by {err.max() / scale:.2e}"
         del eng
         torch.cuda.empty_cache()
 
