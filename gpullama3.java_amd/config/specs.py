@@ -108,3 +108,5 @@ class ModelSpec:
     embedding_scale: Optional[float] = None       # the embedding row times this
     position_table_name: Optional[str] = None     # a stored [max_positions, hidden] table whose row at the token's position is added to it
     logit_scale: Optional[float] = None           # the logits times this
+    head_bias_name: Optional[str] = None          # a stored [vocab] vector added to the logits (before the scale)
+    logit_softcap: Optional[float] = None         # the logits become cap * tanh(logits / cap) (after the scale)

@@ -48,6 +48,22 @@ extern "C" int gl3_scale_f32(float* p, float s, long n, hipStream_t stream) {
   return 0;
 }
 
+// ---- p[i] = cap * tanh(p[i] / cap) (what a model's soft cap of the logits is applied with)
+__global__ void softcap_f32_kernel(float* p, float cap, long n) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = cap * tanhf(p[i] / cap);
+}
+
+extern "C" int gl3_softcap_f32(float* p, float cap, long n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  GL3_REQUIRE(p != nullptr && cap > 0.f, "gl3_softcap_f32: null pointer or a cap that is not positive");
+  long blocks = (n + 255) / 256;
+  GL3_REQUIRE(blocks < (1L << 31), "gl3_softcap_f32: %ld elements is too many", n);
+  softcap_f32_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p, cap, n);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---- scatter of a few integers whose places and values travel in the launch itself: how the host
 // changes entries of a table on the device (a page added to a sequence) without staging memory.
 #define GL3_SCATTER_MAX 128

@@ -50,6 +50,7 @@ def _declare(lib):
         "gl3_fill_u32": [P, c_uint32, L, P],
         "gl3_embed": [P, I, P, P, I, I, P, P, P, F, P, P, P],
         "gl3_scale_f32": [P, F, L, P],
+        "gl3_softcap_f32": [P, F, L, P],
         "gl3_rmsnorm": [P, P, P, I, P, I, I, I, F, P],
         "gl3_gather_rows": [P, P, P, I, I, I, P],
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
@@ -180,6 +181,12 @@ def scale_(t, factor):
     """t *= factor (float32, contiguous)."""
     _dev(t, "tensor", torch.float32)
     _check(library().gl3_scale_f32(_ptr(t), float(factor), t.numel(), _stream()), "scale_f32")
+
+
+def softcap_(t, cap):
+    """t = cap * tanh(t / cap) (float32, contiguous)."""
+    _dev(t, "tensor", torch.float32)
+    _check(library().gl3_softcap_f32(_ptr(t), float(cap), t.numel(), _stream()), "softcap_f32")
 
 
 def embed(table, ids, out, ssq=None, next_weight=None, xg=None, scale=1.0, pos_table=None, positions=None):

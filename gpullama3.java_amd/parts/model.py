@@ -21,6 +21,8 @@ def expected_tensors(spec, dtype=torch.float32, device="cpu"):
         out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden))
     if spec.position_table_name is not None:
         out[spec.position_table_name] = TensorSpec((spec.max_positions, spec.hidden))
+    if spec.head_bias_name is not None:
+        out[spec.head_bias_name] = TensorSpec((spec.vocab_size,), "vector")
     if spec.final_norm is not None:
         out.update(_norm_tensors(spec.final_norm))
     for b in spec.layers:
@@ -68,7 +70,7 @@ class DecoderModel:
                                  "with keys and values of its own")
             self.runs.append(RunInfo(entry=e, kv_entry=e if r.reads is None else r.reads,
                                      writes_kv=r.reads is None))
-        self.embedding = self.head = self.position_table = None
+        self.embedding = self.head = self.position_table = self.head_bias = None
         self.weights = {}
 
     def expected(self):
@@ -77,6 +79,8 @@ class DecoderModel:
             out[self.spec.head_name] = TensorSpec((self.spec.vocab_size, self.spec.hidden))
         if self.spec.position_table_name is not None:
             out[self.spec.position_table_name] = TensorSpec((self.spec.max_positions, self.spec.hidden))
+        if self.spec.head_bias_name is not None:
+            out[self.spec.head_bias_name] = TensorSpec((self.spec.vocab_size,), "vector")
         if self.final_norm is not None:
             out.update(self.final_norm.tensors())
         for b in self.blocks:
@@ -91,6 +95,8 @@ class DecoderModel:
         ops.for_few_rows(self.head, without=self.without)
         if self.spec.position_table_name is not None:
             self.position_table = weights[self.spec.position_table_name].to(self.embedding.dtype)
+        if self.spec.head_bias_name is not None:     # the epilogues read biases as float
+            self.head_bias = weights[self.spec.head_bias_name].float().contiguous()
         if self.final_norm is not None:
             self.final_norm.load(weights)
         for b in self.blocks:
@@ -152,7 +158,9 @@ class DecoderModel:
                 ops.settle_residual(ctx, x)
                 h = ctx.buffer("head_rows", (n, self.spec.hidden), self.dtype)
                 K.gather_rows(x, want_rows, h)
-            ops.linear(h, self.head, logits, ops.EPI_STORE, ctx)
+            ops.linear(h, self.head, logits, ops.EPI_STORE, ctx, bias=self.head_bias)
             if self.spec.logit_scale is not None:
                 K.scale_(logits, self.spec.logit_scale)
+            if self.spec.logit_softcap is not None:
+                K.softcap_(logits, self.spec.logit_softcap)
         return logits

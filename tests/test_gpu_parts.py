@@ -758,12 +758,13 @@ def other_plain(cfg, W, toks):
         x = x + P.linear((act * (P.linear(h, W[p + "u"]) + W[p + "ub"])).astype(np.float32), W[p + "dn"])
         if p + "db" in W:
             x = x + W[p + "db"]
-    return P.linear(P.rmsnorm(x, W["final"], cfg["eps"]), W["emb"]) * np.float32(cfg["logit_scale"])
+    logits = (P.linear(P.rmsnorm(x, W["final"], cfg["eps"]), W["emb"]) + W["head_bias"]) * np.float32(cfg["logit_scale"])
+    return np.float32(cfg["softcap"]) * np.tanh(logits / np.float32(cfg["softcap"]))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_decoder_of_another_make_from_descriptions_alone(tmp_path, dtype):
-    """Embedding multiplier, learned absolute positions, logit scale, biases on every projection,
+    """Embedding multiplier, learned absolute positions, logit scale, a bias and a soft cap on the logits, biases on every projection,
     the other activation and a block kind defined here: all of it is a description and two
     registrations, no file of the framework changes. 40 tokens in one step take the kernels for 33
     to 64 rows, whose products into the residual rows leave their sums in slices (K = 1024): the
@@ -810,17 +811,19 @@ def test_a_decoder_of_another_make_from_descriptions_alone(tmp_path, dtype):
                              run_order=tuple(Run(i) for i in range(c["layers"])),
                              final_norm=NormSpec(dim=c["hidden"], eps=c["eps"], names={"weight": "final"}),
                              max_positions=128, tie_embeddings=True, embedding_name="emb", head_name=None,
-                             embedding_scale=c["embedding_scale"], position_table_name="wpe", logit_scale=c["logit_scale"])
+                             embedding_scale=c["embedding_scale"], position_table_name="wpe", logit_scale=c["logit_scale"],
+                             head_bias_name="head_bias", logit_softcap=c["softcap"])
 
     g.register_architecture("OtherForCausalLM", OtherConfig)
     # three layers: the usual arrangement whose down projection has no bias (its sums stay in slices
     # behind it), then the halving one, which reads the rows, then the usual one again
     cfg = {"architectures": ["OtherForCausalLM"], "hidden": 128, "inter": 1024, "layers": 3, "heads": 4, "kv_heads": 2,
-           "head_dim": 32, "vocab": 300, "eps": 1e-5, "embedding_scale": 3.0, "logit_scale": 0.25,
+           "head_dim": 32, "vocab": 300, "eps": 1e-5, "embedding_scale": 3.0, "logit_scale": 0.25, "softcap": 2.0,
            "halving_layers": [1], "down_bias_layers": [1, 2]}
     rng = np.random.default_rng(4)
     r = lambda *s, scale=0.05: (rng.standard_normal(s) * scale).astype(np.float32)
-    W = {"emb": r(300, 128, scale=0.3), "wpe": r(128, 128, scale=0.3), "final": 1 + r(128, scale=0.1)}
+    W = {"emb": r(300, 128, scale=0.3), "wpe": r(128, 128, scale=0.3), "final": 1 + r(128, scale=0.1),
+         "head_bias": r(300, scale=2.0)}
     for l in range(3):
         p = f"l{l}."
         W.update({p + "n1": 1 + r(128, scale=0.1), p + "n2": 1 + r(128, scale=0.1), p + "q": r(128, 128), p + "k": r(64, 128),
