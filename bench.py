@@ -95,6 +95,8 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=PROMPT, help="tokens every sequence holds before the decode steps")
     ap.add_argument("--prefill-len", type=int, default=PREFILL, help="tokens of the prompt whose prefill is timed")
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=None,
+                    help="the longest sequence (max_position_embeddings) instead of the shape's; reported as seq_len")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma-separated")
     ap.add_argument("--seed", type=int, default=0)
@@ -116,6 +118,8 @@ def main():
     from gpullama3_java_amd.engine import Engine
 
     shape_name, shape = SHAPES[args.shape]
+    if args.context is not None:
+        shape = {**shape, "max_position_embeddings": args.context}
     context = shape["max_position_embeddings"]
     prompt_len, prefill_len = args.prompt_len, args.prefill_len
     if args.layers is None:

@@ -8,7 +8,9 @@
 // A block works on (token, kv head, group of up to 16 query heads, split of the key
 // range); its NW waves take chunks of 32 keys in turn, and a wave asks for the keys and
 // values of CB chunks at once before it works on the first: the work per chunk is short
-// next to a trip to memory, so the trips must overlap. Per chunk, transposed:
+// next to a trip to memory, so the trips must overlap. (Asking for the chunk CB places on as
+// soon as one has been worked on, so that loads are on their way during the work too, was no
+// faster at any context and 2.5% slower at 32,768 keys.) Per chunk, transposed:
 //   S^T[key, head]  = K[key, :] . Q[head, :]^T      two 16x16 tiles, k = head_dim
 //   O^T[dim, head] += V^T[dim, key] . P^T[key, head]  head_dim/16 tiles, k = 32 keys
 // so a lane's 16 bytes of a key row, and of a row of the transposed value page, are the
@@ -21,8 +23,11 @@
 // quarter q of the lanes ends up with keys 8q..8q+7, which is one 16-byte load from a
 // row of the transposed value page. Softmax keeps a
 // running maximum and sum per head in 32-bit. The waves' partial results are merged
-// in shared memory; with more than one split each block writes (max, sum, O) to a
-// workspace and a second kernel merges the splits in split order.
+// in shared memory (heads of more than 64: the upper half of the waves hands its results to
+// the lower half first, so that eight waves' results need the room of four: with four waves a
+// context of 560 keys took three trips to memory one after the other, with eight it takes
+// two, of which the second is nearly empty); with more than one split each block writes
+// (max, sum, O) to a workspace and a second kernel merges the splits in split order.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -53,8 +58,9 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     long out_stride, int n_heads, int n_kv, int page_size, int window, float scale, int n_splits) {
   constexpr int KK = HS / 32;   // k-steps of the first product
   constexpr int DT = HS / 16;   // row tiles of the second product
-  __shared__ float sm_m[NW][16], sm_l[NW][16];
-  __shared__ f32x4 sm_o[NW][DT][64];
+  constexpr int NS = (HS > 64 && NW > 4) ? NW / 2 : NW;   // partial results that shared memory holds at a time
+  __shared__ float sm_m[NS][16], sm_l[NS][16];
+  __shared__ f32x4 sm_o[NS][DT][64];
   AD_STAMP(0); AD_STAMP(1);
   const int g = n_heads / n_kv;
   const int groups = (g + 15) / 16;
@@ -177,17 +183,39 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   // merge the waves, in wave order
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
-  if (qd == 0) { sm_m[wave][j] = m_run; sm_l[wave][j] = l_run; }
+  if (NS < NW) {
+    // wave w + NS hands its results to wave w, which then stands for both
+    if (wave >= NS) {
+      if (qd == 0) { sm_m[wave - NS][j] = m_run; sm_l[wave - NS][j] = l_run; }
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) sm_o[wave][dt][lane] = o[dt];
+      for (int dt = 0; dt < DT; ++dt) sm_o[wave - NS][dt][lane] = o[dt];
+    }
+    __syncthreads();
+    if (wave < NS) {
+      const float m2 = sm_m[wave][j], l2 = sm_l[wave][j];
+      const float m_new = fmaxf(m_run, m2);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float f1 = __expf(m_run - m_use), f2 = __expf(m2 - m_use);   // a maximum of -inf gives 0
+      l_run = l_run * f1 + l2 * f2;
+      m_run = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt] = o[dt] * f1 + sm_o[wave][dt][lane] * f2;
+    }
+    __syncthreads();
+  }
+  if (wave < NS) {
+    if (qd == 0) { sm_m[wave][j] = m_run; sm_l[wave][j] = l_run; }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) sm_o[wave][dt][lane] = o[dt];
+  }
   __syncthreads();
   AD_STAMP(5);
   float M = sm_m[0][j];
 #pragma unroll
-  for (int w = 1; w < NW; ++w) M = fmaxf(M, sm_m[w][j]);
-  float f[NW], L = 0.f;
+  for (int w = 1; w < NS; ++w) M = fmaxf(M, sm_m[w][j]);
+  float f[NS], L = 0.f;
 #pragma unroll
-  for (int w = 0; w < NW; ++w) {
+  for (int w = 0; w < NS; ++w) {
     f[w] = sm_m[w][j] == -INFINITY ? 0.f : __expf(sm_m[w][j] - M);
     L += f[w] * sm_l[w][j];
   }
@@ -195,7 +223,7 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   for (int dt = wave; dt < DT; dt += NW) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < NW; ++w) acc += sm_o[w][dt][lane] * f[w];
+    for (int w = 0; w < NS; ++w) acc += sm_o[w][dt][lane] * f[w];
     if (j >= heads_here) continue;
     const int dim = dt * 16 + 4 * qd;   // lane holds O^T[dim .. dim+3][head j]
     if (n_splits == 1) {
@@ -215,24 +243,51 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   AD_STAMP(9); AD_STAMP(15);
 }
 
-// Merge the splits of one (token, head): in split order, so the result has one order of summation.
-__global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                              bf16_t* __restrict__ out, long out_stride, int n_heads, int head_dim,
-                                              int n_splits) {
+// Merge the splits of one (token, head); one wave. Lane i holds the maxima and sums of splits i, i + 64, ...
+// (all on their way at once; read one after the other, sixteen splits took 11 us), the factors go from
+// lane to lane, and every lane adds up its dims over the splits in split order, eight splits' loads at a time.
+__global__ __launch_bounds__(64) void attention_decode_merge_kernel(const float* __restrict__ part_o,
+                                                                    const float* __restrict__ part_ml,
+                                                                    bf16_t* __restrict__ out, long out_stride, int n_heads,
+                                                                    int head_dim, int n_splits) {
   const long th = blockIdx.x;   // token * n_heads + head
   const long t = th / n_heads, h = th % n_heads;
+  const int lane = threadIdx.x;
   const float* ml = part_ml + th * n_splits * 2;
-  float M = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, ml[2 * s]);
-  float L = 0.f;
-  for (int s = 0; s < n_splits; ++s) L += (ml[2 * s] == -INFINITY ? 0.f : __expf(ml[2 * s] - M)) * ml[2 * s + 1];
-  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+  float m[4], l[4];             // (at most 256 splits)
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int sp = lane + 64 * i;
+    m[i] = sp < n_splits ? ml[2 * sp] : -INFINITY;
+    l[i] = sp < n_splits ? ml[2 * sp + 1] : 0.f;
+  }
+  float M = fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3]));
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) M = fmaxf(M, __shfl_xor(M, d, 64));
+  float f[4], L = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[i] = m[i] == -INFINITY ? 0.f : __expf(m[i] - M);
+    L += f[i] * l[i];
+  }
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) L += __shfl_xor(L, d, 64);
+  const float* po = part_o + th * n_splits * head_dim;
+  for (int d = lane; d < head_dim + lane; d += 64) {     // (every lane walks the same number of times: the factors travel between lanes)
+    const bool mine = d < head_dim;
     float acc = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float f = ml[2 * s] == -INFINITY ? 0.f : __expf(ml[2 * s] - M);
-      acc += f * part_o[(th * n_splits + s) * head_dim + d];
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (mine && s0 + e < n_splits) ? po[(long)(s0 + e) * head_dim + d] : 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int sp = s0 + e;   // (the same for all lanes)
+        const float fs = __shfl(sp < 64 ? f[0] : sp < 128 ? f[1] : sp < 192 ? f[2] : f[3], sp & 63, 64);
+        acc += fs * v[e];
+      }
     }
-    out[t * out_stride + h * head_dim + d] = static_cast<bf16_t>(acc / L);
+    if (mine) out[t * out_stride + h * head_dim + d] = static_cast<bf16_t>(acc / L);
   }
 }
 
@@ -264,9 +319,9 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
   const long blocks = (long)n_tokens * n_kv * groups;
   GL3_REQUIRE(blocks < (1L << 31), "gl3_attention_decode: too many blocks");
   dim3 grid((unsigned)blocks, n_splits);
-  // 8 waves where their partial results fit the block's shared memory, else 4
+  // 8 waves; as many chunks on their way per wave as the registers hold (two waves share a SIMD's registers)
 #define GO(HS)                                                                                                        \
-  attention_decode_kernel<HS, (HS <= 64 ? 8 : 4), (HS <= 64 ? 4 : 2)><<<grid, dim3(HS <= 64 ? 512 : 256), 0, stream>>>(  \
+  attention_decode_kernel<HS, 8, (HS <= 64 ? 4 : HS <= 96 ? 3 : 2)><<<grid, dim3(512), 0, stream>>>(                                  \
       (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token, block_table, \
       table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, n_splits)
   switch (head_dim) {

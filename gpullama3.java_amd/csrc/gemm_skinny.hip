@@ -1237,7 +1237,10 @@ static int launch_skinny(int nw, const SkCall& a) {
     return 0;                                                                                                    \
   } while (0)
       if (steps <= 64) DEC(4);
-      if constexpr (EPI == SK_STORE) {
+      if constexpr (EPI == SK_STORE || EPI == SK_QKV) {
+        if (steps <= 96) DEC(6);   // (the QKV product of the 3B layers, K = 3,072: 13.8 us on the streaming kernel, 11.1 us here)
+      }
+      if constexpr (EPI == SK_STORE) {   // (with the rotation's operands beside 8 k-steps a wave the registers spill: K = 4,096, 17.0 -> 18.6 us)
         if (steps <= 128) DEC(8);
       }
 #undef DEC
@@ -1547,6 +1550,11 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
            : tiles == 3 ? launch_wide<3, 2, SK_QKV, bf16_t>(a, 1, 0)
                         : launch_wide<4, 2, SK_QKV, bf16_t>(a, 1, 0);
   }
+  // a folded norm's product of one token tile over a K too long for the kernel that keeps its operands in registers:
+  // whole lines, one strip a block, of which a CU holds several (so that more strips than CUs do not wait for a
+  // second round)
+  if (ssq && waves == 0 && M <= 16 && K > 3072 && wide_addressable(M, N, K, lda, ldw))
+    return launch_wide<1, 1, SK_QKV, bf16_t, true>(a, 1, 0);
   if (!ssq) return pick_mt<SK_QKV, bf16_t, false, false>(pick_waves(waves, N, K), a);
   return pick_mt<SK_QKV, bf16_t, true, false>(pick_waves(waves, N, K), a);
 }

@@ -692,14 +692,15 @@ def decode_splits(n_tokens, n_heads, n_kv, kv_len, head_dim=64):
     is worth its few microseconds only when a block would otherwise walk hundreds of KB of keys (more
     than 128 K elements, or 256 K and more where the step has more than 16 blocks anyway; ``kv_len`` is
     what the launch is sized for, in a replayed step the next power of two, so 4,096 stands for 2,049
-    to 4,096 keys), then one split per 64 K elements,
+    to 4,096 keys), then one split per 64 K elements (per 32 K where the step has at most 16 blocks: one
+    sequence of the 1B layers at 4,000 keys, 0.865 -> 0.822 ms a step; the same within 1% at 8,000 to 32,768 keys),
     and only until every CU has a block: more splits than that were slower at every batch and context
     measured (heads of 64, 16 sequences at 8,200 keys: 54 us with 2 splits, 63 us with 8)."""
     blocks = n_tokens * n_kv * -(-(n_heads // n_kv) // 16)
     elements = kv_len * head_dim
     if elements <= 131072 or (blocks > 16 and elements < 262144):
         return 1
-    return int(max(1, min(elements // 65536, 256 // blocks, 16)))
+    return int(max(1, min(elements // (32768 if blocks <= 16 else 65536), 256 // blocks, 32)))
 
 
 def attention_decode(q, k_cache, v_cache, positions, seq_of_token, block_table, out, n_heads, n_kv, head_dim,

@@ -30,7 +30,8 @@ def test_decode_attention_splits_the_keys_until_every_cu_has_a_block():
     assert s(1, 32, 8, 1024) == 1 and s(8, 32, 8, 1024, 128) == 1 and s(64, 32, 8, 16384) == 1   # short; blocks enough
     assert s(8, 32, 8, 1024, 128) == 1 and s(8, 32, 8, 2048, 64) == 1                   # 128 K elements, 64 blocks
     assert s(8, 32, 8, 2048, 128) == 4 and s(8, 32, 8, 4096, 64) == 4                   # 256 K elements
-    assert s(1, 32, 8, 4096) == 4 and s(1, 32, 8, 8192) == 8 and s(1, 32, 8, 32768) == 16   # a split per 64 K elements
-    assert s(1, 32, 8, 2048, 128) == 4 and s(1, 32, 8, 4096, 128) == 8
+    assert s(1, 32, 8, 4096) == 8 and s(1, 32, 8, 8192) == 16 and s(1, 32, 8, 32768) == 32   # few blocks: a split per 32 K elements
+    assert s(1, 32, 8, 2048, 128) == 8 and s(2, 32, 8, 4096, 128) == 16
+    assert s(4, 32, 8, 4096, 64) == 4 and s(4, 32, 8, 16384, 64) == 8                    # more than 16 blocks: per 64 K
     assert s(8, 32, 8, 32768) == 4 and s(16, 32, 8, 32768) == 2 and s(32, 32, 8, 32768) == 1   # 256 blocks, not more
-    assert s(2, 64, 2, 100000) == 16                                  # never more than 16
+    assert s(2, 64, 2, 100000) == 32                                  # never more than 32
