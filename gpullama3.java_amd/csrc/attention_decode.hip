@@ -319,11 +319,23 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
   const long blocks = (long)n_tokens * n_kv * groups;
   GL3_REQUIRE(blocks < (1L << 31), "gl3_attention_decode: too many blocks");
   dim3 grid((unsigned)blocks, n_splits);
-  // 8 waves; as many chunks on their way per wave as the registers hold (two waves share a SIMD's registers)
+  // 8 waves; as many chunks on their way per wave as the registers hold (two waves share a SIMD's registers).
+  // More blocks than CUs: 4 waves, so that a CU holds two blocks and the second 256 blocks do not wait for the
+  // first to end (what a block does before its keys arrive is a chain of trips to memory, paid once per round).
+  const bool small = blocks * n_splits > 256;
 #define GO(HS)                                                                                                        \
-  attention_decode_kernel<HS, 8, (HS <= 64 ? 4 : HS <= 96 ? 3 : 2)><<<grid, dim3(512), 0, stream>>>(                                  \
-      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token, block_table, \
-      table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, n_splits)
+  do {                                                                                                                \
+    if (small)                                                                                                        \
+      attention_decode_kernel<HS, 4, (HS <= 64 ? 4 : HS <= 96 ? 3 : 2)><<<grid, dim3(256), 0, stream>>>(                \
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token,         \
+          block_table, table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, \
+          n_splits);                                                                                                  \
+    else                                                                                                              \
+      attention_decode_kernel<HS, 8, (HS <= 64 ? 4 : HS <= 96 ? 3 : 2)><<<grid, dim3(512), 0, stream>>>(                \
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token,         \
+          block_table, table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, \
+          n_splits);                                                                                                  \
+  } while (0)
   switch (head_dim) {
     case 32: GO(32); break;
     case 64: GO(64); break;

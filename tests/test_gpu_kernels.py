@@ -497,14 +497,34 @@ def test_attention_decode(H, Kh, hs, splits):
     np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
 
 
-@pytest.mark.parametrize("splits", [1, 4])
-def test_attention_decode_far_key_and_window_edge(splits):
+@pytest.mark.parametrize("hs", [96, 128])
+def test_attention_decode_more_blocks_than_cus_and_many_splits(hs):
+    """More (token, kv head) pairs than CUs (the blocks then have four waves, not eight), and more splits than
+    chunks, so that most splits are empty and the merge reads more than a lane a split."""
+    rng = np.random.default_rng(hs)
+    H, Kh = 8, 4
+    lens_before = [int(n) for n in rng.integers(0, 300, 70)]
+    new = [1] * 70
+    sk, sv, qs = attention_case(rng, H, Kh, hs, lens_before, new, "bfloat16")
+    got, ref = run_attention(decode_fn(1), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng)
+    np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+    lens_before, new = [5, 700, 2500], [1] * 3
+    sk, sv, qs = attention_case(rng, H, Kh, hs, lens_before, new, "bfloat16")
+    for splits in (70, 200):
+        got, ref = run_attention(decode_fn(splits), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng)
+        np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+
+
+@pytest.mark.parametrize("hs, far", [(64, 13), (128, 13), (128, 170), (96, 235)])
+@pytest.mark.parametrize("splits", [1, 4, 40])
+def test_attention_decode_far_key_and_window_edge(splits, hs, far):
+    """One key among hundreds carries the weight: in the first wave's chunk, and (heads over 64) in a chunk of
+    the upper waves, whose sums reach the result through the lower waves."""
     rng = np.random.default_rng(19)
-    H, Kh, hs, n = 4, 2, 64, 700
+    H, Kh, n = 4, 2, 700
     k = rng.standard_normal((n, Kh, hs)).astype(np.float32) * 0.1
     v = rng.standard_normal((n, Kh, hs)).astype(np.float32)
     q = rng.standard_normal((n, H, hs)).astype(np.float32) * 0.1
-    far = 13
     k[far, 1] = 0; k[far, 1, 5] = 30.0
     q[n - 1, 2] = 0; q[n - 1, 2, 5] = 30.0
     q[n - 1, 0] = 0; q[n - 1, 0, 5] = 30.0
