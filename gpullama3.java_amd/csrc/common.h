@@ -117,6 +117,13 @@ __device__ __forceinline__ long gl3_v_offset(int dim, int position_in_page, int 
   return ((long)((dim >> 4) * (page_size >> 3) + (position_in_page >> 3)) << 7) + ((dim & 15) << 3) + (position_in_page & 7);
 }
 
+// Element (row n, column k) of a matrix that is kept in the order of the matrix operands:
+// [strip of 16 rows][k-step of 32][lane = 16 * (k block of 8) + row][8 elements], `steps` k-steps a strip
+// (lib.tile_weight; 8 consecutive k of a row lie together).
+__host__ __device__ __forceinline__ long gl3_operand_offset(long n, int k, int steps) {
+  return (((n >> 4) * steps + (k >> 5)) << 9) + (((k & 31) >> 3) << 7) + ((n & 15) << 3) + (k & 7);
+}
+
 enum { GL3_ACT_SILU = 0, GL3_ACT_GELU_TANH = 1 };
 
 template <bool FAST>

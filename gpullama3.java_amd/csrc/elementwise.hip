@@ -13,10 +13,13 @@
 template <typename TW, bool VEC>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out, int d,
                              float* __restrict__ ssq, const float* __restrict__ next_weight, bf16_t* __restrict__ xg,
-                             float scale, const TW* __restrict__ pos_table, const int* __restrict__ positions) {
+                             float scale, const TW* __restrict__ pos_table, const int* __restrict__ positions,
+                             int operand_steps) {
   __shared__ float scratch[16];
   const long t = blockIdx.x;
-  const TW* row = table + (long)ids[t] * d;
+  // operand_steps > 0 (VEC only): the table is kept in the matrix operands' order alone (gl3_operand_offset)
+  const TW* row = operand_steps ? table : table + (long)ids[t] * d;
+  const long id = ids[t];
   const TW* prow = pos_table ? pos_table + (long)positions[t] * d : nullptr;
   float* o = out + t * d;
   float ss = 0.f;
@@ -26,7 +29,7 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
     for (int i = threadIdx.x * 8; i < d; i += blockDim.x * 8) {
-      const tw8 r8 = *(const tw8*)(row + i);
+      const tw8 r8 = *(const tw8*)(row + (operand_steps ? gl3_operand_offset(id, i, operand_steps) : (long)i));
       float v[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = to_f32<TW>(r8[e]);
@@ -72,7 +75,7 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
 
 extern "C" int gl3_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens, int d,
                          float* ssq, const float* next_weight, void* xg, float scale, const void* pos_table,
-                         const int* positions, hipStream_t stream) {
+                         const int* positions, int operand_steps, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   GL3_REQUIRE(table && ids && out && n_tokens > 0 && d > 0, "gl3_embed: bad arguments (T=%d d=%d)", n_tokens, d);
   GL3_REQUIRE(!ssq || n_tokens <= 64, "gl3_embed: sums of squares are kept for at most 64 rows");
@@ -84,9 +87,13 @@ extern "C" int gl3_embed(const void* table, int table_dtype, const int* ids, flo
   const bool vec = d % 8 == 0 && (uintptr_t)table % 32 == 0 && (uintptr_t)out % 16 == 0 &&
                    (!pos_table || (uintptr_t)pos_table % 32 == 0) &&
                    (!xg || ((uintptr_t)xg % 16 == 0 && (uintptr_t)next_weight % 16 == 0));
+  // operand_steps > 0: the table lies in the matrix operands' order ([strip of 16 rows][k-step of 32][lane][8]) with
+  // that many k-steps a strip; a row's 8 consecutive elements are still one 16-byte unit
+  GL3_REQUIRE(operand_steps == 0 || (vec && operand_steps * 32 >= d),
+              "gl3_embed: a table in the operands' order needs a width of a multiple of 8 and aligned rows");
 #define GO(TW, VEC)                                                                                              \
   embed_kernel<TW, VEC><<<grid, block, 0, stream>>>((const TW*)table, ids, out, d, ssq, next_weight, (bf16_t*)xg, scale, \
-                                                    (const TW*)pos_table, pos_table ? positions : nullptr)
+                                                    (const TW*)pos_table, pos_table ? positions : nullptr, operand_steps)
   if (table_dtype == GL3_F32) { if (vec) GO(float, true); else GO(float, false); }
   else if (table_dtype == GL3_BF16) { if (vec) GO(bf16_t, true); else GO(bf16_t, false); }
   else GL3_REQUIRE(false, "gl3_embed: unknown dtype %d", table_dtype);

@@ -27,13 +27,13 @@ enum { MF_STORE = 0, MF_ADD = 1, MF_GATED = 2 };
 #define MF_LD (MF_BK + 8)   // padded row, in elements
 
 // WM x WN waves; a wave owns (32*TM) x 64 of the tile.
-template <int EPI, typename TC, int TM, int WM, int WN>
+template <int EPI, typename TC, int TM, int WM, int WN, bool WT = false>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* __restrict__ A,
                                                                   const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                   int M, int N, int K, long lda, long ldw, long ldc,
                                                                   int tiles_m, int tiles_n, int group_m, int k_per_slice,
                                                                   float* __restrict__ P, long p_stride, long ldp,
-                                                                  const float* __restrict__ bias, int act) {
+                                                                  const float* __restrict__ bias, int act, int w_steps) {
   constexpr int NT = 64 * WM * WN;                       // threads
   constexpr int BM = 32 * TM * WM;                       // rows of a block
   constexpr int BN = 64 * WN;                            // rows of W of a block
@@ -65,10 +65,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   // inside the tile, and every load is unconditional (rows and columns beyond the matrix are
   // clamped to its last ones and their values dropped): no branch around a load, whose registers
   // the compiler would then wait for at once.
+  // WT: W is kept in the matrix operands' order alone ([strip of 16 rows][k-step of 32][lane][8], w_steps
+  // k-steps a strip, gl3_operand_offset): a thread's 16 bytes are still 8 consecutive k of one row, only at another
+  // place, and go to the same place in shared memory.
   const bf16_t* a_tile = A + (long)m0 * lda;
   const bf16_t* w_tile[2];
-  w_tile[0] = W + (long)n0 * ldw;
-  w_tile[1] = (EPI == MF_GATED) ? W + ((long)N + n0) * ldw : w_tile[0];
+  w_tile[0] = WT ? W : W + (long)n0 * ldw;
+  w_tile[1] = WT ? W : (EPI == MF_GATED) ? W + ((long)N + n0) * ldw : w_tile[0];
   static_assert(EPI != MF_GATED || (NWC % 2 == 0 && (NT / 8) * (NWC / 2) == BN / 2),
                 "gate rows and up rows must fall to different loads of a thread");
   unsigned aoff[NA], woff[NWC];
@@ -84,7 +87,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
     const int r = (tid + NT * i) >> 3;
     wrow_s[i] = r;
     const int rel = (EPI == MF_GATED && i >= NWC / 2) ? r - BN / 2 : r;
-    woff[i] = (unsigned)(min(n0 + rel, N - 1) - n0) * (unsigned)ldw;
+    const int row = min(n0 + rel, N - 1);
+    woff[i] = WT ? (unsigned)gl3_operand_offset(row + ((EPI == MF_GATED && i >= NWC / 2) ? N : 0), 0, w_steps)
+                 : (unsigned)(row - n0) * (unsigned)ldw;
   }
   // K in slices (blockIdx.y): slice 0 ends in the epilogue proper, the others store their sums
   // as floats into P[slice - 1], for the reader to add up in slice order
@@ -101,10 +106,17 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
     const bf16_t* ak = a_tile + kf;
 #pragma unroll
     for (int i = 0; i < NA; ++i) ra[i] = *(const bf16x8*)(ak + (aoff[i] + col));
+    if (WT) {   // column kf + col of the row lies at its place inside the strip
+      const unsigned kc = (unsigned)kf + col;
+      const unsigned wcol = ((kc >> 5) << 9) + (((kc & 31u) >> 3) << 7);
 #pragma unroll
-    for (int i = 0; i < NWC; ++i) {
-      const bf16_t* wk = w_tile[(EPI == MF_GATED && i >= NWC / 2) ? 1 : 0] + kf;
-      rw[i] = *(const bf16x8*)(wk + (woff[i] + col));
+      for (int i = 0; i < NWC; ++i) rw[i] = *(const bf16x8*)(w_tile[0] + (woff[i] + wcol));
+    } else {
+#pragma unroll
+      for (int i = 0; i < NWC; ++i) {
+        const bf16_t* wk = w_tile[(EPI == MF_GATED && i >= NWC / 2) ? 1 : 0] + kf;
+        rw[i] = *(const bf16x8*)(wk + (woff[i] + col));
+      }
     }
   };
   fetch(k_begin);
@@ -213,9 +225,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   else finish(std::true_type{});
 }
 
-template <int EPI, typename TC, int TM, int WM, int WN>
+template <int EPI, typename TC, int TM, int WM, int WN, bool WT = false>
 static int launch_shape(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                        int slices, float* P, long p_stride, long ldp, const float* bias, int act, hipStream_t stream) {
+                        int slices, float* P, long p_stride, long ldp, const float* bias, int act, int w_steps,
+                        hipStream_t stream) {
   const int bm = 32 * TM * WM;
   const int ncols = (EPI == MF_GATED) ? 32 * WN : 64 * WN;
   const int tiles_n = (N + ncols - 1) / ncols;
@@ -228,22 +241,33 @@ static int launch_shape(const void* A, const void* W, void* C, int M, int N, int
   // them a rectangle of 4 x 8 (8 x 8), which asks memory for a third of the bytes that one column of
   // 32 row tiles does (3 to 5% of the time of the large products)
   const int group_m = tiles_m < (bm == 256 ? 4 : 8) ? tiles_m : (bm == 256 ? 4 : 8);
-  gemm_mfma_kernel<EPI, TC, TM, WM, WN><<<dim3((unsigned)blocks, slices), dim3(64 * WM * WN), 0, stream>>>(
+  gemm_mfma_kernel<EPI, TC, TM, WM, WN, WT><<<dim3((unsigned)blocks, slices), dim3(64 * WM * WN), 0, stream>>>(
       (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n, group_m, k_per_slice, P,
-      p_stride, ldp, bias, act);
+      p_stride, ldp, bias, act, w_steps);
   GL3_LAUNCH_CHECK();
   return 0;
 }
 
 template <int EPI, typename TC>
 static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                       int slices, float* P, long p_stride, long ldp, const float* bias, int act, int shape,
+                       int slices, float* P, long p_stride, long ldp, const float* bias, int act, int shape, int w_steps,
                        hipStream_t stream) {
-  if (shape == 1) return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
-  if (shape == 2) return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
-  if (shape == 3) return launch_shape<EPI, TC, 4, 2, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
-  if (shape == 4) return launch_shape<EPI, TC, 2, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
-  if (shape == 5) return launch_shape<EPI, TC, 1, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
+  if (w_steps) {
+    // W in the operands' order alone: the store epilogue (a head that is held once), tiles of 128 x 128 or 256 x 256
+    if constexpr (EPI == MF_STORE) {
+      const long small = (long)((M + 127) / 128) * ((N + 127) / 128);
+      if (shape == 2 || (shape == 0 && small > 1024))
+        return launch_shape<EPI, TC, 2, 4, 4, true>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
+      return launch_shape<EPI, TC, 1, 4, 2, true>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
+    } else {
+      GL3_REQUIRE(false, "gl3_gemm_mfma: W in the operands' order alone is read by the store epilogue only (epilogue %d)", EPI);
+    }
+  }
+  if (shape == 1) return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
+  if (shape == 2) return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
+  if (shape == 3) return launch_shape<EPI, TC, 4, 2, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
+  if (shape == 4) return launch_shape<EPI, TC, 2, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
+  if (shape == 5) return launch_shape<EPI, TC, 1, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
   // 256 x 256 tiles of sixteen waves, one block a CU, have half the operand traffic per product, and
   // that traffic is what bounds the large products; of the 128 x 128 tiles of eight waves two fit a CU and
   // overlap each other's waits. A step of 64 columns takes a chip full of the large tiles 1.7 us and a chip
@@ -264,10 +288,10 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
   const long small_cost = rounds(small_tiles, 512) * (small_tiles <= 256 ? 84 : 105), big_cost = rounds(big_tiles, 256) * 170;
   const long wide_cost = rounds(wide_tiles, 256) * (wide_tiles <= 128 ? 119 : 95);
   if (wide_cost < small_cost && wide_cost < big_cost && slices == 1)
-    return launch_shape<EPI, TC, 1, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
+    return launch_shape<EPI, TC, 1, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
   if (big_cost < small_cost)
-    return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
-  return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, stream);
+    return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
+  return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
 }
 
 // N counts output columns: for the gated epilogue W has 2N rows (gate, then up).
@@ -278,9 +302,10 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
 // shape: 0 lets the library choose the tile; 1: 128 x 128, eight waves; 2: 256 x 256, sixteen waves of
 // 64 x 64; 3: 256 x 256, eight waves of 128 x 64; 4: 256 rows x 128, eight waves of 64 x 64; 5: 128 rows x 256,
 // sixteen waves of 32 x 64.
+// w_steps: 0, or W is kept in the matrix operands' order alone (lib.tile_weight) with that many k-steps a strip.
 extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
                              long ldc, int epilogue, int slices, float* P, long p_stride, long ldp, const float* bias,
-                             int act, int shape, hipStream_t stream) {
+                             int act, int shape, int w_steps, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_mfma: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gl3_gemm_mfma: K=%d, lda=%ld, ldw=%ld must be multiples of 8",
@@ -299,7 +324,11 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_mfma: a bias goes with one slice of K");
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_mfma: unknown activation %d", act);
   GL3_REQUIRE(shape >= 0 && shape <= 5, "gl3_gemm_mfma: unknown tile shape %d", shape);
-#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, shape, stream
+  // w_steps > 0: W is kept in the matrix operands' order alone, w_steps k-steps of 32 a strip of 16 rows
+  GL3_REQUIRE(w_steps == 0 || (w_steps * 32 >= K && (epilogue == MF_GATED ? 2L * N : (long)N) % 16 == 0 &&
+                               (epilogue == MF_GATED ? 2L * N : (long)N) * w_steps * 32 < (1L << 32)),
+              "gl3_gemm_mfma: W in the operands' order with %d k-steps for K=%d, N=%d", w_steps, K, N);
+#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, shape, w_steps, stream
   if (c_dtype == GL3_F32) {
     if (epilogue == MF_STORE) return launch_mfma<MF_STORE, float>(ARGS);
     if (epilogue == MF_ADD) return launch_mfma<MF_ADD, float>(ARGS);

@@ -48,14 +48,14 @@ def _declare(lib):
     sigs = {
         "gl3_abi_version": [],
         "gl3_fill_u32": [P, c_uint32, L, P],
-        "gl3_embed": [P, I, P, P, I, I, P, P, P, F, P, P, P],
+        "gl3_embed": [P, I, P, P, I, I, P, P, P, F, P, P, I, P],
         "gl3_scale_f32": [P, F, L, P],
         "gl3_softcap_f32": [P, F, L, P],
         "gl3_rmsnorm": [P, P, P, I, P, I, I, I, F, P],
         "gl3_gather_rows": [P, P, P, I, I, I, P],
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
-        "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, P],
+        "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, I, P],
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_sample_work_floats": [I, I],
@@ -67,7 +67,7 @@ def _declare(lib):
         "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, I, P],
         "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
         "gl3_token_facts": [P, P, P, I, I, P, P, I, P, P, P, I, P],
-        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, P],
+        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, I, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
         "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P],
@@ -117,6 +117,23 @@ def _dev(t, name, dtype=None, contiguous=True):
     if contiguous and not t.is_contiguous():
         raise KernelError(f"{name} must be contiguous")
     return t
+
+
+def held_once(w):
+    """Whether the matrix is kept in the matrix operands' order ALONE (``hold_once``): its memory is its copy
+    ``w.tiled``, and only what reads that order may touch it."""
+    return getattr(w, "operand_order_only", False)
+
+
+def _operand_steps(w):
+    """The k-steps of 32 a strip of a matrix that is held once (what the kernels that read both orders take), else 0."""
+    return -(-w.shape[1] // 32) if held_once(w) else 0
+
+
+def _stored(w, who):
+    if held_once(w):
+        raise KernelError(f"{who}: the weight is kept in the matrix operands' order alone, which this kernel does not read")
+    return w
 
 
 def _code(t, name):
@@ -211,7 +228,8 @@ def embed(table, ids, out, ssq=None, next_weight=None, xg=None, scale=1.0, pos_t
             raise KernelError(f"embed: table of positions {tuple(pos_table.shape)} for rows of {d}")
     _check(library().gl3_embed(_ptr(table), _code(table, "table"), _ptr(ids), _ptr(out), T, d, _ptr(ssq),
                                _ptr(next_weight), _ptr(xg), float(scale), _ptr(pos_table),
-                               _ptr(positions) if pos_table is not None else c_void_p(0), _stream()), "embed")
+                               _ptr(positions) if pos_table is not None else c_void_p(0), _operand_steps(table),
+                               _stream()), "embed")
 
 
 def rmsnorm(x, weight, out, eps, rows=None):
@@ -311,7 +329,8 @@ def gemm_generic(a, w, out, epilogue=EPI_STORE, bias=None, act="silu"):
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_generic(_ptr(a), _code(a, "a"), _ptr(w), _code(w, "w"), _ptr(out), _code(out, "out"),
                                       M, N, K, a.stride(0), w.stride(0), out.stride(0), epilogue,
-                                      _bias(bias, rows, "gemm_generic"), _act(act, "gemm_generic"), _stream()),
+                                      _bias(bias, rows, "gemm_generic"), _act(act, "gemm_generic"), _operand_steps(w),
+                                      _stream()),
            "gemm_generic")
 
 
@@ -440,6 +459,8 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows
     _check_next(next_weight, xg, M, N, "gemm_skinny")
     if xg is not None and ssq_out is None:
         raise KernelError("gemm_skinny: the next norm's rows come with the sums of squares")
+    if held_once(w) and (strip_rows != 16 or not _tiled(w, rows, K, n_out=N).value):
+        raise KernelError("gemm_skinny: a weight kept in the operands' order alone is read in strips of 16 rows through its copy")
     _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                      out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _ptr(next_weight),
                                      _ptr(xg), xg.stride(0) if xg is not None else 0, _bias(bias, rows, "gemm_skinny"),
@@ -497,6 +518,28 @@ def tile_weight8(w):
     return wp.view(N // 8, 8, steps, 2, 4, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
 
 
+def untile_weight(t, n_rows, K):
+    """The rows of a matrix out of its copy in the matrix operands' order (``tile_weight`` without a permutation
+    of the rows): a new tensor [n_rows, K] in the stored order."""
+    steps = -(-K // 32)
+    return t.view(n_rows // 16, steps, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(n_rows, steps * 32)[:, :K].contiguous()
+
+
+def hold_once(w):
+    """``w`` (which carries ``w.tiled``, rows in order, K a multiple of 32) as a matrix that is kept in the
+    operands' order alone: a tensor of the same shape and dtype whose memory IS the copy. Whoever drops ``w``
+    then frees the stored order. The kernels that read both orders (the embedding, the generic and the tiled
+    product, and those of few rows that take ``w.tiled``) are told by ``held_once``; the others refuse it."""
+    t = getattr(w, "tiled", None)
+    N, K = w.shape
+    if t is None or getattr(t, "tiled_for", None) is not None or K % 32 or N % 16 or t.numel() != N * K:
+        raise KernelError(f"hold_once: {tuple(w.shape)} has no copy in the operands' order that could stand for it")
+    alias = t.view(N, K)
+    alias.tiled = t
+    alias.operand_order_only = True
+    return alias
+
+
 def _tiled8(w, n_rows, K):
     t = getattr(w, "tiled8", None)
     if t is None or n_rows % 8 or t.numel() != n_rows * -(-K // 64) * 64:
@@ -515,7 +558,7 @@ def _tiled(w, n_rows, K, qkv=None, n_out=None):
 
 
 def gemm_skinny_wide_fits(a, w, out, epilogue):
-    return 8 < a.shape[0] <= 64 and gemm_skinny_fits(a, w, out, epilogue)
+    return 8 < a.shape[0] <= 64 and gemm_skinny_fits(a, w, out, epilogue) and not held_once(w)
 
 
 def wide_slices(N, K):
@@ -529,7 +572,8 @@ def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="si
     """out (=, +=, gated) a @ w.T for 17 to 64 rows of ``a``. ``out`` with three axes [slices, M, N]
     (float32, store epilogue) takes the sums of one slice of K each: the caller adds them up; that form
     also takes 9 to 16 rows."""
-    _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
+    _dev(a, "a", torch.bfloat16, contiguous=False); _dev(_stored(w, "gemm_skinny_wide"), "w", torch.bfloat16)
+    _dev(out, "out", contiguous=False)
     M, K = a.shape
     slices, slice_stride = 1, 0
     rows = out
@@ -585,6 +629,8 @@ def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=
     wrows = 2 * N if epilogue == EPI_GATED else N
     if w.shape != (wrows, K) or out.shape[0] != M or out.stride(1) != 1 or M > 64:
         raise KernelError(f"gemm: rows {tuple(xg.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
+    if held_once(w) and (whole_lines or not _tiled(w, wrows, K, n_out=N).value):
+        raise KernelError("gemm_skinny_norm: a weight kept in the operands' order alone is read through its copy")
     if whole_lines:
         if epilogue != EPI_GATED or rows is not None or M > 16 or waves:
             raise KernelError("gemm_skinny_norm: whole lines go with the gated epilogue, at most 16 rows, all of them")
@@ -642,7 +688,7 @@ def qkv_rope_cache(a, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_toke
     ``a`` holds the rows as they are; else ``a`` = bfloat16(norm weight * x) and the product is that
     of RMSNorm(x), the rows' sums of squares coming as partial sums. ``token_pages``, ``token_rot``: what
     ``token_facts`` made of the same positions, table and rotation (then the kernel does not look them up)."""
-    _dev(w_qkv, "w_qkv", torch.bfloat16); _dev(q_out, "q_out", torch.bfloat16, contiguous=False)
+    _dev(_stored(w_qkv, "qkv_rope_cache"), "w_qkv", torch.bfloat16); _dev(q_out, "q_out", torch.bfloat16, contiguous=False)
     K = w_qkv.shape[1]
     if ssq is None:
         _dev(a, "a", torch.bfloat16, contiguous=False)
@@ -764,7 +810,8 @@ def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None, bias=None, act="s
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
     _check(library().gl3_gemm_mfma(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                    out.stride(0), epilogue, slices, _ptr(more_slices), p_stride, ldp,
-                                   _bias(bias, rows, "gemm_mfma"), _act(act, "gemm_mfma"), int(shape), _stream()),
+                                   _bias(bias, rows, "gemm_mfma"), _act(act, "gemm_mfma"), int(shape), _operand_steps(w),
+                                   _stream()),
            "gemm_mfma")
 
 

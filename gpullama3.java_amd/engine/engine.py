@@ -68,6 +68,8 @@ def _without(without, weight_copies):
     names = set(ops.switches(without))
     if not weight_copies:
         names.add("tiled")
+    elif weight_copies == "both":
+        names.add("once")
     return frozenset(names)
 
 
@@ -76,8 +78,8 @@ class Engine:
 
     ``weight_copies``: a bfloat16 engine keeps, beside each matrix that decode steps read (QKV, output and down
     projection, the head, and the gate/up rows of small models), a copy in the order in which the matrix cores
-    take it: 2.5 -> 4.0 GB for the 1B shape, for about 5% more tokens a second at batch 8. False leaves the
-    copies out. ``without``: names of fast paths (``parts.ops.SWITCHES``) this engine does not use, for
+    take it, and the head (with a tied embedding) in that order alone: 2.5 -> 3.5 GB for the 1B shape, for 16%
+    more tokens a second at batch 8. False leaves the copies out; "both" keeps the stored order of every matrix too. ``without``: names of fast paths (``parts.ops.SWITCHES``) this engine does not use, for
     measurements and tests. ``max_graphs``: captured decode steps kept at a time; the least recently used
     one goes first."""
 
@@ -145,8 +147,11 @@ class Engine:
             return cls.from_folder(tmp, dtype=dtype, device=device, **kw)
 
     def weights(self):
-        """Stored name -> device tensor (stacked matrices appear as views under their stored names)."""
-        return self.model.weights
+        """Stored name -> device tensor (stacked matrices appear as views under their stored names). A matrix that
+        the engine keeps in the matrix operands' order alone is put back into the stored order for the caller: a
+        tensor of the caller's own, made at each call."""
+        from ..csrc import lib as K
+        return {name: K.untile_weight(w.tiled, *w.shape) if K.held_once(w) else w for name, w in self.model.weights.items()}
 
     # ------------------------------------------------------------------ slots
     def take_slot(self):

@@ -93,6 +93,13 @@ class DecoderModel:
         self.embedding = weights[self.spec.embedding_name]
         self.head = self.embedding if self.spec.head_name is None else weights[self.spec.head_name]
         ops.for_few_rows(self.head, without=self.without)
+        if ops.can_hold_once(self.head, self.without):
+            # every reader of the head (and of a tied embedding) takes the matrix operands' order: the stored
+            # order is let go, the copy stands for the matrix under its stored name
+            name = self.spec.embedding_name if self.spec.head_name is None else self.spec.head_name
+            self.head = weights[name] = K.hold_once(self.head)
+            if self.spec.head_name is None:
+                self.embedding = self.head
         if self.spec.position_table_name is not None:
             self.position_table = weights[self.spec.position_table_name].to(self.embedding.dtype)
         if self.spec.head_bias_name is not None:     # the epilogues read biases as float

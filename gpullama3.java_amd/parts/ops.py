@@ -28,9 +28,10 @@ CHUNK_ROWS = 128
 # the decoder sets before ``load``). "skinny", "wide", "mfma", "attn_decode", "attn_prefill": a family of kernels;
 # "fused": norms, rotation and cache write folded into products; "tiled", "packed": the weights' copies in operand
 # order and the rows handed over in the packed tiles' order; "widefold", "wide916": the kernel of whole lines for
-# the gated product with a folded norm and for products of 9 to 16 rows over a long K.
+# the gated product with a folded norm and for products of 9 to 16 rows over a long K; "once": a weight whose
+# readers all take the operands' order kept in that order alone (with any switch set, both orders are kept).
 SWITCHES = frozenset({"skinny", "wide", "mfma", "attn_decode", "attn_prefill", "fused", "tiled", "packed", "widefold",
-                      "wide916"})
+                      "wide916", "once"})
 _NONE = frozenset()
 
 
@@ -60,6 +61,16 @@ def for_few_rows(w, qkv=None, without=_NONE):
             and w.is_contiguous()):
         w.tiled = K.tile_weight(w, qkv)
     return w
+
+
+def can_hold_once(w, without=_NONE):
+    """Whether a weight whose readers all take the matrix operands' order (the head: the embedding look-up of a
+    tied head, the products of few rows, the tiled product's store epilogue, the generic product) can be kept in
+    that order alone: it has the copy, rows in order, whole k-steps, and the engine has no fast path switched
+    off (a comparison wants both orders at hand; ``Engine(weight_copies="both")`` asks for exactly that)."""
+    t = getattr(w, "tiled", None)
+    return (not without and t is not None and getattr(t, "tiled_for", None) is None and w.shape[1] % 32 == 0
+            and w.shape[0] % 16 == 0 and t.numel() == w.numel())
 
 
 def for_gated(w, without=_NONE):
@@ -234,7 +245,7 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
             return
         if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
             N = out.shape[1]
-            rows = K.skinny_strip_rows(a.shape[0], N, a.shape[1], epilogue)
+            rows = 16 if K.held_once(w) else K.skinny_strip_rows(a.shape[0], N, a.shape[1], epilogue)
             if (epilogue == EPI_ADD and ctx is not None and getattr(ctx, "fuse", False) and N % 16 == 0
                     and "fused" not in disabled and out.shape[0] == ctx.n_tokens <= FUSE_ROWS):
                 # the rows are complete after this product: leave what the norm that follows needs

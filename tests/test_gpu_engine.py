@@ -456,3 +456,39 @@ def test_one_step_with_a_decode_token_a_fresh_prompt_and_a_chunk(name, dtype):
     assert [eng.cache.length(s) for s in (s_old, s_new, s_old2)] == [71, 37, 135]
     out = eng.step([(s_old, [old[71]]), (s_new, [new[37]]), (s_old2, [old2[135]])]).cpu().numpy()
     close(out, np.stack([refs[0][71], refs[1][37], refs[2][135]]), dtype, "the decode step after the mixed step")
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_the_head_is_held_once_and_gives_the_same_logits(name):
+    """A bfloat16 engine keeps the head (A: and the tied embedding with it) in the matrix operands' order alone.
+    Every way a step reads it gives what an engine that keeps both orders gives, bit for bit: a prompt with all
+    rows wanted (the tiled product), its last row (a product of one row), decode steps (the folded norm), a
+    batch of 40 (the product of 17 to 64 rows); ``weights()`` hands back the stored order."""
+    from gpullama3_java_amd.csrc import lib
+    from safetensors.torch import load_file
+    import os
+    once, both = engine(name, "bfloat16", n_slots=64, max_tokens=8192), engine(name, "bfloat16", weight_copies="both",
+                                                                                n_slots=64, max_tokens=8192)
+    head = once.model.head
+    assert lib.held_once(head) and head.data_ptr() == head.tiled.data_ptr()
+    assert (once.model.embedding is head) == CONFIGS[name]["tie_word_embeddings"]
+    assert not lib.held_once(both.model.head) and both.model.head.tiled is not None
+    folder, _, _ = model(name)
+    stored = load_file(os.path.join(folder, "model.safetensors"))
+    given = once.weights()
+    assert set(given) == set(stored)
+    for k, v in stored.items():
+        assert torch.equal(given[k].cpu(), v.to(given[k].dtype)), k
+    toks = rand_tokens(name, 5, 100)
+    outs = []
+    for eng in (once, both):
+        s = eng.take_slot()
+        got = [eng.step([(s, toks[:90])], want="all"), eng.step([(s, toks[90:95])]), eng.step([(s, toks[95:96])])]
+        got += [eng.step([(s, [t])]) for t in toks[96:]]
+        many = [eng.take_slot() for _ in range(40)]
+        eng.step([(m, toks[i:i + 3]) for i, m in enumerate(many)], want="none")
+        got.append(eng.step([(m, [toks[i]]) for i, m in enumerate(many)]))
+        outs.append([g_.clone() for g_ in got])
+    for i, (u, v) in enumerate(zip(*outs)):
+        assert torch.equal(u, v), f"{name}: result {i} differs between the head held once and both orders"
+    close(torch.cat(outs[0][:1]).cpu().numpy(), plain_logits(name, toks[:90]), "bfloat16", f"{name} held once, whole")

@@ -1112,6 +1112,70 @@ def test_products_read_a_weight_copy_in_operand_order(M, N, Kd):
     assert torch.equal(p2, res[False][2])
 
 
+@pytest.mark.parametrize("N, Kd", [(48, 96), (2048, 2048), (272, 1568), (8208, 160)])
+def test_a_weight_kept_in_operand_order_alone(N, Kd):
+    """``hold_once``: the matrix's memory is its copy in the operands' order. The embedding look-up, the generic
+    product, the tiled product (store epilogue, both tiles) and the products of few rows give what they give
+    for the stored order, bit for bit; ``untile_weight`` gives the stored order back; what cannot read it refuses."""
+    rng = np.random.default_rng(N + Kd)
+    lib = K()
+    w = dev(rounded(rng.standard_normal((N, Kd)) / math.sqrt(Kd), "bfloat16"), torch.bfloat16)
+    w.tiled = lib.tile_weight(w)
+    once = lib.hold_once(w)
+    assert lib.held_once(once) and not lib.held_once(w) and once.shape == w.shape and once.data_ptr() == w.tiled.data_ptr()
+    assert torch.equal(lib.untile_weight(once.tiled, N, Kd), w)
+    # the embedding look-up, with and without what a folded norm wants
+    ids = torch.tensor(rng.integers(0, N, 19), dtype=torch.int32, device=DEV)
+    e1, e2 = torch.zeros(19, Kd, device=DEV), torch.zeros(19, Kd, device=DEV)
+    lib.embed(w, ids, e1); lib.embed(once, ids, e2)
+    assert torch.equal(e1, e2) and torch.equal(e1, w[ids.long()].float())
+    nw = dev(1 + 0.1 * rng.standard_normal(Kd))
+    got = []
+    for table in (w, once):
+        o, q, g_ = torch.zeros(19, Kd, device=DEV), torch.zeros(64, device=DEV), torch.zeros(19, Kd, device=DEV, dtype=torch.bfloat16)
+        lib.embed(table, ids, o, q, nw, g_, scale=1.5)
+        got.append((o, q, g_))
+    assert all(torch.equal(u, v) for u, v in zip(*got))
+    # products of many rows: the generic kernel and both tiles of the tiled one, odd row counts
+    for M in (3, 65, 300):
+        a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
+        ref = P.linear(a.float().cpu().numpy(), w.float().cpu().numpy())
+        g1, g2 = torch.zeros(M, N, device=DEV), torch.zeros(M, N, device=DEV)
+        lib.gemm_generic(a, w, g1); lib.gemm_generic(a, once, g2)
+        assert torch.equal(g1, g2)
+        for shape in (1, 2, 0):
+            m1, m2 = torch.zeros(M, N, device=DEV), torch.full((M, N + 3), -7.0, device=DEV)
+            lib.gemm_mfma(a, w, m1, shape=shape); lib.gemm_mfma(a, once, m2[:, :N], shape=shape)
+            assert torch.equal(m1, m2[:, :N]) and torch.all(m2[:, N:] == -7.0), (M, shape)
+            np.testing.assert_allclose(m1.cpu().numpy(), ref, atol=2e-5 * np.abs(ref).max() * math.sqrt(Kd))
+        b1, b2 = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16), torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+        lib.gemm_mfma(a, w, b1, shape=1); lib.gemm_mfma(a, once, b2, shape=1)
+        assert torch.equal(b1, b2)
+        with pytest.raises(lib.KernelError, match="store epilogue"):
+            lib.gemm_mfma(a, once, torch.zeros(M, N, device=DEV), lib.EPI_ADD)
+    # products of few rows read the copy as before
+    for M in (1, 8, 16, 40, 64):
+        a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
+        s1, s2 = torch.zeros(M, N, device=DEV), torch.zeros(M, N, device=DEV)
+        lib.gemm_skinny(a, w, s1); lib.gemm_skinny(a, once, s2)
+        assert torch.equal(s1, s2), M
+    x = (rng.standard_normal((9, Kd)) * 2).astype(np.float32)
+    xg, ssq = times_weight(x, rounded(1 + 0.2 * rng.standard_normal(Kd), "bfloat16")).to(DEV), dev(ssq_partials(x, 3))
+    n1, n2 = torch.zeros(9, N, device=DEV), torch.zeros(9, N, device=DEV)
+    lib.gemm_skinny_norm(xg, ssq, 3, 1e-5, w, n1); lib.gemm_skinny_norm(xg, ssq, 3, 1e-5, once, n2)
+    assert torch.equal(n1, n2)
+    # what reads the stored order only says so
+    a = dev(rounded(rng.standard_normal((8, Kd)), "bfloat16"), torch.bfloat16)
+    with pytest.raises(lib.KernelError, match="strips of 16"):
+        lib.gemm_skinny(a, once, torch.zeros(8, N, device=DEV), strip_rows=8)
+    a40 = dev(rounded(rng.standard_normal((40, Kd)), "bfloat16"), torch.bfloat16)
+    assert not lib.gemm_skinny_wide_fits(a40, once, torch.zeros(40, N, device=DEV), lib.EPI_STORE)
+    with pytest.raises(lib.KernelError, match="operands' order alone"):
+        lib.gemm_skinny_wide(a40, once, torch.zeros(40, N, device=DEV))
+    with pytest.raises(lib.KernelError, match="hold_once"):
+        lib.hold_once(dev(np.zeros((16, 40)), torch.bfloat16))              # no copy, and K is no whole k-step
+
+
 @pytest.mark.parametrize("pairing", ["adjacent", "half", None])
 @pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 16), (5, 5, 48), (8, 1, 128)])
 def test_qkv_rope_cache_reads_a_weight_copy_in_operand_order(pairing, H, Kh, hs):
