@@ -123,6 +123,18 @@ __device__ __forceinline__ long gl3_v_offset(int dim, int position_in_page, int 
 __host__ __device__ __forceinline__ long gl3_operand_offset(long n, int k, int steps) {
   return (((n >> 4) * steps + (k >> 5)) << 9) + (((k & 31) >> 3) << 7) + ((n & 15) << 3) + (k & 7);
 }
+// The same for the packed strips of 8 rows: [strip of 8 rows][step of 64 k][lane = 16 * (k block of 8 inside its
+// half) + 8 * (half of the step) + row][8 elements], `steps` steps of 64 a strip (lib.tile_weight8).
+__host__ __device__ __forceinline__ long gl3_packed_offset(long n, int k, int steps) {
+  return (((n >> 3) * steps + (k >> 6)) << 9) + (((k & 31) >> 3) << 7) + (((k >> 5) & 1) << 6) + ((n & 7) << 3) + (k & 7);
+}
+// Where element (n, k) of W lies. order 0: rows as stored (ldw); 1: the operands' order; 2: the packed strips of 8.
+// `pos` (order 1, may be null): the place of each row in a copy whose strips hold the rows in another order.
+__host__ __device__ __forceinline__ long gl3_w_offset(int order, long n, int k, long ldw, int steps, const int* pos) {
+  if (order == 0) return n * ldw + k;
+  if (order == 1) return gl3_operand_offset(pos ? pos[n] : n, k, steps);
+  return gl3_packed_offset(n, k, steps);
+}
 
 enum { GL3_ACT_SILU = 0, GL3_ACT_GELU_TANH = 1 };
 

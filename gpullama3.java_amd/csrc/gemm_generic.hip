@@ -25,9 +25,10 @@ template <typename TA, typename TW, typename TC, int EPI>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
                                                             TC* __restrict__ C, int M, int N, int K, long lda,
                                                             long ldw, long ldc, long up_offset,
-                                                            const float* __restrict__ bias, int act, int w_steps) {
+                                                            const float* __restrict__ bias, int act, int w_order, int w_steps,
+                                                            const int* __restrict__ w_pos) {
   // N is the number of output columns; for EPI_GATED the up rows of W start at
-  // row `up_offset`. w_steps > 0: W is kept in the matrix operands' order (gl3_operand_offset).
+  // row `up_offset`. w_order, w_steps, w_pos: how W lies (gl3_w_offset).
   __shared__ float As[GK][GT + 1];
   __shared__ float Ws[GK][GT + 1];
   __shared__ float Us[EPI == EPI_GATED ? GK : 1][GT + 1];
@@ -45,9 +46,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
       if (k < K) {
         if (m0 + r < M) a = to_f32<TA>(A[(m0 + r) * lda + k]);
         if (n0 + r < N) {
-          w = to_f32<TW>(W[w_steps ? gl3_operand_offset(n0 + r, k, w_steps) : (n0 + r) * ldw + k]);
-          if (EPI == EPI_GATED)
-            u = to_f32<TW>(W[w_steps ? gl3_operand_offset(up_offset + n0 + r, k, w_steps) : (up_offset + n0 + r) * ldw + k]);
+          w = to_f32<TW>(W[gl3_w_offset(w_order, n0 + r, k, ldw, w_steps, w_pos)]);
+          if (EPI == EPI_GATED) u = to_f32<TW>(W[gl3_w_offset(w_order, up_offset + n0 + r, k, ldw, w_steps, w_pos)]);
         }
       }
       As[kk][r] = a;
@@ -100,42 +100,46 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
 
 template <typename TA, typename TW, typename TC>
 static int launch_generic(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                          int epi, const float* bias, int act, int w_steps, hipStream_t stream) {
+                          int epi, const float* bias, int act, int w_order, int w_steps, const int* w_pos, hipStream_t stream) {
   dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT), block(256);
   GL3_REQUIRE(grid.y <= 65535, "gl3_gemm_generic: M=%d is too large for one launch", M);
   const TA* a = (const TA*)A;
   const TW* w = (const TW*)W;
   TC* c = (TC*)C;
-  if (epi == EPI_STORE) gemm_generic_kernel<TA, TW, TC, EPI_STORE><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act, w_steps);
-  else if (epi == EPI_ADD) gemm_generic_kernel<TA, TW, TC, EPI_ADD><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act, w_steps);
-  else gemm_generic_kernel<TA, TW, TC, EPI_GATED><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, N, bias, act, w_steps);
+  if (epi == EPI_STORE) gemm_generic_kernel<TA, TW, TC, EPI_STORE><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act, w_order, w_steps, w_pos);
+  else if (epi == EPI_ADD) gemm_generic_kernel<TA, TW, TC, EPI_ADD><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, 0, bias, act, w_order, w_steps, w_pos);
+  else gemm_generic_kernel<TA, TW, TC, EPI_GATED><<<grid, block, 0, stream>>>(a, w, c, M, N, K, lda, ldw, ldc, N, bias, act, w_order, w_steps, w_pos);
   GL3_LAUNCH_CHECK();
   return 0;
 }
 
 // N counts output columns: for the gated epilogue W has 2N rows (gate, then up).
 // bias (may be null): N floats (gated: 2N). act: the gated epilogue's activation (GL3_ACT_*).
-// w_steps: 0, or W is kept in the matrix operands' order alone with that many k-steps of 32 a strip.
+// w_order, w_pos: how W lies (see below): as stored, or one of its copies in the matrix cores' order alone.
 extern "C" int gl3_gemm_generic(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M,
                                 int N, int K, long lda, long ldw, long ldc, int epilogue, const float* bias, int act,
-                                int w_steps, hipStream_t stream) {
+                                int w_order, const int* w_pos, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_generic: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gl3_gemm_generic: leading dimensions %ld %ld %ld too small", lda, ldw, ldc);
   GL3_REQUIRE(epilogue >= 0 && epilogue <= 2, "gl3_gemm_generic: unknown epilogue %d", epilogue);
   GL3_REQUIRE(epilogue != EPI_ADD || c_dtype == GL3_F32, "gl3_gemm_generic: the add epilogue needs a float output");
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_generic: unknown activation %d", act);
-  // w_steps > 0: W is kept in the matrix operands' order, [strip of 16 rows][k-step of 32][lane][8], w_steps k-steps a strip
-  GL3_REQUIRE(w_steps == 0 || (w_steps * 32 >= K && (epilogue == EPI_GATED ? 2 * N : N) % 16 == 0),
-              "gl3_gemm_generic: W in the operands' order with %d k-steps for K=%d, N=%d", w_steps, K, N);
+  // w_order: 0: W holds the rows as stored. 1: W is the copy in the matrix operands' order (lib.tile_weight); w_pos (may be
+  // null) then names each row's place in it. 2: the copy in packed strips of 8 rows (lib.tile_weight8).
+  const long w_rows = epilogue == EPI_GATED ? 2L * N : N;
+  GL3_REQUIRE(w_order >= 0 && w_order <= 2 && (w_order != 1 || w_rows % 16 == 0) && (w_order != 2 || w_rows % 8 == 0) &&
+                  (w_order == 1 || !w_pos),
+              "gl3_gemm_generic: W in order %d with N=%d, epilogue %d", w_order, N, epilogue);
+  const int w_steps = w_order == 1 ? (K + 31) / 32 : (K + 63) / 64;
   const int key = a_dtype * 4 + w_dtype * 2 + c_dtype;
   switch (key) {
-    case 0: return launch_generic<float, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_steps, stream);
-    case 2: return launch_generic<float, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_steps, stream);
-    case 4: return launch_generic<bf16_t, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_steps, stream);
-    case 5: return launch_generic<bf16_t, float, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_steps, stream);
-    case 6: return launch_generic<bf16_t, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_steps, stream);
-    case 7: return launch_generic<bf16_t, bf16_t, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_steps, stream);
+    case 0: return launch_generic<float, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
+    case 2: return launch_generic<float, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
+    case 4: return launch_generic<bf16_t, float, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
+    case 5: return launch_generic<bf16_t, float, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
+    case 6: return launch_generic<bf16_t, bf16_t, float>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
+    case 7: return launch_generic<bf16_t, bf16_t, bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, epilogue, bias, act, w_order, w_steps, w_pos, stream);
     default:
       GL3_REQUIRE(false, "gl3_gemm_generic: unsupported dtypes A=%d W=%d C=%d", a_dtype, w_dtype, c_dtype);
   }

@@ -27,13 +27,14 @@ enum { MF_STORE = 0, MF_ADD = 1, MF_GATED = 2 };
 #define MF_LD (MF_BK + 8)   // padded row, in elements
 
 // WM x WN waves; a wave owns (32*TM) x 64 of the tile.
-template <int EPI, typename TC, int TM, int WM, int WN, bool WT = false>
+template <int EPI, typename TC, int TM, int WM, int WN, int WT = 0>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* __restrict__ A,
                                                                   const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                   int M, int N, int K, long lda, long ldw, long ldc,
                                                                   int tiles_m, int tiles_n, int group_m, int k_per_slice,
                                                                   float* __restrict__ P, long p_stride, long ldp,
-                                                                  const float* __restrict__ bias, int act, int w_steps) {
+                                                                  const float* __restrict__ bias, int act, int w_steps,
+                                                                  const int* __restrict__ w_pos) {
   constexpr int NT = 64 * WM * WN;                       // threads
   constexpr int BM = 32 * TM * WM;                       // rows of a block
   constexpr int BN = 64 * WN;                            // rows of W of a block
@@ -65,9 +66,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   // inside the tile, and every load is unconditional (rows and columns beyond the matrix are
   // clamped to its last ones and their values dropped): no branch around a load, whose registers
   // the compiler would then wait for at once.
-  // WT: W is kept in the matrix operands' order alone ([strip of 16 rows][k-step of 32][lane][8], w_steps
-  // k-steps a strip, gl3_operand_offset): a thread's 16 bytes are still 8 consecutive k of one row, only at another
-  // place, and go to the same place in shared memory.
+  // WT 1: W is the copy in the matrix operands' order alone ([strip of 16 rows][k-step of 32][lane][8], w_steps
+  // k-steps a strip, gl3_operand_offset; w_pos, may be null: each row's place in a copy whose strips hold the rows
+  // in another order). WT 2: the copy in packed strips of 8 rows (gl3_packed_offset, w_steps steps of 64). A
+  // thread's 16 bytes are still 8 consecutive k of one row, only at another place, and go to the same place in
+  // shared memory.
   const bf16_t* a_tile = A + (long)m0 * lda;
   const bf16_t* w_tile[2];
   w_tile[0] = WT ? W : W + (long)n0 * ldw;
@@ -75,7 +78,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   static_assert(EPI != MF_GATED || (NWC % 2 == 0 && (NT / 8) * (NWC / 2) == BN / 2),
                 "gate rows and up rows must fall to different loads of a thread");
   unsigned aoff[NA], woff[NWC];
-  int arow_s[NA], wrow_s[NWC];
+  int arow_s[NA], wrow_s[NWC], wcol_s[NWC];
   const int scol = (tid & 7) * 8;
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
@@ -84,12 +87,33 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   }
 #pragma unroll
   for (int i = 0; i < NWC; ++i) {
-    const int r = (tid + NT * i) >> 3;
+    int r = (tid + NT * i) >> 3, c = tid & 7;
+    if (WT) {
+      // Which 16 bytes of the tile a thread brings is free (they go to their own place in shared memory). In a copy's
+      // order 8 rows of a strip at one block of 8 k are a 128-byte line, and the lines of a strip's k-step lie side by
+      // side: a wave that took them in order would ask one small region of memory for all its 8 lines, where rows of
+      // the stored order lie far apart (the products of 2,048 rows were 13 to 20% slower that way). So a wave takes
+      // the same line of 8 different strips: lane l the row l % 8 of strip l / 8 of its group.
+      const int idx = (tid >> 6) * NWC + i, l = tid & 63;
+      if (WT == 1) {   // [strip of 16][k-step of 32][k block q][row][8]: 16 lines a strip and step of 64 k
+        const int combo = idx & 15;
+        r = ((idx >> 4) * 8 + (l >> 3)) * 16 + (combo & 1) * 8 + (l & 7);
+        c = (combo >> 3) * 4 + ((combo >> 1) & 3);
+      } else {         // [strip of 8][step of 64 k][k block q][half][row][8]: 8 lines a strip and step
+        const int combo = idx & 7;
+        r = ((idx >> 3) * 8 + (l >> 3)) * 8 + (l & 7);
+        c = (combo & 1) * 4 + (combo >> 1);
+      }
+    }
     wrow_s[i] = r;
+    wcol_s[i] = c * 8;
     const int rel = (EPI == MF_GATED && i >= NWC / 2) ? r - BN / 2 : r;
     const int row = min(n0 + rel, N - 1);
-    woff[i] = WT ? (unsigned)gl3_operand_offset(row + ((EPI == MF_GATED && i >= NWC / 2) ? N : 0), 0, w_steps)
-                 : (unsigned)(row - n0) * (unsigned)ldw;
+    const int wrow = row + ((EPI == MF_GATED && i >= NWC / 2) ? N : 0);
+    // (WT: K is a multiple of 64, so a thread's column inside a k-step of 64 is at the same place of every step)
+    woff[i] = WT == 1   ? (unsigned)gl3_operand_offset(w_pos ? w_pos[wrow] : wrow, c * 8, w_steps)
+              : WT == 2 ? (unsigned)gl3_packed_offset(wrow, c * 8, w_steps)
+                        : (unsigned)(row - n0) * (unsigned)ldw;
   }
   // K in slices (blockIdx.y): slice 0 ends in the epilogue proper, the others store their sums
   // as floats into P[slice - 1], for the reader to add up in slice order
@@ -106,11 +130,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
     const bf16_t* ak = a_tile + kf;
 #pragma unroll
     for (int i = 0; i < NA; ++i) ra[i] = *(const bf16x8*)(ak + (aoff[i] + col));
-    if (WT) {   // column kf + col of the row lies at its place inside the strip
-      const unsigned kc = (unsigned)kf + col;
-      const unsigned wcol = ((kc >> 5) << 9) + (((kc & 31u) >> 3) << 7);
+    if (WT) {
+      // a k-step of 64 lies 2 KB (the operands' order: two k-steps of 32) or 1 KB (the packed strips of 8) further in
+      // every strip: the same step for all threads, whose offsets stay what they are
+      const bf16_t* wk = w_tile[0] + (long)(min(k0, K - 64) >> 6) * (WT == 1 ? 1024 : 512);   // (the step after the last reads the last again)
 #pragma unroll
-      for (int i = 0; i < NWC; ++i) rw[i] = *(const bf16x8*)(w_tile[0] + (woff[i] + wcol));
+      for (int i = 0; i < NWC; ++i) rw[i] = *(const bf16x8*)(wk + woff[i]);
     } else {
 #pragma unroll
       for (int i = 0; i < NWC; ++i) {
@@ -139,12 +164,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
 #pragma unroll
       for (int i = 0; i < NA; ++i) *(bf16x8*)&As[buf][arow_s[i]][scol] = ra[i];
 #pragma unroll
-      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[buf][wrow_s[i]][scol] = rw[i];
+      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[buf][wrow_s[i]][WT ? wcol_s[i] : scol] = rw[i];
     } else {
 #pragma unroll
       for (int i = 0; i < NA; ++i) *(bf16x8*)&As[buf][arow_s[i]][scol] = r_ok ? ra[i] : zero;
 #pragma unroll
-      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[buf][wrow_s[i]][scol] = r_ok ? rw[i] : zero;
+      for (int i = 0; i < NWC; ++i) *(bf16x8*)&Ws[buf][wrow_s[i]][WT ? wcol_s[i] : scol] = r_ok ? rw[i] : zero;
     }
   };
   auto products = [&](int buf, int kk) {
@@ -225,10 +250,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
   else finish(std::true_type{});
 }
 
-template <int EPI, typename TC, int TM, int WM, int WN, bool WT = false>
+template <int EPI, typename TC, int TM, int WM, int WN, int WT = 0>
 static int launch_shape(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
                         int slices, float* P, long p_stride, long ldp, const float* bias, int act, int w_steps,
-                        hipStream_t stream) {
+                        const int* w_pos, hipStream_t stream) {
   const int bm = 32 * TM * WM;
   const int ncols = (EPI == MF_GATED) ? 32 * WN : 64 * WN;
   const int tiles_n = (N + ncols - 1) / ncols;
@@ -243,43 +268,25 @@ static int launch_shape(const void* A, const void* W, void* C, int M, int N, int
   const int group_m = tiles_m < (bm == 256 ? 4 : 8) ? tiles_m : (bm == 256 ? 4 : 8);
   gemm_mfma_kernel<EPI, TC, TM, WM, WN, WT><<<dim3((unsigned)blocks, slices), dim3(64 * WM * WN), 0, stream>>>(
       (const bf16_t*)A, (const bf16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, tiles_m, tiles_n, group_m, k_per_slice, P,
-      p_stride, ldp, bias, act, w_steps);
+      p_stride, ldp, bias, act, w_steps, w_pos);
   GL3_LAUNCH_CHECK();
   return 0;
 }
 
-template <int EPI, typename TC>
-static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                       int slices, float* P, long p_stride, long ldp, const float* bias, int act, int shape, int w_steps,
-                       hipStream_t stream) {
-  if (w_steps) {
-    // W in the operands' order alone: the store epilogue (a head that is held once), tiles of 128 x 128 or 256 x 256
-    if constexpr (EPI == MF_STORE) {
-      const long small = (long)((M + 127) / 128) * ((N + 127) / 128);
-      if (shape == 2 || (shape == 0 && small > 1024))
-        return launch_shape<EPI, TC, 2, 4, 4, true>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
-      return launch_shape<EPI, TC, 1, 4, 2, true>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
-    } else {
-      GL3_REQUIRE(false, "gl3_gemm_mfma: W in the operands' order alone is read by the store epilogue only (epilogue %d)", EPI);
-    }
-  }
-  if (shape == 1) return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
-  if (shape == 2) return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
-  if (shape == 3) return launch_shape<EPI, TC, 4, 2, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
-  if (shape == 4) return launch_shape<EPI, TC, 2, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
-  if (shape == 5) return launch_shape<EPI, TC, 1, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
-  // 256 x 256 tiles of sixteen waves, one block a CU, have half the operand traffic per product, and
-  // that traffic is what bounds the large products; of the 128 x 128 tiles of eight waves two fit a CU and
-  // overlap each other's waits. A step of 64 columns takes a chip full of the large tiles 1.7 us and a chip
-  // full of the small ones (twice as many blocks, a quarter of the work each) 1.05 us, and the blocks need
-  // rounds on the chip: the tile whose rounds take less time is chosen (240 large tiles are one round
-  // where 960 small ones are two; 276 large ones are two where 1,104 small ones are three).
-  // A third tile, 128 rows x 256 of sixteen waves of 32 x 64, is for the products in between: more tiles of 128 x 128
-  // than one for every CU, but not enough work to fill the chip with the large tiles (2,048 rows of the 1B layers'
-  // QKV product, 384 tiles of 128 x 128 or 192 of 128 x 256: 45 -> 40 us); a step of it takes a full chip about 0.95 us.
-  // Tiles of 128 x 128 that are at most one a CU run faster than two that share one (0.8 of the time a step).
-  const long small_n = (EPI == MF_GATED) ? (N + 63) / 64 : (N + 127) / 128;
-  const long big_n = (EPI == MF_GATED) ? (N + 127) / 128 : (N + 255) / 256;
+// The tile the library takes where the caller names none: 1 (128 x 128), 2 (256 x 256) or 5 (128 rows x 256).
+// 256 x 256 tiles of sixteen waves, one block a CU, have half the operand traffic per product, and
+// that traffic is what bounds the large products; of the 128 x 128 tiles of eight waves two fit a CU and
+// overlap each other's waits. A step of 64 columns takes a chip full of the large tiles 1.7 us and a chip
+// full of the small ones (twice as many blocks, a quarter of the work each) 1.05 us, and the blocks need
+// rounds on the chip: the tile whose rounds take less time is chosen (240 large tiles are one round
+// where 960 small ones are two; 276 large ones are two where 1,104 small ones are three).
+// A third tile, 128 rows x 256 of sixteen waves of 32 x 64, is for the products in between: more tiles of 128 x 128
+// than one for every CU, but not enough work to fill the chip with the large tiles (2,048 rows of the 1B layers'
+// QKV product, 384 tiles of 128 x 128 or 192 of 128 x 256: 45 -> 40 us); a step of it takes a full chip about 0.95 us.
+// Tiles of 128 x 128 that are at most one a CU run faster than two that share one (0.8 of the time a step).
+static int choose_shape(int M, int N, int slices, bool gated) {
+  const long small_n = gated ? (N + 63) / 64 : (N + 127) / 128;
+  const long big_n = gated ? (N + 127) / 128 : (N + 255) / 256;
   const long small_tiles = (long)((M + 127) / 128) * small_n * slices, wide_tiles = (long)((M + 127) / 128) * big_n * slices;
   const long big_tiles = (long)((M + 255) / 256) * big_n * slices;
   // rounds on the chip, in thousandths: whole rounds, and a last, partly empty one that costs half a round and
@@ -287,11 +294,37 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
   auto rounds = [](long tiles, long places) { return tiles / places * 1000 + (tiles % places ? 500 + tiles % places * 500 / places : 0); };
   const long small_cost = rounds(small_tiles, 512) * (small_tiles <= 256 ? 84 : 105), big_cost = rounds(big_tiles, 256) * 170;
   const long wide_cost = rounds(wide_tiles, 256) * (wide_tiles <= 128 ? 119 : 95);
-  if (wide_cost < small_cost && wide_cost < big_cost && slices == 1)
-    return launch_shape<EPI, TC, 1, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
-  if (big_cost < small_cost)
-    return launch_shape<EPI, TC, 2, 4, 4>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
-  return launch_shape<EPI, TC, 1, 4, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, stream);
+  if (wide_cost < small_cost && wide_cost < big_cost && slices == 1) return 5;
+  return big_cost < small_cost ? 2 : 1;
+}
+
+template <int EPI, typename TC>
+static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
+                       int slices, float* P, long p_stride, long ldp, const float* bias, int act, int shape, int w_order,
+                       const int* w_pos, hipStream_t stream) {
+  const int w_steps = w_order == 1 ? (K + 31) / 32 : w_order == 2 ? (K + 63) / 64 : 0;
+  if (shape == 0) shape = choose_shape(M, N, slices, EPI == MF_GATED);
+#define MF_ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, w_pos, stream
+  if (w_order) {
+    // W is one of its copies in the matrix cores' order (a weight that is held once): the store and add epilogues,
+    // the three tiles that the library chooses between
+    if constexpr (EPI != MF_GATED) {
+      GL3_REQUIRE(shape == 1 || shape == 2 || shape == 5, "gl3_gemm_mfma: tile shape %d does not read W in a copy's order", shape);
+      if (w_order == 1)
+        return shape == 1 ? launch_shape<EPI, TC, 1, 4, 2, 1>(MF_ARGS)
+               : shape == 2 ? launch_shape<EPI, TC, 2, 4, 4, 1>(MF_ARGS) : launch_shape<EPI, TC, 1, 4, 4, 1>(MF_ARGS);
+      return shape == 1 ? launch_shape<EPI, TC, 1, 4, 2, 2>(MF_ARGS)
+             : shape == 2 ? launch_shape<EPI, TC, 2, 4, 4, 2>(MF_ARGS) : launch_shape<EPI, TC, 1, 4, 4, 2>(MF_ARGS);
+    } else {
+      GL3_REQUIRE(false, "gl3_gemm_mfma: W in a copy's order alone is not read by the gated epilogue (order %d)", w_order);
+    }
+  }
+  if (shape == 1) return launch_shape<EPI, TC, 1, 4, 2>(MF_ARGS);
+  if (shape == 2) return launch_shape<EPI, TC, 2, 4, 4>(MF_ARGS);
+  if (shape == 3) return launch_shape<EPI, TC, 4, 2, 4>(MF_ARGS);
+  if (shape == 4) return launch_shape<EPI, TC, 2, 4, 2>(MF_ARGS);
+  return launch_shape<EPI, TC, 1, 4, 4>(MF_ARGS);
+#undef MF_ARGS
 }
 
 // N counts output columns: for the gated epilogue W has 2N rows (gate, then up).
@@ -302,10 +335,10 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
 // shape: 0 lets the library choose the tile; 1: 128 x 128, eight waves; 2: 256 x 256, sixteen waves of
 // 64 x 64; 3: 256 x 256, eight waves of 128 x 64; 4: 256 rows x 128, eight waves of 64 x 64; 5: 128 rows x 256,
 // sixteen waves of 32 x 64.
-// w_steps: 0, or W is kept in the matrix operands' order alone (lib.tile_weight) with that many k-steps a strip.
+// w_order, w_pos: how W lies (see below): as stored, or one of its copies in the matrix cores' order alone.
 extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda, long ldw,
                              long ldc, int epilogue, int slices, float* P, long p_stride, long ldp, const float* bias,
-                             int act, int shape, int w_steps, hipStream_t stream) {
+                             int act, int shape, int w_order, const int* w_pos, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   GL3_REQUIRE(A && W && C && M > 0 && N > 0 && K > 0, "gl3_gemm_mfma: bad arguments (M=%d N=%d K=%d)", M, N, K);
   GL3_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gl3_gemm_mfma: K=%d, lda=%ld, ldw=%ld must be multiples of 8",
@@ -324,11 +357,15 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
   GL3_REQUIRE(!bias || slices == 1, "gl3_gemm_mfma: a bias goes with one slice of K");
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_mfma: unknown activation %d", act);
   GL3_REQUIRE(shape >= 0 && shape <= 5, "gl3_gemm_mfma: unknown tile shape %d", shape);
-  // w_steps > 0: W is kept in the matrix operands' order alone, w_steps k-steps of 32 a strip of 16 rows
-  GL3_REQUIRE(w_steps == 0 || (w_steps * 32 >= K && (epilogue == MF_GATED ? 2L * N : (long)N) % 16 == 0 &&
-                               (epilogue == MF_GATED ? 2L * N : (long)N) * w_steps * 32 < (1L << 32)),
-              "gl3_gemm_mfma: W in the operands' order with %d k-steps for K=%d, N=%d", w_steps, K, N);
-#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, shape, w_steps, stream
+  // w_order: 0: W holds the rows as stored. 1: W is the copy in the matrix operands' order (lib.tile_weight), w_pos (may be
+  // null) naming each row's place in it. 2: the copy in packed strips of 8 rows (lib.tile_weight8).
+  {
+    const long w_rows = epilogue == MF_GATED ? 2L * N : (long)N;
+    GL3_REQUIRE(w_order >= 0 && w_order <= 2 && (w_order == 0 || (K % 64 == 0 && (long)w_rows * K < (1L << 32))) &&
+                    (w_order != 1 || w_rows % 16 == 0) && (w_order != 2 || w_rows % 8 == 0) && (w_order == 1 || !w_pos),
+                "gl3_gemm_mfma: W in order %d with K=%d (a copy's order is read over whole steps of 64), N=%d", w_order, K, N);
+  }
+#define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, shape, w_order, w_pos, stream
   if (c_dtype == GL3_F32) {
     if (epilogue == MF_STORE) return launch_mfma<MF_STORE, float>(ARGS);
     if (epilogue == MF_ADD) return launch_mfma<MF_ADD, float>(ARGS);

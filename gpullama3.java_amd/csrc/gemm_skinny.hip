@@ -972,7 +972,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
                                                                    const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                    int M, int N, int K, long lda, long ldw, long ldc,
                                                                    long slice_stride, int pairs_per_slice, SkRope rp,
-                                                                   SkNext nx, SkNorm nrm) {
+                                                                   SkNext nx, SkNorm nrm, int wl) {
+  // wl: how W lies. 0: rows as they are stored. 1: the matrix operands' order alone, [strip of 16 rows][k-step of 32]
+  // [lane][8] (lib.tile_weight; for the stacked q, k, v rows the strips hold the rows that sk_strip_row names).
+  // 2: the packed strips of 8 rows, [strip of 8][step of 64 k][lane][8] (lib.tile_weight8). In both a wave's load
+  // is 1 KB of consecutive memory (a k-step of a strip, or 64 k of 8 rows), and its 16-byte pieces go to the same
+  // places of the staged tile as the stored order's.
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   constexpr int NWT = NS * NG;        // tiles of W a pair of k-steps
   constexpr int NT = NWT + MT;        // tiles a wave stages for a pair of k-steps: 16 rows x 128 bytes each
@@ -995,12 +1000,26 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   const int line = r < 8 ? r : 8 + ((r + 1) & 7);
   const int get0 = line * 128 + ((q ^ (r & 7)) * 16);
   const int get1 = line * 128 + (((4 + q) ^ (r & 7)) * 16);
+  // where the lane's two loads of a tile of W go: (row, 16-byte piece) is (l8, c8) and (8 + l8, c8) for stored rows,
+  // (r, q) and (r, 4 + q) for a k-step of the operands' order each, (lane % 8 [+ 8], 4 * (lane / 8 % 2) + q) for the
+  // packed strips of 8
+  int putw0 = put0, putw1 = put1;
+  if (wl == 1) {
+    putw0 = get0;
+    putw1 = get1;
+  } else if (wl == 2) {
+    const int r8 = lane & 7, c = 4 * ((lane >> 3) & 1) + q;
+    putw0 = r8 * 128 + ((c ^ r8) * 16);
+    putw1 = (8 + ((r8 + 1) & 7)) * 128 + ((c ^ r8) * 16);
+  }
 
   // Both operands are read through buffer descriptors: a lane whose row or k does not exist gives
   // an offset beyond the buffer and gets zeros without a branch around the load, so every wave issues
   // the same loads in the same order and can wait for exactly the ones it needs.
-  const __amdgpu_buffer_rsrc_t w_buf =
-      __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)((((long)NG * N - 1) * ldw + K) * 2), 0x00020000);
+  const unsigned strip_bytes = wl == 1 ? (unsigned)((K + 31) >> 5) << 10 : (unsigned)((K + 63) >> 6) << 10;   // (wl 1, 2)
+  const long w_bytes = wl == 0 ? (((long)NG * N - 1) * ldw + K) * 2
+                       : wl == 1 ? (long)NG * (N >> 4) * strip_bytes : (long)(N >> 3) * strip_bytes;
+  const __amdgpu_buffer_rsrc_t w_buf = __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)w_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t a_buf =
       __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)((((long)M - 1) * lda + K) * 2), 0x00020000);
   constexpr unsigned NOWHERE = SK_NOWHERE;   // beyond any buffer the entry point lets in
@@ -1011,10 +1030,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   for (int g = 0; g < NS; ++g)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int wr = sk_strip_row<EPI>(min(strip0 + g, n_strips - 1), 8 * j + l8, N, rp, hd[g], sub[g], rotated[g]);
+      const int strip_g = min(strip0 + g, n_strips - 1);
+      const int wr = sk_strip_row<EPI>(strip_g, 8 * j + l8, N, rp, hd[g], sub[g], rotated[g]);
 #pragma unroll
       for (int h = 0; h < NG; ++h)   // (32-bit: the entry point lets in operands below 2 GiB only)
-        wo[g * NG + h][j] = ((unsigned)(wr + h * N) * (unsigned)ldw + (unsigned)c8 * 8u) * 2u;
+        wo[g * NG + h][j] = wl == 0   ? ((unsigned)(wr + h * N) * (unsigned)ldw + (unsigned)c8 * 8u) * 2u
+                            : wl == 1 ? (unsigned)(strip_g + h * (N >> 4)) * strip_bytes + (unsigned)j * 1024u + (unsigned)lane * 16u
+                                      : (unsigned)(2 * strip_g + j) * strip_bytes + (unsigned)lane * 16u;
     }
   unsigned xo[MT][2];
 #pragma unroll
@@ -1067,12 +1089,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
     return i < n_it ? p_begin + wave + NW * (j < n_it ? j : j - n_it) : p_end;
   };
   bf16x8 held[NT][2];
+  const unsigned w_pair = wl == 0 ? 128u : wl == 1 ? 2048u : 1024u;   // bytes from one pair of k-steps to the next
+  const int k_steps = (K + 31) >> 5;
   auto ask = [&](int p) {
     const unsigned k2 = (p < p_end && p * 64 + c8 * 8 < K) ? (unsigned)p * 128u : NOWHERE;   // (K is a multiple of 8)
+    // (the copies are padded with zeros to whole steps; the operands' order may end after a pair's first k-step)
+    const unsigned kw0 = wl == 0 ? k2 : p < p_end ? (unsigned)p * w_pair : NOWHERE;
+    const unsigned kw1 = (wl == 1 && 2 * p + 1 >= k_steps) ? NOWHERE : kw0;
 #pragma unroll
-    for (int t = 0; t < NWT; ++t)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) held[t][j] = sk_ld_b128(w_buf, wo[t][j] + k2);
+    for (int t = 0; t < NWT; ++t) {
+      held[t][0] = sk_ld_b128(w_buf, wo[t][0] + kw0);   // (offsets are below 2^31: with NOWHERE added they are beyond any buffer)
+      held[t][1] = sk_ld_b128(w_buf, wo[t][1] + kw1);
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -1102,8 +1130,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   for (int i = 0; i < n_it; ++i) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      *(bf16x8*)(stage + t * 2048 + put0) = held[t][0];
-      *(bf16x8*)(stage + t * 2048 + put1) = held[t][1];
+      *(bf16x8*)(stage + t * 2048 + (t < NWT ? putw0 : put0)) = held[t][0];
+      *(bf16x8*)(stage + t * 2048 + (t < NWT ? putw1 : put1)) = held[t][1];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -1180,6 +1208,7 @@ struct SkCall {
   const void* Wt = nullptr;   // W in the operands' order (the resident kernel reads it where it is given)
   const void* Wt8 = nullptr;  // W in the order of the packed tiles of strips of 8 rows
   int a_packed = 0;           // the rows of A lie in the packed tiles' order (strips of 8 rows, M <= 8 only)
+  int wl = 0;                 // (kernel of whole lines) W points at: 0 the stored rows, 1 the operands' order, 2 the packed strips of 8
 };
 
 // Blocks of the resident kernel: every strip its own block while that still leaves CUs idle, else
@@ -1388,7 +1417,7 @@ static int launch_wide(const SkCall& a, int slices, long slice_stride) {
   gemm_skinny_wide_kernel<MT, NS, NW, EPI, TC, XNORM>
       <<<dim3((n_strips + NS - 1) / NS, slices), dim3(NW * 64), 0, a.stream>>>(
           (const bf16_t*)a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, slice_stride, per_slice,
-          a.rp, a.nx, a.nrm);
+          a.rp, a.nx, a.nrm, a.wl);
   GL3_LAUNCH_CHECK();
   return 0;
 }
@@ -1430,9 +1459,17 @@ static int wide_strips(int N, int slices, int epilogue) {
 extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, long lda,
                                     long ldw, long ldc, int epilogue, int slices, long slice_stride,
                                     int strips_per_block, const float* bias, int act, const float* ssq, int n_partials,
-                                    float eps, int pack_out, hipStream_t stream) {
+                                    float eps, int pack_out, int w_order, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   if (check_common("gl3_gemm_skinny_wide", A, W, C, M, N, K, lda, ldw, 0)) return -1;
+  // w_order: 0: W holds the rows as they are stored. 1: W is the copy in the matrix operands' order (lib.tile_weight,
+  // rows in order; gated: the gate strips, then the up strips). 2: the copy in packed strips of 8 rows (lib.tile_weight8).
+  {
+    const long w_rows = epilogue == SK_GATED ? 2L * N : N;
+    GL3_REQUIRE(w_order >= 0 && w_order <= 2 && (w_order != 1 || (N % 16 == 0 && w_rows * ((K + 31) / 32 * 64) < (1L << 31))) &&
+                    (w_order != 2 || (N % 8 == 0 && epilogue != SK_GATED && (long)N * ((K + 63) / 64 * 128) < (1L << 31))),
+                "gl3_gemm_skinny_wide: W in order %d with N=%d, K=%d, epilogue %d", w_order, N, K, epilogue);
+  }
   GL3_REQUIRE(ssq || M > 16 || (M > 8 && epilogue == SK_STORE && c_dtype == GL3_F32),
               "gl3_gemm_skinny_wide: M=%d; up to 16 rows are gl3_gemm_skinny's (but 9 to 16 with a float output stored)", M);
   GL3_REQUIRE(!ssq || (M <= 16 && epilogue == SK_GATED && c_dtype == GL3_BF16 && slices == 1 && n_partials > 0),
@@ -1460,6 +1497,7 @@ extern "C" int gl3_gemm_skinny_wide(const void* A, const void* W, void* C, int c
   GL3_REQUIRE(act == GL3_ACT_SILU || act == GL3_ACT_GELU_TANH, "gl3_gemm_skinny_wide: unknown activation %d", act);
   SkCall a = {A, W, C, M, N, K, lda, ldw, ldc, SkNorm{ssq, n_partials, eps, nullptr}, nullptr, SkRope{}, stream, false};
   a.nx = SkNext{nullptr, nullptr, 0, bias, act, pack_out};
+  a.wl = w_order;
   if (ssq)
     return strips_per_block == big ? launch_wide<1, 2, SK_GATED, bf16_t, true>(a, 1, 0)
                                    : launch_wide<1, 1, SK_GATED, bf16_t, true>(a, 1, 0);
@@ -1517,7 +1555,8 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
                                   const int* seq_of_token, const int* block_table, int table_stride,
                                   const float* cos_tab, const float* sin_tab, void* k_cache, void* v_cache,
                                   int n_heads, int n_kv, int head_dim, int adjacent, int page_size, int waves,
-                                  const void* w_tiled, const int* token_pages, const float* token_rot, hipStream_t stream) {
+                                  const void* w_tiled, const int* token_pages, const float* token_rot, int w_once,
+                                  hipStream_t stream) {
   if (M == 0) return 0;
   const int N = (n_heads + 2 * n_kv) * head_dim;
   if (check_common("gl3_qkv_rope_cache", a_rows, Wqkv, q_out, M, N, K, lda, ldw, waves)) return -1;
@@ -1537,6 +1576,11 @@ extern "C" int gl3_qkv_rope_cache(const void* a_rows, const float* ssq, int n_pa
   SkCall a = {a_rows, Wqkv, q_out, M, N, K, lda, ldw, ldq, nrm, nullptr, rp, stream, waves == 0};
   GL3_REQUIRE(!w_tiled || (uintptr_t)w_tiled % 16 == 0, "gl3_qkv_rope_cache: the copy of W must be 16-byte aligned");
   a.Wt = w_tiled;   // (its strips hold the rows that sk_strip_row names: for half-split pairing 8 rows and the 8 half a head further)
+  // w_once: the stored order is gone, Wqkv is that copy: the kernels of few rows read it as before, the kernel of
+  // whole lines reads it in its own order
+  GL3_REQUIRE(!w_once || (w_tiled && N % 16 == 0 && (long)N * ((K + 31) / 32 * 64) < (1L << 31)),
+              "gl3_qkv_rope_cache: weights in the operands' order alone need that copy (N=%d, K=%d)", N, K);
+  if (w_once) { a.W = w_tiled; a.wl = 1; }
   if (!ssq && waves == 0 && M > 16 && wide_addressable(M, N, K, lda, ldw)) {
     // many rows, read in whole lines: two strips a block, so that the rows are read half as often, where one
     // strip a block would be more blocks than CUs (N = 3,072, K = 2,048, 64 rows: 10.0 us with two, 8.9 us with

@@ -55,7 +55,7 @@ def _declare(lib):
         "gl3_gather_rows": [P, P, P, I, I, I, P],
         "gl3_add_slices_rmsnorm": [P, P, P, I, L, L, P, I, P, I, I, I, F, P],
         "gl3_rope_cache_write": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
-        "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, I, P],
+        "gl3_gemm_generic": [P, I, P, I, P, I, I, I, I, L, L, L, I, P, I, I, P, P],
         "gl3_attention_generic": [P, L, P, P, I, P, P, P, I, P, L, I, I, I, I, I, I, F, P],
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_sample_work_floats": [I, I],
@@ -63,11 +63,11 @@ def _declare(lib):
         "gl3_argmax_static": [P, L, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
         "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P, I, P],
-        "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P, I, F, I, P],
+        "gl3_gemm_skinny_wide": [P, P, P, I, I, I, I, L, L, L, I, I, L, I, P, I, P, I, F, I, I, P],
         "gl3_gemm_skinny_norm": [P, P, P, I, F, P, P, I, I, I, I, L, L, L, I, I, P, I, P, I, P],
-        "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
+        "gl3_qkv_rope_cache": [P, P, I, F, P, P, L, I, I, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, P, P, P, I, P],
         "gl3_token_facts": [P, P, P, I, I, P, P, I, P, P, P, I, P],
-        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, I, P],
+        "gl3_gemm_mfma": [P, P, P, I, I, I, I, L, L, L, I, I, P, L, L, P, I, I, I, P, P],
         "gl3_attention_decode_supports": [I, I],
         "gl3_attention_prefill_supports": [I, I],
         "gl3_attention_prefill": [P, L, P, P, P, P, P, P, I, P, L, I, I, I, I, I, I, I, F, I, P],
@@ -120,19 +120,25 @@ def _dev(t, name, dtype=None, contiguous=True):
 
 
 def held_once(w):
-    """Whether the matrix is kept in the matrix operands' order ALONE (``hold_once``): its memory is its copy
-    ``w.tiled``, and only what reads that order may touch it."""
+    """Whether the matrix is kept in the matrix cores' order ALONE (``hold_once``): its memory is one of its
+    copies (``w.tiled``, ``w.tiled8``), and only what reads such an order may touch it."""
     return getattr(w, "operand_order_only", False)
 
 
-def _operand_steps(w):
-    """The k-steps of 32 a strip of a matrix that is held once (what the kernels that read both orders take), else 0."""
-    return -(-w.shape[1] // 32) if held_once(w) else 0
+def _w_order(w):
+    """How a weight lies, for the kernels that read any order: (0, the stored rows, no table), (1, the copy in
+    the operands' order, each row's place in it or nothing), (2, the copy in packed strips of 8 rows, nothing)."""
+    if not held_once(w):
+        return 0, _ptr(w), c_void_p(0)
+    t = getattr(w, "tiled", None)
+    if t is not None:
+        return 1, _ptr(t), _ptr(getattr(t, "row_pos", None))
+    return 2, _ptr(w.tiled8), c_void_p(0)
 
 
 def _stored(w, who):
     if held_once(w):
-        raise KernelError(f"{who}: the weight is kept in the matrix operands' order alone, which this kernel does not read")
+        raise KernelError(f"{who}: the weight is kept in the matrix cores' order alone, which this kernel does not read")
     return w
 
 
@@ -206,6 +212,16 @@ def softcap_(t, cap):
     _check(library().gl3_softcap_f32(_ptr(t), float(cap), t.numel(), _stream()), "softcap_f32")
 
 
+def _table_steps(table):
+    """0, or the k-steps of 32 a strip of a table that is held once (in the operands' order, rows in order)."""
+    if not held_once(table):
+        return 0
+    t = getattr(table, "tiled", None)
+    if t is None or getattr(t, "row_pos", None) is not None or t.data_ptr() != table.data_ptr():
+        raise KernelError("embed: a table that is held once must be its copy in the operands' order, rows in order")
+    return -(-table.shape[1] // 32)
+
+
 def embed(table, ids, out, ssq=None, next_weight=None, xg=None, scale=1.0, pos_table=None, positions=None):
     """out[t] = scale * table[ids[t]] (+ pos_table[positions[t]]) as float32. The caller has checked
     ids < rows and positions < rows of ``pos_table``. ``ssq`` (at least 64 floats, at most 64 tokens)
@@ -228,7 +244,7 @@ def embed(table, ids, out, ssq=None, next_weight=None, xg=None, scale=1.0, pos_t
             raise KernelError(f"embed: table of positions {tuple(pos_table.shape)} for rows of {d}")
     _check(library().gl3_embed(_ptr(table), _code(table, "table"), _ptr(ids), _ptr(out), T, d, _ptr(ssq),
                                _ptr(next_weight), _ptr(xg), float(scale), _ptr(pos_table),
-                               _ptr(positions) if pos_table is not None else c_void_p(0), _operand_steps(table),
+                               _ptr(positions) if pos_table is not None else c_void_p(0), _table_steps(table),
                                _stream()), "embed")
 
 
@@ -327,10 +343,10 @@ def gemm_generic(a, w, out, epilogue=EPI_STORE, bias=None, act="silu"):
     rows = 2 * N if epilogue == EPI_GATED else N
     if w.shape != (rows, K) or out.shape[0] != M:
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
-    _check(library().gl3_gemm_generic(_ptr(a), _code(a, "a"), _ptr(w), _code(w, "w"), _ptr(out), _code(out, "out"),
+    order, wp, pos = _w_order(w)
+    _check(library().gl3_gemm_generic(_ptr(a), _code(a, "a"), wp, _code(w, "w"), _ptr(out), _code(out, "out"),
                                       M, N, K, a.stride(0), w.stride(0), out.stride(0), epilogue,
-                                      _bias(bias, rows, "gemm_generic"), _act(act, "gemm_generic"), _operand_steps(w),
-                                      _stream()),
+                                      _bias(bias, rows, "gemm_generic"), _act(act, "gemm_generic"), order, pos, _stream()),
            "gemm_generic")
 
 
@@ -459,8 +475,10 @@ def gemm_skinny(a, w, out, epilogue=EPI_STORE, waves=0, ssq_out=None, strip_rows
     _check_next(next_weight, xg, M, N, "gemm_skinny")
     if xg is not None and ssq_out is None:
         raise KernelError("gemm_skinny: the next norm's rows come with the sums of squares")
-    if held_once(w) and (strip_rows != 16 or not _tiled(w, rows, K, n_out=N).value):
-        raise KernelError("gemm_skinny: a weight kept in the operands' order alone is read in strips of 16 rows through its copy")
+    if held_once(w) and not (skinny_takes(w, M, strip_rows) and (strip_rows == 8 or _tiled(w, rows, K, n_out=N).value)
+                             and a.stride(0) < 2 ** 24 and K < 2 ** 24):
+        raise KernelError("gemm_skinny: a weight kept in the matrix cores' order alone is read through the copy whose strips "
+                          f"the call names (strips of {strip_rows} rows, {M} rows of a)")
     _check(library().gl3_gemm_skinny(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                      out.stride(0), epilogue, waves, _ptr(ssq_out), strip_rows, _ptr(next_weight),
                                      _ptr(xg), xg.stride(0) if xg is not None else 0, _bias(bias, rows, "gemm_skinny"),
@@ -501,6 +519,10 @@ def tile_weight(w, qkv=None):
     wp[:, :K] = w[rows]
     t = wp.view(N // 16, 16, steps, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
     t.tiled_for = qkv
+    if not torch.equal(rows, torch.arange(N, device=rows.device)):
+        # the place of each stored row in the copy, for the kernels that read the copy row by row
+        t.row_pos = torch.empty(N, dtype=torch.int32, device=w.device)
+        t.row_pos[rows] = torch.arange(N, dtype=torch.int32, device=w.device)
     return t
 
 
@@ -519,25 +541,67 @@ def tile_weight8(w):
 
 
 def untile_weight(t, n_rows, K):
-    """The rows of a matrix out of its copy in the matrix operands' order (``tile_weight`` without a permutation
-    of the rows): a new tensor [n_rows, K] in the stored order."""
+    """The rows of a matrix out of its copy in the matrix operands' order (``tile_weight``): a new tensor
+    [n_rows, K] in the stored order."""
     steps = -(-K // 32)
-    return t.view(n_rows // 16, steps, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(n_rows, steps * 32)[:, :K].contiguous()
+    rows = t.view(n_rows // 16, steps, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(n_rows, steps * 32)[:, :K]
+    pos = getattr(t, "row_pos", None)
+    return (rows[pos.long()] if pos is not None else rows).contiguous()
+
+
+def untile_weight8(t, n_rows, K):
+    """The same out of the copy in packed strips of 8 rows (``tile_weight8``)."""
+    steps = -(-K // 64)
+    # [strip, step, q, half, row, element] -> [strip, row, step, half, q, element]
+    return t.view(n_rows // 8, steps, 4, 2, 8, 8).permute(0, 4, 1, 3, 2, 5).reshape(n_rows, steps * 64)[:, :K].contiguous()
+
+
+def stored_order(w):
+    """``w`` as the rows lie in the model's file: ``w`` itself, or (held once) rebuilt from a copy, a new tensor."""
+    if not held_once(w):
+        return w
+    t = getattr(w, "tiled", None)
+    return untile_weight(t, *w.shape) if t is not None else untile_weight8(w.tiled8, *w.shape)
+
+
+def can_hold_once(w):
+    """Whether one of the copies that ``w`` carries has exactly the matrix's elements, over whole steps of 64 k
+    (the tiled product's step), so that it can stand for the matrix."""
+    N, K = w.shape
+    t, t8 = getattr(w, "tiled", None), getattr(w, "tiled8", None)
+    return K % 64 == 0 and ((t is not None and N % 16 == 0 and t.numel() == N * K)
+                            or (t8 is not None and N % 8 == 0 and t8.numel() == N * K))
 
 
 def hold_once(w):
-    """``w`` (which carries ``w.tiled``, rows in order, K a multiple of 32) as a matrix that is kept in the
-    operands' order alone: a tensor of the same shape and dtype whose memory IS the copy. Whoever drops ``w``
-    then frees the stored order. The kernels that read both orders (the embedding, the generic and the tiled
-    product, and those of few rows that take ``w.tiled``) are told by ``held_once``; the others refuse it."""
-    t = getattr(w, "tiled", None)
+    """``w`` (which carries ``w.tiled`` and/or ``w.tiled8``, over whole steps of k) as a matrix that is kept in
+    the matrix cores' order alone: a tensor of the same shape and dtype whose memory IS a copy. Whoever drops
+    ``w`` then frees the stored order. The kernels that read any order (the embedding, the generic and the tiled
+    product, the kernel of whole lines, and those of few rows that take the copies anyway) are told by
+    ``held_once``; the others refuse it."""
+    if not can_hold_once(w):
+        raise KernelError(f"hold_once: {tuple(w.shape)} has no copy in the matrix cores' order that could stand for it")
     N, K = w.shape
-    if t is None or getattr(t, "tiled_for", None) is not None or K % 32 or N % 16 or t.numel() != N * K:
-        raise KernelError(f"hold_once: {tuple(w.shape)} has no copy in the operands' order that could stand for it")
-    alias = t.view(N, K)
-    alias.tiled = t
+    t, t8 = getattr(w, "tiled", None), getattr(w, "tiled8", None)
+    base = t if (t is not None and N % 16 == 0 and t.numel() == N * K) else t8
+    alias = base.view(N, K)
     alias.operand_order_only = True
+    if t is not None:
+        alias.tiled = t
+    if t8 is not None:
+        alias.tiled8 = t8
     return alias
+
+
+def skinny_takes(w, M, strip_rows, qkv=None):
+    """Whether the products of few rows can read ``w`` in strips of ``strip_rows``: always when the stored order
+    is there; a weight that is held once through the copy whose strips those are (rows in order, or for ``qkv``)."""
+    if not held_once(w):
+        return True
+    N, K = w.shape
+    if strip_rows == 8:
+        return M <= 8 and bool(_tiled8(w, N, K).value)
+    return bool(_tiled(w, N, K, qkv=qkv).value)
 
 
 def _tiled8(w, n_rows, K):
@@ -558,7 +622,8 @@ def _tiled(w, n_rows, K, qkv=None, n_out=None):
 
 
 def gemm_skinny_wide_fits(a, w, out, epilogue):
-    return 8 < a.shape[0] <= 64 and gemm_skinny_fits(a, w, out, epilogue) and not held_once(w)
+    return (8 < a.shape[0] <= 64 and gemm_skinny_fits(a, w, out, epilogue)
+            and not (held_once(w) and getattr(getattr(w, "tiled", None), "row_pos", None) is not None))
 
 
 def wide_slices(N, K):
@@ -572,8 +637,7 @@ def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="si
     """out (=, +=, gated) a @ w.T for 17 to 64 rows of ``a``. ``out`` with three axes [slices, M, N]
     (float32, store epilogue) takes the sums of one slice of K each: the caller adds them up; that form
     also takes 9 to 16 rows."""
-    _dev(a, "a", torch.bfloat16, contiguous=False); _dev(_stored(w, "gemm_skinny_wide"), "w", torch.bfloat16)
-    _dev(out, "out", contiguous=False)
+    _dev(a, "a", torch.bfloat16, contiguous=False); _dev(w, "w", torch.bfloat16); _dev(out, "out", contiguous=False)
     M, K = a.shape
     slices, slice_stride = 1, 0
     rows = out
@@ -584,10 +648,13 @@ def gemm_skinny_wide(a, w, out, epilogue=EPI_STORE, strips=0, bias=None, act="si
     if (w.shape != (wrows, K) or rows.shape[0] != M or rows.stride(1) != 1 or a.stride(1) != 1
             or not (16 < M <= 64 or (8 < M <= 16 and epilogue == EPI_STORE and out.dtype == torch.float32))):
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
-    _check(library().gl3_gemm_skinny_wide(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0),
+    order, wp, pos = _w_order(w)
+    if pos.value:
+        raise KernelError("gemm_skinny_wide: a copy whose strips hold the rows in another order is not read row by row")
+    _check(library().gl3_gemm_skinny_wide(_ptr(a), wp, _ptr(out), _code(out, "out"), M, N, K, a.stride(0),
                                           w.stride(0), rows.stride(0), epilogue, slices, slice_stride, strips,
                                           _bias(bias, wrows, "gemm_skinny_wide"), _act(act, "gemm_skinny_wide"),
-                                          None, 0, 0.0, 0, _stream()), "gemm_skinny_wide")
+                                          None, 0, 0.0, 0, order, _stream()), "gemm_skinny_wide")
 
 
 def _check_norm_args(xg, ssq, n_partials, K):
@@ -629,15 +696,18 @@ def gemm_skinny_norm(xg, ssq, n_partials, eps, w, out, epilogue=EPI_STORE, rows=
     wrows = 2 * N if epilogue == EPI_GATED else N
     if w.shape != (wrows, K) or out.shape[0] != M or out.stride(1) != 1 or M > 64:
         raise KernelError(f"gemm: rows {tuple(xg.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
-    if held_once(w) and (whole_lines or not _tiled(w, wrows, K, n_out=N).value):
-        raise KernelError("gemm_skinny_norm: a weight kept in the operands' order alone is read through its copy")
+    if held_once(w) and not whole_lines and not _tiled(w, wrows, K, n_out=N).value:
+        raise KernelError("gemm_skinny_norm: a weight kept in the matrix cores' order alone is read through its copy")
     if whole_lines:
         if epilogue != EPI_GATED or rows is not None or M > 16 or waves:
             raise KernelError("gemm_skinny_norm: whole lines go with the gated epilogue, at most 16 rows, all of them")
+        order, wp, pos = _w_order(w)
+        if pos.value or order == 2:
+            raise KernelError("gemm_skinny_norm: the gated product of whole lines reads stored rows or the operands' order")
         return _check(library().gl3_gemm_skinny_wide(
-            _ptr(xg), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, xg.stride(0), w.stride(0), out.stride(0), epilogue,
+            _ptr(xg), wp, _ptr(out), _code(out, "out"), M, N, K, xg.stride(0), w.stride(0), out.stride(0), epilogue,
             1, 0, 0, _bias(bias, wrows, "gemm_skinny_norm"), _act(act, "gemm_skinny_norm"), _ptr(ssq), n_partials,
-            float(eps), int(bool(pack_out)), _stream()), "gemm_skinny_wide")
+            float(eps), int(bool(pack_out)), order, _stream()), "gemm_skinny_wide")
     _check(library().gl3_gemm_skinny_norm(
         _ptr(xg), _ptr(rows), _ptr(ssq), n_partials, float(eps), _ptr(w), _ptr(out), _code(out, "out"), M, N, K,
         xg.stride(0), w.stride(0), out.stride(0), epilogue, waves, _bias(bias, wrows, "gemm_skinny_norm"),
@@ -688,7 +758,7 @@ def qkv_rope_cache(a, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_toke
     ``a`` holds the rows as they are; else ``a`` = bfloat16(norm weight * x) and the product is that
     of RMSNorm(x), the rows' sums of squares coming as partial sums. ``token_pages``, ``token_rot``: what
     ``token_facts`` made of the same positions, table and rotation (then the kernel does not look them up)."""
-    _dev(_stored(w_qkv, "qkv_rope_cache"), "w_qkv", torch.bfloat16); _dev(q_out, "q_out", torch.bfloat16, contiguous=False)
+    _dev(w_qkv, "w_qkv", torch.bfloat16); _dev(q_out, "q_out", torch.bfloat16, contiguous=False)
     K = w_qkv.shape[1]
     if ssq is None:
         _dev(a, "a", torch.bfloat16, contiguous=False)
@@ -719,12 +789,15 @@ def qkv_rope_cache(a, ssq, n_partials, eps, w_qkv, q_out, positions, seq_of_toke
                                                              or token_rot.shape != (T, head_dim) or not token_rot.is_cuda
                                                              or not token_rot.is_contiguous())):
             raise KernelError("qkv_rope_cache: a page per token, and with a rotation a row [head_dim] of cos and sin per token")
+    copy = _tiled(w_qkv, w_qkv.shape[0], K, qkv=(n_heads, n_kv, head_dim, cos is not None, bool(adjacent)))
+    if held_once(w_qkv) and not copy.value:
+        raise KernelError("qkv_rope_cache: weights kept in the operands' order alone need the copy made for this rotation")
     _check(library().gl3_qkv_rope_cache(
         _ptr(a), _ptr(ssq), n_partials, float(eps), _ptr(w_qkv), _ptr(q_out), q_out.stride(0), T, K, a.stride(0),
         w_qkv.stride(0), _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], _ptr(cos),
         _ptr(sin), _ptr(k_cache), _ptr(v_cache), n_heads, n_kv, head_dim, int(adjacent), page_size, waves,
-        _tiled(w_qkv, w_qkv.shape[0], K, qkv=(n_heads, n_kv, head_dim, cos is not None, bool(adjacent))),
-        _ptr(token_pages), _ptr(token_rot if token_pages is not None and cos is not None else None), _stream()),
+        copy, _ptr(token_pages), _ptr(token_rot if token_pages is not None and cos is not None else None),
+        int(held_once(w_qkv)), _stream()),
         "qkv_rope_cache")
 
 
@@ -808,10 +881,10 @@ def gemm_mfma(a, w, out, epilogue=EPI_STORE, more_slices=None, bias=None, act="s
     rows = 2 * N if epilogue == EPI_GATED else N
     if w.shape != (rows, K) or out.shape[0] != M:
         raise KernelError(f"gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}, epilogue {epilogue}")
-    _check(library().gl3_gemm_mfma(_ptr(a), _ptr(w), _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
+    order, wp, pos = _w_order(w)
+    _check(library().gl3_gemm_mfma(_ptr(a), wp, _ptr(out), _code(out, "out"), M, N, K, a.stride(0), w.stride(0),
                                    out.stride(0), epilogue, slices, _ptr(more_slices), p_stride, ldp,
-                                   _bias(bias, rows, "gemm_mfma"), _act(act, "gemm_mfma"), int(shape), _operand_steps(w),
-                                   _stream()),
+                                   _bias(bias, rows, "gemm_mfma"), _act(act, "gemm_mfma"), int(shape), order, pos, _stream()),
            "gemm_mfma")
 
 

@@ -78,8 +78,10 @@ class Engine:
 
     ``weight_copies``: a bfloat16 engine keeps, beside each matrix that decode steps read (QKV, output and down
     projection, the head, and the gate/up rows of small models), a copy in the order in which the matrix cores
-    take it, and the head (with a tied embedding) in that order alone: 2.5 -> 3.5 GB for the 1B shape, for 16%
-    more tokens a second at batch 8. False leaves the copies out; "both" keeps the stored order of every matrix too. ``without``: names of fast paths (``parts.ops.SWITCHES``) this engine does not use, for
+    take it, and lets the stored order of those go (the gate/up rows of large models, which no step reads in
+    another order, stay as stored; the output projection may keep two copies, in strips of 16 and of 8): 2.5 ->
+    2.6 GB for the 1B shape, for 16% more tokens a second at batch 8. False leaves the copies out; "both" keeps
+    the stored order of every matrix too (4.0 GB). ``without``: names of fast paths (``parts.ops.SWITCHES``) this engine does not use, for
     measurements and tests. ``max_graphs``: captured decode steps kept at a time; the least recently used
     one goes first."""
 
@@ -148,10 +150,10 @@ class Engine:
 
     def weights(self):
         """Stored name -> device tensor (stacked matrices appear as views under their stored names). A matrix that
-        the engine keeps in the matrix operands' order alone is put back into the stored order for the caller: a
+        the engine keeps in the matrix cores' order alone is put back into the stored order for the caller: a
         tensor of the caller's own, made at each call."""
-        from ..csrc import lib as K
-        return {name: K.untile_weight(w.tiled, *w.shape) if K.held_once(w) else w for name, w in self.model.weights.items()}
+        from ..parts import ops
+        return {name: ops.stored(w) for name, w in self.model.weights.items()}
 
     # ------------------------------------------------------------------ slots
     def take_slot(self):

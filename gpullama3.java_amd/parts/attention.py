@@ -14,6 +14,7 @@ import math
 import torch
 
 from ..cache import KVNeed
+from ..csrc import lib as K
 from ..weights.loader import TensorSpec
 from . import ops
 from .base import build_part, register_part
@@ -62,6 +63,16 @@ class GQAAttention:
         ops.for_few_rows(self.w_qkv, (self.H, self.Kh, self.hs, self.position is not None,
                                       bool(self.position is not None and self.position.adjacent)), without=without)
         self.w_o = ops.for_eight_rows(weights[n["o"]], without=without)
+        if getattr(self, "may_hold_once", False):
+            # the stored order is let go where a copy in the matrix cores' order can stand for the matrix; the stored
+            # names then name rows that are put together on request
+            if ops.can_hold_once(self.w_qkv, without):
+                self.w_qkv, self.w_q = K.hold_once(self.w_qkv), None
+                weights[n["q"]], weights[n["k"]], weights[n["v"]] = (
+                    ops.StoredRows(self, "w_qkv", 0, qn), ops.StoredRows(self, "w_qkv", qn, qn + kn),
+                    ops.StoredRows(self, "w_qkv", qn + kn, qn + 2 * kn))
+            if ops.can_hold_once(self.w_o, without):
+                self.w_o = weights[n["o"]] = K.hold_once(self.w_o)
         if self.biased:     # the epilogues read biases as float
             self.b_qkv = torch.cat([weights[n[k]].float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()
         if "o_bias" in n:

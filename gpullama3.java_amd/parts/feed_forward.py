@@ -8,6 +8,7 @@ from __future__ import annotations
 import torch
 
 from ..csrc.lib import ACTIVATIONS
+from ..csrc import lib as K
 from ..weights.loader import TensorSpec
 from . import ops
 from .base import register_part
@@ -47,6 +48,8 @@ class GatedFeedForward:
         without = getattr(self, "without", frozenset())      # the fast paths that the engine does without
         ops.for_gated(self.w_gate_up, without=without)
         self.w_down = ops.for_eight_rows(weights[n["down"]], without=without)
+        if getattr(self, "may_hold_once", False) and ops.can_hold_once(self.w_down, without):
+            self.w_down = weights[n["down"]] = K.hold_once(self.w_down)      # (the stored order is let go)
         if self.biased:     # the epilogues read biases as float
             self.b_gate_up = torch.cat([weights[n["gate_bias"]].float(), weights[n["up_bias"]].float()]).contiguous()
         if "down_bias" in n:

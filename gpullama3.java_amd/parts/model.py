@@ -58,9 +58,13 @@ class DecoderModel:
         self.without = ops.switches(without)
         self.blocks = [build_part("block", b, dtype=dtype, device=device) for b in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm, dtype=dtype) if spec.final_norm is not None else None
+        # (a layer whose queries read another entry's keys and values needs the q rows alone: then stacked rows keep
+        # their stored order)
+        may_hold_once = not any(r.reads is not None for r in spec.run_order)
         for part in [p for b in self.blocks for p in b.parts()] + [self.final_norm]:
             if part is not None:
                 part.without = self.without
+                part.may_hold_once = may_hold_once
         self.runs = []
         for e, r in enumerate(spec.run_order):
             if not 0 <= r.layer < len(self.blocks):

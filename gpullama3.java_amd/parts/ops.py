@@ -64,13 +64,31 @@ def for_few_rows(w, qkv=None, without=_NONE):
 
 
 def can_hold_once(w, without=_NONE):
-    """Whether a weight whose readers all take the matrix operands' order (the head: the embedding look-up of a
-    tied head, the products of few rows, the tiled product's store epilogue, the generic product) can be kept in
-    that order alone: it has the copy, rows in order, whole k-steps, and the engine has no fast path switched
-    off (a comparison wants both orders at hand; ``Engine(weight_copies="both")`` asks for exactly that)."""
-    t = getattr(w, "tiled", None)
-    return (not without and t is not None and getattr(t, "tiled_for", None) is None and w.shape[1] % 32 == 0
-            and w.shape[0] % 16 == 0 and t.numel() == w.numel())
+    """Whether a weight can be kept in the order of one of its copies alone (``lib.hold_once``): it carries a copy
+    over whole steps of k, and the engine has no fast path switched off (a comparison wants both orders at hand;
+    ``Engine(weight_copies="both")`` asks for exactly that). Every kernel that a step may take for such a weight
+    reads the copies' orders: the embedding look-up, the products of few rows (through the copy whose strips they
+    walk), the kernel of whole lines, the tiled product's store and add epilogues, the generic product."""
+    # (a weight with packed strips of 8 only: steps of 9 to 64 rows must find the kernel of whole lines, which takes
+    # it with K in slices; else they would fall back to the tiled product, which is right but slow for so few rows)
+    return (not without and K.can_hold_once(w)
+            and (getattr(w, "tiled", None) is not None or K.wide_slices(w.shape[0], w.shape[1]) >= 2))
+
+
+class StoredRows:
+    """Rows ``lo .. hi`` of a matrix that a part keeps in another order than the stored one, under the name the
+    model's file gives them: put together when somebody asks (``Engine.weights``)."""
+
+    def __init__(self, part, attribute, lo, hi):
+        self.part, self.attribute, self.lo, self.hi = part, attribute, lo, hi
+
+    def stored(self):
+        return K.stored_order(getattr(self.part, self.attribute))[self.lo:self.hi]
+
+
+def stored(w):
+    """What ``Engine.weights`` hands out for an entry of a model's weights: the tensor in the stored order."""
+    return w.stored() if isinstance(w, StoredRows) else K.stored_order(w)
 
 
 def for_gated(w, without=_NONE):
@@ -227,7 +245,8 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
         return
     if isinstance(a, Normed):
         if ("fused" not in disabled and w.dtype == torch.bfloat16 and K.gemm_skinny_norm_fits(a.xg, w, out, epilogue)
-                and a.xg.shape[0] <= 64 and not _streams_rows_for_many_strips(out.shape[0], w, epilogue)):
+                and a.xg.shape[0] <= 64 and not _streams_rows_for_many_strips(out.shape[0], w, epilogue)
+                and (_whole_lines(a, w, epilogue) or K.skinny_takes(w, out.shape[0], 16))):
             return K.gemm_skinny_norm(a.xg, a.ssq, a.n_partials, a.eps, w, out, epilogue, rows=a.rows, bias=bias, act=act,
                                       whole_lines=_whole_lines(a, w, epilogue))
         a = a.materialize()
@@ -235,7 +254,9 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
         chunks = row_chunks(a.shape[0], ctx)
         if (chunks and ctx is not None and getattr(ctx, "fuse", False) and not disabled & {"wide", "fused", "skinny"}
                 and K.gemm_skinny_fits(a[:1], w, out[:1], epilogue)
-                and not (epilogue == EPI_STORE and out.shape[1] >= 128 * 512)):     # (the head: the tiled kernel)
+                and not (epilogue == EPI_STORE and out.shape[1] >= 128 * 512)      # (the head: the tiled kernel)
+                and (K.skinny_takes(w, 64, 16) or (epilogue == EPI_ADD and bias is None
+                                                   and K.wide_slices(out.shape[1], a.shape[1]) >= 2))):
             return _linear_in_chunks(a, w, out, epilogue, ctx, chunks, bias, act)
         if (_streams_rows_for_many_strips(a.shape[0], w, epilogue) and "mfma" not in disabled
                 and K.gemm_mfma_fits(a, w, out, epilogue)):
@@ -243,9 +264,11 @@ def linear(a, w, out, epilogue=EPI_STORE, ctx=None, bias=None, act="silu", pack_
         if ("wide" not in disabled and (a.shape[0] > FUSE_ROWS or _long_k_of_9_to_16_rows(a, out, epilogue, bias, disabled))
                 and K.gemm_skinny_wide_fits(a, w, out, epilogue) and _linear_wide(a, w, out, epilogue, ctx, bias, act)):
             return
-        if "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
+        rows = K.skinny_strip_rows(a.shape[0], out.shape[1], a.shape[1], epilogue)
+        if not K.skinny_takes(w, a.shape[0], rows):      # (held once: through the copy it has, if it has one for these rows)
+            rows = 24 - rows if K.skinny_takes(w, a.shape[0], 24 - rows) and epilogue != EPI_GATED else 0
+        if rows and "skinny" not in disabled and K.gemm_skinny_fits(a, w, out, epilogue):
             N = out.shape[1]
-            rows = 16 if K.held_once(w) else K.skinny_strip_rows(a.shape[0], N, a.shape[1], epilogue)
             if (epilogue == EPI_ADD and ctx is not None and getattr(ctx, "fuse", False) and N % 16 == 0
                     and "fused" not in disabled and out.shape[0] == ctx.n_tokens <= FUSE_ROWS):
                 # the rows are complete after this product: leave what the norm that follows needs
@@ -398,6 +421,9 @@ def qkv_project(ctx, h, w_qkv, w_q, rotary, k_cache, v_cache, block_table, n_hea
         qkv = ctx.buffer("qkv", (T, (n_heads + 2 * n_kv) * head_dim), dtype)
         linear(h, w_qkv, qkv, bias=bias)
     else:
+        if w_q is None:
+            raise ValueError("a layer that reads another entry's keys and values needs the query rows alone, which a "
+                             "mixer that keeps its stacked rows in the operands' order only does not have")
         qkv = ctx.buffer("qkv", (T, n_heads * head_dim), dtype)
         linear(h, w_q, qkv, bias=None if bias is None else bias[:n_heads * head_dim])
     K.rope_cache_write(qkv, ctx.positions, _table_rows(ctx), block_table, cos, sin, k_cache, v_cache,

@@ -458,37 +458,53 @@ def test_one_step_with_a_decode_token_a_fresh_prompt_and_a_chunk(name, dtype):
     close(out, np.stack([refs[0][71], refs[1][37], refs[2][135]]), dtype, "the decode step after the mixed step")
 
 
-@pytest.mark.parametrize("name", ["A", "B"])
-def test_the_head_is_held_once_and_gives_the_same_logits(name):
-    """A bfloat16 engine keeps the head (A: and the tied embedding with it) in the matrix operands' order alone.
-    Every way a step reads it gives what an engine that keeps both orders gives, bit for bit: a prompt with all
-    rows wanted (the tiled product), its last row (a product of one row), decode steps (the folded norm), a
-    batch of 40 (the product of 17 to 64 rows); ``weights()`` hands back the stored order."""
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_weights_held_once_give_the_same_logits(name):
+    """A bfloat16 engine keeps the matrices that decode steps read in the matrix cores' order ALONE where a copy
+    can stand for them (whole steps of 64 k): the head (A: with the tied embedding), the stacked q, k, v rows, the
+    output and the down projection. Every way a step reads them gives what an engine that keeps both orders gives,
+    bit for bit: a prompt with all rows wanted (the tiled products), a chunk, single tokens (the folded norms), a
+    batch of 12 and of 40 (the kernel of whole lines); ``weights()`` hands back the stored order under the stored names."""
     from gpullama3_java_amd.csrc import lib
     from safetensors.torch import load_file
     import os
     once, both = engine(name, "bfloat16", n_slots=64, max_tokens=8192), engine(name, "bfloat16", weight_copies="both",
                                                                                 n_slots=64, max_tokens=8192)
-    head = once.model.head
-    assert lib.held_once(head) and head.data_ptr() == head.tiled.data_ptr()
-    assert (once.model.embedding is head) == CONFIGS[name]["tie_word_embeddings"]
-    assert not lib.held_once(both.model.head) and both.model.head.tiled is not None
+    cfg = CONFIGS[name]
+    d, F, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    mixer, ffn = once.model.blocks[0].mixer, once.model.blocks[0].ffn
+    # which matrices a copy can stand for follows from the sizes alone
+    assert lib.held_once(once.model.head) == (d % 64 == 0 and V % 16 == 0)
+    assert lib.held_once(mixer.w_qkv) == (d % 64 == 0 and mixer.w_qkv.shape[0] % 16 == 0)
+    from gpullama3_java_amd.parts import ops
+    assert lib.held_once(mixer.w_o) == ops.can_hold_once(both.model.blocks[0].mixer.w_o)
+    assert lib.held_once(ffn.w_down) == ops.can_hold_once(both.model.blocks[0].ffn.w_down)
+    if name == "A":
+        assert lib.held_once(once.model.head) and lib.held_once(mixer.w_qkv) and lib.held_once(mixer.w_o) and lib.held_once(ffn.w_down)
+        assert (once.model.embedding is once.model.head) == cfg["tie_word_embeddings"]
+        assert once.model.head.data_ptr() == once.model.head.tiled.data_ptr() and mixer.w_q is None
+    for m in (both.model.head, both.model.blocks[0].mixer.w_qkv, both.model.blocks[0].ffn.w_down):
+        assert not lib.held_once(m)
     folder, _, _ = model(name)
     stored = load_file(os.path.join(folder, "model.safetensors"))
     given = once.weights()
     assert set(given) == set(stored)
     for k, v in stored.items():
         assert torch.equal(given[k].cpu(), v.to(given[k].dtype)), k
-    toks = rand_tokens(name, 5, 100)
+    n = min(100, cfg["max_position_embeddings"] - 8)
+    toks = rand_tokens(name, 5, n)
     outs = []
     for eng in (once, both):
         s = eng.take_slot()
-        got = [eng.step([(s, toks[:90])], want="all"), eng.step([(s, toks[90:95])]), eng.step([(s, toks[95:96])])]
-        got += [eng.step([(s, [t])]) for t in toks[96:]]
-        many = [eng.take_slot() for _ in range(40)]
-        eng.step([(m, toks[i:i + 3]) for i, m in enumerate(many)], want="none")
-        got.append(eng.step([(m, [toks[i]]) for i, m in enumerate(many)]))
+        got = [eng.step([(s, toks[:n - 10])], want="all"), eng.step([(s, toks[n - 10:n - 5])]), eng.step([(s, toks[n - 5:n - 4])])]
+        got += [eng.step([(s, [t])]) for t in toks[n - 4:]]
+        for B in (12, 40):
+            many = [eng.take_slot() for _ in range(B)]
+            eng.step([(m, toks[i:i + 3]) for i, m in enumerate(many)], want="none")
+            got.append(eng.step([(m, [toks[i]]) for i, m in enumerate(many)]))
+            for m in many:
+                eng.give_back_slot(m)
         outs.append([g_.clone() for g_ in got])
     for i, (u, v) in enumerate(zip(*outs)):
-        assert torch.equal(u, v), f"{name}: result {i} differs between the head held once and both orders"
-    close(torch.cat(outs[0][:1]).cpu().numpy(), plain_logits(name, toks[:90]), "bfloat16", f"{name} held once, whole")
+        assert torch.equal(u, v), f"{name}: result {i} differs between weights held once and both orders"
+    close(outs[0][0].cpu().numpy(), plain_logits(name, toks[:n - 10]), "bfloat16", f"{name} held once, whole")

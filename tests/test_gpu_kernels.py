@@ -1112,7 +1112,7 @@ def test_products_read_a_weight_copy_in_operand_order(M, N, Kd):
     assert torch.equal(p2, res[False][2])
 
 
-@pytest.mark.parametrize("N, Kd", [(48, 96), (2048, 2048), (272, 1568), (8208, 160)])
+@pytest.mark.parametrize("N, Kd", [(48, 64), (2048, 2048), (272, 1600), (8208, 192)])
 def test_a_weight_kept_in_operand_order_alone(N, Kd):
     """``hold_once``: the matrix's memory is its copy in the operands' order. The embedding look-up, the generic
     product, the tiled product (store epilogue, both tiles) and the products of few rows give what they give
@@ -1151,8 +1151,6 @@ def test_a_weight_kept_in_operand_order_alone(N, Kd):
         b1, b2 = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16), torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
         lib.gemm_mfma(a, w, b1, shape=1); lib.gemm_mfma(a, once, b2, shape=1)
         assert torch.equal(b1, b2)
-        with pytest.raises(lib.KernelError, match="store epilogue"):
-            lib.gemm_mfma(a, once, torch.zeros(M, N, device=DEV), lib.EPI_ADD)
     # products of few rows read the copy as before
     for M in (1, 8, 16, 40, 64):
         a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
@@ -1166,14 +1164,13 @@ def test_a_weight_kept_in_operand_order_alone(N, Kd):
     assert torch.equal(n1, n2)
     # what reads the stored order only says so
     a = dev(rounded(rng.standard_normal((8, Kd)), "bfloat16"), torch.bfloat16)
-    with pytest.raises(lib.KernelError, match="strips of 16"):
-        lib.gemm_skinny(a, once, torch.zeros(8, N, device=DEV), strip_rows=8)
-    a40 = dev(rounded(rng.standard_normal((40, Kd)), "bfloat16"), torch.bfloat16)
-    assert not lib.gemm_skinny_wide_fits(a40, once, torch.zeros(40, N, device=DEV), lib.EPI_STORE)
-    with pytest.raises(lib.KernelError, match="operands' order alone"):
-        lib.gemm_skinny_wide(a40, once, torch.zeros(40, N, device=DEV))
+    with pytest.raises(lib.KernelError, match="matrix cores' order alone"):
+        lib.gemm_skinny(a, once, torch.zeros(8, N, device=DEV), strip_rows=8)          # it has no copy in strips of 8
     with pytest.raises(lib.KernelError, match="hold_once"):
-        lib.hold_once(dev(np.zeros((16, 40)), torch.bfloat16))              # no copy, and K is no whole k-step
+        lib.hold_once(dev(np.zeros((16, 40)), torch.bfloat16))              # no copy
+    odd = dev(np.zeros((16, 96)), torch.bfloat16)
+    odd.tiled = lib.tile_weight(odd)
+    assert not lib.can_hold_once(odd)                                       # K is no whole number of the tiled product's steps
 
 
 @pytest.mark.parametrize("pairing", ["adjacent", "half", None])
@@ -1212,6 +1209,122 @@ def test_qkv_rope_cache_reads_a_weight_copy_in_operand_order(pairing, H, Kh, hs)
                        dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
                        pairing == "adjacent", page)
     assert torch.equal(q2, got[False][0])
+
+
+@pytest.mark.parametrize("N, Kd", [(48, 64), (2048, 2048), (272, 1600), (2048, 8192), (136, 320)])
+def test_a_weight_kept_in_either_copy_s_order_alone(N, Kd):
+    """A weight of a product into the residual stream that is held once, as its copy in the operands' order
+    (strips of 16) or in packed strips of 8: the kernel of whole lines (17 to 64 rows, 9 to 16 into slices),
+    the tiled product's add epilogue with K in slices, the generic product and the products of few rows give what
+    they give for the stored rows, bit for bit; ``stored_order`` gives the rows back."""
+    rng = np.random.default_rng(N * 3 + Kd)
+    lib = K()
+    w = dev(rounded(rng.standard_normal((N, Kd)) / math.sqrt(Kd), "bfloat16"), torch.bfloat16)
+    holders = {}
+    if N % 16 == 0:
+        w16 = w.clone(); w16.tiled = lib.tile_weight(w16); holders["strips of 16"] = lib.hold_once(w16)
+    if N % 8 == 0 and Kd % 64 == 0:
+        w8 = w.clone(); w8.tiled8 = lib.tile_weight8(w8); holders["strips of 8"] = lib.hold_once(w8)
+        assert holders["strips of 8"].data_ptr() == w8.tiled8.data_ptr()
+    for how, once in holders.items():
+        assert lib.held_once(once) and torch.equal(lib.stored_order(once), w), how
+        for M in (9, 16, 17, 40, 64):
+            a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
+            assert lib.gemm_skinny_wide_fits(a, once, torch.zeros(M, N, device=DEV), lib.EPI_STORE)
+            slices = max(2, min(4, Kd // 64)) if Kd >= 128 else 1
+            if M > 16 or slices > 1:
+                shape = (slices, M, N) if slices > 1 else (M, N)
+                p1, p2 = torch.zeros(shape, device=DEV), torch.zeros(shape, device=DEV)
+                lib.gemm_skinny_wide(a, w, p1); lib.gemm_skinny_wide(a, once, p2)
+                assert torch.equal(p1, p2), (how, M, "slices")
+            if M > 16:
+                res = rng.standard_normal((M, N)).astype(np.float32)
+                x1, x2 = dev(res), dev(res)
+                lib.gemm_skinny_wide(a, w, x1, lib.EPI_ADD); lib.gemm_skinny_wide(a, once, x2, lib.EPI_ADD)
+                assert torch.equal(x1, x2), (how, M, "add")
+                b1, b2 = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16), torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+                lib.gemm_skinny_wide(a, w, b1); lib.gemm_skinny_wide(a, once, b2)
+                assert torch.equal(b1, b2), (how, M, "store")
+        for M in (5, 130, 300):
+            a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
+            res = rng.standard_normal((M, N)).astype(np.float32)
+            g1, g2 = dev(res), dev(res)
+            lib.gemm_generic(a, w, g1, lib.EPI_ADD); lib.gemm_generic(a, once, g2, lib.EPI_ADD)
+            assert torch.equal(g1, g2), (how, M, "generic")
+            for shape in (1, 2, 0):
+                for n_more in (0, 1, 2):
+                    if n_more and Kd // (n_more + 1) < 64:
+                        continue
+                    x1, x2 = dev(res), dev(res)
+                    m1 = torch.zeros(n_more, M, N, device=DEV) if n_more else None
+                    m2 = torch.zeros(n_more, M, N, device=DEV) if n_more else None
+                    lib.gemm_mfma(a, w, x1, lib.EPI_ADD, more_slices=m1, shape=shape)
+                    lib.gemm_mfma(a, once, x2, lib.EPI_ADD, more_slices=m2, shape=shape)
+                    assert torch.equal(x1, x2) and (m1 is None or torch.equal(m1, m2)), (how, M, shape, n_more)
+        for M in (1, 8, 12):                                # the products of few rows, in the strips the copy has
+            a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
+            rows = 8 if how == "strips of 8" else 16
+            res = rng.standard_normal((M, N)).astype(np.float32)
+            if lib.skinny_takes(once, M, rows):
+                x1, x2 = dev(res), dev(res)
+                lib.gemm_skinny(a, w if rows == 16 else w8, x1, lib.EPI_ADD, strip_rows=rows)
+                lib.gemm_skinny(a, once, x2, lib.EPI_ADD, strip_rows=rows)
+                assert torch.equal(x1, x2), (how, M, "skinny")
+            else:
+                assert rows == 8 and M > 8
+                with pytest.raises(lib.KernelError, match="matrix cores' order alone"):
+                    lib.gemm_skinny(a, once, dev(res), lib.EPI_ADD, strip_rows=rows)
+
+
+@pytest.mark.parametrize("pairing", ["adjacent", "half", None])
+@pytest.mark.parametrize("H, Kh, hs, d", [(32, 8, 64, 128), (6, 2, 16, 64), (5, 5, 48, 3200), (8, 1, 128, 4096)])
+def test_stacked_qkv_rows_kept_in_operand_order_alone(pairing, H, Kh, hs, d):
+    """The stacked q, k, v rows held once, as the copy whose strips pair up what the rotation's end pairs: the fused
+    product of 1 to 64 rows (the kernels of few rows, and the kernel of whole lines for 17 rows and more and for a
+    folded norm over a long K), and the plain product through the tiled and the generic kernels, which find each
+    row's place in the copy, all give what the stored rows give, bit for bit."""
+    rng = np.random.default_rng(hs + H + d)
+    lib = K()
+    page = 64
+    N = (H + 2 * Kh) * hs
+    w = dev(rounded(rng.standard_normal((N, d)) / math.sqrt(d), "bfloat16"), torch.bfloat16)
+    wq = w.clone()
+    wq.tiled = lib.tile_weight(wq, qkv=(H, Kh, hs, pairing is not None, pairing == "adjacent"))
+    once = lib.hold_once(wq)
+    assert torch.equal(lib.stored_order(once), w)
+    cos, sin = P.rope_table(256, hs, 50000.0)
+    nw = rounded(1 + 0.2 * rng.standard_normal(d), "bfloat16")
+    for T in (7, 16, 30, 64):
+        x = (rng.standard_normal((T, d)) * 2).astype(np.float32)
+        positions = rng.integers(0, 200, T)
+        zk = [np.zeros((b + 1, Kh, hs), np.float32) for b in positions]
+        for folded in ((True, False) if T <= 16 else (False,)):
+            got = []
+            for weight in (w, once):
+                kc, vc, table = paged(zk, zk, Kh, hs, page, "bfloat16", np.random.default_rng(1))
+                q_out = torch.zeros(T, H * hs, device=DEV, dtype=torch.bfloat16)
+                rows = times_weight(x, nw).to(DEV) if folded else dev(rounded(x, "bfloat16"), torch.bfloat16)
+                lib.qkv_rope_cache(rows, dev(ssq_partials(x, 6)) if folded else None, 6 if folded else 0, 1e-5, weight, q_out,
+                                   dev(positions, torch.int32), dev(np.arange(T), torch.int32), table,
+                                   dev(cos) if pairing else None, dev(sin) if pairing else None, kc, vc, H, Kh, hs,
+                                   pairing == "adjacent", page)
+                got.append((q_out, kc, vc))
+            for u, v in zip(*got):
+                assert torch.equal(u, v), (T, folded)
+    for M in (3, 200):
+        a = dev(rounded(rng.standard_normal((M, d)), "bfloat16"), torch.bfloat16)
+        g1, g2 = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16), torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+        lib.gemm_generic(a, w, g1); lib.gemm_generic(a, once, g2)
+        assert torch.equal(g1, g2)
+        for shape in (0, 1, 2, 5):
+            m1, m2 = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16), torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+            lib.gemm_mfma(a, w, m1, shape=shape); lib.gemm_mfma(a, once, m2, shape=shape)
+            assert torch.equal(m1, m2), (M, shape)
+    a = dev(rounded(rng.standard_normal((4, d)), "bfloat16"), torch.bfloat16)
+    if pairing == "half" and hs > 16:                       # (rows in another order: the plain products of few rows cannot read it)
+        assert not lib.skinny_takes(once, 4, 16)
+        with pytest.raises(lib.KernelError, match="matrix cores' order alone"):
+            lib.gemm_skinny(a, once, torch.zeros(4, N, device=DEV))
 
 
 @pytest.mark.parametrize("N, Kd", [(2048, 2048), (2048, 8192), (40, 72), (136, 1544), (3072, 200)])
