@@ -975,9 +975,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
                                                                    SkNext nx, SkNorm nrm, int wl) {
   // wl: how W lies. 0: rows as they are stored. 1: the matrix operands' order alone, [strip of 16 rows][k-step of 32]
   // [lane][8] (lib.tile_weight; for the stacked q, k, v rows the strips hold the rows that sk_strip_row names).
-  // 2: the packed strips of 8 rows, [strip of 8][step of 64 k][lane][8] (lib.tile_weight8). In both a wave's load
-  // is 1 KB of consecutive memory (a k-step of a strip, or 64 k of 8 rows), and its 16-byte pieces go to the same
-  // places of the staged tile as the stored order's.
+  // 2: the packed strips of 8 rows, [strip of 8][step of 64 k][lane][8] (lib.tile_weight8). In both orders a lane can
+  // load what it holds as the matrix instruction's operand straight from memory, in whole 128-byte lines (the
+  // operands' order IS that layout; of the packed strips lane (r, q) takes row r % 8 of strip r / 8 at the k block q
+  // of the k-step's half): the tiles of W then do not pass through shared memory at all, only the rows of A do.
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   constexpr int NWT = NS * NG;        // tiles of W a pair of k-steps
   constexpr int NT = NWT + MT;        // tiles a wave stages for a pair of k-steps: 16 rows x 128 bytes each
@@ -1003,15 +1004,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   // where the lane's two loads of a tile of W go: (row, 16-byte piece) is (l8, c8) and (8 + l8, c8) for stored rows,
   // (r, q) and (r, 4 + q) for a k-step of the operands' order each, (lane % 8 [+ 8], 4 * (lane / 8 % 2) + q) for the
   // packed strips of 8
-  int putw0 = put0, putw1 = put1;
-  if (wl == 1) {
-    putw0 = get0;
-    putw1 = get1;
-  } else if (wl == 2) {
-    const int r8 = lane & 7, c = 4 * ((lane >> 3) & 1) + q;
-    putw0 = r8 * 128 + ((c ^ r8) * 16);
-    putw1 = (8 + ((r8 + 1) & 7)) * 128 + ((c ^ r8) * 16);
-  }
+  const int putw0 = put0, putw1 = put1;   // (stored rows: as the rows of A)
 
   // Both operands are read through buffer descriptors: a lane whose row or k does not exist gives
   // an offset beyond the buffer and gets zeros without a branch around the load, so every wave issues
@@ -1034,9 +1027,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
       const int wr = sk_strip_row<EPI>(strip_g, 8 * j + l8, N, rp, hd[g], sub[g], rotated[g]);
 #pragma unroll
       for (int h = 0; h < NG; ++h)   // (32-bit: the entry point lets in operands below 2 GiB only)
+        // (wl 1, 2: j is the k-step of the pair, and the lane's 16 bytes are its operand of that k-step)
         wo[g * NG + h][j] = wl == 0   ? ((unsigned)(wr + h * N) * (unsigned)ldw + (unsigned)c8 * 8u) * 2u
                             : wl == 1 ? (unsigned)(strip_g + h * (N >> 4)) * strip_bytes + (unsigned)j * 1024u + (unsigned)lane * 16u
-                                      : (unsigned)(2 * strip_g + j) * strip_bytes + (unsigned)lane * 16u;
+                                      : (unsigned)(2 * strip_g + (r >> 3)) * strip_bytes + (unsigned)(2 * q + j) * 128u + (unsigned)(r & 7) * 16u;
     }
   unsigned xo[MT][2];
 #pragma unroll
@@ -1128,10 +1122,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
   }
   if (XNORM) sk_ssq_ask<NW, MT>(sq, M, nrm, sq_row);
   for (int i = 0; i < n_it; ++i) {
+    bf16x8 wnow[NWT][2];   // (wl 1, 2) this pair's operands of W, which the next pair's loads are about to replace
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      *(bf16x8*)(stage + t * 2048 + (t < NWT ? putw0 : put0)) = held[t][0];
-      *(bf16x8*)(stage + t * 2048 + (t < NWT ? putw1 : put1)) = held[t][1];
+      if (t < NWT && wl != 0) {
+        wnow[t][0] = held[t][0];
+        wnow[t][1] = held[t][1];
+      } else {
+        *(bf16x8*)(stage + t * 2048 + (t < NWT ? putw0 : put0)) = held[t][0];
+        *(bf16x8*)(stage + t * 2048 + (t < NWT ? putw1 : put1)) = held[t][1];
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -1147,7 +1147,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t*
       for (int g = 0; g < NS; ++g)
 #pragma unroll
         for (int h = 0; h < NG; ++h) {
-          const bf16x8 wf = *(const bf16x8*)(stage + (g * NG + h) * 2048 + get);
+          const bf16x8 wf = wl != 0 ? wnow[g * NG + h][s] : *(const bf16x8*)(stage + (g * NG + h) * 2048 + get);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
             acc[g][h][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[mt], acc[g][h][mt], 0, 0, 0);
