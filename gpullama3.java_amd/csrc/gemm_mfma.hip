@@ -90,10 +90,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
     int r = (tid + NT * i) >> 3, c = tid & 7;
     if (WT) {
       // Which 16 bytes of the tile a thread brings is free (they go to their own place in shared memory). In a copy's
-      // order 8 rows of a strip at one block of 8 k are a 128-byte line, and the lines of a strip's k-step lie side by
-      // side: a wave that took them in order would ask one small region of memory for all its 8 lines, where rows of
-      // the stored order lie far apart (the products of 2,048 rows were 13 to 20% slower that way). So a wave takes
-      // the same line of 8 different strips: lane l the row l % 8 of strip l / 8 of its group.
+      // order 8 rows of a strip at one block of 8 k are a 128-byte line. With the stored order's assignment (eight
+      // neighbouring threads: the eight pieces of one row's 64 k) eight threads would touch eight lines, 16 bytes of
+      // each, which a CU's first-level cache takes at a third of the rate of whole lines (the products of 2,048 rows
+      // were 13 to 20% slower that way). So eight neighbouring threads take one whole line, and a wave the same
+      // line of 8 different strips: lane l the row l % 8 of strip l / 8 of its group.
       const int idx = (tid >> 6) * NWC + i, l = tid & 63;
       if (WT == 1) {   // [strip of 16][k-step of 32][k block q][row][8]: 16 lines a strip and step of 64 k
         const int combo = idx & 15;

@@ -1228,6 +1228,10 @@ def test_a_weight_kept_in_either_copy_s_order_alone(N, Kd):
         assert holders["strips of 8"].data_ptr() == w8.tiled8.data_ptr()
     for how, once in holders.items():
         assert lib.held_once(once) and torch.equal(lib.stored_order(once), w), how
+        # (over the packed strips of 8 the kernel of whole lines deals the k-steps to its waves in runs, not in turn:
+        # the same products summed in another order)
+        same = (lambda u, v: torch.equal(u, v)) if how == "strips of 16" else (
+            lambda u, v: bool(((u.float() - v.float()).abs().max() <= 2e-2 * max(1e-6, float(u.float().abs().max())))))
         for M in (9, 16, 17, 40, 64):
             a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
             assert lib.gemm_skinny_wide_fits(a, once, torch.zeros(M, N, device=DEV), lib.EPI_STORE)
@@ -1236,15 +1240,15 @@ def test_a_weight_kept_in_either_copy_s_order_alone(N, Kd):
                 shape = (slices, M, N) if slices > 1 else (M, N)
                 p1, p2 = torch.zeros(shape, device=DEV), torch.zeros(shape, device=DEV)
                 lib.gemm_skinny_wide(a, w, p1); lib.gemm_skinny_wide(a, once, p2)
-                assert torch.equal(p1, p2), (how, M, "slices")
+                assert same(p1.sum(0) if slices > 1 else p1, p2.sum(0) if slices > 1 else p2), (how, M, "slices")
             if M > 16:
                 res = rng.standard_normal((M, N)).astype(np.float32)
                 x1, x2 = dev(res), dev(res)
                 lib.gemm_skinny_wide(a, w, x1, lib.EPI_ADD); lib.gemm_skinny_wide(a, once, x2, lib.EPI_ADD)
-                assert torch.equal(x1, x2), (how, M, "add")
+                assert same(x1, x2), (how, M, "add")
                 b1, b2 = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16), torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
                 lib.gemm_skinny_wide(a, w, b1); lib.gemm_skinny_wide(a, once, b2)
-                assert torch.equal(b1, b2), (how, M, "store")
+                assert same(b1, b2), (how, M, "store")
         for M in (5, 130, 300):
             a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
             res = rng.standard_normal((M, N)).astype(np.float32)
