@@ -136,12 +136,6 @@ def _w_order(w):
     return 2, _ptr(w.tiled8), c_void_p(0)
 
 
-def _stored(w, who):
-    if held_once(w):
-        raise KernelError(f"{who}: the weight is kept in the matrix cores' order alone, which this kernel does not read")
-    return w
-
-
 def _code(t, name):
     try:
         return _CODES[t.dtype]

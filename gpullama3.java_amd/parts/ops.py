@@ -71,8 +71,8 @@ def can_hold_once(w, without=_NONE):
     walk), the kernel of whole lines, the tiled product's store and add epilogues, the generic product."""
     # (a weight with packed strips of 8 only: steps of 9 to 64 rows must find the kernel of whole lines, which takes
     # it with K in slices; else they would fall back to the tiled product, which is right but slow for so few rows)
-    return (not without and K.can_hold_once(w)
-            and (getattr(w, "tiled", None) is not None or K.wide_slices(w.shape[0], w.shape[1]) >= 2))
+    strips_of_16 = getattr(w, "tiled", None) is not None and w.shape[0] % 16 == 0
+    return not without and K.can_hold_once(w) and (strips_of_16 or K.wide_slices(w.shape[0], w.shape[1]) >= 2)
 
 
 class StoredRows:

@@ -35,3 +35,34 @@ def test_decode_attention_splits_the_keys_until_every_cu_has_a_block():
     assert s(4, 32, 8, 4096, 64) == 4 and s(4, 32, 8, 16384, 64) == 8                    # more than 16 blocks: per 64 K
     assert s(8, 32, 8, 32768) == 4 and s(16, 32, 8, 32768) == 2 and s(32, 32, 8, 32768) == 1   # 256 blocks, not more
     assert s(2, 64, 2, 100000) == 32                                  # never more than 32
+
+
+def test_which_weights_a_copy_can_stand_for():
+    """``lib.can_hold_once`` / ``ops.can_hold_once``: a copy in the matrix cores' order can stand for the matrix when it
+    has exactly the matrix's elements over whole steps of 64 k; a weight with packed strips of 8 only must also be
+    one whose products of 9 to 64 rows the kernel of whole lines takes with K in slices; any fast path switched off
+    keeps both orders."""
+    import torch
+    from gpullama3_java_amd.parts import ops
+
+    def weight(N, K, strips16, strips8):
+        w = torch.zeros(N, K, dtype=torch.bfloat16)
+        if strips16:
+            w.tiled = torch.zeros(N * -(-K // 32) * 32, dtype=torch.bfloat16)
+            w.tiled.tiled_for = None
+        if strips8:
+            w.tiled8 = torch.zeros(N * -(-K // 64) * 64, dtype=torch.bfloat16)
+        return w
+
+    assert lib.can_hold_once(weight(2048, 2048, True, False)) and lib.can_hold_once(weight(2048, 8192, False, True))
+    assert not lib.can_hold_once(weight(2048, 2048, False, False))                     # no copy
+    assert not lib.can_hold_once(weight(96, 96, True, False))                          # K is no whole number of steps of 64
+    assert not lib.can_hold_once(weight(136, 512, True, False))                        # rows in no whole strips of 16
+    assert lib.can_hold_once(weight(136, 512, False, True))                            # ... but in strips of 8
+    assert ops.can_hold_once(weight(2048, 8192, False, True))                          # down projection of the 1B layers
+    assert not ops.can_hold_once(weight(136, 512, False, True))                        # no slices of K for 9 to 64 rows
+    assert not ops.can_hold_once(weight(136, 512, True, True))                         # (136 rows are no whole strips of 16)
+    assert ops.can_hold_once(weight(128, 512, True, True))
+    assert not ops.can_hold_once(weight(2048, 2048, True, False), frozenset({"once"}))
+    assert not ops.can_hold_once(weight(2048, 2048, True, False), frozenset({"wide"}))
+    assert not lib.held_once(weight(64, 64, True, True))
