@@ -66,3 +66,33 @@ def test_which_weights_a_copy_can_stand_for():
     assert not ops.can_hold_once(weight(2048, 2048, True, False), frozenset({"once"}))
     assert not ops.can_hold_once(weight(2048, 2048, True, False), frozenset({"wide"}))
     assert not lib.held_once(weight(64, 64, True, True))
+
+
+def test_strips_slices_and_pieces_of_the_products_of_few_rows():
+    """The rules that decide a decode step's kernels, at the sizes they were measured at."""
+    from gpullama3_java_amd.parts import ops
+    rows = lib.skinny_strip_rows
+    # strips of 8 weight rows where strips of 16 would leave more than a third of the CUs without a block
+    assert rows(8, 2048, 2048, lib.EPI_ADD) == 8 and rows(8, 2048, 8192, lib.EPI_ADD) == 8            # 1B output, down
+    assert rows(8, 3072, 3072, lib.EPI_ADD) == 16 and rows(8, 4096, 14336, lib.EPI_ADD) == 16         # 3B, 8B: strips enough
+    assert rows(12, 2048, 2048, lib.EPI_ADD) == 16 and rows(12, 2048, 8192, lib.EPI_ADD) == 8          # 9 to 16 rows: only a long K
+    assert rows(40, 2048, 8192, lib.EPI_ADD) == 16 and rows(8, 2048, 2048, lib.EPI_GATED) == 16
+    # the kernel of whole lines cuts K so that the chip has blocks enough, never below 512 columns a slice
+    assert lib.wide_slices(2048, 2048) == 4 and lib.wide_slices(2048, 8192) == 4 and lib.wide_slices(4096, 14336) == 2
+    assert lib.wide_slices(3072, 3072) == 2 and lib.wide_slices(136, 512) == 1 and lib.wide_slices(128256, 2048) == 1
+    # which kernel keeps the rows of a step in registers
+    assert lib.skinny_keeps_operands(8, 4096) and not lib.skinny_keeps_operands(8, 8192)
+    assert lib.skinny_keeps_operands(40, 2048) and not lib.skinny_keeps_operands(40, 3072)
+    # a replayed step of 66 to 128 rows is worked on in two pieces; other steps are not
+    class Ctx:
+        replayed = True
+    assert ops.row_chunks(64, Ctx) is None and ops.row_chunks(65, Ctx) is None and ops.row_chunks(129, Ctx) is None
+    assert ops.row_chunks(66, Ctx) == [(0, 33), (33, 66)] and ops.row_chunks(128, Ctx) == [(0, 64), (64, 128)]
+    Ctx.replayed = False
+    assert ops.row_chunks(100, Ctx) is None
+    assert ops.FUSE_ROWS == 16 and ops.CHUNK_ROWS == 128
+    # the gated product of few rows runs on the kernel of whole lines where it has blocks enough (and then needs no copy)
+    import torch
+    assert ops.gated_on_whole_lines(torch.empty(2 * 8192, 8, dtype=torch.bfloat16))
+    assert not ops.gated_on_whole_lines(torch.empty(2 * 320, 8, dtype=torch.bfloat16))
+    assert not ops.gated_on_whole_lines(torch.empty(2 * 8192, 8, dtype=torch.bfloat16), frozenset({"widefold"}))
