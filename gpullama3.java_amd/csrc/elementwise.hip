@@ -327,9 +327,12 @@ __global__ __launch_bounds__(256) void rope_cache_vec_kernel(
     const int* __restrict__ block_table, int table_stride, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int n_heads, int n_kv,
     int head_dim, int rot_dim, int adjacent, int page_size, int write_kv, long row_stride, int n_tokens) {
-  // Blocks with consecutive numbers go to different XCDs, each with a second-level cache of its own. The values
-  // of 8 consecutive positions of a sequence share 16 bytes of a transposed page, one 2-byte store per token;
-  // with neighbouring tokens on one XCD those stores meet in one cache and leave it as whole lines.
+  // Blocks with consecutive numbers go to different XCDs, each with a second-level cache of its own; neighbouring
+  // tokens go to one XCD. The values of 8 consecutive positions of a sequence share 16 bytes of a transposed page.
+  // The first of the step's tokens in such a group of 8 positions writes the values of all of them that the step
+  // brings (they follow it in the packed order): 16 bytes a dim where the group is whole, single elements at the
+  // ends of a sequence's tokens. (One 2-byte store per token and dim before: a million partial writes a layer for
+  // 2,048 tokens.)
   const int per_xcd = (n_tokens + 7) / 8;
   const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (t >= n_tokens) return;
@@ -344,17 +347,42 @@ __global__ __launch_bounds__(256) void rope_cache_vec_kernel(
   const int pair_units = rotate ? half / 8 : 0;              // per head
   const int plain_units = (head_dim - (rotate ? rot_dim : 0)) / 8;
   const int per_head = pair_units + plain_units;
-  const int v_units = write_kv ? n_kv * (head_dim / 8) : 0;
+  int v_units = 0, run = 0;                      // units of the value heads, and how many tokens' values this block writes
+  if (write_kv) {
+    const int seq = seq_of_token[t];
+    const bool first = (pos & 7) == 0 || t == 0 || seq_of_token[t - 1] != seq || positions[t - 1] != pos - 1;
+    if (first) {
+      v_units = n_kv * (head_dim / 8);
+      run = 1;
+      while (run < 8 - (pos & 7) && t + run < n_tokens && seq_of_token[t + run] == seq && positions[t + run] == pos + run) ++run;
+    }
+  }
   const int total = rot_heads * per_head + v_units;
   for (int w = threadIdx.x; w < total; w += blockDim.x) {
     if (w >= rot_heads * per_head) {            // a unit of a value head: transposed into the cache
       const int u = w - rot_heads * per_head;
       const int ch = u / (head_dim / 8), e0 = (u % (head_dim / 8)) * 8;
-      const rc_bf16x8 v = *(const rc_bf16x8*)(row + (long)(n_heads + n_kv + ch) * head_dim + e0);
       bf16_t* vpage = v_cache + ((long)page * n_kv + ch) * page_size * head_dim;
       const long at = gl3_v_offset(e0, in_page, page_size);   // dims e0 .. e0+7 lie in one tile, 8 elements apart
+      const bf16_t* from = row + (long)(n_heads + n_kv + ch) * head_dim + e0;
+      if (run == 8) {                            // a whole group of 8 positions (pos % 8 == 0): 16 bytes a dim
+        rc_bf16x8 v[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) vpage[at + 8 * e] = v[e];
+        for (int i = 0; i < 8; ++i) v[i] = *(const rc_bf16x8*)(from + (long)i * row_stride);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          rc_bf16x8 o;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) o[i] = v[i][e];
+          *(rc_bf16x8*)(vpage + at + 8 * e) = o;
+        }
+      } else {
+        for (int i = 0; i < run; ++i) {
+          const rc_bf16x8 v = *(const rc_bf16x8*)(from + (long)i * row_stride);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) vpage[at + i + 8 * e] = v[e];
+        }
+      }
       continue;
     }
     const int head = w / per_head, u = w % per_head;
