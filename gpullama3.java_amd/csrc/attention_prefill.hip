@@ -149,7 +149,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   // one chunk of one head: scores, running softmax, weighted values. MASKED: some query of the
   // wave does not see some key of the chunk (the diagonal, a window's edge).
   auto head_chunk = [&](int hh, const bf16x8 (&ka)[KK], const bf16x8 (&kb2)[KK], const bf16x8 (&vt)[DT], int key0,
-                        auto masked) {
+                        bool masked) {
     f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
       s[v] = sa[v];
       s[4 + v] = sb[v];
     }
-    if (decltype(masked)::value) {
+    if (masked) {                               // (the same for the whole wave: a branch around the tests, one body)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int k1 = key0 + 8 * qd + v, k2 = k1 + 4;
@@ -220,13 +220,9 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) vt[dt] = *(const bf16x8*)&vs[buf][dt * 16 + j][8 * qd];
         // every query of the wave sees the whole chunk: no mask (the same for the whole wave)
-        if (key0 + 31 <= p_first && key0 >= lo_last) {
+        const bool masked = !(key0 + 31 <= p_first && key0 >= lo_last);
 #pragma unroll
-          for (int hh = 0; hh < GH; ++hh) head_chunk(hh, ka, kb2, vt, key0, std::false_type{});
-        } else {
-#pragma unroll
-          for (int hh = 0; hh < GH; ++hh) head_chunk(hh, ka, kb2, vt, key0, std::true_type{});
-        }
+        for (int hh = 0; hh < GH; ++hh) head_chunk(hh, ka, kb2, vt, key0, masked);
       }
       if (ck < ck1) stage(buf ^ 1, rk[(r + 1) % AHEAD], rv[(r + 1) % AHEAD]);
       __syncthreads();
@@ -363,7 +359,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
   // where they are used, no more than four ahead of their products (the scheduler would read them
   // all first, and they do not fit into the registers beside the sums). MASKED: some query of the
   // wave does not see some key of the chunk (the diagonal, a window's edge).
-  auto chunk = [&](int buf, int key0, auto masked) {
+  auto chunk = [&](int buf, int key0, bool masked) {
     f32x16 s[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t)
@@ -378,7 +374,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
       }
       if (kk % 4 == 3) __builtin_amdgcn_sched_barrier(0);
     }
-    if (decltype(masked)::value) {
+    if (masked) {                               // (the same for the whole wave: a branch around the tests, one body)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -446,8 +442,7 @@ __global__ __launch_bounds__(256, OCC) void attention_prefill_wide_kernel(
       fetch(min(ck + AHEAD, ck1), rk[r], rv[r]);
       if (ck >= ck_first && ck <= ck_last) {
         // every query of the wave sees the whole chunk: no mask (the same for the whole wave)
-        if (key0 + CK - 1 <= p_first && key0 >= lo_last) chunk(buf, key0, std::false_type{});
-        else chunk(buf, key0, std::true_type{});
+        chunk(buf, key0, !(key0 + CK - 1 <= p_first && key0 >= lo_last));
       }
       if (ck < ck1) stage(buf ^ 1, rk[(r + 1) % AHEAD], rv[(r + 1) % AHEAD]);
       __syncthreads();
