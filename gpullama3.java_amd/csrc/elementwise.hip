@@ -107,32 +107,52 @@ extern "C" int gl3_embed(const void* table, int table_dtype, const int* ids, flo
 // (J/inference/InferenceCore.java:47-56). One block per row; `rows` (may be
 // null) picks the rows of x that are normalised, so that the final norm runs on
 // the wanted positions only. The order of the sum depends on d alone.
-template <typename TW, typename TO>
-__global__ void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows, const TW* __restrict__ w,
-                               TO* __restrict__ out, int d, float eps) {
+// VEC 4 (rows of a multiple of 4 floats, 16-byte aligned): 16-byte loads, and a thread's first four
+// elements stay in registers between the two passes, so rows of up to 4,096 floats are read once.
+template <typename TW, typename TO, int VEC>
+__global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                                                       const TW* __restrict__ w, TO* __restrict__ out, int d, float eps) {
+  typedef float vec_t __attribute__((ext_vector_type(VEC)));
   __shared__ float scratch[16];
   const long r = blockIdx.x;
   const long src = rows ? rows[r] : r;
   const float* xr = x + src * d;
+  const int first = threadIdx.x * VEC, stride = blockDim.x * VEC;
+  vec_t kept = vec_t(0.f);
   float ss = 0.f;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    float v = xr[i];
-    ss += v * v;
+  for (int i = first; i < d; i += stride) {
+    const vec_t v = *(const vec_t*)(xr + i);
+    if (i == first) kept = v;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) ss += ((const float*)&v)[e] * ((const float*)&v)[e];
   }
   ss = block_sum(ss, scratch);
   ss = ss / (float)d;
   ss = ss + eps;
   ss = 1.0f / sqrtf(ss);
   TO* o = out + r * d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_f32<TO>(to_f32<TW>(w[i]) * (ss * xr[i]));
+  for (int i = first; i < d; i += stride) {
+    const vec_t v = i == first ? kept : *(const vec_t*)(xr + i);
+    typedef TO out_t __attribute__((ext_vector_type(VEC)));
+    out_t res;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) res[e] = from_f32<TO>(to_f32<TW>(w[i + e]) * (ss * ((const float*)&v)[e]));
+    *(out_t*)(o + i) = res;      // (VEC 4: the launcher has checked the output's alignment)
+  }
 }
 
 extern "C" int gl3_rmsnorm(const float* x, const int* rows, const void* w, int w_dtype, void* out, int out_dtype,
                            int n_rows, int d, float eps, hipStream_t stream) {
   if (n_rows == 0) return 0;
   GL3_REQUIRE(x && w && out && n_rows > 0 && d > 0, "gl3_rmsnorm: bad arguments (rows=%d d=%d)", n_rows, d);
-  dim3 grid(n_rows), block(256);
-#define GO(TW, TO) rmsnorm_kernel<TW, TO><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, d, eps)
+  const bool vec4 = d % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0;
+  const int threads = !vec4 ? 256 : d / 4 >= 1024 ? 1024 : d / 4 > 256 ? 512 : 256;
+  dim3 grid(n_rows), block(threads);
+#define GO(TW, TO)                                                                                              \
+  do {                                                                                                          \
+    if (vec4) rmsnorm_kernel<TW, TO, 4><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, d, eps);   \
+    else rmsnorm_kernel<TW, TO, 1><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, d, eps);        \
+  } while (0)
   if (w_dtype == GL3_F32 && out_dtype == GL3_F32) GO(float, float);
   else if (w_dtype == GL3_F32 && out_dtype == GL3_BF16) GO(float, bf16_t);
   else if (w_dtype == GL3_BF16 && out_dtype == GL3_F32) GO(bf16_t, float);
@@ -218,8 +238,11 @@ __global__ __launch_bounds__(1024) void add_slices_rmsnorm_kernel(float* __restr
   for (int i = first; i < d; i += stride) {
     // beyond the kept elements: this thread's own stores, or the sum again when x was not written
     const vec_t v = i == first ? kept : (rows ? summed(i) : *(const vec_t*)(xr + i));
+    typedef TO out_t __attribute__((ext_vector_type(VEC)));
+    out_t res;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) o[i + e] = from_f32<TO>(to_f32<TW>(w[i + e]) * (ss * ((const float*)&v)[e]));
+    for (int e = 0; e < VEC; ++e) res[e] = from_f32<TO>(to_f32<TW>(w[i + e]) * (ss * ((const float*)&v)[e]));
+    *(out_t*)(o + i) = res;      // (VEC 4: the launcher has checked the output's alignment)
   }
 }
 
@@ -230,7 +253,8 @@ extern "C" int gl3_add_slices_rmsnorm(float* x, const int* rows, const float* P,
   GL3_REQUIRE(x && P && n_rows > 0 && d > 0 && n_slices > 0 && ldp >= d,
               "gl3_add_slices_rmsnorm: bad arguments (rows=%d d=%d slices=%d)", n_rows, d, n_slices);
   GL3_REQUIRE((w != nullptr) == (out != nullptr), "gl3_add_slices_rmsnorm: weight and output come together");
-  const bool vec4 = d % 4 == 0 && ldp % 4 == 0 && slice_stride % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)P % 16 == 0;
+  const bool vec4 = d % 4 == 0 && ldp % 4 == 0 && slice_stride % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)P % 16 == 0 &&
+                    (uintptr_t)out % 16 == 0;
   const int per = vec4 ? 4 : 1;
   const int threads = d / per >= 1024 ? 1024 : d / per > 256 ? 512 : 256;
   dim3 grid(n_rows), block(threads);
