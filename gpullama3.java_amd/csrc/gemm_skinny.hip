@@ -967,12 +967,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
 //
 // XNORM (one slice of K): the product is that of an RMSNorm, as in the other kernels: A holds
 // bfloat16(weight * x) and the rows' 1/rms, from the partial sums of squares, is applied to the sums.
-template <int MT, int NS, int NW, int EPI, typename TC, bool XNORM>
+template <int MT, int NS, int NW, int EPI, typename TC, bool XNORM, int WL>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_wide_kernel(const bf16_t* __restrict__ A,
                                                                    const bf16_t* __restrict__ W, TC* __restrict__ C,
                                                                    int M, int N, int K, long lda, long ldw, long ldc,
                                                                    long slice_stride, int pairs_per_slice, SkRope rp,
-                                                                   SkNext nx, SkNorm nrm, int wl) {
+                                                                   SkNext nx, SkNorm nrm) {
+  constexpr int wl = WL;   // (a template parameter: as a run-time value every tile of every pair took a branch and two copies)
   // wl: how W lies. 0: rows as they are stored. 1: the matrix operands' order alone, [strip of 16 rows][k-step of 32]
   // [lane][8] (lib.tile_weight; for the stacked q, k, v rows the strips hold the rows that sk_strip_row names).
   // 2: the packed strips of 8 rows, [strip of 8][step of 64 k][lane][8] (lib.tile_weight8). In both orders a lane can
@@ -1420,10 +1421,19 @@ static int launch_wide(const SkCall& a, int slices, long slice_stride) {
   const int n_strips = (a.N + 15) / 16;
   const int pairs = (a.K + 63) / 64;   // pairs of k-steps
   const int per_slice = (pairs + slices - 1) / slices;
-  gemm_skinny_wide_kernel<MT, NS, NW, EPI, TC, XNORM>
-      <<<dim3((n_strips + NS - 1) / NS, slices), dim3(NW * 64), 0, a.stream>>>(
-          (const bf16_t*)a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, slice_stride, per_slice,
-          a.rp, a.nx, a.nrm, a.wl);
+#define SK_WIDE(WL)                                                                                               \
+  gemm_skinny_wide_kernel<MT, NS, NW, EPI, TC, XNORM, WL>                                                         \
+      <<<dim3((n_strips + NS - 1) / NS, slices), dim3(NW * 64), 0, a.stream>>>(                                   \
+          (const bf16_t*)a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, slice_stride, per_slice, \
+          a.rp, a.nx, a.nrm)
+  if (a.wl == 0) SK_WIDE(0);
+  else if (a.wl == 1) SK_WIDE(1);
+  else {
+    // the packed strips of 8 rows: the copies of the output and down projections
+    if constexpr ((EPI == SK_STORE || EPI == SK_ADD) && !XNORM) SK_WIDE(2);
+    else GL3_REQUIRE(false, "gl3_gemm_skinny_wide: W in packed strips of 8 is read by the store and add epilogues (epilogue %d)", EPI);
+  }
+#undef SK_WIDE
   GL3_LAUNCH_CHECK();
   return 0;
 }
