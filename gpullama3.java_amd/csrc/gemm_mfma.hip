@@ -108,9 +108,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_mfma_kernel(const bf16_t* _
     }
     wrow_s[i] = r;
     wcol_s[i] = c * 8;
-    const int rel = (EPI == MF_GATED && i >= NWC / 2) ? r - BN / 2 : r;
+    // (gated: the tile's second half of rows are the up rows of the same columns; in a copy's order which half a
+    // load falls into goes by its row, not by its number)
+    const bool up = EPI == MF_GATED && (WT ? r >= BN / 2 : i >= NWC / 2);
+    const int rel = up ? r - BN / 2 : r;
     const int row = min(n0 + rel, N - 1);
-    const int wrow = row + ((EPI == MF_GATED && i >= NWC / 2) ? N : 0);
+    const int wrow = row + (up ? N : 0);
     // (WT: K is a multiple of 64, so a thread's column inside a k-step of 64 is at the same place of every step)
     woff[i] = WT == 1   ? (unsigned)gl3_operand_offset(w_pos ? w_pos[wrow] : wrow, c * 8, w_steps)
               : WT == 2 ? (unsigned)gl3_packed_offset(wrow, c * 8, w_steps)
@@ -307,17 +310,17 @@ static int launch_mfma(const void* A, const void* W, void* C, int M, int N, int 
   if (shape == 0) shape = choose_shape(M, N, slices, EPI == MF_GATED);
 #define MF_ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, w_steps, w_pos, stream
   if (w_order) {
-    // W is one of its copies in the matrix cores' order (a weight that is held once): the store and add epilogues,
-    // the three tiles that the library chooses between
+    // W is one of its copies in the matrix cores' order (a weight that is held once): the three tiles that the library
+    // chooses between
+    GL3_REQUIRE(shape == 1 || shape == 2 || shape == 5, "gl3_gemm_mfma: tile shape %d does not read W in a copy's order", shape);
+    if (w_order == 1)
+      return shape == 1 ? launch_shape<EPI, TC, 1, 4, 2, 1>(MF_ARGS)
+             : shape == 2 ? launch_shape<EPI, TC, 2, 4, 4, 1>(MF_ARGS) : launch_shape<EPI, TC, 1, 4, 4, 1>(MF_ARGS);
     if constexpr (EPI != MF_GATED) {
-      GL3_REQUIRE(shape == 1 || shape == 2 || shape == 5, "gl3_gemm_mfma: tile shape %d does not read W in a copy's order", shape);
-      if (w_order == 1)
-        return shape == 1 ? launch_shape<EPI, TC, 1, 4, 2, 1>(MF_ARGS)
-               : shape == 2 ? launch_shape<EPI, TC, 2, 4, 4, 1>(MF_ARGS) : launch_shape<EPI, TC, 1, 4, 4, 1>(MF_ARGS);
       return shape == 1 ? launch_shape<EPI, TC, 1, 4, 2, 2>(MF_ARGS)
              : shape == 2 ? launch_shape<EPI, TC, 2, 4, 4, 2>(MF_ARGS) : launch_shape<EPI, TC, 1, 4, 4, 2>(MF_ARGS);
     } else {
-      GL3_REQUIRE(false, "gl3_gemm_mfma: W in a copy's order alone is not read by the gated epilogue (order %d)", w_order);
+      GL3_REQUIRE(false, "gl3_gemm_mfma: the gated epilogue reads the copy in the operands' order, not the packed strips of 8 (order %d)", w_order);
     }
   }
   if (shape == 1) return launch_shape<EPI, TC, 1, 4, 2>(MF_ARGS);
@@ -363,7 +366,7 @@ extern "C" int gl3_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
   {
     const long w_rows = epilogue == MF_GATED ? 2L * N : (long)N;
     GL3_REQUIRE(w_order >= 0 && w_order <= 2 && (w_order == 0 || (K % 64 == 0 && (long)w_rows * K < (1L << 32))) &&
-                    (w_order != 1 || w_rows % 16 == 0) && (w_order != 2 || w_rows % 8 == 0) && (w_order == 1 || !w_pos),
+                    (w_order != 1 || (w_rows % 16 == 0 && N % 16 == 0)) && (w_order != 2 || w_rows % 8 == 0) && (w_order == 1 || !w_pos),
                 "gl3_gemm_mfma: W in order %d with K=%d (a copy's order is read over whole steps of 64), N=%d", w_order, K, N);
   }
 #define ARGS A, W, C, M, N, K, lda, ldw, ldc, slices, P, p_stride, ldp, bias, act, shape, w_order, w_pos, stream

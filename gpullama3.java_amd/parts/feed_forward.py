@@ -46,9 +46,15 @@ class GatedFeedForward:
         self.w_gate_up = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
         weights[n["gate"]], weights[n["up"]] = self.w_gate_up[:self.F], self.w_gate_up[self.F:]
         without = getattr(self, "without", frozenset())      # the fast paths that the engine does without
-        ops.for_gated(self.w_gate_up, without=without)
+        may_hold_once = getattr(self, "may_hold_once", False)
+        ops.for_gated(self.w_gate_up, without=without, alone=may_hold_once)
+        if may_hold_once and ops.gated_alone(self.w_gate_up, without) and ops.can_hold_once(self.w_gate_up, without):
+            # the stored order is let go; the stored names then name rows that are put together on request
+            self.w_gate_up = K.hold_once(self.w_gate_up)
+            weights[n["gate"]] = ops.StoredRows(self, "w_gate_up", 0, self.F)
+            weights[n["up"]] = ops.StoredRows(self, "w_gate_up", self.F, 2 * self.F)
         self.w_down = ops.for_eight_rows(weights[n["down"]], without=without)
-        if getattr(self, "may_hold_once", False) and ops.can_hold_once(self.w_down, without):
+        if may_hold_once and ops.can_hold_once(self.w_down, without):
             self.w_down = weights[n["down"]] = K.hold_once(self.w_down)      # (the stored order is let go)
         if self.biased:     # the epilogues read biases as float
             self.b_gate_up = torch.cat([weights[n["gate_bias"]].float(), weights[n["up_bias"]].float()]).contiguous()

@@ -1173,6 +1173,54 @@ def test_a_weight_kept_in_operand_order_alone(N, Kd):
     assert not lib.can_hold_once(odd)                                       # K is no whole number of the tiled product's steps
 
 
+@pytest.mark.parametrize("F, Kd", [(48, 64), (4096, 2048), (272, 1600), (6160, 192)])
+def test_stacked_gate_and_up_rows_kept_in_operand_order_alone(F, Kd):
+    """The gate rows and the up rows of a feed-forward, stacked and held once: in the copy the up strips follow the
+    F / 16 gate strips. The tiled product (all three tiles, whole and cut tiles), the kernel of whole lines, the
+    products of few rows and the generic product give, with the gated epilogue, what they give over the stored
+    rows, bit for bit."""
+    rng = np.random.default_rng(F + Kd)
+    lib = K()
+    w = dev(rounded(rng.standard_normal((2 * F, Kd)) / math.sqrt(Kd), "bfloat16"), torch.bfloat16)
+    w.tiled = lib.tile_weight(w)
+    once = lib.hold_once(w)
+    assert lib.held_once(once) and torch.equal(lib.stored_order(once), w)
+    for M in (1, 8, 13, 24, 64, 65, 300, 1100):
+        a = dev(rounded(rng.standard_normal((M, Kd)), "bfloat16"), torch.bfloat16)
+        g, u = P.linear(a.float().cpu().numpy(), w[:F].float().cpu().numpy()), P.linear(a.float().cpu().numpy(), w[F:].float().cpu().numpy())
+        ref = g / (1 + np.exp(-g)) * u
+        if M in (1, 13, 65):
+            g1, g2 = torch.zeros(M, F, device=DEV), torch.zeros(M, F, device=DEV)
+            lib.gemm_generic(a, w, g1, lib.EPI_GATED); lib.gemm_generic(a, once, g2, lib.EPI_GATED)
+            assert torch.equal(g1, g2)
+        if M >= 65:
+            for shape in (1, 2, 5, 0):
+                m1 = torch.zeros(M, F, device=DEV, dtype=torch.bfloat16)
+                m2 = torch.full((M, F + 3), -7.0, device=DEV, dtype=torch.bfloat16)
+                lib.gemm_mfma(a, w, m1, lib.EPI_GATED, shape=shape); lib.gemm_mfma(a, once, m2[:, :F], lib.EPI_GATED, shape=shape)
+                assert torch.equal(m1, m2[:, :F]) and torch.all(m2[:, F:] == -7.0), (M, shape)
+                np.testing.assert_allclose(m1.float().cpu().numpy(), ref, atol=2e-2 * np.abs(ref).max())
+            f1, f2 = torch.zeros(M, F, device=DEV), torch.zeros(M, F, device=DEV)
+            lib.gemm_mfma(a, w, f1, lib.EPI_GATED); lib.gemm_mfma(a, once, f2, lib.EPI_GATED)
+            assert torch.equal(f1, f2)
+        if 16 < M <= 64:
+            s1, s2 = torch.zeros(M, F, device=DEV, dtype=torch.bfloat16), torch.zeros(M, F, device=DEV, dtype=torch.bfloat16)
+            lib.gemm_skinny_wide(a, w, s1, lib.EPI_GATED); lib.gemm_skinny_wide(a, once, s2, lib.EPI_GATED)
+            assert torch.equal(s1, s2), M
+        if M <= 64:
+            s1, s2 = torch.zeros(M, F, device=DEV, dtype=torch.bfloat16), torch.zeros(M, F, device=DEV, dtype=torch.bfloat16)
+            lib.gemm_skinny(a, w, s1, lib.EPI_GATED); lib.gemm_skinny(a, once, s2, lib.EPI_GATED)
+            assert torch.equal(s1, s2), M
+    # a folded norm in front, on the kernel of few rows and on the kernel of whole lines
+    x = (rng.standard_normal((9, Kd)) * 2).astype(np.float32)
+    xg, ssq = times_weight(x, rounded(1 + 0.2 * rng.standard_normal(Kd), "bfloat16")).to(DEV), dev(ssq_partials(x, 3))
+    for whole in (False, True):
+        n1, n2 = torch.zeros(9, F, device=DEV, dtype=torch.bfloat16), torch.zeros(9, F, device=DEV, dtype=torch.bfloat16)
+        lib.gemm_skinny_norm(xg, ssq, 3, 1e-5, w, n1, lib.EPI_GATED, whole_lines=whole)
+        lib.gemm_skinny_norm(xg, ssq, 3, 1e-5, once, n2, lib.EPI_GATED, whole_lines=whole)
+        assert torch.equal(n1, n2), whole
+
+
 @pytest.mark.parametrize("pairing", ["adjacent", "half", None])
 @pytest.mark.parametrize("H, Kh, hs", [(32, 8, 64), (6, 2, 16), (5, 5, 48), (8, 1, 128)])
 def test_qkv_rope_cache_reads_a_weight_copy_in_operand_order(pairing, H, Kh, hs):
