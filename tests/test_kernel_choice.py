@@ -68,6 +68,37 @@ def test_which_weights_a_copy_can_stand_for():
     assert not lib.held_once(weight(64, 64, True, True))
 
 
+def test_which_stacked_gate_and_up_rows_stand_alone_in_operand_order():
+    """``ops.gated_alone``: the up strips must follow the gate strips (N a multiple of 16), K comes in whole steps
+    of 64, byte offsets of 32 bits reach all of it, and no fast path is switched off."""
+    import torch
+    from gpullama3_java_amd.parts import ops
+
+    class OnGpu:                       # what the rule looks at, without a GPU
+        is_cuda, dtype = True, torch.bfloat16
+
+        def __init__(self, rows, K):
+            self.shape = (rows, K)
+
+        def dim(self):
+            return 2
+
+        def is_contiguous(self):
+            return True
+
+        def numel(self):
+            return self.shape[0] * self.shape[1]
+
+    assert ops.gated_alone(OnGpu(2 * 8192, 2048)) and ops.gated_alone(OnGpu(2 * 14336, 4096))     # 1B, 8B layers
+    assert ops.gated_alone(OnGpu(2 * 48, 64))
+    assert not ops.gated_alone(OnGpu(2 * 40, 64))            # 40 gate rows: the up rows would begin inside a strip
+    assert not ops.gated_alone(OnGpu(2 * 48, 96))            # K in no whole steps of 64
+    assert not ops.gated_alone(OnGpu(2 * 8192, 2048), frozenset({"once"}))
+    assert not ops.gated_alone(OnGpu(2 * 65536, 16384))      # beyond 32-bit byte offsets
+    cpu = torch.zeros(96, 64, dtype=torch.bfloat16)
+    assert not ops.gated_alone(cpu)
+
+
 def test_strips_slices_and_pieces_of_the_products_of_few_rows():
     """The rules that decide a decode step's kernels, at the sizes they were measured at."""
     from gpullama3_java_amd.parts import ops
