@@ -60,6 +60,7 @@ def _declare(lib):
         "gl3_sample": [P, L, P, P, P, P, P, I, I, P, I, P],
         "gl3_sample_work_floats": [I, I],
         "gl3_argmax": [P, L, P, P, I, I, P],
+        "gl3_argmax_advance": [P, L, P, P, I, I, P, P, P, P, I, P, P],
         "gl3_argmax_static": [P, L, P, I, I, P],
         "gl3_decode_advance": [P, P, P, P, P, I, P, I, P],
         "gl3_gemm_skinny": [P, P, P, I, I, I, I, L, L, L, I, I, P, I, P, P, L, P, I, P, P, I, P],
@@ -386,6 +387,21 @@ def argmax(logits, work, out):
     if logits.stride(1) != 1 or work.numel() < 128 * R or out.numel() < R:
         raise KernelError("argmax: argument sizes")
     _check(library().gl3_argmax(_ptr(logits), logits.stride(0), _ptr(work), _ptr(out), R, V, _stream()), "argmax")
+
+
+def argmax_advance(logits, work, out, token_ids, positions, kv_before, history, step):
+    """``argmax`` into ``out`` and ``decode_advance`` with its result, in two launches instead of three."""
+    _dev(logits, "logits", torch.float32, contiguous=False); _dev(work, "work", torch.float32)
+    R, V = logits.shape
+    for t, name in ((out, "out"), (token_ids, "token_ids"), (positions, "positions"), (kv_before, "kv_before"),
+                    (history, "history"), (step, "step")):
+        _dev(t, name, torch.int32)
+    if (logits.stride(1) != 1 or work.numel() < 128 * R or out.numel() < R or token_ids.numel() != R
+            or positions.numel() != R or kv_before.numel() != R or history.dim() != 2 or history.shape[1] < R or R > 1024):
+        raise KernelError("argmax_advance: argument sizes")
+    _check(library().gl3_argmax_advance(_ptr(logits), logits.stride(0), _ptr(work), _ptr(out), R, V, _ptr(token_ids),
+                                        _ptr(positions), _ptr(kv_before), _ptr(history), history.stride(0), _ptr(step),
+                                        _stream()), "argmax_advance")
 
 
 def sample_work_size(rows, vocab):

@@ -588,6 +588,56 @@ extern "C" int gl3_argmax(const float* logits, long ld, float* work, int* out, i
   return 0;
 }
 
+// The greedy pick of a decode step inside a run, and what follows it between two steps of the run (as
+// gl3_decode_advance does): each row's winner is the sequence's next token, goes into row step[0] of `history`, the
+// sequence moves on by one position, and the step counter goes up. One block does the second stage for all rows
+// (a wave a row, in turn), so the counter is read by everyone before it changes: one launch instead of two.
+__global__ __launch_bounds__(1024) void argmax_final_advance_kernel(const float* __restrict__ part_val,
+                                                                    const int* __restrict__ part_idx, int* __restrict__ out,
+                                                                    int n_rows, int* __restrict__ token_ids,
+                                                                    int* __restrict__ positions, int* __restrict__ kv_before,
+                                                                    int* __restrict__ history, int history_stride,
+                                                                    int* __restrict__ step) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int s = step[0];
+  __syncthreads();
+  for (int row = wave; row < n_rows; row += 16) {
+    float best = part_val[row * ARG_SLICES + lane];
+    int idx = part_idx[row * ARG_SLICES + lane];
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(idx, o, 64);
+      if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
+    }
+    if (lane == 0) {
+      const int t = idx == 0x7fffffff ? 0 : idx;
+      out[row] = t;
+      token_ids[row] = t;
+      history[(long)s * history_stride + row] = t;
+      positions[row] += 1;
+      kv_before[row] += 1;
+    }
+  }
+  if (threadIdx.x == 0) step[0] = s + 1;
+}
+
+extern "C" int gl3_argmax_advance(const float* logits, long ld, float* work, int* out, int n_rows, int V, int* token_ids,
+                                  int* positions, int* kv_before, int* history, int history_stride, int* step,
+                                  hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  GL3_REQUIRE(logits && work && out && n_rows > 0 && V > 0 && ld >= V, "gl3_argmax_advance: bad arguments");
+  GL3_REQUIRE(token_ids && positions && kv_before && history && step && history_stride >= n_rows && n_rows <= 1024,
+              "gl3_argmax_advance: rows=%d stride=%d", n_rows, history_stride);
+  float* pv = work;
+  int* pi = (int*)(work + (long)n_rows * ARG_SLICES);
+  argmax_slice_kernel<<<dim3(n_rows, ARG_SLICES), dim3(256), 0, stream>>>(logits, ld, pv, pi, V);
+  GL3_LAUNCH_CHECK();
+  argmax_final_advance_kernel<<<dim3(1), dim3(1024), 0, stream>>>(pv, pi, out, n_rows, token_ids, positions, kv_before,
+                                                                  history, history_stride, step);
+  GL3_LAUNCH_CHECK();
+  return 0;
+}
+
 // The same without a workspace from the caller (see gl3_noalloc.h): the slices' partial results live
 // in a device array of this library. In host code `scratch` is only a handle for the runtime, not a
 // device address; the address on each GPU is asked for once, with that GPU current, and kept.

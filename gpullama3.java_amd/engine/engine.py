@@ -449,10 +449,9 @@ class Engine:
         def body():
             logits = self.model.forward(ctx, rows)
             if run == "greedy":
-                K.argmax(logits, work, sampled)
+                K.argmax_advance(logits, work, sampled, ctx.token_ids, ctx.positions, ctx.kv_before, hist, step)
             elif run:
                 K.sample(logits, work, temps, tops, us, sampled, step=step, uniform_stride=B_pad)
-            if run:
                 K.decode_advance(ctx.token_ids, ctx.positions, ctx.kv_before, sampled, hist, step)
             return logits
 

@@ -936,6 +936,35 @@ def test_argmax_kernel_takes_the_first_of_the_greatest(V):
     assert out.tolist() == [P.argmax(row) for row in logits]
 
 
+@pytest.mark.parametrize("R, V", [(1, 1000), (9, 63), (40, 128256), (64, 5000)])
+def test_greedy_pick_and_the_run_s_bookkeeping_in_one(R, V):
+    """``argmax_advance`` is ``argmax`` followed by ``decode_advance``: the winners (first of the greatest) become the
+    next tokens, go into the history row that the step counter names, every sequence moves on by one, the counter
+    goes up; more rows than the block has waves, two steps in a row."""
+    rng = np.random.default_rng(R + V)
+    lib = K()
+    work = torch.empty(128 * R, device=DEV)
+    tok = torch.full((R,), -1, dtype=torch.int32, device=DEV)
+    pos = dev(rng.integers(0, 500, R), torch.int32)
+    before = pos.clone()
+    pos0 = pos.cpu().numpy().copy()
+    hist = torch.full((4, R + 2), -3, dtype=torch.int32, device=DEV)
+    step = torch.tensor([1], dtype=torch.int32, device=DEV)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    for n in range(2):
+        logits = rng.standard_normal((R, V)).astype(np.float32)
+        logits[0, [V // 3, V - 1]] = 50.0                      # a tie: the lower index
+        if R > 2:
+            logits[2, :] = -np.inf                               # nothing greater than -inf: index 0
+        want = [P.argmax(row) for row in logits]
+        lib.argmax_advance(dev(logits), work, out, tok, pos, before, hist, step)
+        assert out.tolist() == want and tok.tolist() == want
+        assert hist[1 + n, :R].tolist() == want and torch.all(hist[1 + n, R:] == -3)
+        assert step.item() == 2 + n
+        assert np.array_equal(pos.cpu().numpy(), pos0 + n + 1) and torch.equal(before, pos)
+    assert torch.all(hist[0] == -3) and torch.all(hist[3] == -3)
+
+
 # ------------------------------------------------------------------ biases and the other activation in the products' epilogues
 def gelu_tanh(v):
     return 0.5 * v * (1 + np.tanh(math.sqrt(2 / math.pi) * (v + 0.044715 * v ** 3)))
