@@ -678,11 +678,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_pack_kernel(const bf16_t*
 }
 
 // The resident kernel: K <= 32 * NW * KS. `n_strips` strips are shared out over the blocks.
-template <int MT, int NW, int KS, int EPI, typename TC, bool XNORM, bool SSQ>
+template <int MT, int NW, int KS, int EPI, typename TC, bool XNORM, bool SSQ, int WO>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
     const void* __restrict__ Av, const bf16_t* __restrict__ W, TC* __restrict__ C, int M, int N, int K, long lda,
     long ldw, long ldc, SkNorm nrm, float* __restrict__ ssq_out, SkNext nx, SkRope rp, int n_strips,
-    const bf16_t* __restrict__ Wt) {
+    const bf16_t* __restrict__ Wt_) {
+  // WO 1: W comes as the copy in the operands' order (Wt_); 0: as stored rows; 2: whichever Wt_ says, at run time.
+  // (A template parameter: decided at run time, every load of every strip takes a branch, 250 to 400 of the kernel's
+  // 800 to 1,070 instructions. Sixteen waves with eight k-steps each have no register to spare, and without those
+  // branches the compiler asks for everything at once and spills: they keep the run-time form.)
+  const bool WT = WO == 2 ? Wt_ != nullptr : WO == 1;
+  const bf16_t* const Wt = WT ? Wt_ : nullptr;
   constexpr int NG = (EPI == SK_GATED) ? 2 : 1;
   __shared__ f32x4 red[NW][NG * MT][64];
   __shared__ float sm_ssq[XNORM ? NW : 1][64];
@@ -708,12 +714,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
   // consecutive memory, which the CU's first-level cache takes in less than half the time. Either way the
   // strip lies behind a descriptor that starts at its first row (see sk_rsrc).
   const int steps_all = (K + 31) / 32;
-  const unsigned w_step = Wt ? 1024u : 64u;                // bytes from one k-step to the next
+  const unsigned w_step = WT ? 1024u : 64u;                // bytes from one k-step to the next
   const long tile = (long)steps_all * 512;                 // elements of a strip of the copy
   struct Strip { __amdgpu_buffer_rsrc_t w, u; unsigned lane_at; };
   auto strip_at = [&](int strip_) {
     Strip t;
-    if (Wt) {   // (the same for the whole grid)
+    if (WT) {
       t.w = sk_rsrc(Wt + strip_ * tile, tile * 2);
       t.u = sk_rsrc(Wt + ((long)(N / 16) + strip_) * tile, tile * 2);
       t.lane_at = (unsigned)lane * 16u;
@@ -730,7 +736,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_resident_kernel(
     return t;
   };
   auto step_at = [&](const Strip& t, int st) {   // the offset of this lane's 16 bytes of k-step st
-    return (Wt ? st < steps_all : st * 32 + q * 8 < K) ? t.lane_at + (unsigned)st * w_step : SK_NOWHERE;
+    return (WT ? st < steps_all : st * 32 + q * 8 < K) ? t.lane_at + (unsigned)st * w_step : SK_NOWHERE;
   };
   int strip = blockIdx.x;
   Strip cur = strip_at(strip);
@@ -1233,10 +1239,21 @@ static int launch_skinny(int nw, const SkCall& a) {
   const int steps = (a.K + 31) / 32;
 #define RES(NW, KS)                                                                                               \
   do {                                                                                                            \
-    gemm_skinny_resident_kernel<MT, NW, KS, EPI, TC, XNORM, SSQ>                                                  \
-        <<<dim3(resident_blocks(n_strips, NW)), dim3(NW * 64), 0, a.stream>>>(                                    \
-            a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp, n_strips, \
-            (const bf16_t*)a.Wt);                                                                                 \
+    if constexpr (NW == 16 && KS >= 8)                                                                            \
+      gemm_skinny_resident_kernel<MT, NW, KS, EPI, TC, XNORM, SSQ, 2>                                             \
+          <<<dim3(resident_blocks(n_strips, NW)), dim3(NW * 64), 0, a.stream>>>(                                  \
+              a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp, n_strips, \
+              (const bf16_t*)a.Wt);                                                                               \
+    else if (a.Wt)                                                                                                \
+      gemm_skinny_resident_kernel<MT, NW, KS, EPI, TC, XNORM, SSQ, 1>                                             \
+          <<<dim3(resident_blocks(n_strips, NW)), dim3(NW * 64), 0, a.stream>>>(                                  \
+              a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp, n_strips, \
+              (const bf16_t*)a.Wt);                                                                               \
+    else                                                                                                          \
+      gemm_skinny_resident_kernel<MT, NW, KS, EPI, TC, XNORM, SSQ, 0>                                             \
+          <<<dim3(resident_blocks(n_strips, NW)), dim3(NW * 64), 0, a.stream>>>(                                  \
+              a.A, (const bf16_t*)a.W, (TC*)a.C, a.M, a.N, a.K, a.lda, a.ldw, a.ldc, a.nrm, a.ssq_out, a.nx, a.rp, n_strips, \
+              (const bf16_t*)nullptr);                                                                            \
     GL3_LAUNCH_CHECK();                                                                                           \
     return 0;                                                                                                     \
   } while (0)
