@@ -50,24 +50,30 @@ extern "C" int gl3_ad_stamps(long long* out) {
 #define AD_STAMP(i) do {} while (0)
 #endif
 
-template <int HS, int NW, int CB>
+// P2: a page holds a power of two of positions (page_size == 1 << page_shift): a chunk's page and its place in it are
+// a shift and a mask. A division by a number only known at run time is some forty scalar instructions, and the
+// kernel has eight of them in front of its first loads.
+template <int HS, int NW, int CB, bool P2>
 __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
     int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out,
-    long out_stride, int n_heads, int n_kv, int page_size, int window, float scale, int n_splits) {
+    long out_stride, int n_heads, int n_kv, int g, int page_size, int page_shift, int window, float scale, int n_splits) {
   constexpr int KK = HS / 32;   // k-steps of the first product
   constexpr int DT = HS / 16;   // row tiles of the second product
   constexpr int NS = (HS > 64 && NW > 4) ? NW / 2 : NW;   // partial results that shared memory holds at a time
   __shared__ float sm_m[NS][16], sm_l[NS][16];
   __shared__ f32x4 sm_o[NS][DT][64];
   AD_STAMP(0); AD_STAMP(1);
-  const int g = n_heads / n_kv;
+  // the grid: (kv head and group of 16 query heads, split, token)
+  // (g = n_heads / n_kv comes from the host: the division would stand in front of everything else)
   const int groups = (g + 15) / 16;
-  const int t = blockIdx.x / (n_kv * groups);
-  const int c = (blockIdx.x / groups) % n_kv;
-  const int hg = blockIdx.x % groups;
+  const int t = blockIdx.z;
+  const int c = groups == 1 ? (int)blockIdx.x : (int)blockIdx.x / groups;
+  const int hg = groups == 1 ? 0 : (int)blockIdx.x % groups;
   const int split = blockIdx.y;
+  auto page_of = [&](int key) { return P2 ? key >> page_shift : key / page_size; };
+  auto in_page = [&](int key) { return P2 ? key & (page_size - 1) : key % page_size; };
   // the wave's number as a scalar: what depends on it alone (chunk, page) then lives in scalar
   // registers and its table look-ups are scalar loads, not a trip to memory per lane
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -83,11 +89,11 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
   int first_pages[CB];
 #pragma unroll
   for (int b = 0; b < CB; ++b)
-    first_pages[b] = __builtin_amdgcn_readfirstlane(bt[min(((wave + b * NW) * 32) / page_size, table_stride - 1)]);
+    first_pages[b] = __builtin_amdgcn_readfirstlane(bt[min(page_of((wave + b * NW) * 32), table_stride - 1)]);
   const int kv_len = __builtin_amdgcn_readfirstlane(positions[t]) + 1;
   const int lo = (window > 0 && kv_len > window) ? kv_len - window : 0;
   const int chunk_lo = lo / 32, chunk_hi = (kv_len + 31) / 32;
-  const int per_split = (chunk_hi - chunk_lo + n_splits - 1) / n_splits;
+  const int per_split = n_splits == 1 ? chunk_hi - chunk_lo : (chunk_hi - chunk_lo + n_splits - 1) / n_splits;
   const int c_begin = chunk_lo + split * per_split;
   const int c_end = min(chunk_hi, c_begin + per_split);
   AD_STAMP(2);
@@ -113,8 +119,8 @@ __global__ __launch_bounds__(NW * 64) void attention_decode_kernel(
       if (ck < c_end) {
         const int key0 = ck * 32;
         // (the first chunks from the sequence's start: their pages are here already)
-        const long page = (c_begin == 0 && ck0 == wave) ? first_pages[b] : __builtin_amdgcn_readfirstlane(bt[key0 / page_size]);
-        const int po = key0 % page_size;
+        const long page = (c_begin == 0 && ck0 == wave) ? first_pages[b] : __builtin_amdgcn_readfirstlane(bt[page_of(key0)]);
+        const int po = in_page(key0);
         // the chunk's two key tiles lie one after the other, 16 * HS elements each; a k-step's operand
         // is 512 consecutive elements of a tile in lane order (gl3_k_offset)
         const bf16_t* kb = k_cache + ((page * n_kv + c) * page_size + po) * HS + lane * 8;
@@ -317,24 +323,26 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
                 "gl3_attention_decode: workspace of %ld floats is too small", part_floats);
   const int groups = (n_heads / n_kv + 15) / 16;
   const long blocks = (long)n_tokens * n_kv * groups;
-  GL3_REQUIRE(blocks < (1L << 31), "gl3_attention_decode: too many blocks");
-  dim3 grid((unsigned)blocks, n_splits);
+  GL3_REQUIRE((long)n_kv * groups < (1L << 31) && n_tokens <= 65535, "gl3_attention_decode: too many blocks (%d tokens)", n_tokens);
+  dim3 grid((unsigned)(n_kv * groups), n_splits, n_tokens);
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  const bool p2 = (1 << page_shift) == page_size;
   // 8 waves; as many chunks on their way per wave as the registers hold (two waves share a SIMD's registers).
   // More blocks than CUs: 4 waves, so that a CU holds two blocks and the second 256 blocks do not wait for the
   // first to end (what a block does before its keys arrive is a chain of trips to memory, paid once per round).
   const bool small = blocks * n_splits > 256;
+#define AD_ARGS                                                                                                       \
+  (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token, block_table,    \
+      table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, n_heads / n_kv, page_size, page_shift, window,  \
+      scale, n_splits
 #define GO(HS)                                                                                                        \
   do {                                                                                                                \
-    if (small)                                                                                                        \
-      attention_decode_kernel<HS, 4, (HS <= 64 ? 4 : HS <= 96 ? 3 : 2)><<<grid, dim3(256), 0, stream>>>(                \
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token,         \
-          block_table, table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, \
-          n_splits);                                                                                                  \
-    else                                                                                                              \
-      attention_decode_kernel<HS, 8, (HS <= 64 ? 4 : HS <= 96 ? 3 : 2)><<<grid, dim3(512), 0, stream>>>(                \
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, seq_of_token,         \
-          block_table, table_stride, part_o, part_ml, (bf16_t*)out, out_stride, n_heads, n_kv, page_size, window, scale, \
-          n_splits);                                                                                                  \
+    constexpr int CB = HS <= 64 ? 4 : HS <= 96 ? 3 : 2;                                                               \
+    if (small && p2) attention_decode_kernel<HS, 4, CB, true><<<grid, dim3(256), 0, stream>>>(AD_ARGS);                \
+    else if (small) attention_decode_kernel<HS, 4, CB, false><<<grid, dim3(256), 0, stream>>>(AD_ARGS);                \
+    else if (p2) attention_decode_kernel<HS, 8, CB, true><<<grid, dim3(512), 0, stream>>>(AD_ARGS);                    \
+    else attention_decode_kernel<HS, 8, CB, false><<<grid, dim3(512), 0, stream>>>(AD_ARGS);                           \
   } while (0)
   switch (head_dim) {
     case 32: GO(32); break;
@@ -343,6 +351,7 @@ extern "C" int gl3_attention_decode(const void* q, long q_stride, const void* k_
     default: GO(128); break;
   }
 #undef GO
+#undef AD_ARGS
   GL3_LAUNCH_CHECK();
   if (n_splits > 1) {
     attention_decode_merge_kernel<<<dim3((unsigned)((long)n_tokens * n_heads)), dim3(64), 0, stream>>>(
