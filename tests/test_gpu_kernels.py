@@ -495,6 +495,10 @@ def test_attention_decode(H, Kh, hs, splits):
     sk, sv, qs = attention_case(rng, H, Kh, hs, lens_before, new, "bfloat16")
     got, ref = run_attention(decode_fn(splits), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng)
     np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max())
+    # pages of 32 positions (a chunk a page) and of 96 (no power of two: a chunk's page by division)
+    for page in (32, 96):
+        got, ref = run_attention(decode_fn(splits), sk, sv, qs, lens_before, new, H, Kh, hs, "bfloat16", rng, page=page)
+        np.testing.assert_allclose(got, ref, atol=1e-2 * np.abs(ref).max(), err_msg=f"pages of {page}")
 
 
 @pytest.mark.parametrize("hs", [96, 128])
