@@ -1307,8 +1307,10 @@ static int launch_skinny(int nw, const SkCall& a) {
     if constexpr (NG * MT == 1 && EPI != SK_QKV && !XNORM) {
       if (steps <= 64 && n_strips >= 2048) RES(4, 16);
     }
-    // 16 waves a strip where their partial tiles fit, so that a strip's rows are asked for at once
-    if constexpr (NG * MT <= 2) {
+    // 16 waves a strip where their partial tiles fit, so that a strip's rows are asked for at once; with three and
+    // four token tiles only for the plain store (the head of 33 to 64 rows: 122.5 -> 115.5 us at 64), whose registers
+    // hold them; a folded norm, the sums of squares or the rotation's operands beside them spill
+    if constexpr (NG * MT <= 2 || (EPI == SK_STORE && !XNORM && !SSQ && MT <= 4)) {
       if (steps <= 64) RES(16, 4);
     }
     // (more token tiles, the gated epilogue or the rotation's operands would not fit the registers with
