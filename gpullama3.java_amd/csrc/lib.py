@@ -912,7 +912,7 @@ def mfma_plan(M, N, K):
     """(tile shape, slices of K) for the tiled product [M, K] x [N, K] into the residual stream, whose
     slices the norm that follows adds up. Few tiles: tiles of 128 x 128 and ``mfma_slices``. More tiles
     than places: the plan with the least estimated time among tiles of 128 (512 places) or 256 (256
-    places) and one to four slices, the estimate being (rounds the blocks need on their places) x
+    places) with one to four slices and tiles of 128 rows x 256 (256 places) with one, the estimate being (rounds the blocks need on their places) x
     (steps of 64 columns a block walks) x (time of such a step with the chip full: 1.05 us and 1.7 us)
     + what the norm pays per slice (0.35 us per MB). What decides is the last, partly empty round:
     276 tiles of 256 take two rounds for the work of 1.08, and two slices of them 2.16 of 3. Fitted to
@@ -922,11 +922,15 @@ def mfma_plan(M, N, K):
     if -(-M // 128) * -(-N // 128) <= 256:
         return 1, mfma_slices(M, N, K)
     best = None
-    for shape, tile, places, step_us in ((1, 128, 512, 1.05), (2, 256, 256, 1.7)):
-        for slices in (1, 2, 3, 4):
+    # (tile rows, tile columns, places on the chip, time of a step of 64 columns with the chip full); the tile of 128
+    # rows x 256, one block a CU, whole K only: 0.95 us a step. It is the plan where its tiles are one round and the
+    # others need two rounds or slices: the output projection of 2,048 rows of the 3B layers 81 -> 68 us with its norm,
+    # of the 8B layers 110 -> 97 us, of 5,886 rows 307 -> 280 us, of 4,096 rows of the 1B layers 64 -> 60 us.
+    for shape, rows, cols, places, step_us in ((1, 128, 128, 512, 1.05), (2, 256, 256, 256, 1.7), (5, 128, 256, 256, 0.95)):
+        for slices in ((1,) if shape == 5 else (1, 2, 3, 4)):
             if slices > 1 and K // slices < 512:
                 continue
-            blocks = -(-M // tile) * -(-N // tile) * slices
+            blocks = -(-M // rows) * -(-N // cols) * slices
             estimate = -(-blocks // places) * -(-K // (64 * slices)) * step_us + 0.35e-6 * (slices + 1.5) * M * N * 4
             if best is None or estimate < best[0]:
                 best = (estimate, shape, slices)

@@ -22,7 +22,15 @@ def test_many_tiles_take_the_plan_with_the_fewest_idle_places():
     for M in range(300, 9000, 431):
         for N, K in ((2048, 8192), (3072, 3072), (4096, 14336), (1000, 520), (3072, 272), (6144, 8)):
             shape, slices = lib.mfma_plan(M, N, K)
-            assert shape in (1, 2) and 1 <= slices <= 8 and (slices == 1 or K // slices >= 512)
+            assert shape in (1, 2, 5) and 1 <= slices <= 8 and (slices == 1 or K // slices >= 512)
+            assert shape != 5 or slices == 1
+    # tiles of 128 rows x 256 where they are one round and the others need two rounds or slices (the output projection
+    # of 2,048 rows of the 3B and 8B layers: 81 -> 68 and 110 -> 97 us with the norm; 4,096 rows of the 1B layers 64 -> 60)
+    assert lib.mfma_plan(2048, 3072, 3072) == (5, 1) and lib.mfma_plan(2048, 4096, 4096) == (5, 1)
+    assert lib.mfma_plan(4096, 2048, 2048) == (5, 1) and lib.mfma_plan(5886, 4096, 4096) == (5, 1)
+    # ... and not where the large tiles are one round themselves or K is long
+    assert lib.mfma_plan(8192, 2048, 2048) == (2, 1) and lib.mfma_plan(4096, 4096, 4096) == (2, 1)
+    assert lib.mfma_plan(2048, 4096, 14336) == (2, 2) and lib.mfma_plan(3072, 3072, 3072)[0] == 2
 
 
 def test_decode_attention_splits_the_keys_until_every_cu_has_a_block():
