@@ -880,16 +880,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
   const unsigned s_at = ((unsigned)wave + (unsigned)q * NW) * 256u + (unsigned)a_row * 4u;   // partial wave + NW (4 i + q) of the row (they are stored by row of A)
 #pragma unroll
   for (int i = 0; i < SK_SQN(NW); ++i) sq[i] = sk_ld_f32(s_buf, s_at + (unsigned)i * (NW * 1024u));
-  // DEEP (the plain store: the head, whose blocks walk over some thirty strips each): two strips are on their way
-  // while one is worked on. With one ahead a CU has 64 KB in flight, which is what it gets in the 2.9 us a strip
-  // takes (5.9 TB/s for the chip).
-  constexpr bool DEEP = EPI == SK_STORE && KS <= 6;   // (eight k-steps a wave: the registers do not hold a third set)
-  bf16x8 wn[KS];
-  if (DEEP && strip + (int)gridDim.x < n_strips) {
-    const __amdgpu_buffer_rsrc_t w_buf = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Wt + (long)(strip + (int)gridDim.x) * tile_bytes), 0, (int)tile_bytes, 0x00020000);
-#pragma unroll
-    for (int i = 0; i < KS; ++i) wn[i] = sk_ld_b128(w_buf, w_at + (unsigned)i * (NW * 1024u));
-  }
   __builtin_amdgcn_sched_barrier(0);   // all of that is on its way before anything else is computed
   SK_STAMP(2);
   bool first_strip = true;
@@ -902,12 +892,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
       pre = sk_preload<MT, EPI, TC>(C, M, N, ldc, strip, hd, sub, rotated, rp, nx, tok);
     }
     const int next = strip + gridDim.x;
-    const int ask = DEEP ? next + (int)gridDim.x : next;   // the strip whose rows are asked for now
-    bf16x8 wl[KS], un[KS];
-    if (ask < n_strips) {   // (the same for the block; what is loaded here is used after the strip's end)
-      const __amdgpu_buffer_rsrc_t w_buf = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Wt + (long)ask * tile_bytes), 0, (int)tile_bytes, 0x00020000);
+    bf16x8 wn[KS], un[KS];
+    if (next < n_strips) {   // (the same for the block; what is loaded here is used after the strip's end)
+      const __amdgpu_buffer_rsrc_t w_buf = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Wt + (long)next * tile_bytes), 0, (int)tile_bytes, 0x00020000);
 #pragma unroll
-      for (int i = 0; i < KS; ++i) wl[i] = sk_ld_b128(w_buf, w_at + (unsigned)i * (NW * 1024u));
+      for (int i = 0; i < KS; ++i) wn[i] = sk_ld_b128(w_buf, w_at + (unsigned)i * (NW * 1024u));
       if (EPI == SK_GATED) {
         const __amdgpu_buffer_rsrc_t u_buf = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Wt + (long)(up_strips + next) * tile_bytes), 0, (int)tile_bytes, 0x00020000);
 #pragma unroll
@@ -954,8 +943,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_decode_kernel(
     __syncthreads();   // the partial tiles in shared memory are free again
 #pragma unroll
     for (int i = 0; i < KS; ++i) {
-      wf[i] = DEEP ? wn[i] : wl[i];
-      if (DEEP) wn[i] = wl[i];
+      wf[i] = wn[i];
       if (EPI == SK_GATED) uf[i] = un[i];
     }
     strip = next;
